@@ -1,0 +1,80 @@
+/*
+ * megalodon_hip.h -- C ABI of libmegalodon_hip.so (gfx950 / MI355X).
+ *
+ * Drop-in boundary for the fused-op hot path of XuezheMax/megalodon.  Each
+ * entry point replaces one function of the reference's pybind module
+ * `megalodon_extension.ops` (registered in megalodon/csrc/megalodon_extension.cc:14-24).
+ *
+ * Conventions (all entry points):
+ *   - every pointer is a DEVICE pointer to contiguous memory unless stated;
+ *   - the caller owns and allocates inputs AND outputs (the reference's
+ *     callee-allocates `torch::empty` moves to the Python wrapper);
+ *   - `stream` is a hipStream_t passed as void*; kernels are enqueued on it and
+ *     the call returns without synchronising (the reference enqueues on the
+ *     current CUDA stream the same way, e.g. ema_parameters_kernel.cu:1033);
+ *   - return value 0 = MEGA_OK; otherwise an error code, with a message kept
+ *     in a thread-local buffer readable through mega_last_error() (the
+ *     reference raises c10::Error through TORCH_CHECK);
+ *   - complex tensors are interleaved (re, im) float pairs = torch.complex64;
+ *   - no entry point allocates device memory except where a `workspace`
+ *     argument is documented.
+ */
+#ifndef MEGALODON_HIP_H_
+#define MEGALODON_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MEGA_OK 0
+#define MEGA_ERR_INVALID_ARG 1
+#define MEGA_ERR_UNSUPPORTED 2
+#define MEGA_ERR_HIP 3
+
+/* element types of activation tensors (x, y, dy, dx, q, k, v ...) */
+#define MEGA_F32 0
+#define MEGA_BF16 1
+#define MEGA_F16 2
+
+/* Library version (major*10000 + minor*100 + patch). */
+int mega_version(void);
+
+/* Message of the last error raised on the calling thread ("" if none). */
+const char* mega_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * CEMA convolution-kernel generation (weight path).
+ *
+ * Replaces ema_parameters_fwd(p, log_q, gamma, h=None, L) -> (w, None, None)
+ *   reference: megalodon/csrc/ops/ema_parameters.cc:17-52 (CPU),
+ *              ema_parameters_kernel.cu:74-121 (CUDA), binding ema_parameters.cc:289.
+ *   w[d, j] = sum_n Re(p[d,n] * gamma[d,n] * exp(log_q[d,n] * j)),  j = 0..L-1
+ *   p      (D, N)  float32
+ *   log_q  (D, N)  complex64
+ *   gamma  (D, N)  complex64
+ *   w      (D, L)  float32 (output)
+ *   1 <= N <= 32 (reference limit, ema_parameters_kernel.cu:1026).
+ * ---------------------------------------------------------------------- */
+int mega_ema_weight_fwd(const float* p, const float* log_q, const float* gamma,
+                        int64_t D, int64_t N, int64_t L, float* w,
+                        void* stream);
+
+/* Replaces ema_parameters_bwd(dw, None, p, log_q, gamma, None, None)
+ *   -> (dp, dq, dgamma, None)
+ *   reference: ema_parameters.cc:80-98,141-156 (CPU),
+ *              ema_parameters_kernel.cu:396-472 (CUDA), binding ema_parameters.cc:290.
+ *   S1 = sum_j dw[j] * j * q^(j-1),  S2 = sum_j dw[j] * q^j
+ *   dp = Re(S2 * gamma), dq = conj(S1 * p * gamma), dgamma = conj(S2 * p)
+ *   (gradients w.r.t. q, not log q; PyTorch conjugate convention)
+ *   dw (D, L) float32; dp (D, N) float32; dq, dgamma (D, N) complex64. */
+int mega_ema_weight_bwd(const float* dw, const float* p, const float* log_q,
+                        const float* gamma, int64_t D, int64_t N, int64_t L,
+                        float* dp, float* dq, float* dgamma, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MEGALODON_HIP_H_ */

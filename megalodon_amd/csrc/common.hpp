@@ -1,0 +1,100 @@
+// Shared host/device helpers for the gfx950 kernels of libmegalodon_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/megalodon_hip.h"
+
+namespace mega {
+
+constexpr int kWave = 64;  // gfx950 wavefront width
+
+// ---- error reporting --------------------------------------------------
+char* last_error_buf();  // thread-local, 512 bytes
+int set_error(int code, const char* fmt, ...);
+
+#define MEGA_CHECK_ARG(cond, ...)                                  \
+  do {                                                             \
+    if (!(cond)) return mega::set_error(MEGA_ERR_INVALID_ARG, __VA_ARGS__); \
+  } while (0)
+
+#define MEGA_CHECK_HIP(expr)                                               \
+  do {                                                                     \
+    hipError_t e_ = (expr);                                                \
+    if (e_ != hipSuccess)                                                  \
+      return mega::set_error(MEGA_ERR_HIP, "%s failed: %s", #expr,         \
+                             hipGetErrorString(e_));                       \
+  } while (0)
+
+#define MEGA_CHECK_LAUNCH() MEGA_CHECK_HIP(hipGetLastError())
+
+// ---- 16-bit element conversion (bit-level, round-to-nearest-even) -------
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t v) {
+  return __uint_as_float(static_cast<uint32_t>(v) << 16);
+}
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);  // NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+__device__ __forceinline__ float f16_bits_to_float(uint16_t v) {
+  return __half2float(__ushort_as_half(v));
+}
+__device__ __forceinline__ uint16_t float_to_f16_bits(float f) {
+  return __half_as_ushort(__float2half_rn(f));
+}
+
+// Element traits: storage type + conversion to/from float.
+template <int DT> struct Elem;
+template <> struct Elem<MEGA_F32> {
+  using type = float;
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <> struct Elem<MEGA_BF16> {
+  using type = uint16_t;
+  static __device__ __forceinline__ float load(const uint16_t* p) { return bf16_bits_to_float(*p); }
+  static __device__ __forceinline__ void store(uint16_t* p, float v) { *p = float_to_bf16_bits(v); }
+};
+template <> struct Elem<MEGA_F16> {
+  using type = uint16_t;
+  static __device__ __forceinline__ float load(const uint16_t* p) { return f16_bits_to_float(*p); }
+  static __device__ __forceinline__ void store(uint16_t* p, float v) { *p = float_to_f16_bits(v); }
+};
+
+inline int elem_size(int dt) { return dt == MEGA_F32 ? 4 : 2; }
+inline bool valid_dtype(int dt) { return dt == MEGA_F32 || dt == MEGA_BF16 || dt == MEGA_F16; }
+
+// ---- complex helpers ------------------------------------------------------
+struct cf {
+  float x, y;
+};
+__device__ __forceinline__ cf cmul(cf a, cf b) {
+  return {a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x};
+}
+__device__ __forceinline__ cf cmulc(cf a, cf b) {  // a * conj(b)
+  return {a.x * b.x + a.y * b.y, a.y * b.x - a.x * b.y};
+}
+__device__ __forceinline__ cf cadd(cf a, cf b) { return {a.x + b.x, a.y + b.y}; }
+__device__ __forceinline__ cf csub(cf a, cf b) { return {a.x - b.x, a.y - b.y}; }
+
+// ---- wave64 reductions ------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+}  // namespace mega

@@ -1,0 +1,299 @@
+// CEMA convolution-kernel generation for gfx950: w[d,j] = sum_n Re(c_n q_n^j)
+// and its backward reductions.
+//
+// Follows the math of the reference weight path
+//   megalodon/csrc/ops/ema_parameters.cc:17-52 (forward), :80-98 (backward)
+// with a different evaluation scheme: every power q^j is factored as
+// q^(T*h) * q^lo with both factors taken from small per-channel tables whose
+// entries are evaluated directly (phase reduced in float64 "turns", so the
+// angle j*arg(q) never loses bits for j up to 2^31), instead of the
+// reference's repeated multiplication (ema_parameters_kernel.cu:115-117) or
+// fp32 exp(log_q*j) (ema_parameters.cc:45-46).
+//
+// Forward: one workgroup per (channel, 64-tile slab).  Each lane keeps the 4
+// (or 2) consecutive low powers q^lo of all N modes in registers, reads the
+// per-tile factor c*q^(T*h) from LDS (wave-uniform broadcast) and emits one
+// float4 (float2) per tile: 2 FMA per (element, mode), one coalesced store.
+//
+// Backward: same factorisation turned into per-lane partial sums
+//   A[lo] = sum_h dw[h,lo] q^(T h),  B[lo] = sum_h j dw[h,lo] q^(T h)
+// followed by one multiplication with q^lo and a workgroup reduction.
+#include "common.hpp"
+
+namespace mega {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kSlab = 64;  // tiles handled per table fill
+
+// q^j for log q = (a, phi), evaluated directly.
+__device__ __forceinline__ cf qpow(float a, float phi, int64_t j) {
+  if (j == 0) return {1.0f, 0.0f};
+  const double jj = static_cast<double>(j);
+  const double turns = static_cast<double>(phi) * 0.15915494309189535 * jj;
+  const double fr = turns - rint(turns);  // in [-0.5, 0.5]
+  float s, c;
+  sincospif(2.0f * static_cast<float>(fr), &s, &c);
+  const float mag = static_cast<float>(exp(static_cast<double>(a) * jj));
+  return {mag * c, mag * s};
+}
+
+template <int NMAX, int PT>
+struct LowTables {
+  cf p1[NMAX][64];  // q^b, b < 64
+  cf p2[NMAX][(kThreads * PT) / 64];  // q^(64 a)
+};
+
+template <int NMAX, int PT>
+__device__ __forceinline__ void fill_low_tables(LowTables<NMAX, PT>& t, const cf* lq, int N) {
+  constexpr int kA = (kThreads * PT) / 64;
+  for (int i = threadIdx.x; i < NMAX * 64; i += kThreads) {
+    const int n = i >> 6, b = i & 63;
+    t.p1[n][b] = n < N ? qpow(lq[n].x, lq[n].y, b) : cf{0.f, 0.f};
+  }
+  for (int i = threadIdx.x; i < NMAX * kA; i += kThreads) {
+    const int n = i / kA, a = i % kA;
+    t.p2[n][a] = n < N ? qpow(lq[n].x, lq[n].y, 64 * a) : cf{0.f, 0.f};
+  }
+}
+
+// ------------------------------ forward ------------------------------------
+template <int NMAX, int PT, bool VEC>
+__global__ __launch_bounds__(kThreads) void ema_weight_fwd_kernel(
+    const float* __restrict__ p, const cf* __restrict__ log_q,
+    const cf* __restrict__ gamma, int N, int64_t L, float* __restrict__ w) {
+  constexpr int kTile = kThreads * PT;
+  __shared__ LowTables<NMAX, PT> low;
+  __shared__ cf hi[kSlab][NMAX];  // c_n * q_n^(kTile * h)
+
+  const int64_t d = blockIdx.x;
+  const int64_t h0 = static_cast<int64_t>(blockIdx.y) * kSlab;
+  const int64_t n_tiles = (L + kTile - 1) / kTile;
+  const int nh = static_cast<int>(min<int64_t>(kSlab, n_tiles - h0));
+  const cf* lq = log_q + d * N;
+
+  fill_low_tables<NMAX, PT>(low, lq, N);
+  for (int i = threadIdx.x; i < nh * NMAX; i += kThreads) {
+    const int h = i / NMAX, n = i % NMAX;
+    cf v{0.f, 0.f};
+    if (n < N) {
+      const cf g = gamma[d * N + n];
+      const float pp = p[d * N + n];
+      v = cmul(cf{pp * g.x, pp * g.y}, qpow(lq[n].x, lq[n].y, (h0 + h) * kTile));
+    }
+    hi[h][n] = v;
+  }
+  __syncthreads();
+
+  float qx[PT][NMAX], qny[PT][NMAX];  // Re(q^lo), -Im(q^lo)
+#pragma unroll
+  for (int r = 0; r < PT; ++r) {
+    const int lo = threadIdx.x * PT + r;
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n) {
+      const cf v = cmul(low.p2[n][lo >> 6], low.p1[n][lo & 63]);
+      qx[r][n] = v.x;
+      qny[r][n] = -v.y;
+    }
+  }
+
+  float* wrow = w + d * L;
+  for (int h = 0; h < nh; ++h) {
+    float acc[PT];
+#pragma unroll
+    for (int r = 0; r < PT; ++r) acc[r] = 0.f;
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n) {
+      const cf t = hi[h][n];
+#pragma unroll
+      for (int r = 0; r < PT; ++r) {
+        acc[r] = fmaf(t.x, qx[r][n], acc[r]);
+        acc[r] = fmaf(t.y, qny[r][n], acc[r]);
+      }
+    }
+    const int64_t j0 = (h0 + h) * kTile + static_cast<int64_t>(threadIdx.x) * PT;
+    if (VEC && j0 + PT <= L) {
+      if constexpr (PT == 4) {
+        *reinterpret_cast<float4*>(wrow + j0) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      } else {
+        *reinterpret_cast<float2*>(wrow + j0) = make_float2(acc[0], acc[1]);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < PT; ++r)
+        if (j0 + r < L) wrow[j0 + r] = acc[r];
+    }
+  }
+}
+
+// ------------------------------ backward -----------------------------------
+template <int NMAX, int PT, bool VEC>
+__global__ __launch_bounds__(kThreads) void ema_weight_bwd_kernel(
+    const float* __restrict__ dw, const float* __restrict__ p,
+    const cf* __restrict__ log_q, const cf* __restrict__ gamma, int N,
+    int64_t L, float* __restrict__ dp, cf* __restrict__ dq,
+    cf* __restrict__ dgamma) {
+  constexpr int kTile = kThreads * PT;
+  __shared__ LowTables<NMAX, PT> low;
+  __shared__ cf hi[kSlab][NMAX];                // q_n^(kTile * h)
+  __shared__ float red[kThreads / kWave][4 * NMAX];
+
+  const int64_t d = blockIdx.x;
+  const cf* lq = log_q + d * N;
+  const float* drow = dw + d * L;
+  const int64_t n_tiles = (L + kTile - 1) / kTile;
+
+  fill_low_tables<NMAX, PT>(low, lq, N);
+
+  float ax[PT][NMAX], ay[PT][NMAX], bx[PT][NMAX], by[PT][NMAX];
+#pragma unroll
+  for (int r = 0; r < PT; ++r)
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n) ax[r][n] = ay[r][n] = bx[r][n] = by[r][n] = 0.f;
+
+  for (int64_t h0 = 0; h0 < n_tiles; h0 += kSlab) {
+    const int nh = static_cast<int>(min<int64_t>(kSlab, n_tiles - h0));
+    __syncthreads();  // previous slab fully consumed (also orders the low-table fill)
+    for (int i = threadIdx.x; i < nh * NMAX; i += kThreads) {
+      const int h = i / NMAX, n = i % NMAX;
+      hi[h][n] = n < N ? qpow(lq[n].x, lq[n].y, (h0 + h) * kTile) : cf{0.f, 0.f};
+    }
+    __syncthreads();
+    for (int h = 0; h < nh; ++h) {
+      const int64_t j0 = (h0 + h) * kTile + static_cast<int64_t>(threadIdx.x) * PT;
+      float g[PT];
+      if (VEC && PT == 2 && j0 + PT <= L) {
+        const float2 v = *reinterpret_cast<const float2*>(drow + j0);
+        g[0] = v.x;
+        g[PT - 1] = v.y;
+      } else {
+#pragma unroll
+        for (int r = 0; r < PT; ++r) g[r] = j0 + r < L ? drow[j0 + r] : 0.f;
+      }
+      float gj[PT];
+#pragma unroll
+      for (int r = 0; r < PT; ++r) gj[r] = g[r] * static_cast<float>(j0 + r);
+#pragma unroll
+      for (int n = 0; n < NMAX; ++n) {
+        const cf t = hi[h][n];
+#pragma unroll
+        for (int r = 0; r < PT; ++r) {
+          ax[r][n] = fmaf(g[r], t.x, ax[r][n]);
+          ay[r][n] = fmaf(g[r], t.y, ay[r][n]);
+          bx[r][n] = fmaf(gj[r], t.x, bx[r][n]);
+          by[r][n] = fmaf(gj[r], t.y, by[r][n]);
+        }
+      }
+    }
+  }
+
+  // fold in q^lo, then reduce over the workgroup
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+#pragma unroll
+  for (int n = 0; n < NMAX; ++n) {
+    cf s2{0.f, 0.f}, s1{0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < PT; ++r) {
+      const int lo = threadIdx.x * PT + r;
+      const cf ql = cmul(low.p2[n][lo >> 6], low.p1[n][lo & 63]);
+      s2 = cadd(s2, cmul(ql, cf{ax[r][n], ay[r][n]}));
+      s1 = cadd(s1, cmul(ql, cf{bx[r][n], by[r][n]}));
+    }
+    const float v0 = wave_sum(s2.x), v1 = wave_sum(s2.y);
+    const float v2 = wave_sum(s1.x), v3 = wave_sum(s1.y);
+    if (lane == 0) {
+      red[wave][4 * n + 0] = v0;
+      red[wave][4 * n + 1] = v1;
+      red[wave][4 * n + 2] = v2;
+      red[wave][4 * n + 3] = v3;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < N) {
+    const int n = threadIdx.x;
+    cf s2{0.f, 0.f}, s1q{0.f, 0.f};
+#pragma unroll
+    for (int wv = 0; wv < kThreads / kWave; ++wv) {
+      s2.x += red[wv][4 * n + 0];
+      s2.y += red[wv][4 * n + 1];
+      s1q.x += red[wv][4 * n + 2];
+      s1q.y += red[wv][4 * n + 3];
+    }
+    // S1 = sum_j j dw_j q^(j-1) = (sum_j j dw_j q^j) / q
+    const cf s1 = cmul(s1q, qpow(lq[n].x, lq[n].y, -1));
+    const cf g = gamma[d * N + n];
+    const float pp = p[d * N + n];
+    dp[d * N + n] = s2.x * g.x - s2.y * g.y;
+    const cf t = cmul(s1, cf{pp * g.x, pp * g.y});
+    dq[d * N + n] = cf{t.x, -t.y};
+    dgamma[d * N + n] = cf{s2.x * pp, -s2.y * pp};
+  }
+}
+
+}  // namespace
+}  // namespace mega
+
+using namespace mega;
+
+extern "C" int mega_ema_weight_fwd(const float* p, const float* log_q,
+                                   const float* gamma, int64_t D, int64_t N,
+                                   int64_t L, float* w, void* stream) {
+  MEGA_CHECK_ARG(p && log_q && gamma && w, "mega_ema_weight_fwd: null pointer");
+  MEGA_CHECK_ARG(D >= 0 && L >= 0, "mega_ema_weight_fwd: negative size");
+  MEGA_CHECK_ARG(N >= 1 && N <= 32, "mega_ema_weight_fwd: N=%lld outside [1,32]", (long long)N);
+  MEGA_CHECK_ARG(D <= 0x7fffffff, "mega_ema_weight_fwd: D too large");
+  if (D == 0 || L == 0) return MEGA_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const cf* lq = reinterpret_cast<const cf*>(log_q);
+  const cf* gm = reinterpret_cast<const cf*>(gamma);
+  const bool vec = (L % 4 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0);
+  if (N <= 16) {
+    constexpr int kTile = kThreads * 4;
+    const int64_t tiles = (L + kTile - 1) / kTile;
+    dim3 grid(static_cast<unsigned>(D), static_cast<unsigned>((tiles + kSlab - 1) / kSlab));
+    if (vec)
+      ema_weight_fwd_kernel<16, 4, true><<<grid, kThreads, 0, s>>>(p, lq, gm, (int)N, L, w);
+    else
+      ema_weight_fwd_kernel<16, 4, false><<<grid, kThreads, 0, s>>>(p, lq, gm, (int)N, L, w);
+  } else {
+    constexpr int kTile = kThreads * 2;
+    const int64_t tiles = (L + kTile - 1) / kTile;
+    dim3 grid(static_cast<unsigned>(D), static_cast<unsigned>((tiles + kSlab - 1) / kSlab));
+    if (vec)
+      ema_weight_fwd_kernel<32, 2, true><<<grid, kThreads, 0, s>>>(p, lq, gm, (int)N, L, w);
+    else
+      ema_weight_fwd_kernel<32, 2, false><<<grid, kThreads, 0, s>>>(p, lq, gm, (int)N, L, w);
+  }
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
+}
+
+extern "C" int mega_ema_weight_bwd(const float* dw, const float* p,
+                                   const float* log_q, const float* gamma,
+                                   int64_t D, int64_t N, int64_t L, float* dp,
+                                   float* dq, float* dgamma, void* stream) {
+  MEGA_CHECK_ARG(dw && p && log_q && gamma && dp && dq && dgamma,
+                 "mega_ema_weight_bwd: null pointer");
+  MEGA_CHECK_ARG(D >= 0 && L >= 0, "mega_ema_weight_bwd: negative size");
+  MEGA_CHECK_ARG(N >= 1 && N <= 32, "mega_ema_weight_bwd: N=%lld outside [1,32]", (long long)N);
+  MEGA_CHECK_ARG(D <= 0x7fffffff, "mega_ema_weight_bwd: D too large");
+  MEGA_CHECK_ARG(L <= 0x7fffffff, "mega_ema_weight_bwd: L too large");
+  if (D == 0) return MEGA_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const cf* lq = reinterpret_cast<const cf*>(log_q);
+  const cf* gm = reinterpret_cast<const cf*>(gamma);
+  cf* dqc = reinterpret_cast<cf*>(dq);
+  cf* dgc = reinterpret_cast<cf*>(dgamma);
+  const bool vec = (L % 2 == 0) && (reinterpret_cast<uintptr_t>(dw) % 8 == 0);
+  dim3 grid(static_cast<unsigned>(D));
+  if (N <= 16) {
+    if (vec)
+      ema_weight_bwd_kernel<16, 2, true><<<grid, kThreads, 0, s>>>(dw, p, lq, gm, (int)N, L, dp, dqc, dgc);
+    else
+      ema_weight_bwd_kernel<16, 2, false><<<grid, kThreads, 0, s>>>(dw, p, lq, gm, (int)N, L, dp, dqc, dgc);
+  } else {
+    ema_weight_bwd_kernel<32, 1, false><<<grid, kThreads, 0, s>>>(dw, p, lq, gm, (int)N, L, dp, dqc, dgc);
+  }
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
+}

@@ -1,0 +1,102 @@
+"""Python face of the C ABI with the reference's operator signatures.
+
+Each function here has the name, argument order, returned tuple and error
+behaviour of one function of the reference's pybind module
+``megalodon_extension.ops`` (megalodon/csrc/megalodon_extension.cc:14-24) and
+forwards to the matching ``mega_*`` entry point of ``libmegalodon_hip.so``.
+Outputs are allocated here with ``torch.empty`` on the inputs' device (the
+reference allocates them inside the C++ op); kernels run on the current
+stream; nothing synchronises.  Non-CUDA tensors raise ``RuntimeError``: there
+is no CPU path in this package.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+
+def _require_cuda(*tensors) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("megalodon_amd ops need GPU (HIP) tensors; there is no CPU fallback")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError("all tensors must be on the same device")
+    return dev
+
+
+def _as_c64(t: torch.Tensor, name: str) -> torch.Tensor:
+    if t.dtype != torch.complex64:
+        raise RuntimeError(f"{name} must be complex64 (got {t.dtype})")
+    return t.contiguous()
+
+
+# --------------------------------------------------------------------------
+# ema_parameters (reference: csrc/ops/ema_parameters.cc:195-290)
+# --------------------------------------------------------------------------
+def ema_parameters_fwd(
+    p: torch.Tensor,
+    log_q: torch.Tensor,
+    gamma: torch.Tensor,
+    h: Optional[torch.Tensor],
+    L: int,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """(w, b, v) = ema_parameters_fwd(p, log_q, gamma, h, L); weight path only.
+
+    p (D,N[,1]) float32, log_q/gamma complex64 -> w (D, L) float32.  With
+    ``h`` given the reference also returns the bias of the carried state
+    (ema_parameters.cc:56-77); that branch is not part of this library yet.
+    """
+    dev = _require_cuda(p, log_q, gamma, h)
+    if h is not None:
+        raise NotImplementedError("ema_parameters with a carried state (h) is not implemented")
+    if p.dtype != torch.float32:
+        raise RuntimeError(f"p must be float32 (got {p.dtype})")
+    D, N = p.shape[0], p.shape[1]
+    p_c = p.contiguous()
+    lq = _as_c64(log_q, "log_q")
+    gm = _as_c64(gamma, "gamma")
+    w = torch.empty((D, L), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_ema_weight_fwd", _lib.ptr(p_c), _lib.ptr(lq), _lib.ptr(gm),
+                  _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(w), _lib.stream_ptr(dev))
+    return w, None, None
+
+
+def ema_parameters_bwd(
+    w_grad: torch.Tensor,
+    b_grad: Optional[torch.Tensor],
+    p: torch.Tensor,
+    log_q: torch.Tensor,
+    gamma: torch.Tensor,
+    h: Optional[torch.Tensor],
+    v: Optional[torch.Tensor],
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """(dp, dq, dgamma, dh); gradients w.r.t. q (not log q), PyTorch conjugate
+    convention (ema_parameters.cc:80-98)."""
+    dev = _require_cuda(w_grad, p, log_q, gamma, h, b_grad)
+    if h is not None or b_grad is not None:
+        raise NotImplementedError("ema_parameters with a carried state (h) is not implemented")
+    if p.dtype != torch.float32 or w_grad.dtype != torch.float32:
+        raise RuntimeError("p and w_grad must be float32")
+    D, N = p.shape[0], p.shape[1]
+    L = w_grad.shape[-1]
+    dw = w_grad.contiguous()
+    p_c = p.contiguous()
+    lq = _as_c64(log_q, "log_q")
+    gm = _as_c64(gamma, "gamma")
+    dp = torch.empty_like(p_c)
+    dq = torch.empty_like(lq)
+    dg = torch.empty_like(gm)
+    with torch.cuda.device(dev):
+        _lib.call("mega_ema_weight_bwd", _lib.ptr(dw), _lib.ptr(p_c), _lib.ptr(lq), _lib.ptr(gm),
+                  _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg),
+                  _lib.stream_ptr(dev))
+    return dp, dq, dg, None

@@ -1,0 +1,29 @@
+"""The C-ABI library loads and exports every symbol the public header declares
+(no compute calls: runs without a GPU)."""
+import ctypes
+
+from megalodon_amd import _lib
+
+
+def test_library_loads_and_reports_version():
+    lib = _lib.load()
+    assert lib.mega_version() >= 100
+    assert lib.mega_last_error() == b"" or isinstance(lib.mega_last_error(), bytes)
+
+
+def test_every_declared_symbol_is_exported():
+    lib = _lib.load()
+    names = _lib.declared_symbols()
+    assert "mega_ema_weight_fwd" in names and "mega_version" in names
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, f"declared in include/megalodon_hip.h but not exported: {missing}"
+
+
+def test_invalid_argument_is_reported_not_raised_in_c():
+    lib = _lib.load()
+    fn = lib.mega_ema_weight_fwd
+    fn.restype = ctypes.c_int
+    null = ctypes.c_void_p(0)
+    code = fn(null, null, null, ctypes.c_int64(1), ctypes.c_int64(16), ctypes.c_int64(8), null, null)
+    assert code == 1
+    assert b"null" in lib.mega_last_error()
