@@ -25,8 +25,8 @@ def pytest_collection_modifyitems(config, items):
 def rel_err(a, b):
     """max|a-b| / max|b| with float64 accumulation (the parity metric)."""
     import torch
-    a = a.detach().double().cpu() if not a.is_complex() else torch.view_as_real(a.detach().cpu()).double()
-    b = b.detach().double().cpu() if not b.is_complex() else torch.view_as_real(b.detach().cpu()).double()
+    a = a.detach().double().cpu() if not a.is_complex() else torch.view_as_real(a.detach().cpu().resolve_conj()).double()
+    b = b.detach().double().cpu() if not b.is_complex() else torch.view_as_real(b.detach().cpu().resolve_conj()).double()
     denom = b.abs().max().item()
     if denom == 0.0:
         return (a - b).abs().max().item()
