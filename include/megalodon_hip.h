@@ -73,6 +73,39 @@ int mega_ema_weight_bwd(const float* dw, const float* p, const float* log_q,
                         const float* gamma, int64_t D, int64_t N, int64_t L,
                         float* dp, float* dq, float* dgamma, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Causal FFT convolution.
+ *
+ * Replaces fftconv_fwd(x, k_f) -> (y, x_f) and the torch.fft branch used for
+ * L > 16384, i.e. `_fftconv_fwd` / `fused_fftconv_fwd`
+ *   reference: megalodon/modules/fused_ops/fftconv.py:30-50,79-93,
+ *              megalodon/csrc/ops/fftconv_kernel.cu:34-78,480-501, binding fftconv.cc:22-33.
+ *   y[b,d,t] = sum_{s<=t} k[d,t-s] x[b,d,s]
+ *            = irfft(rfft(x, 2N) * rfft(k, 2N))[:L],  N = 2^ceil(log2 L)
+ *   x, y (B, D, L) of `dtype` (MEGA_F32 / MEGA_BF16 / MEGA_F16);
+ *   k (D, L) float32 in the TIME domain (the reference passes rfft(k); here
+ *   the transform of k happens inside the kernel and nothing is saved).
+ *   Arithmetic is float32 throughout; y is rounded once on store.
+ *   L <= mega_fftconv_max_length() (32768); longer rows return
+ *   MEGA_ERR_UNSUPPORTED.
+ *   The first call for a transform size on a device allocates the twiddle
+ *   tables and a per-workgroup scratch (kept until process exit) and
+ *   synchronises `stream` once.
+ * ---------------------------------------------------------------------- */
+int mega_fftconv_max_length(void);
+int mega_fftconv_fwd(const void* x, int dtype, const float* k, int64_t B,
+                     int64_t D, int64_t L, void* y, void* stream);
+
+/* Replaces fftconv_bwd(dy, x_f, k_f, k_dtype) -> (dx, dk) / `_fftconv_bwd`
+ *   reference: fftconv.py:53-75,96-106, fftconv_kernel.cu:80-164,503-520.
+ *   dx[b,d,t] = sum_{s>=t} dy[b,d,s] k[d,s-t]
+ *   dk[d,j]   = sum_b sum_{t>=j} dy[b,d,t] x[b,d,t-j]
+ *   Takes x and k themselves (the spectra are recomputed, not saved).
+ *   dy, x, dx (B, D, L) of `dtype`; k, dk (D, L) float32. */
+int mega_fftconv_bwd(const void* dy, const void* x, int dtype, const float* k,
+                     int64_t B, int64_t D, int64_t L, void* dx, float* dk,
+                     void* stream);
+
 #ifdef __cplusplus
 }
 #endif

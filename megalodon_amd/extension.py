@@ -100,3 +100,48 @@ def ema_parameters_bwd(
                   _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg),
                   _lib.stream_ptr(dev))
     return dp, dq, dg, None
+
+
+# --------------------------------------------------------------------------
+# fftconv (reference: csrc/ops/fftconv.cc:22-33, fused_ops/fftconv.py:30-106)
+# --------------------------------------------------------------------------
+def fftconv_max_length() -> int:
+    return int(_lib.load().mega_fftconv_max_length())
+
+
+def fftconv_fwd(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
+    """y = causal_conv(x, k).  x (B, D, L) float32/bfloat16/float16, k (D, L).
+
+    Differs from the reference's ``fftconv_fwd(x, k_f) -> (y, x_f)`` in taking
+    the time-domain kernel and returning no saved spectrum: backward recomputes
+    it (1 GiB of ``x_f`` is not kept alive between forward and backward)."""
+    dev = _require_cuda(x, k)
+    if x.dim() != 3 or k.dim() != 2 or k.shape[0] != x.shape[1] or k.shape[1] != x.shape[2]:
+        raise RuntimeError(f"fftconv: x {tuple(x.shape)} and k {tuple(k.shape)} do not match (B,D,L)/(D,L)")
+    B, D, L = x.shape
+    xc = x.contiguous()
+    kc = k.contiguous().float()
+    y = torch.empty_like(xc)
+    with torch.cuda.device(dev):
+        _lib.call("mega_fftconv_fwd", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)), _lib.ptr(kc),
+                  _lib.i64(B), _lib.i64(D), _lib.i64(L), _lib.ptr(y), _lib.stream_ptr(dev))
+    return y
+
+
+def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
+                k_dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(dx, dk) with dk of dtype ``k_dtype`` (fftconv.py:53-75)."""
+    dev = _require_cuda(y_grad, x, k)
+    B, D, L = x.shape
+    if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
+        raise RuntimeError("fftconv_bwd: y_grad must match x in shape and dtype")
+    dy = y_grad.contiguous()
+    xc = x.contiguous()
+    kc = k.contiguous().float()
+    dx = torch.empty_like(xc)
+    dk = torch.empty((D, L), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_fftconv_bwd", _lib.ptr(dy), _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
+                  _lib.ptr(kc), _lib.i64(B), _lib.i64(D), _lib.i64(L), _lib.ptr(dx), _lib.ptr(dk),
+                  _lib.stream_ptr(dev))
+    return dx, dk.to(k_dtype)

@@ -1,0 +1,122 @@
+"""Parity of the HIP causal FFT convolution with the float64 oracle.
+Tolerances: rel err (max|a-b|/max|b|) <= 1e-4 for float32 rows, <= 2e-2 for
+bfloat16 / float16 rows (forward values and both gradients)."""
+import pytest
+import torch
+
+from conftest import rel_err
+from megalodon_amd import extension as ops
+from megalodon_amd import synthetic
+from megalodon_amd.fused_ops import ema_parameters, fftconv as fftconv_op
+from oracle import cema, fftconv
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+SHAPES = [
+    (1, 3, 1), (2, 3, 31), (2, 5, 50), (1, 4, 2048), (2, 3, 1000),     # direct (time-domain) kernel
+    (1, 3, 2049), (2, 2, 4096), (1, 3, 4097), (2, 2, 6001),            # M = 2048, 4096
+    (1, 3, 8192), (1, 2, 8193), (2, 2, 16384), (1, 2, 12345),          # M = 4096, 8192
+    (1, 3, 16385), (2, 3, 32768), (1, 2, 32767), (1, 2, 20001),        # M = 16384 (even and odd L)
+]
+
+
+def _data(B, D, L, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, D, L, generator=g).to(dtype)
+    k = torch.randn(D, L, generator=g) * (0.97 ** torch.arange(L, dtype=torch.float32))
+    dy = torch.randn(B, D, L, generator=g).to(dtype)
+    return x, k, dy
+
+
+@pytest.mark.parametrize("B,D,L", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fwd_matches_oracle(B, D, L, dtype):
+    x, k, _ = _data(B, D, L, dtype, 31 * L + B)
+    y = ops.fftconv_fwd(x.cuda(), k.cuda())
+    assert y.dtype == dtype and y.shape == x.shape
+    want = fftconv.fftconv_fwd(x, k)
+    assert rel_err(y, want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("B,D,L", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_bwd_matches_oracle(B, D, L, dtype):
+    x, k, dy = _data(B, D, L, dtype, 17 * L + B)
+    dx, dk = ops.fftconv_bwd(dy.cuda(), x.cuda(), k.cuda(), torch.float32)
+    assert dx.dtype == dtype and dk.dtype == torch.float32 and dk.shape == k.shape
+    wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
+    assert rel_err(dx, wdx) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= TOL[dtype]
+
+
+def test_float16_rows():
+    x, k, dy = _data(2, 3, 5000, torch.float16, 5)
+    y = ops.fftconv_fwd(x.cuda(), k.cuda())
+    assert rel_err(y, fftconv.fftconv_fwd(x, k)) <= TOL[torch.float16]
+
+
+def test_config0_cema_forward_fp32():
+    """BASELINE config 0: CEMA forward fp32, B=1, L=2048, D=1024, ndim=16."""
+    D, N, L = 1024, 16, 2048
+    prm = synthetic.cema_params(D, N, 1000)
+    x = synthetic.cema_inputs(1, D, L, 1000)["x"]
+    k, _ = ema_parameters(prm["p"].cuda(), prm["q"].cuda(), prm["gamma"].cuda(), None, L)
+    out = fftconv_op(x.cuda(), k) + x.cuda() * prm["omega"].cuda()
+    kk = cema.ema_weight_fwd(prm["p"], prm["q"].log(), prm["gamma"], L)
+    want = fftconv.fftconv_fwd(x, kk) + x.double() * prm["omega"].double()
+    assert rel_err(out, want) <= 1e-4
+
+
+def test_config1_rows_bf16_fwd_bwd_with_ema_kernel():
+    """BASELINE config 1 row shape (L=32768, ndim=16, x bf16), a slice of the channels."""
+    D, N, L = 48, 16, 32768
+    prm = synthetic.cema_params(D, N, 1001)
+    io = synthetic.cema_inputs(1, D, L, 1001, torch.bfloat16)
+    kk = cema.ema_weight_fwd(prm["p"], prm["q"].log(), prm["gamma"], L)
+    k = kk.float()
+    y = ops.fftconv_fwd(io["x"].cuda(), k.cuda())
+    assert rel_err(y, fftconv.fftconv_fwd(io["x"], k)) <= 2e-2
+    dx, dk = ops.fftconv_bwd(io["dy"].cuda(), io["x"].cuda(), k.cuda(), torch.float32)
+    wdx, wdk = fftconv.fftconv_bwd(io["dy"], io["x"], k)
+    assert rel_err(dx, wdx) <= 2e-2
+    assert rel_err(dk, wdk) <= 2e-2
+
+
+def test_full_size_linearity_and_shift_properties():
+    """Size-independent checks at the full benchmark shape of one launch:
+    linearity in x and the unit-impulse identity conv(x, delta) = x."""
+    B, D, L = 1, 512, 32768
+    g = torch.Generator().manual_seed(77)
+    x1 = torch.randn(B, D, L, generator=g).cuda()
+    x2 = torch.randn(B, D, L, generator=g).cuda()
+    k = (torch.randn(D, L, generator=g) * (0.999 ** torch.arange(L, dtype=torch.float32))).cuda()
+    y1 = ops.fftconv_fwd(x1, k)
+    y2 = ops.fftconv_fwd(x2, k)
+    y12 = ops.fftconv_fwd(x1 + 2.0 * x2, k)
+    assert rel_err(y12, y1 + 2.0 * y2) <= 1e-4
+    delta = torch.zeros(D, L, device="cuda")
+    delta[:, 0] = 1.0
+    assert rel_err(ops.fftconv_fwd(x1, delta), x1) <= 1e-5
+    shift = torch.zeros(D, L, device="cuda")
+    shift[:, 5] = 1.0
+    ys = ops.fftconv_fwd(x1, shift)
+    assert rel_err(ys[..., 5:], x1[..., :-5]) <= 1e-5 and ys[..., :5].abs().max().item() <= 1e-4
+
+
+def test_autograd_function():
+    B, D, L = 2, 4, 3000
+    x, k, dy = _data(B, D, L, torch.float32, 9)
+    xc = x.cuda().requires_grad_(True)
+    kc = k.cuda().requires_grad_(True)
+    y = fftconv_op(xc, kc)
+    y.backward(dy.cuda())
+    wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
+    assert rel_err(xc.grad, wdx) <= 1e-4 and rel_err(kc.grad, wdk) <= 1e-4
+
+
+def test_too_long_rows_fail_loudly():
+    x = torch.zeros(1, 1, 32769, device="cuda")
+    k = torch.zeros(1, 32769, device="cuda")
+    with pytest.raises(RuntimeError, match="exceeds"):
+        ops.fftconv_fwd(x, k)
