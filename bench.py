@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Benchmark of the Megalodon fused-op hot path on one MI355X.
+
+A step is one CEMA layer forward+backward at the 7B layer width (BASELINE
+config 1): k = ema_parameters(p, q, gamma) -> y = fftconv(x, k) + x*omega, then
+backward through both ops to dx, d(alpha, delta, theta, gamma, omega), with
+B=1, L=32768, D=4096, ndim=16, x and the upstream gradient in bf16, arithmetic
+in fp32.  Inputs are synthetic, seeded, and resident in HBM before the timed
+region.  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+
+def cpu_baseline(B, D, N, L, seed, budget_s=25.0):
+    """The same step on the host cores through the reference's CPU formulation:
+    ema_parameters by the C/OpenMP restatement of its C++ loop nest, the
+    convolution by torch.fft on CPU tensors (which is the reference's CPU
+    path), on a bounded slice of the channels (every loop nest is linear in D).
+    """
+    import torch
+    from megalodon_amd import synthetic
+    from oracle import native, fftconv as offt
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16) if os.environ.get("OMP_NUM_THREADS") is None else int(os.environ["OMP_NUM_THREADS"])
+    torch.set_num_threads(cores)
+    os.environ.setdefault("OMP_NUM_THREADS", str(cores))
+    lib = native.port()
+    Ds = 64
+    prm = synthetic.cema_params(D, N, seed)
+    io = synthetic.cema_inputs(B, Ds, L, seed, torch.bfloat16)
+    p, lq, g = prm["p"][:Ds], prm["q"][:Ds].log(), prm["gamma"][:Ds]
+    om = prm["omega"][:Ds]
+
+    def step():
+        k = native.ema_weight_fwd(lib, "oracle_", p, lq, g, L)
+        x = io["x"].float()
+        L_ = x.shape[-1]
+        n = 2 * (L_ if (L_ & (L_ - 1)) == 0 else (1 << L_.bit_length()))
+        x_f = torch.fft.rfft(x, n=n)
+        k_f = torch.fft.rfft(k, n=n, norm="forward")
+        y = torch.fft.irfft(x_f * k_f, n=n, norm="forward")[..., :L_].to(torch.bfloat16)
+        out = y + io["x"] * om
+        dy = io["dy"].float()
+        dy_f = torch.fft.rfft(dy.flip(dims=(-1,)), n=n)
+        dx = torch.fft.irfft(dy_f * k_f, n=n, norm="forward")[..., :L_].flip(dims=(-1,)).to(torch.bfloat16)
+        dk = torch.fft.irfft((dy_f * x_f).sum(dim=0), n=n)[..., :L_].flip(dims=(-1,))
+        dx = dx + io["dy"] * om
+        dom = (io["dy"].float() * x).sum(dim=(0, 2))
+        grads = native.ema_weight_bwd(lib, "oracle_", dk, p, lq, g)
+        return out, dx, dom, grads
+
+    t0 = time.perf_counter()
+    step()
+    one = time.perf_counter() - t0
+    reps = max(1, min(5, int(budget_s / max(one, 1e-3)) - 1))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        step()
+    dt = (time.perf_counter() - t0) / reps
+    tokens_per_s = B * L / (dt * D / Ds)
+    return {
+        "value": tokens_per_s, "unit": "tokens/s", "cores": cores, "kind": "port",
+        "sample": f"{Ds} of {D} channels, {reps} rep(s) of the full fwd+bwd step at L={L}, "
+                  f"{dt:.3f} s each, scaled by D/{Ds}",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every op shards "
+              "without communication along channels / batch / heads); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from megalodon_amd import _lib, synthetic
+    from megalodon_amd.modules import MultiHeadComplexEMA
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    _lib.load()  # fails loudly when the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, D, N, L, seed = 1, 4096, 16, 32768, 1001
+
+    layer = MultiHeadComplexEMA(D, N).to(dev)
+    layer.train()
+    io = synthetic.cema_inputs(B, D, L, seed, torch.bfloat16)
+    x = io["x"].to(dev).requires_grad_(True)
+    dy = io["dy"].to(dev)
+
+    def step():
+        x.grad = None
+        for prm in layer.parameters():
+            prm.grad = None
+        out, _ = layer(x, None, False)
+        out.backward(dy.to(out.dtype))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    log = {"mega_fftconv_fwd": [], "mega_fftconv_bwd": [], "mega_ema_weight_fwd": [], "mega_ema_weight_bwd": []}
+    _lib.set_event_log(log)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    _lib.set_event_log(None)
+
+    def avg_ms(name):
+        ev = log[name]
+        return sum(a.elapsed_time(b) for a, b in ev) / max(1, len(ev))
+
+    E = B * D * L
+    ms_step = dt / args.steps * 1e3
+    conv_ms = avg_ms("mega_fftconv_fwd")  # one launch of the convolution kernel
+    conv_bytes = 8 * E  # x 2E + k 4E in, y 2E out (bf16 rows, fp32 kernel)
+    achieved = conv_bytes / (conv_ms * 1e-3) / 1e9
+    kernels = {
+        "fftconv_fwd_ms": conv_ms,
+        "fftconv_bwd_ms": avg_ms("mega_fftconv_bwd"),
+        "ema_weight_fwd_ms": avg_ms("mega_ema_weight_fwd"),
+        "ema_weight_bwd_ms": avg_ms("mega_ema_weight_bwd"),
+    }
+    kernels["fftconv_bwd_GBps"] = 16 * E / (kernels["fftconv_bwd_ms"] * 1e-3) / 1e9
+    kernels["ema_weight_fwd_GBps"] = 4 * E / (kernels["ema_weight_fwd_ms"] * 1e-3) / 1e9
+    kernels["ema_weight_bwd_GBps"] = 4 * E / (kernels["ema_weight_bwd_ms"] * 1e-3) / 1e9
+
+    result = {
+        "metric": "Megalodon layer fwd+bwd tokens/s at L=32K, 1 GPU; CEMA+FFT-conv HBM GB/s (% peak)",
+        "value": B * L / (dt / args.steps),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: CEMA + causal FFT convolution forward+backward, "
+                               "B=1 L=32768 D=4096 ndim=16, x/dy bf16, fp32 arithmetic",
+                   "global_batch": B, "seq_len": L},
+        "roofline": {
+            "bound": "hbm", "kernel": "fftconv_kernel<LOGM=14, bf16, MODE=0> (one launch = forward conv of all rows)",
+            "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+        },
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(B, D, N, L, seed)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -80,7 +80,30 @@ def stream_ptr(device=None) -> ctypes.c_void_p:
     return _c_ptr(torch.cuda.current_stream(device).cuda_stream)
 
 
+# Optional per-entry-point device timing: when a dict is installed with
+# ``set_event_log``, every call of an entry point named in it is bracketed by
+# events recorded on the current stream (the stream the kernels are enqueued
+# on); the (start, end) pairs are appended to the list under that name.
+_event_log = None
+
+
+def set_event_log(log) -> None:
+    global _event_log
+    _event_log = log
+
+
 def call(name: str, *args) -> None:
     fn = getattr(load(), name)
     fn.restype = ctypes.c_int
+    log = _event_log
+    if log is not None and name in log:
+        import torch
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        code = fn(*args)
+        e1.record()
+        log[name].append((e0, e1))
+        check(code, name)
+        return
     check(fn(*args), name)

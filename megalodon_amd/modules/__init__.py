@@ -1,0 +1,4 @@
+"""Modules with the reference's names (megalodon/modules/__init__.py:1-15) for the hot path."""
+from .complex_exponential_moving_average import MultiHeadComplexEMA
+
+__all__ = ["MultiHeadComplexEMA"]

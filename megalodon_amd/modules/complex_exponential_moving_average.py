@@ -1,0 +1,100 @@
+"""`MultiHeadComplexEMA` with the reference's constructor, parameters and forward
+(megalodon/modules/complex_exponential_moving_average.py:42-150), minus the
+`megalodon.distributed` look-ups: model-parallel world size is 1, so
+``dim_per_partition == embed_dim`` and the theta permutation is drawn locally
+instead of being broadcast (:21-26)."""
+from typing import Optional, Tuple
+import math
+
+import torch
+from torch import nn
+
+from ..fused_ops import ema_parameters, fftconv
+
+_r2c = torch.view_as_complex
+
+
+def _reset_parameters(alpha, delta, theta, gamma, omega, embed_dim):
+    # delta & alpha
+    nn.init.normal_(alpha, mean=0.0, std=0.2)
+    nn.init.normal_(delta, mean=0.0, std=0.2)
+    idx = torch.randperm(embed_dim)
+    # theta: logit of permuted log-spaced frequencies exp(-i ln(D)/D), i = 1..D
+    freqs = math.log(embed_dim) / embed_dim
+    freqs = torch.exp(torch.arange(1, embed_dim + 1) * -freqs)
+    freqs = freqs[idx].to(theta).view(embed_dim, 1, 1)
+    freqs = torch.log(freqs / (1.0 - freqs))
+    with torch.no_grad():
+        theta.copy_(freqs)
+    # gamma (imaginary part zero at init), omega
+    nn.init.normal_(gamma, mean=0.0, std=1.0)
+    with torch.no_grad():
+        gamma[:, :, 1] = 0.
+    nn.init.trunc_normal_(omega, mean=0.0, std=0.25, a=-1.0, b=1.0)
+
+
+class MultiHeadComplexEMA(nn.Module):
+    """Complex Exponential Moving Average layer."""
+
+    def __init__(self, embed_dim, ndim=16):
+        super().__init__()
+        self.embed_dim = embed_dim
+        self.ndim = ndim
+        self.scale = math.sqrt(1.0 / self.ndim)
+        self.dim_per_partition = embed_dim
+
+        self.alpha = nn.Parameter(torch.Tensor(self.dim_per_partition, ndim, 1))
+        self.delta = nn.Parameter(torch.Tensor(self.dim_per_partition, ndim, 1))
+        self.theta = nn.Parameter(torch.Tensor(self.dim_per_partition, 1, 1))
+        self.gamma = nn.Parameter(torch.Tensor(self.dim_per_partition, ndim, 2))
+        self.omega = nn.Parameter(torch.Tensor(self.dim_per_partition, 1))
+        self._coeffs = None
+        self._init_parameters()
+
+    def _init_parameters(self):
+        _reset_parameters(self.alpha, self.delta, self.theta, self.gamma, self.omega, self.embed_dim)
+
+    def _calc_coeffs(self):
+        self._coeffs = None
+        # D x 1 x 1
+        theta = torch.sigmoid(self.theta.float()) * (2 * math.pi / self.ndim)
+        # 1 x N
+        wavelets = torch.arange(1, self.ndim + 1, dtype=theta.dtype, device=theta.device).view(1, self.ndim)
+        # D x N x 1
+        theta = wavelets.unsqueeze(2) * theta
+        alpha = torch.sigmoid(self.alpha.float())
+        delta = torch.sigmoid(self.delta.float())
+        p = alpha
+        q = torch.polar(1.0 - alpha * delta, theta)
+        # D x N
+        gamma = _r2c(self.gamma.float()) * self.scale
+        return p, q, gamma
+
+    def coeffs(self):
+        if self.training:
+            return self._calc_coeffs()
+        if self._coeffs is None:
+            self._coeffs = self._calc_coeffs()
+        return self._coeffs
+
+    def forward(
+        self,
+        x: torch.Tensor,
+        hx: Optional[torch.Tensor] = None,
+        compute_last_state: bool = False,
+    ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        # B x D x L
+        if hx is not None or compute_last_state:
+            raise NotImplementedError(
+                "carried EMA state (hx / compute_last_state) is outside the single-sequence training path")
+        bsz, _, seq_len = x.size()
+        residual = x * self.omega
+
+        p, q, gamma = self.coeffs()
+        k, b = ema_parameters(p, q, gamma, hx, seq_len)
+        output = fftconv(x, k)
+        output = output + residual
+        return output, None
+
+    def extra_repr(self) -> str:
+        return 'edim={} ({}), ndim={}'.format(self.embed_dim, self.dim_per_partition, self.ndim)

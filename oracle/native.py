@@ -1,0 +1,124 @@
+"""ctypes access to the compiled CPU checkers (TEST INFRASTRUCTURE ONLY).
+
+``port()``  -> oracle/liboracle_cpu.so, the C/OpenMP restatement (oracle/cpu_ref.c)
+``ref()``   -> oracle/_ref/libmegalodon_ref_cpu.so, the reference's own C++ CPU
+               operators compiled from /root/reference (None when not built)
+Both take and return float32 torch CPU tensors.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from typing import Optional
+
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+PORT_PATH = os.path.join(HERE, "liboracle_cpu.so")
+REF_PATH = os.path.join(HERE, "_ref", "libmegalodon_ref_cpu.so")
+
+_port = None
+_ref = None
+
+
+def build(with_reference: bool = True) -> None:
+    """Compile the checkers (make); the reference build is skipped when
+    /root/reference is absent."""
+    subprocess.run(["make", "-C", HERE, "liboracle_cpu.so"], check=True, capture_output=True)
+    if with_reference:
+        subprocess.run(["make", "-C", HERE, "ref"], check=True, capture_output=True)
+
+
+def port() -> ctypes.CDLL:
+    global _port
+    if _port is None:
+        if not os.path.exists(PORT_PATH):
+            build(with_reference=False)
+        _port = ctypes.CDLL(PORT_PATH)
+    return _port
+
+
+def ref() -> Optional[ctypes.CDLL]:
+    global _ref
+    if _ref is None and os.path.exists(REF_PATH):
+        _ref = ctypes.CDLL(REF_PATH)
+    return _ref
+
+
+def _p(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _i(v):
+    return ctypes.c_int64(int(v))
+
+
+def _c64_as_f32(t):
+    return torch.view_as_real(t.to(torch.complex64).contiguous().resolve_conj()).contiguous()
+
+
+def ema_weight_fwd(lib, prefix, p, log_q, gamma, L):
+    D = p.shape[0]
+    pf = p.reshape(D, -1).float().contiguous()
+    N = pf.shape[1]
+    lq = _c64_as_f32(log_q.reshape(D, N))
+    gm = _c64_as_f32(gamma.reshape(D, N))
+    w = torch.empty(D, L, dtype=torch.float32)
+    getattr(lib, prefix + "ema_weight_fwd")(_p(pf), _p(lq), _p(gm), _i(D), _i(N), _i(L), _p(w))
+    return w
+
+
+def ema_weight_bwd(lib, prefix, dw, p, log_q, gamma):
+    D = p.shape[0]
+    pf = p.reshape(D, -1).float().contiguous()
+    N = pf.shape[1]
+    L = dw.shape[-1]
+    lq = _c64_as_f32(log_q.reshape(D, N))
+    gm = _c64_as_f32(gamma.reshape(D, N))
+    dwf = dw.float().contiguous()
+    dp = torch.empty(D, N, dtype=torch.float32)
+    dq = torch.empty(D, N, 2, dtype=torch.float32)
+    dg = torch.empty(D, N, 2, dtype=torch.float32)
+    getattr(lib, prefix + "ema_weight_bwd")(_p(dwf), _p(pf), _p(lq), _p(gm), _i(D), _i(N), _i(L),
+                                            _p(dp), _p(dq), _p(dg))
+    return dp, torch.view_as_complex(dq), torch.view_as_complex(dg)
+
+
+def group_timestep_norm_fwd(lib, prefix, x, prev_count, prev_mean, prev_var, gamma, beta, mask, G, eps):
+    B, L, H = x.shape
+    xf = x.float().contiguous()
+    pc = prev_count.to(torch.int64).contiguous()
+    pm, pv = prev_mean.float().contiguous(), prev_var.float().contiguous()
+    gm, bt = gamma.float().contiguous(), beta.float().contiguous()
+    mk = None if mask is None else mask.to(torch.uint8).contiguous()
+    y = torch.empty_like(xf)
+    count = torch.empty(B, dtype=torch.int64)
+    mean = torch.empty(B, G)
+    var = torch.empty(B, G)
+    cummean = torch.empty(B, L, G)
+    cumrstd = torch.empty(B, L, G)
+    getattr(lib, prefix + "group_timestep_norm_fwd")(
+        _p(xf), _p(pc), _p(pm), _p(pv), _p(gm), _p(bt), _p(mk), _i(B), _i(L), _i(H), _i(G),
+        ctypes.c_double(eps), _p(y), _p(count), _p(mean), _p(var), _p(cummean), _p(cumrstd))
+    return y, count, mean, var, cummean, cumrstd
+
+
+def group_timestep_norm_bwd(lib, prefix, dy, dmean, dvar, x, prev_mean, count, cummean, cumrstd, gamma, mask, G):
+    B, L, H = x.shape
+    dyf, xf = dy.float().contiguous(), x.float().contiguous()
+    dm, dv = dmean.float().contiguous(), dvar.float().contiguous()
+    pm = prev_mean.float().contiguous()
+    cnt = count.to(torch.int64).contiguous()
+    cm, cr = cummean.float().contiguous(), cumrstd.float().contiguous()
+    gm = gamma.float().contiguous()
+    mk = None if mask is None else mask.to(torch.uint8).contiguous()
+    dx = torch.empty_like(xf)
+    dpm = torch.empty(B, G)
+    dpv = torch.empty(B, G)
+    dg = torch.empty(H)
+    db = torch.empty(H)
+    getattr(lib, prefix + "group_timestep_norm_bwd")(
+        _p(dyf), _p(dm), _p(dv), _p(xf), _p(pm), _p(cnt), _p(cm), _p(cr), _p(gm), _p(mk),
+        _i(B), _i(L), _i(H), _i(G), _p(dx), _p(dpm), _p(dpv), _p(dg), _p(db))
+    return dx, dpm, dpv, dg, db

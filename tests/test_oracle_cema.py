@@ -110,3 +110,47 @@ def test_weight_bwd_finite_differences():
             fr = (loss(p, q, gamma + ec) - loss(p, q, gamma - ec)) / (2 * eps)
             fi = (loss(p, q, gamma + 1j * ec) - loss(p, q, gamma - 1j * ec)) / (2 * eps)
             assert abs(complex(fr, fi) - complex(dg[d, n])) < 1e-6
+
+
+# ---- compiled checkers: the C restatement and the reference's own C++ CPU path ----
+from oracle import native
+
+
+def _f32_case(D, N, seed):
+    p, q, gamma = _params(D, N, seed)
+    return p.float(), q.to(torch.complex64).log(), gamma.to(torch.complex64)
+
+
+def test_c_port_matches_float64_oracle():
+    lib = native.port()
+    p, lq, gamma = _f32_case(6, 16, 11)
+    L = 300
+    w = native.ema_weight_fwd(lib, "oracle_", p, lq, gamma, L)
+    want = cema.ema_weight_fwd(p, lq, gamma, L)
+    assert (w.double() - want).abs().max() / want.abs().max() < 2e-5
+    g = torch.Generator().manual_seed(3)
+    dw = torch.randn(6, L, generator=g)
+    dp, dq, dg = native.ema_weight_bwd(lib, "oracle_", dw, p, lq, gamma)
+    wp, wq, wg = cema.ema_weight_bwd(dw, p, lq, gamma)
+    assert (dp.double() - wp).abs().max() / wp.abs().max() < 1e-4
+    assert (dq.to(torch.complex128) - wq).abs().max() / wq.abs().max() < 1e-4
+    assert (dg.to(torch.complex128) - wg).abs().max() / wg.abs().max() < 1e-4
+
+
+@pytest.mark.skipif(native.ref() is None, reason="oracle/_ref not built (needs /root/reference)")
+def test_reference_cpp_cpu_path_matches_oracle():
+    """The reference's EMAParametersCPUFwd/Bwd (compiled from its own sources)
+    against the float64 restatement, float32 tolerance."""
+    lib = native.ref()
+    for D, N, L, seed in [(5, 16, 257, 1), (3, 4, 64, 2), (2, 1, 33, 3)]:
+        p, lq, gamma = _f32_case(D, N, seed)
+        w = native.ema_weight_fwd(lib, "ref_", p, lq, gamma, L)
+        want = cema.ema_weight_fwd(p, lq, gamma, L)
+        assert (w.double() - want).abs().max() / want.abs().max() < 2e-5
+        g = torch.Generator().manual_seed(seed)
+        dw = torch.randn(D, L, generator=g)
+        dp, dq, dg = native.ema_weight_bwd(lib, "ref_", dw, p, lq, gamma)
+        wp, wq, wg = cema.ema_weight_bwd(dw, p, lq, gamma)
+        assert (dp.double() - wp).abs().max() / wp.abs().max() < 1e-4
+        assert (dq.to(torch.complex128) - wq).abs().max() / wq.abs().max() < 1e-4
+        assert (dg.to(torch.complex128) - wg).abs().max() / wg.abs().max() < 1e-4
