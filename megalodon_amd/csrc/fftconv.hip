@@ -16,6 +16,7 @@
 #include "fftconv_core.hpp"
 
 #include <mutex>
+#include <vector>
 
 namespace mega {
 namespace {
@@ -23,37 +24,6 @@ namespace {
 using namespace fftc;
 
 // ------------------------------ tables --------------------------------------
-template <int LOGM>
-__global__ void fftconv_tables_kernel(c32* tab) {
-  using C = Cfg<LOGM>;
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= C::TABLE) return;
-  const double N = 2.0 * C::M;
-  double num, den;
-  if (i < 32 * C::T) {
-    const int a2 = i / C::T, t = i % C::T;
-    num = static_cast<double>(t) * a2;
-    den = C::M;
-  } else if (i < 64 * C::T) {
-    const int j = i - 32 * C::T;
-    const int a2 = j / C::T, t = j % C::T;
-    num = static_cast<double>(t) * (2 * a2 + 1);
-    den = N;
-  } else if (i < 64 * C::T + 32 * C::R3) {
-    const int j = i - 64 * C::T;
-    num = static_cast<double>(j / 32) * (j % 32);
-    den = C::T;
-  } else {
-    const int j = i - 64 * C::T - 32 * C::R3;
-    num = 2.0 * (j % 1024) + (j / 1024);
-    den = N;
-  }
-  const double fr = fmod(num, den) / den;  // exact: num < 2^53
-  double s, c;
-  sincospi(-2.0 * fr, &s, &c);
-  tab[i] = c32{static_cast<float>(c), static_cast<float>(s)};
-}
-
 constexpr int kMaxDevices = 16;
 struct TableCache {
   c32* ptr[kMaxDevices][4] = {};
@@ -86,8 +56,9 @@ int get_tables(hipStream_t stream, const c32** out, float** scratch, int* slots)
     g_tables.slots[dev][LOGM - 11] = nslots;
     c32* p = nullptr;
     MEGA_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&p), sizeof(c32) * C::TABLE));
-    fftconv_tables_kernel<LOGM><<<(C::TABLE + 255) / 256, 256, 0, stream>>>(p);
-    hipError_t e = hipGetLastError();
+    std::vector<c32> host(C::TABLE);
+    fill_tables<LOGM>(host.data());
+    hipError_t e = hipMemcpyAsync(p, host.data(), sizeof(c32) * C::TABLE, hipMemcpyHostToDevice, stream);
     if (e == hipSuccess) e = hipStreamSynchronize(stream);
     if (e != hipSuccess) {
       (void)hipFree(p);
@@ -227,7 +198,8 @@ __device__ __forceinline__ void store_row(const float* re, const float* im, void
 // twiddles are re-read from L1/L2 at each use instead of being kept live in
 // registers across transforms (which would spill).
 __device__ __forceinline__ Tables launder(Tables tb) {
-  asm volatile("" : "+s"(tb.tw1e), "+s"(tb.tw1o), "+s"(tb.tw2), "+s"(tb.pw));
+  asm volatile("" : "+s"(tb.kr), "+s"(tb.kbo), "+s"(tb.kbe), "+s"(tb.kbo2));
+  asm volatile("" : "+s"(tb.kp2), "+s"(tb.ki3), "+s"(tb.kre), "+s"(tb.kro), "+s"(tb.pw));
   return tb;
 }
 

@@ -214,32 +214,103 @@ struct Cfg {
   static constexpr int LD1 = T + R3;        // row pitch of exchange 1 (floats)
   static constexpr int LD2 = R3 + (R3 >= 4 ? 2 : 0);  // pitch of exchange 2
   static constexpr int PLANE = (32 * LD1 > 1024 * LD2) ? 32 * LD1 : 1024 * LD2;
-  static constexpr int TABLE = 64 * T + 32 * R3 + 2048;  // c32 entries
+  static constexpr int TABLE = 4 * T + R3 + 96 + 2048;  // c32 entries
   static_assert(LOGM >= 11 && LOGM <= 14, "M must be 2048..16384");
 };
 
-// Twiddle tables for one M (device memory, W_X^k = exp(-2 pi i k / X)):
-//   tw1e[a2*T + t]  = W_M^(t a2)            pass-1 twiddle, even half
-//   tw1o[a2*T + t]  = W_N^(t (2 a2 + 1))    pass-1 twiddle, odd half
-//   tw2[n0*32 + a1] = W_T^(n0 a1)           pass-2 twiddle
-//   pw[h*1024 + c]  = W_N^(2c + h)          pointwise twiddle
+// Per-lane twiddle seeds for one M (device memory, W_X^k = exp(-2 pi i k / X)).
+// Every twiddle of a pass is a geometric sequence base * ratio^k whose base
+// and ratio depend only on the lane, so a pass loads two seeds and generates
+// the rest with multiplications instead of 31 dependent table loads.
+//   kr[t]   = W_M^t                      ratio, forward pass 1 (t = lane)
+//   kbo[t]  = W_N^t                      base,  forward pass 1, odd half
+//   kp2[n0] = W_T^n0                     ratio, forward pass 2
+//   ki3[a1] = W_T^a1                     ratio, inverse pass 3
+//   kbe[t]  = W_M^(n0 a2)                base,  inverse pass 2, even (t = a2*R3 + n0)
+//   kre[a2] = W_M^(R3 a2)                ratio, inverse pass 2, even
+//   kbo2[t] = W_N^(n0 (2 a2 + 1))        base,  inverse pass 2, odd
+//   kro[a2] = W_N^(R3 (2 a2 + 1))        ratio, inverse pass 2, odd
+//   pw[h*1024 + c] = W_N^(2c + h)        pointwise twiddle
 struct Tables {
-  const c32* tw1e;
-  const c32* tw1o;
-  const c32* tw2;
+  const c32* kr;
+  const c32* kbo;
+  const c32* kp2;
+  const c32* ki3;
+  const c32* kbe;
+  const c32* kre;
+  const c32* kbo2;
+  const c32* kro;
   const c32* pw;
 };
 
 template <int LOGM>
 MEGA_HD Tables make_tables(const c32* base) {
   using C = Cfg<LOGM>;
-  return Tables{base, base + 32 * C::T, base + 64 * C::T, base + 64 * C::T + 32 * C::R3};
+  Tables tb;
+  tb.kr = base;
+  tb.kbo = tb.kr + C::T;
+  tb.kbe = tb.kbo + C::T;
+  tb.kbo2 = tb.kbe + C::T;
+  tb.kp2 = tb.kbo2 + C::T;
+  tb.ki3 = tb.kp2 + C::R3;
+  tb.kre = tb.ki3 + 32;
+  tb.kro = tb.kre + 32;
+  tb.pw = tb.kro + 32;
+  return tb;
+}
+
+// Host-side fill of the seed table (float64 trigonometry, exact argument reduction).
+template <int LOGM>
+inline void fill_tables(c32* out) {
+  using C = Cfg<LOGM>;
+  const double N = 2.0 * C::M;
+  auto w = [](double num, double den) {
+    const double fr = __builtin_fmod(num, den) / den;
+    const double a = -6.283185307179586476925286766559 * fr;
+    return c32{static_cast<float>(__builtin_cos(a)), static_cast<float>(__builtin_sin(a))};
+  };
+  c32* p = out;
+  for (int t = 0; t < C::T; ++t) *p++ = w(t, C::M);
+  for (int t = 0; t < C::T; ++t) *p++ = w(t, N);
+  for (int t = 0; t < C::T; ++t) *p++ = w(static_cast<double>(t % C::R3) * (t / C::R3), C::M);
+  for (int t = 0; t < C::T; ++t) *p++ = w(static_cast<double>(t % C::R3) * (2 * (t / C::R3) + 1), N);
+  for (int n0 = 0; n0 < C::R3; ++n0) *p++ = w(n0, C::T);
+  for (int a1 = 0; a1 < 32; ++a1) *p++ = w(a1, C::T);
+  for (int a2 = 0; a2 < 32; ++a2) *p++ = w(static_cast<double>(C::R3) * a2, C::M);
+  for (int a2 = 0; a2 < 32; ++a2) *p++ = w(static_cast<double>(C::R3) * (2 * a2 + 1), N);
+  for (int h = 0; h < 2; ++h)
+    for (int c = 0; c < 1024; ++c) *p++ = w(2.0 * c + h, N);
 }
 
 // table[idx] addressed as uniform base + 32-bit unsigned byte offset (lets the
 // compiler use the scalar-base addressing form instead of a 64-bit lane address)
 MEGA_HD c32 ldc(const c32* base, unsigned idx) {
   return *reinterpret_cast<const c32*>(reinterpret_cast<const char*>(base) + idx * 8u);
+}
+
+MEGA_HD c32 cmulv(c32 a, c32 b) { return c32{a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x}; }
+MEGA_HD c32 csqv(c32 a) { return c32{a.x * a.x - a.y * a.y, 2.f * a.x * a.y}; }
+MEGA_HD c32 conjv(c32 a) { return c32{a.x, -a.y}; }
+
+// Calls f(k, base * r^k) for k = 0..COUNT-1.  Powers are built in blocks of 8
+// (block seeds by r^8, then a chain of 7), so no twiddle is more than 10
+// multiplications away from a table value.
+template <int COUNT, typename F>
+MEGA_HD void geo_twiddles(c32 base, c32 r, F&& f) {
+  const c32 r8 = csqv(csqv(csqv(r)));
+  c32 blk = base;
+#pragma unroll
+  for (int a = 0; a < COUNT; a += 8) {
+    c32 s = blk;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      if (a + b < COUNT) {
+        f(a + b, s);
+        if (b + 1 < 8 && a + b + 1 < COUNT) s = cmulv(s, r);
+      }
+    }
+    if (a + 8 < COUNT) blk = cmulv(blk, r8);
+  }
 }
 
 MEGA_HD void cmul_ip(float& xr, float& xi, c32 w) {
@@ -270,15 +341,15 @@ MEGA_HD void slot_residues(int s, int& c0, int& c1) {
 // outputs in registers (output a2 at position bitrev5(a2)).
 template <int LOGM, int H>
 MEGA_HD void fwd_pass1(float* re, float* im, int t, const Tables& tb) {
-  using C = Cfg<LOGM>;
+  const c32 r = ldc(tb.kr, t);
+  const c32 base = H == 0 ? c32{1.f, 0.f} : ldc(tb.kbo, t);
   if (H == 0) dif<32, 1>(re, im); else shifted_dif32(re, im);
-  const c32* tw = H == 0 ? tb.tw1e : tb.tw1o;
-#pragma unroll
-  for (int a2 = (H == 0 ? 1 : 0); a2 < 32; ++a2) {
+  // W_M^(t a2) (even) or W_N^(t (2 a2 + 1)) = W_N^t (W_M^t)^a2 (odd)
+  geo_twiddles<32>(base, r, [&](int a2, c32 w) {
+    if (H == 0 && a2 == 0) return;
     const int pos = bitrev<5>(a2);
-    if (a2 % 8 == 0) MEGA_MEM_FENCE();
-    cmul_ip(re[pos], im[pos], ldc(tw, a2 * C::T + t));
-  }
+    cmul_ip(re[pos], im[pos], w);
+  });
 }
 template <int LOGM>
 MEGA_HD void x1_write(const float* re, const float* im, int t, float* lre, float* lim) {
@@ -304,14 +375,13 @@ MEGA_HD void x1_read(float* re, float* im, int t, const float* lre, const float*
 template <int LOGM>
 MEGA_HD void fwd_pass2(float* re, float* im, int t, const Tables& tb) {
   using C = Cfg<LOGM>;
-  const int n0p = t % C::R3;
+  const c32 r = ldc(tb.kp2, t % C::R3);  // W_T^n0'
   dif<32, 1>(re, im);
-#pragma unroll
-  for (int a1 = 1; a1 < 32; ++a1) {
+  geo_twiddles<32>(c32{1.f, 0.f}, r, [&](int a1, c32 w) {
+    if (a1 == 0) return;
     const int pos = bitrev<5>(a1);
-    if (a1 % 8 == 0) MEGA_MEM_FENCE();
-    cmul_ip(re[pos], im[pos], ldc(tb.tw2, n0p * 32 + a1));
-  }
+    cmul_ip(re[pos], im[pos], w);
+  });
 }
 // element (a2', a1, n0') goes to residue c = a2' + 32 a1
 template <int LOGM>
@@ -442,21 +512,24 @@ MEGA_HD void pointwise(float* re, float* im, const float* bre, const float* bim,
 template <int LOGM, int H>
 MEGA_HD void inv_pass3(float* re, float* im, int t, const Tables& tb) {
   using C = Cfg<LOGM>;
-#pragma unroll
-  for (int g = 0; g < 2 * C::NSLOT; ++g) dit<C::R3, 1>(im + g * C::R3, re + g * C::R3);
+  c32 rr[2 * C::NSLOT];
 #pragma unroll
   for (int u = 0; u < C::NSLOT; ++u) {
     int c[2];
     slot_residues<H>(t + C::T * u, c[0], c[1]);
+    rr[2 * u] = conjv(ldc(tb.ki3, c[0] >> 5));
+    rr[2 * u + 1] = conjv(ldc(tb.ki3, c[1] >> 5));
+  }
 #pragma unroll
-    for (int w = 0; w < 2; ++w) {
-      const int a1 = c[w] >> 5;
+  for (int g = 0; g < 2 * C::NSLOT; ++g) dit<C::R3, 1>(im + g * C::R3, re + g * C::R3);
 #pragma unroll
-      for (int n0 = 1; n0 < C::R3; ++n0) {
-        const int i = sidx<LOGM>(u, w, n0);
-        cmulc_ip(re[i], im[i], ldc(tb.tw2, n0 * 32 + a1));
-      }
-    }
+  for (int g = 0; g < 2 * C::NSLOT; ++g) {
+    // conj(W_T^(n0 a1)), a1 = residue >> 5
+    geo_twiddles<C::R3>(c32{1.f, 0.f}, rr[g], [&](int n0, c32 w) {
+      if (n0 == 0) return;
+      const int i = g * C::R3 + n0;
+      cmul_ip(re[i], im[i], w);
+    });
   }
 }
 template <int LOGM, int H>
@@ -490,19 +563,18 @@ MEGA_HD void ix2_read(float* re, float* im, int t, const float* lre, const float
   }
 }
 // pass 2': inverse radix-32 over a1 -> n1 at bitrev5(n1); conj pass-1 twiddle
+// conj(W^((n1 R3 + n0') ...)) = conj(base) conj(ratio)^n1
 template <int LOGM, int H>
 MEGA_HD void inv_pass2(float* re, float* im, int t, const Tables& tb) {
   using C = Cfg<LOGM>;
-  const int a2p = t / C::R3, n0p = t % C::R3;
+  const int a2p = t / C::R3;
+  const c32 base = conjv(ldc(H == 0 ? tb.kbe : tb.kbo2, t));
+  const c32 r = conjv(ldc(H == 0 ? tb.kre : tb.kro, a2p));
   dif<32, 1>(im, re);
-  const c32* tw = (H == 0 ? tb.tw1e : tb.tw1o);
-  const unsigned tw0 = a2p * C::T + n0p;
-#pragma unroll
-  for (int n1 = 0; n1 < 32; ++n1) {
+  geo_twiddles<32>(base, r, [&](int n1, c32 w) {
     const int pos = bitrev<5>(n1);
-    if (n1 % 8 == 0) MEGA_MEM_FENCE();
-    cmulc_ip(re[pos], im[pos], ldc(tw, tw0 + n1 * C::R3));
-  }
+    cmul_ip(re[pos], im[pos], w);
+  });
 }
 template <int LOGM>
 MEGA_HD void ix1_write(const float* re, const float* im, int t, float* lre, float* lim) {

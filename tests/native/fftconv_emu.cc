@@ -11,25 +11,8 @@ using namespace mega::fftc;
 
 template <int LOGM>
 static void build_tables(std::vector<c32>& tab) {
-  using C = Cfg<LOGM>;
-  const double N = 2.0 * C::M;
-  tab.resize(C::TABLE);
-  auto w = [](double num, double den) {
-    const double a = -2.0 * M_PI * std::fmod(num, den) / den;
-    return c32{(float)std::cos(a), (float)std::sin(a)};
-  };
-  c32* p = tab.data();
-  for (int a2 = 0; a2 < 32; ++a2)
-    for (int t = 0; t < C::T; ++t) p[a2 * C::T + t] = w((double)t * a2, C::M);
-  p += 32 * C::T;
-  for (int a2 = 0; a2 < 32; ++a2)
-    for (int t = 0; t < C::T; ++t) p[a2 * C::T + t] = w((double)t * (2 * a2 + 1), N);
-  p += 32 * C::T;
-  for (int n0 = 0; n0 < C::R3; ++n0)
-    for (int a1 = 0; a1 < 32; ++a1) p[n0 * 32 + a1] = w((double)n0 * a1, C::T);
-  p += 32 * C::R3;
-  for (int h = 0; h < 2; ++h)
-    for (int c = 0; c < 1024; ++c) p[h * 1024 + c] = w(2.0 * c + h, N);
+  tab.resize(Cfg<LOGM>::TABLE);
+  fill_tables<LOGM>(tab.data());
 }
 
 static float seq_at(const float* s, int L, int m, int flip) {
