@@ -106,6 +106,49 @@ int mega_fftconv_bwd(const void* dy, const void* x, int dtype, const float* k,
                      int64_t B, int64_t D, int64_t L, void* dx, float* dk,
                      void* stream);
 
+/* ------------------------------------------------------------------------
+ * Group TimestepNorm (cumulative group mean / variance over time).
+ *
+ * Replaces group_timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma,
+ *   beta, padding_mask?, num_groups, eps)
+ *   -> (y, count, mean, var, cummean, cumrstd)
+ *   reference: megalodon/csrc/ops/timestep_norm.cc:218-316 (CPU),
+ *              timestep_norm_kernel.cu:453-681,1252-1326 (CUDA), binding timestep_norm.cc:702.
+ *   x, y (B, L, D) of `dtype`; gamma, beta (D); prev_mean, prev_var, mean, var
+ *   (B, G), all of `dtype`; prev_count, count (B) int64; padding_mask (B, L)
+ *   bytes (non-zero = padding) or NULL; cummean, cumrstd (B, L, G) float32.
+ *   Masked steps leave the running statistics unchanged and give y = 0; the
+ *   stored cummean / cumrstd at a masked step are those of the unchanged state.
+ *   `workspace`: mega_group_timestep_norm_workspace_bytes(B, L, D, G, 0) bytes
+ *   of device memory, contents irrelevant on entry (cleared by the call).
+ * ---------------------------------------------------------------------- */
+int64_t mega_group_timestep_norm_workspace_bytes(int64_t B, int64_t L, int64_t D,
+                                                 int64_t G, int backward);
+int mega_group_timestep_norm_fwd(const void* x, int dtype, const int64_t* prev_count,
+                                 const void* prev_mean, const void* prev_var,
+                                 const void* gamma, const void* beta,
+                                 const uint8_t* padding_mask, int64_t B, int64_t L,
+                                 int64_t D, int64_t G, double eps, void* y,
+                                 int64_t* count, void* mean, void* var,
+                                 float* cummean, float* cumrstd, void* workspace,
+                                 void* stream);
+
+/* Replaces group_timestep_norm_bwd(dy, dmean, dvar, x, prev_mean, count,
+ *   cummean, cumrstd, gamma, padding_mask?, num_groups)
+ *   -> (dx, dprev_mean, dprev_var, dgamma, dbeta)
+ *   reference: timestep_norm.cc:318-450 (CPU), timestep_norm_kernel.cu:683-1086,
+ *              1328-1439 (CUDA), binding timestep_norm.cc:704.
+ *   `count` is the forward's output count; dgamma, dbeta (D) of `dtype`.
+ *   `workspace`: mega_group_timestep_norm_workspace_bytes(B, L, D, G, 1) bytes. */
+int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, const void* dvar,
+                                 const void* x, int dtype, const void* prev_mean,
+                                 const int64_t* count, const float* cummean,
+                                 const float* cumrstd, const void* gamma,
+                                 const uint8_t* padding_mask, int64_t B, int64_t L,
+                                 int64_t D, int64_t G, void* dx, void* dprev_mean,
+                                 void* dprev_var, void* dgamma, void* dbeta,
+                                 void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,941 @@
+// Group TimestepNorm for gfx950: cumulative (over time) group mean / variance
+// normalisation, forward and backward, one pass over the activations.
+//
+// Math follows megalodon/csrc/ops/timestep_norm.cc:218-316 (forward) and
+// :318-450 (backward), merge operator megalodon/csrc/utils.h:154-164; masked
+// steps behave as in the reference's CUDA kernels (state unchanged, y = dx = 0,
+// stored statistics are those of the unchanged state,
+// timestep_norm_kernel.cu:621-626).
+//
+// Design.  The reference scans time in B*ceil(G/32) blocks and reads x two to
+// three times.  Here the (batch, group) chains are cut into tiles of 64
+// timesteps; a workgroup loads one tile (64 rows x D/G features) into
+// registers, reduces every row to its moments, scans the 64 rows inside one
+// wavefront (lane = timestep) and obtains the carry of all earlier tiles by a
+// decoupled look-back over per-tile records in device memory (aggregate /
+// inclusive-prefix words published with relaxed device-scope atomics, value and
+// ready-flag in one 64-bit word).  The tile is then normalised from registers:
+// x is read once and y written once.  The backward pass runs the same scheme
+// in reverse time with 2x2 upper-triangular affine maps as the carried
+// quantity (the reverse recurrence on (dmean, dvar) is affine in the state).
+// Tiles are handed out in time order by a ticket counter, so every tile a
+// workgroup waits for is already resident or finished.
+#include "common.hpp"
+
+#include <algorithm>
+
+namespace mega {
+namespace {
+
+constexpr int kTL = 64;        // timesteps per tile = lanes per wavefront
+constexpr int kThreads = 256;  // 4 wavefronts
+constexpr int kWaves = kThreads / kWave;
+
+struct TsnParams {
+  const void* x;
+  const void* dy;          // backward only
+  const void* gamma;
+  const void* beta;        // forward only
+  const uint8_t* mask;     // (B, L) or null; 1 = padding
+  const int64_t* prev_count;  // forward: (B); backward: final count (B)
+  const void* prev_mean;
+  const void* prev_var;    // forward only
+  const void* dmean;       // backward only
+  const void* dvar;
+  const float* cummean_in;  // backward
+  const float* cumrstd_in;
+  void* y;                 // forward y / backward dx
+  int64_t* count;
+  void* mean;              // forward mean / backward dprev_mean
+  void* var;               // forward var / backward dprev_var
+  float* cummean;
+  float* cumrstd;
+  float* part_g;           // backward partial sums (B*NT, D)
+  float* part_b;
+  int* ticket;
+  const int* nbefore;      // (B, NT+1) unmasked steps before tile j
+  unsigned long long* rec; // per (chain, tile) records
+  int B, L, D, G, Dg, NT;
+  float eps;
+};
+
+// ---- 64-bit (value, flag) words -------------------------------------------
+__device__ __forceinline__ void put_word(unsigned long long* p, float v) {
+  const unsigned long long w = (static_cast<unsigned long long>(1u) << 32) | __float_as_uint(v);
+  __hip_atomic_store(p, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool get_word(const unsigned long long* p, float& v) {
+  const unsigned long long w =
+      __hip_atomic_load(const_cast<unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  v = __uint_as_float(static_cast<uint32_t>(w));
+  return (w >> 32) != 0;
+}
+
+// ---- Welford triple ----------------------------------------------------------
+struct Wel {
+  float n, u, v;
+};
+__device__ __forceinline__ Wel wel_merge(Wel a, Wel b) {  // utils.h:154-164
+  const float n = a.n + b.n;
+  const float inv = n > 0.f ? 1.f / n : 0.f;
+  const float c1 = a.n * inv, c2 = b.n * inv;
+  const float d = b.u - a.u;
+  return Wel{n, c1 * a.u + c2 * b.u, c1 * a.v + c2 * b.v + (c1 * d) * (c2 * d)};
+}
+__device__ __forceinline__ Wel wel_shfl_up(Wel a, int d) {
+  return Wel{__shfl_up(a.n, d, 64), __shfl_up(a.u, d, 64), __shfl_up(a.v, d, 64)};
+}
+__device__ __forceinline__ Wel wel_shfl_xor(Wel a, int d) {
+  return Wel{__shfl_xor(a.n, d, 64), __shfl_xor(a.u, d, 64), __shfl_xor(a.v, d, 64)};
+}
+
+// ---- affine map on the carried gradient (ug, vg) -----------------------------
+//   ug' = a ug + e vg + bu,   vg' = a vg + bv
+struct Aff {
+  float a, e, bu, bv;
+};
+// apply x first (later time), then y (earlier time)
+__device__ __forceinline__ Aff aff_compose(Aff y, Aff x) {
+  return Aff{y.a * x.a, y.a * x.e + y.e * x.a, y.a * x.bu + y.e * x.bv + y.bu, y.a * x.bv + y.bv};
+}
+__device__ __forceinline__ Aff aff_shfl_down(Aff m, int d) {
+  return Aff{__shfl_down(m.a, d, 64), __shfl_down(m.e, d, 64), __shfl_down(m.bu, d, 64),
+             __shfl_down(m.bv, d, 64)};
+}
+__device__ __forceinline__ Aff aff_shfl_up(Aff m, int d) {
+  return Aff{__shfl_up(m.a, d, 64), __shfl_up(m.e, d, 64), __shfl_up(m.bu, d, 64),
+             __shfl_up(m.bv, d, 64)};
+}
+
+// ---- element vectors (16 bytes) -----------------------------------------------
+template <int DT> struct Vec;
+template <> struct Vec<MEGA_F32> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void unpack(const uint4& r, float* f) {
+    f[0] = __uint_as_float(r.x); f[1] = __uint_as_float(r.y);
+    f[2] = __uint_as_float(r.z); f[3] = __uint_as_float(r.w);
+  }
+  static __device__ __forceinline__ uint4 pack(const float* f) {
+    return make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),
+                      __float_as_uint(f[3]));
+  }
+};
+template <> struct Vec<MEGA_BF16> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void unpack(const uint4& r, float* f) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(w[i] << 16);
+      f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ uint4 pack(const float* f) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      w[i] = static_cast<uint32_t>(float_to_bf16_bits(f[2 * i])) |
+             (static_cast<uint32_t>(float_to_bf16_bits(f[2 * i + 1])) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+  }
+};
+template <> struct Vec<MEGA_F16> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void unpack(const uint4& r, float* f) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = f16_bits_to_float(static_cast<uint16_t>(w[i] & 0xffffu));
+      f[2 * i + 1] = f16_bits_to_float(static_cast<uint16_t>(w[i] >> 16));
+    }
+  }
+  static __device__ __forceinline__ uint4 pack(const float* f) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      w[i] = static_cast<uint32_t>(float_to_f16_bits(f[2 * i])) |
+             (static_cast<uint32_t>(float_to_f16_bits(f[2 * i + 1])) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+  }
+};
+
+template <int DT>
+__device__ __forceinline__ float ldT(const void* p, int64_t i) {
+  return Elem<DT>::load(static_cast<const typename Elem<DT>::type*>(p) + i);
+}
+template <int DT>
+__device__ __forceinline__ void stT(void* p, int64_t i, float v) {
+  Elem<DT>::store(static_cast<typename Elem<DT>::type*>(p) + i, v);
+}
+
+template <int LPR>
+__device__ __forceinline__ float row_sum(float v) {  // sum over the LPR lanes of a row
+#pragma unroll
+  for (int off = LPR / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// ---- preparation: clear ticket / records, count unmasked steps per tile --------
+__global__ void tsn_prep_kernel(int* ticket, unsigned long long* rec, int64_t rec_words,
+                                const uint8_t* mask, int* nbefore, int B, int L, int NT) {
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = gid; i < rec_words; i += stride) rec[i] = 0ull;
+  if (gid == 0) *ticket = 0;
+  // block b (< B) also builds nbefore[b][0..NT]
+  if (blockIdx.x < static_cast<unsigned>(B)) {
+    __shared__ int sums[256];
+    const int b = blockIdx.x;
+    const int per = (NT + 255) / 256;  // tiles per thread
+    const int j0 = threadIdx.x * per;
+    int local = 0;
+    for (int j = j0; j < j0 + per && j < NT; ++j) {
+      int c = 0;
+      for (int t = j * kTL; t < (j + 1) * kTL && t < L; ++t)
+        c += (mask == nullptr || mask[static_cast<int64_t>(b) * L + t] == 0) ? 1 : 0;
+      local += c;
+    }
+    sums[threadIdx.x] = local;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int run = 0;
+      for (int i = 0; i < 256; ++i) {
+        const int v = sums[i];
+        sums[i] = run;
+        run += v;
+      }
+    }
+    __syncthreads();
+    int run = sums[threadIdx.x];
+    for (int j = j0; j < j0 + per && j < NT; ++j) {
+      nbefore[b * (NT + 1) + j] = run;
+      for (int t = j * kTL; t < (j + 1) * kTL && t < L; ++t)
+        run += (mask == nullptr || mask[static_cast<int64_t>(b) * L + t] == 0) ? 1 : 0;
+      if (j == NT - 1) nbefore[b * (NT + 1) + NT] = run;
+    }
+  }
+}
+
+// ------------------------------ forward ---------------------------------------
+constexpr int kFwdWords = 4;  // aggregate (u, v), inclusive (u, v)
+
+// carry of all tiles before tile j of this chain (wave 0 only)
+__device__ __forceinline__ Wel fwd_lookback(const TsnParams& p, int b, int g, int j, int lane,
+                                            Wel prior) {
+  const int64_t chain = static_cast<int64_t>(b) * p.G + g;
+  const unsigned long long* rec = p.rec + chain * p.NT * kFwdWords;
+  const int* nb = p.nbefore + b * (p.NT + 1);
+  Wel total{0.f, 0.f, 0.f};
+  int base = j - 1;
+  while (true) {
+    const int idx = base - lane;
+    int kind = 3;  // 1 aggregate, 2 inclusive prefix, 3 beyond the chain start
+    Wel val{0.f, 0.f, 0.f};
+    if (idx >= 0) {
+      const unsigned long long* r = rec + static_cast<int64_t>(idx) * kFwdWords;
+      while (true) {
+        float iu, iv, au, av;
+        const bool fi = get_word(r + 2, iu) & get_word(r + 3, iv);
+        if (fi) {
+          kind = 2;
+          val = Wel{prior.n + static_cast<float>(nb[idx + 1]), iu, iv};
+          break;
+        }
+        const bool fa = get_word(r + 0, au) & get_word(r + 1, av);
+        if (fa) {
+          kind = 1;
+          val = Wel{static_cast<float>(nb[idx + 1] - nb[idx]), au, av};
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+    } else if (idx == -1) {
+      kind = 2;
+      val = prior;
+    }
+    const unsigned long long m2 = __ballot(kind == 2);
+    const int k = m2 ? __ffsll(static_cast<long long>(m2)) - 1 : 64;
+    if (lane > k || kind == 3) val = Wel{0.f, 0.f, 0.f};
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) val = wel_merge(val, wel_shfl_xor(val, off));
+    total = wel_merge(val, total);
+    if (m2) break;
+    base -= 64;
+  }
+  return total;
+}
+
+template <int DT, int LPR>
+__global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
+  constexpr int VEC = Vec<DT>::N;
+  constexpr int RPW = kWave / LPR;         // rows per wave per pass
+  constexpr int RPP = RPW * kWaves;        // rows per pass
+  constexpr int P = kTL / RPP;             // passes
+  __shared__ float s_a[kTL], s_b[kTL];
+  __shared__ int s_valid[kTL];
+  __shared__ int s_ticket;
+
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  if (threadIdx.x == 0) s_ticket = atomicAdd(p.ticket, 1);
+  __syncthreads();
+  const int NC = p.B * p.G;
+  const int j = s_ticket / NC;
+  const int chain = s_ticket % NC;
+  const int b = chain / p.G, g = chain % p.G;
+  const int t0 = j * kTL;
+  const int col = lane % LPR;
+  const bool col_ok = col * VEC < p.Dg;
+  const float inv_dg = 1.f / static_cast<float>(p.Dg);
+
+  uint4 xv[P];
+#pragma unroll
+  for (int q = 0; q < P; ++q) {
+    const int r = q * RPP + wave * RPW + lane / LPR;
+    const int t = t0 + r;
+    xv[q] = make_uint4(0, 0, 0, 0);
+    if (t < p.L && col_ok) {
+      const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
+      xv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.x) + off);
+    }
+    float f[VEC];
+    Vec<DT>::unpack(xv[q], f);
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) s += f[e];
+    const float mu = row_sum<LPR>(s) * inv_dg;
+    float s2 = 0.f;
+    if (col_ok) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) s2 += (f[e] - mu) * (f[e] - mu);
+    }
+    const float var = row_sum<LPR>(s2) * inv_dg;
+    if (col == 0) {
+      s_a[r] = mu;
+      s_b[r] = var;
+    }
+  }
+  __syncthreads();
+
+  if (wave == 0) {
+    const int t = t0 + lane;
+    const bool valid = t < p.L && (p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0);
+    Wel me{valid ? 1.f : 0.f, valid ? s_a[lane] : 0.f, valid ? s_b[lane] : 0.f};
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const Wel o = wel_shfl_up(me, d);
+      if (lane >= d) me = wel_merge(o, me);
+    }
+    const int64_t chain64 = static_cast<int64_t>(b) * p.G + g;
+    unsigned long long* rec = p.rec + (chain64 * p.NT + j) * kFwdWords;
+    const Wel agg{__shfl(me.n, 63, 64), __shfl(me.u, 63, 64), __shfl(me.v, 63, 64)};
+    if (lane == 0 && j + 1 < p.NT) {
+      put_word(rec + 0, agg.u);
+      put_word(rec + 1, agg.v);
+    }
+    const Wel prior{static_cast<float>(p.prev_count[b]), ldT<DT>(p.prev_mean, chain64),
+                    ldT<DT>(p.prev_var, chain64)};
+    const Wel prefix = j == 0 ? prior : fwd_lookback(p, b, g, j, lane, prior);
+    if (lane == 0 && j + 1 < p.NT) {
+      const Wel inc = wel_merge(prefix, agg);
+      put_word(rec + 2, inc.u);
+      put_word(rec + 3, inc.v);
+    }
+    const Wel st = wel_merge(prefix, me);
+    const float rstd = 1.f / sqrtf(st.v + p.eps);
+    if (t < p.L) {
+      const int64_t o = (static_cast<int64_t>(b) * p.L + t) * p.G + g;
+      p.cummean[o] = st.u;
+      p.cumrstd[o] = rstd;
+    }
+    s_valid[lane] = valid ? 1 : 0;
+    if (j == p.NT - 1 && lane == 63) {
+      stT<DT>(p.mean, chain64, st.u);
+      stT<DT>(p.var, chain64, st.v);
+      if (g == 0) p.count[b] = p.prev_count[b] + p.nbefore[b * (p.NT + 1) + p.NT];
+    }
+    __builtin_amdgcn_s_waitcnt(0);  // s_a/s_b reads retired before they are overwritten
+    __builtin_amdgcn_wave_barrier();
+    s_a[lane] = st.u;
+    s_b[lane] = rstd;
+  }
+  __syncthreads();
+
+  float gm[VEC], bt[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    gm[e] = col_ok ? ldT<DT>(p.gamma, g * p.Dg + col * VEC + e) : 0.f;
+    bt[e] = col_ok ? ldT<DT>(p.beta, g * p.Dg + col * VEC + e) : 0.f;
+  }
+#pragma unroll
+  for (int q = 0; q < P; ++q) {
+    const int r = q * RPP + wave * RPW + lane / LPR;
+    const int t = t0 + r;
+    if (t < p.L && col_ok) {
+      float f[VEC], o[VEC];
+      Vec<DT>::unpack(xv[q], f);
+      const float u = s_a[r], rs = s_b[r];
+      const bool valid = s_valid[r] != 0;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) o[e] = valid ? (f[e] - u) * rs * gm[e] + bt[e] : 0.f;
+      const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
+      *reinterpret_cast<uint4*>(static_cast<typename Elem<DT>::type*>(p.y) + off) = Vec<DT>::pack(o);
+    }
+  }
+}
+
+// Any shape: one wavefront per (batch, group) walks the sequence step by step.
+template <int DT>
+__global__ __launch_bounds__(kWave) void tsn_fwd_serial_kernel(const TsnParams p) {
+  const int chain = blockIdx.x;
+  const int b = chain / p.G, g = chain % p.G;
+  const int lane = threadIdx.x;
+  const float inv_dg = 1.f / static_cast<float>(p.Dg);
+  Wel st{static_cast<float>(p.prev_count[b]), ldT<DT>(p.prev_mean, chain), ldT<DT>(p.prev_var, chain)};
+  int64_t cnt = p.prev_count[b];
+  for (int t = 0; t < p.L; ++t) {
+    const int64_t row = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg;
+    const bool valid = p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0;
+    float s = 0.f;
+    for (int i = lane; i < p.Dg; i += kWave) s += ldT<DT>(p.x, row + i);
+    const float mu = wave_sum(s) * inv_dg;
+    float s2 = 0.f;
+    for (int i = lane; i < p.Dg; i += kWave) {
+      const float d = ldT<DT>(p.x, row + i) - mu;
+      s2 += d * d;
+    }
+    const float var = wave_sum(s2) * inv_dg;
+    if (valid) {
+      st = wel_merge(st, Wel{1.f, mu, var});
+      ++cnt;
+    }
+    const float rstd = 1.f / sqrtf(st.v + p.eps);
+    if (lane == 0) {
+      const int64_t o = (static_cast<int64_t>(b) * p.L + t) * p.G + g;
+      p.cummean[o] = st.u;
+      p.cumrstd[o] = rstd;
+    }
+    for (int i = lane; i < p.Dg; i += kWave) {
+      const float xx = ldT<DT>(p.x, row + i);
+      const float o = valid ? (xx - st.u) * rstd * ldT<DT>(p.gamma, g * p.Dg + i) +
+                                  ldT<DT>(p.beta, g * p.Dg + i)
+                            : 0.f;
+      stT<DT>(p.y, row + i, o);
+    }
+  }
+  if (lane == 0) {
+    stT<DT>(p.mean, chain, st.u);
+    stT<DT>(p.var, chain, st.v);
+    if (g == 0) p.count[b] = cnt;
+  }
+}
+
+// ------------------------------ backward --------------------------------------
+constexpr int kBwdWords = 6;  // aggregate (a, e, bu, bv), outgoing state (ug, vg)
+
+struct State2 {
+  float ug, vg;
+};
+__device__ __forceinline__ State2 aff_apply(Aff m, State2 s) {
+  return State2{m.a * s.ug + m.e * s.vg + m.bu, m.a * s.vg + m.bv};
+}
+
+// state entering tile j from the later tiles of this chain (wave 0 only)
+__device__ __forceinline__ State2 bwd_lookahead(const TsnParams& p, int64_t chain, int j, int lane,
+                                                State2 init) {
+  const unsigned long long* rec = p.rec + chain * p.NT * kBwdWords;
+  Aff total{1.f, 0.f, 0.f, 0.f};
+  int base = j + 1;
+  while (true) {
+    const int idx = base + lane;
+    int kind = 3;
+    Aff val{1.f, 0.f, 0.f, 0.f};
+    State2 sv{0.f, 0.f};
+    if (idx < p.NT) {
+      const unsigned long long* r = rec + static_cast<int64_t>(idx) * kBwdWords;
+      while (true) {
+        float a, e, bu, bv, ug, vg;
+        const bool fs = get_word(r + 4, ug) & get_word(r + 5, vg);
+        if (fs) {
+          kind = 2;
+          sv = State2{ug, vg};
+          break;
+        }
+        const bool fa = get_word(r + 0, a) & get_word(r + 1, e) & get_word(r + 2, bu) & get_word(r + 3, bv);
+        if (fa) {
+          kind = 1;
+          val = Aff{a, e, bu, bv};
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+    } else if (idx == p.NT) {
+      kind = 2;
+      sv = init;
+    }
+    const unsigned long long m2 = __ballot(kind == 2);
+    const int k = m2 ? __ffsll(static_cast<long long>(m2)) - 1 : 64;
+    if (lane >= k || kind != 1) val = Aff{1.f, 0.f, 0.f, 0.f};
+    // ordered prefix composition: lane l holds A_base o ... o A_(base+l)
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const Aff o = aff_shfl_up(val, d);
+      if (lane >= d) val = aff_compose(o, val);
+    }
+    const Aff win{__shfl(val.a, 63, 64), __shfl(val.e, 63, 64), __shfl(val.bu, 63, 64),
+                  __shfl(val.bv, 63, 64)};
+    total = aff_compose(total, win);
+    if (m2) {
+      const State2 s{__shfl(sv.ug, k, 64), __shfl(sv.vg, k, 64)};
+      return aff_apply(total, s);
+    }
+    base += 64;
+  }
+}
+
+template <int DT, int LPR>
+__global__ __launch_bounds__(kThreads) void tsn_bwd_kernel(const TsnParams p) {
+  constexpr int VEC = Vec<DT>::N;
+  constexpr int RPW = kWave / LPR;
+  constexpr int RPP = RPW * kWaves;
+  constexpr int P = kTL / RPP;
+  __shared__ float s_ux[kTL], s_ds[kTL], s_db[kTL];   // row stats, then (ux, dux, dvx)
+  __shared__ float s_u[kTL], s_r[kTL];
+  __shared__ int s_valid[kTL];
+  __shared__ float s_pg[kWaves][LPR * VEC], s_pb[kWaves][LPR * VEC];
+  __shared__ int s_ticket;
+
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  if (threadIdx.x == 0) s_ticket = atomicAdd(p.ticket, 1);
+  __syncthreads();
+  const int NC = p.B * p.G;
+  const int j = p.NT - 1 - s_ticket / NC;  // later tiles first
+  const int chain = s_ticket % NC;
+  const int b = chain / p.G, g = chain % p.G;
+  const int t0 = j * kTL;
+  const int col = lane % LPR;
+  const bool col_ok = col * VEC < p.Dg;
+  const float inv_dg = 1.f / static_cast<float>(p.Dg);
+
+  float gm[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) gm[e] = col_ok ? ldT<DT>(p.gamma, g * p.Dg + col * VEC + e) : 0.f;
+
+  // statistics saved by the forward pass, one row per lane of every wave
+  {
+    const int t = t0 + lane;
+    if (wave == 0) {
+      const bool in = t < p.L;
+      const int64_t o = (static_cast<int64_t>(b) * p.L + (in ? t : 0)) * p.G + g;
+      s_u[lane] = in ? p.cummean_in[o] : 0.f;
+      s_r[lane] = in ? p.cumrstd_in[o] : 0.f;
+      s_valid[lane] = (in && (p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0)) ? 1 : 0;
+    }
+  }
+  __syncthreads();
+
+  uint4 xv[P], dv[P];
+#pragma unroll
+  for (int q = 0; q < P; ++q) {
+    const int r = q * RPP + wave * RPW + lane / LPR;
+    const int t = t0 + r;
+    xv[q] = make_uint4(0, 0, 0, 0);
+    dv[q] = make_uint4(0, 0, 0, 0);
+    if (t < p.L && col_ok) {
+      const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
+      xv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.x) + off);
+      dv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.dy) + off);
+    }
+    float f[VEC], d[VEC];
+    Vec<DT>::unpack(xv[q], f);
+    Vec<DT>::unpack(dv[q], d);
+    const float u = s_u[r];
+    float sx = 0.f, sds = 0.f, sdb = 0.f;
+    if (col_ok) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        sx += f[e];
+        sds += d[e] * (f[e] - u) * gm[e];
+        sdb += d[e] * gm[e];
+      }
+    }
+    sx = row_sum<LPR>(sx);
+    sds = row_sum<LPR>(sds);
+    sdb = row_sum<LPR>(sdb);
+    if (col == 0) {
+      s_ux[r] = sx * inv_dg;
+      s_ds[r] = sds;
+      s_db[r] = sdb;
+    }
+  }
+  __syncthreads();
+
+  if (wave == 0) {
+    const int64_t chain64 = static_cast<int64_t>(b) * p.G + g;
+    const int t = t0 + lane;
+    const bool valid = s_valid[lane] != 0;
+    const int* nb = p.nbefore + b * (p.NT + 1);
+    // n_t = number of valid steps up to and including t, prior included
+    const unsigned long long vm = __ballot(valid);
+    const int incl = __popcll(vm & ((lane == 63) ? ~0ull : ((1ull << (lane + 1)) - 1ull)));
+    const int64_t n0 = p.prev_count[b] - nb[p.NT];  // prior count
+    const float nt = static_cast<float>(n0 + nb[j] + incl);
+    const float c1 = valid ? (nt - 1.f) / nt : 0.f;
+    const float c2 = valid ? 1.f / nt : 0.f;
+    const float r = s_r[lane], ux = s_ux[lane];
+    float prev_u;
+    if (t == 0) {
+      prev_u = ldT<DT>(p.prev_mean, chain64);
+    } else if (lane == 0) {
+      prev_u = p.cummean_in[(static_cast<int64_t>(b) * p.L + t - 1) * p.G + g];
+    } else {
+      prev_u = s_u[lane - 1];
+    }
+    const float delta = ux - prev_u;
+    const float pu = -r * s_db[lane];
+    const float pv = -0.5f * r * r * r * s_ds[lane];
+    const float e = -2.f * c1 * c2 * delta;
+    const Aff mine = valid ? Aff{c1, e, c1 * pu + e * pv, c1 * pv} : Aff{1.f, 0.f, 0.f, 0.f};
+    // inclusive suffix composition: I_i = X_i o X_(i+1) o ... o X_63
+    Aff inc = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const Aff o = aff_shfl_down(inc, d);
+      if (lane + d < 64) inc = aff_compose(inc, o);
+    }
+    unsigned long long* rec = p.rec + (chain64 * p.NT + j) * kBwdWords;
+    if (lane == 0 && j > 0) {
+      put_word(rec + 0, inc.a);
+      put_word(rec + 1, inc.e);
+      put_word(rec + 2, inc.bu);
+      put_word(rec + 3, inc.bv);
+    }
+    const State2 init{ldT<DT>(p.dmean, chain64), ldT<DT>(p.dvar, chain64)};
+    const State2 sin = j == p.NT - 1 ? init : bwd_lookahead(p, chain64, j, lane, init);
+    // state entering row i = (X_(i+1) o ... o X_63)(sin)
+    Aff exc = aff_shfl_down(inc, 1);
+    if (lane == 63) exc = Aff{1.f, 0.f, 0.f, 0.f};
+    const State2 si = aff_apply(exc, sin);
+    if (lane == 0) {
+      const State2 sout = aff_apply(inc, sin);
+      if (j > 0) {
+        put_word(rec + 4, sout.ug);
+        put_word(rec + 5, sout.vg);
+      } else {
+        stT<DT>(p.mean, chain64, sout.ug);
+        stT<DT>(p.var, chain64, sout.vg);
+      }
+    }
+    const float du = si.ug + pu;
+    const float dvv = si.vg + pv;
+    const float dux = c2 * du + 2.f * c1 * c2 * dvv * delta;
+    const float dvx = c2 * dvv;
+    __builtin_amdgcn_s_waitcnt(0);
+    __builtin_amdgcn_wave_barrier();
+    s_ds[lane] = dux;
+    s_db[lane] = dvx;
+  }
+  __syncthreads();
+
+  float pg[VEC], pb[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) pg[e] = pb[e] = 0.f;
+#pragma unroll
+  for (int q = 0; q < P; ++q) {
+    const int r = q * RPP + wave * RPW + lane / LPR;
+    const int t = t0 + r;
+    if (t < p.L && col_ok) {
+      float f[VEC], d[VEC], o[VEC];
+      Vec<DT>::unpack(xv[q], f);
+      Vec<DT>::unpack(dv[q], d);
+      const bool valid = s_valid[r] != 0;
+      const float u = s_u[r], rs = s_r[r], ux = s_ux[r], dux = s_ds[r], dvx = s_db[r];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        o[e] = valid ? d[e] * rs * gm[e] + (dux + 2.f * dvx * (f[e] - ux)) * inv_dg : 0.f;
+        if (valid) {
+          pg[e] += d[e] * (f[e] - u) * rs;
+          pb[e] += d[e];
+        }
+      }
+      const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
+      *reinterpret_cast<uint4*>(static_cast<typename Elem<DT>::type*>(p.y) + off) = Vec<DT>::pack(o);
+    }
+  }
+  // per-tile column sums of the gamma / beta gradients
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1) {
+      pg[e] += __shfl_xor(pg[e], off, 64);
+      pb[e] += __shfl_xor(pb[e], off, 64);
+    }
+    if (lane < LPR) {
+      s_pg[wave][col * VEC + e] = pg[e];
+      s_pb[wave][col * VEC + e] = pb[e];
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < LPR * VEC; i += kThreads) {
+    if (i < p.Dg) {
+      float a = 0.f, c = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        a += s_pg[w][i];
+        c += s_pb[w][i];
+      }
+      const int64_t o = (static_cast<int64_t>(b) * p.NT + j) * p.D + g * p.Dg + i;
+      p.part_g[o] = a;
+      p.part_b[o] = c;
+    }
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kWave) void tsn_bwd_serial_kernel(const TsnParams p) {
+  const int chain = blockIdx.x;
+  const int b = chain / p.G, g = chain % p.G;
+  const int lane = threadIdx.x;
+  const float inv_dg = 1.f / static_cast<float>(p.Dg);
+  float ug = ldT<DT>(p.dmean, chain), vg = ldT<DT>(p.dvar, chain);
+  int64_t m0 = p.prev_count[b];
+  // per-(batch) partial sums live in part_g/part_b rows [b] (NT == 1 layout)
+  for (int i = lane; i < p.Dg; i += kWave) {
+    p.part_g[static_cast<int64_t>(b) * p.D + g * p.Dg + i] = 0.f;
+    p.part_b[static_cast<int64_t>(b) * p.D + g * p.Dg + i] = 0.f;
+  }
+  for (int t = p.L - 1; t >= 0; --t) {
+    const int64_t row = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg;
+    const bool valid = p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0;
+    if (!valid) {
+      for (int i = lane; i < p.Dg; i += kWave) stT<DT>(p.y, row + i, 0.f);
+      continue;
+    }
+    const int64_t so = (static_cast<int64_t>(b) * p.L + t) * p.G + g;
+    const float u = p.cummean_in[so], r = p.cumrstd_in[so];
+    const float prev_u = t == 0 ? ldT<DT>(p.prev_mean, chain) : p.cummean_in[so - p.G];
+    const float c1 = static_cast<float>(m0 - 1) / static_cast<float>(m0);
+    const float c2 = 1.f / static_cast<float>(m0);
+    --m0;
+    float sx = 0.f, sds = 0.f, sdb = 0.f;
+    for (int i = lane; i < p.Dg; i += kWave) {
+      const float xx = ldT<DT>(p.x, row + i), d = ldT<DT>(p.dy, row + i);
+      const float w = ldT<DT>(p.gamma, g * p.Dg + i);
+      sx += xx;
+      sds += d * (xx - u) * w;
+      sdb += d * w;
+    }
+    const float ux = wave_sum(sx) * inv_dg;
+    const float ds = wave_sum(sds), db = wave_sum(sdb);
+    const float du = ug - r * db;
+    const float dvv = vg - 0.5f * r * r * r * ds;
+    const float dux = c2 * du + 2.f * c1 * c2 * dvv * (ux - prev_u);
+    const float dvx = c2 * dvv;
+    for (int i = lane; i < p.Dg; i += kWave) {
+      const float xx = ldT<DT>(p.x, row + i), d = ldT<DT>(p.dy, row + i);
+      const float w = ldT<DT>(p.gamma, g * p.Dg + i);
+      stT<DT>(p.y, row + i, d * r * w + (dux + 2.f * dvx * (xx - ux)) * inv_dg);
+      p.part_g[static_cast<int64_t>(b) * p.D + g * p.Dg + i] += d * (xx - u) * r;
+      p.part_b[static_cast<int64_t>(b) * p.D + g * p.Dg + i] += d;
+    }
+    ug = c1 * du - 2.f * c1 * c2 * dvv * (ux - prev_u);
+    vg = c1 * dvv;
+  }
+  if (lane == 0) {
+    stT<DT>(p.mean, chain, ug);
+    stT<DT>(p.var, chain, vg);
+  }
+}
+
+// dgamma[h] = sum_rows part_g[row][h] (same for dbeta), rows = B*NT
+template <int DT>
+__global__ void tsn_param_grad_kernel(const float* part_g, const float* part_b, int rows, int D,
+                                      void* dgamma, void* dbeta) {
+  const int h = blockIdx.x * blockDim.x + threadIdx.x;
+  if (h >= D) return;
+  float a = 0.f, c = 0.f, ca = 0.f, cc = 0.f;  // Kahan-compensated column sums
+  for (int r = 0; r < rows; ++r) {
+    const float ya = part_g[static_cast<int64_t>(r) * D + h] - ca;
+    const float ta = a + ya;
+    ca = (ta - a) - ya;
+    a = ta;
+    const float yc = part_b[static_cast<int64_t>(r) * D + h] - cc;
+    const float tc = c + yc;
+    cc = (tc - c) - yc;
+    c = tc;
+  }
+  stT<DT>(dgamma, h, a);
+  stT<DT>(dbeta, h, c);
+}
+
+// ------------------------------ host side --------------------------------------
+inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+struct WsLayout {
+  int64_t ticket_off, nbefore_off, rec_off, rec_words, part_off, total;
+};
+WsLayout ws_layout(int64_t B, int64_t L, int64_t D, int64_t G, int words, bool partials) {
+  const int64_t NT = (L + kTL - 1) / kTL;
+  WsLayout w;
+  w.ticket_off = 0;
+  w.nbefore_off = 256;
+  w.rec_off = align_up(w.nbefore_off + B * (NT + 1) * 4, 256);
+  w.rec_words = B * G * NT * words;
+  w.part_off = align_up(w.rec_off + w.rec_words * 8, 256);
+  w.total = w.part_off + (partials ? 2 * B * NT * D * 4 : 0);
+  return w;
+}
+
+bool fast_path_ok(int dtype, int64_t D, int64_t Dg, const void* a, const void* b, const void* c) {
+  const int vec = dtype == MEGA_F32 ? 4 : 8;
+  const auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  return Dg % vec == 0 && D % vec == 0 && Dg / vec <= 64 && al(a) && al(b) && (c == nullptr || al(c));
+}
+
+template <int DT, bool FWD>
+int launch_fast(const TsnParams& p, int64_t tiles, hipStream_t s) {
+  const int vec = DT == MEGA_F32 ? 4 : 8;
+  const int lanes = p.Dg / vec;
+  const dim3 grid(static_cast<unsigned>(tiles));
+#define MEGA_TSN_LAUNCH(LPR)                                              \
+  do {                                                                    \
+    if (FWD) tsn_fwd_kernel<DT, LPR><<<grid, kThreads, 0, s>>>(p);        \
+    else tsn_bwd_kernel<DT, LPR><<<grid, kThreads, 0, s>>>(p);            \
+  } while (0)
+  if (lanes <= 4) MEGA_TSN_LAUNCH(4);
+  else if (lanes <= 8) MEGA_TSN_LAUNCH(8);
+  else if (lanes <= 16) MEGA_TSN_LAUNCH(16);
+  else if (lanes <= 32) MEGA_TSN_LAUNCH(32);
+  else MEGA_TSN_LAUNCH(64);
+#undef MEGA_TSN_LAUNCH
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
+}
+
+template <int DT>
+int tsn_fwd_impl(TsnParams p, void* workspace, hipStream_t s) {
+  const int64_t NT = p.NT;
+  if (fast_path_ok(DT, p.D, p.Dg, p.x, p.y, nullptr)) {
+    const WsLayout w = ws_layout(p.B, p.L, p.D, p.G, kFwdWords, false);
+    char* ws = static_cast<char*>(workspace);
+    p.ticket = reinterpret_cast<int*>(ws + w.ticket_off);
+    int* nbefore = reinterpret_cast<int*>(ws + w.nbefore_off);
+    p.nbefore = nbefore;
+    p.rec = reinterpret_cast<unsigned long long*>(ws + w.rec_off);
+    const int prep_blocks = static_cast<int>(std::max<int64_t>(p.B, std::min<int64_t>(1024, (w.rec_words + 255) / 256)));
+    tsn_prep_kernel<<<prep_blocks, 256, 0, s>>>(p.ticket, p.rec, w.rec_words, p.mask, nbefore, p.B,
+                                                p.L, static_cast<int>(NT));
+    MEGA_CHECK_LAUNCH();
+    return launch_fast<DT, true>(p, static_cast<int64_t>(p.B) * p.G * NT, s);
+  }
+  tsn_fwd_serial_kernel<DT><<<p.B * p.G, kWave, 0, s>>>(p);
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
+}
+
+template <int DT>
+int tsn_bwd_impl(TsnParams p, void* dgamma, void* dbeta, void* workspace, hipStream_t s) {
+  const int64_t NT = p.NT;
+  char* ws = static_cast<char*>(workspace);
+  const WsLayout w = ws_layout(p.B, p.L, p.D, p.G, kBwdWords, true);
+  p.part_g = reinterpret_cast<float*>(ws + w.part_off);
+  p.part_b = p.part_g + static_cast<int64_t>(p.B) * NT * p.D;
+  int rows;
+  if (fast_path_ok(DT, p.D, p.Dg, p.x, p.y, p.dy)) {
+    p.ticket = reinterpret_cast<int*>(ws + w.ticket_off);
+    int* nbefore = reinterpret_cast<int*>(ws + w.nbefore_off);
+    p.nbefore = nbefore;
+    p.rec = reinterpret_cast<unsigned long long*>(ws + w.rec_off);
+    const int prep_blocks = static_cast<int>(std::max<int64_t>(p.B, std::min<int64_t>(1024, (w.rec_words + 255) / 256)));
+    tsn_prep_kernel<<<prep_blocks, 256, 0, s>>>(p.ticket, p.rec, w.rec_words, p.mask, nbefore, p.B,
+                                                p.L, static_cast<int>(NT));
+    MEGA_CHECK_LAUNCH();
+    const int rc = launch_fast<DT, false>(p, static_cast<int64_t>(p.B) * p.G * NT, s);
+    if (rc != MEGA_OK) return rc;
+    rows = static_cast<int>(p.B * NT);
+  } else {
+    tsn_bwd_serial_kernel<DT><<<p.B * p.G, kWave, 0, s>>>(p);
+    MEGA_CHECK_LAUNCH();
+    rows = p.B;
+  }
+  tsn_param_grad_kernel<DT><<<(p.D + 255) / 256, 256, 0, s>>>(p.part_g, p.part_b, rows, p.D, dgamma, dbeta);
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
+}
+
+}  // namespace
+}  // namespace mega
+
+using namespace mega;
+
+extern "C" int64_t mega_group_timestep_norm_workspace_bytes(int64_t B, int64_t L, int64_t D,
+                                                            int64_t G, int backward) {
+  if (B <= 0 || L <= 0 || D <= 0 || G <= 0) return 256;
+  return ws_layout(B, L, D, G, backward ? kBwdWords : kFwdWords, backward != 0).total;
+}
+
+static int check_dims(const char* who, int64_t B, int64_t L, int64_t D, int64_t G) {
+  MEGA_CHECK_ARG(B >= 0 && L >= 0 && D >= 1 && G >= 1, "%s: bad sizes", who);
+  MEGA_CHECK_ARG(D % G == 0, "%s: num_features %lld not divisible by num_groups %lld", who,
+                 (long long)D, (long long)G);
+  MEGA_CHECK_ARG(B * G <= 0x7fffffff && L <= 0x7fffffff && D <= 0x7fffffff, "%s: size too large", who);
+  MEGA_CHECK_ARG(B * G * ((L + kTL - 1) / kTL) <= 0x7fffffff, "%s: too many tiles", who);
+  return MEGA_OK;
+}
+
+extern "C" int mega_group_timestep_norm_fwd(const void* x, int dtype, const int64_t* prev_count,
+                                            const void* prev_mean, const void* prev_var,
+                                            const void* gamma, const void* beta,
+                                            const uint8_t* padding_mask, int64_t B, int64_t L,
+                                            int64_t D, int64_t G, double eps, void* y,
+                                            int64_t* count, void* mean, void* var, float* cummean,
+                                            float* cumrstd, void* workspace, void* stream) {
+  MEGA_CHECK_ARG(valid_dtype(dtype), "mega_group_timestep_norm_fwd: bad dtype %d", dtype);
+  int rc = check_dims("mega_group_timestep_norm_fwd", B, L, D, G);
+  if (rc != MEGA_OK) return rc;
+  MEGA_CHECK_ARG(x && prev_count && prev_mean && prev_var && gamma && beta && y && count && mean &&
+                     var && cummean && cumrstd && workspace,
+                 "mega_group_timestep_norm_fwd: null pointer");
+  if (B == 0) return MEGA_OK;
+  TsnParams p{};
+  p.x = x; p.gamma = gamma; p.beta = beta; p.mask = padding_mask; p.prev_count = prev_count;
+  p.prev_mean = prev_mean; p.prev_var = prev_var; p.y = y; p.count = count; p.mean = mean;
+  p.var = var; p.cummean = cummean; p.cumrstd = cumrstd;
+  p.B = (int)B; p.L = (int)L; p.D = (int)D; p.G = (int)G; p.Dg = (int)(D / G);
+  p.NT = (int)((L + kTL - 1) / kTL); p.eps = (float)eps;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MEGA_CHECK_ARG(L >= 1, "mega_group_timestep_norm_fwd: empty sequence");
+  switch (dtype) {
+    case MEGA_F32: return tsn_fwd_impl<MEGA_F32>(p, workspace, s);
+    case MEGA_BF16: return tsn_fwd_impl<MEGA_BF16>(p, workspace, s);
+    default: return tsn_fwd_impl<MEGA_F16>(p, workspace, s);
+  }
+}
+
+extern "C" int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, const void* dvar,
+                                            const void* x, int dtype, const void* prev_mean,
+                                            const int64_t* count, const float* cummean,
+                                            const float* cumrstd, const void* gamma,
+                                            const uint8_t* padding_mask, int64_t B, int64_t L,
+                                            int64_t D, int64_t G, void* dx, void* dprev_mean,
+                                            void* dprev_var, void* dgamma, void* dbeta,
+                                            void* workspace, void* stream) {
+  MEGA_CHECK_ARG(valid_dtype(dtype), "mega_group_timestep_norm_bwd: bad dtype %d", dtype);
+  int rc = check_dims("mega_group_timestep_norm_bwd", B, L, D, G);
+  if (rc != MEGA_OK) return rc;
+  MEGA_CHECK_ARG(dy && dmean && dvar && x && prev_mean && count && cummean && cumrstd && gamma &&
+                     dx && dprev_mean && dprev_var && dgamma && dbeta && workspace,
+                 "mega_group_timestep_norm_bwd: null pointer");
+  MEGA_CHECK_ARG(B >= 1 && L >= 1, "mega_group_timestep_norm_bwd: empty input");
+  TsnParams p{};
+  p.x = x; p.dy = dy; p.gamma = gamma; p.mask = padding_mask; p.prev_count = count;
+  p.prev_mean = prev_mean; p.dmean = dmean; p.dvar = dvar; p.cummean_in = cummean;
+  p.cumrstd_in = cumrstd; p.y = dx; p.mean = dprev_mean; p.var = dprev_var;
+  p.B = (int)B; p.L = (int)L; p.D = (int)D; p.G = (int)G; p.Dg = (int)(D / G);
+  p.NT = (int)((L + kTL - 1) / kTL);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case MEGA_F32: return tsn_bwd_impl<MEGA_F32>(p, dgamma, dbeta, workspace, s);
+    case MEGA_BF16: return tsn_bwd_impl<MEGA_BF16>(p, dgamma, dbeta, workspace, s);
+    default: return tsn_bwd_impl<MEGA_F16>(p, dgamma, dbeta, workspace, s);
+  }
+}

@@ -145,3 +145,104 @@ def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
                   _lib.ptr(kc), _lib.i64(B), _lib.i64(D), _lib.i64(L), _lib.ptr(dx), _lib.ptr(dk),
                   _lib.stream_ptr(dev))
     return dx, dk.to(k_dtype)
+
+
+# --------------------------------------------------------------------------
+# group_timestep_norm (reference: csrc/ops/timestep_norm.cc:621-705)
+# --------------------------------------------------------------------------
+def _tsn_workspace(B, L, D, G, backward, dev):
+    fn = _lib.load().mega_group_timestep_norm_workspace_bytes
+    fn.restype = _lib.ctypes.c_int64
+    nbytes = int(fn(_lib.i64(B), _lib.i64(L), _lib.i64(D), _lib.i64(G), _lib.i32(1 if backward else 0)))
+    return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+
+def _mask_bytes(padding_mask):
+    if padding_mask is None:
+        return None
+    if padding_mask.dtype != torch.bool:
+        raise RuntimeError("padding_mask must be a bool tensor")
+    return padding_mask.contiguous().view(torch.uint8)
+
+
+def group_timestep_norm_fwd(
+    x: torch.Tensor,
+    prev_count: torch.Tensor,
+    prev_mean: torch.Tensor,
+    prev_var: torch.Tensor,
+    gamma: torch.Tensor,
+    beta: torch.Tensor,
+    padding_mask: Optional[torch.Tensor],
+    num_groups: int,
+    eps: float,
+):
+    """(y, count, mean, var, cummean, cumrstd); tensors other than count /
+    mask / the float32 statistics must share x's dtype, as in the reference
+    (timestep_norm_kernel.cu:1270-1273)."""
+    dev = _require_cuda(x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask)
+    if x.dim() != 3:
+        raise RuntimeError("x must be (B, L, D)")
+    B, L, D = x.shape
+    for name, t in (("prev_mean", prev_mean), ("prev_var", prev_var), ("gamma", gamma), ("beta", beta)):
+        if t.dtype != x.dtype:
+            raise RuntimeError(f"{name} must have x's dtype {x.dtype} (got {t.dtype})")
+    if prev_count.dtype != torch.int64:
+        raise RuntimeError("prev_count must be int64")
+    G = int(num_groups)
+    xc = x.contiguous()
+    y = torch.empty_like(xc)
+    count = torch.empty_like(prev_count, memory_format=torch.contiguous_format)
+    mean = torch.empty((B, G), dtype=x.dtype, device=dev)
+    var = torch.empty((B, G), dtype=x.dtype, device=dev)
+    cummean = torch.empty((B, L, G), dtype=torch.float32, device=dev)
+    cumrstd = torch.empty((B, L, G), dtype=torch.float32, device=dev)
+    mask = _mask_bytes(padding_mask)
+    ws = _tsn_workspace(B, L, D, G, False, dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_group_timestep_norm_fwd", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
+                  _lib.ptr(prev_count.contiguous()), _lib.ptr(prev_mean.contiguous()),
+                  _lib.ptr(prev_var.contiguous()), _lib.ptr(gamma.contiguous()), _lib.ptr(beta.contiguous()),
+                  _lib.ptr(mask), _lib.i64(B), _lib.i64(L), _lib.i64(D), _lib.i64(G), _lib.f64(eps),
+                  _lib.ptr(y), _lib.ptr(count), _lib.ptr(mean), _lib.ptr(var), _lib.ptr(cummean),
+                  _lib.ptr(cumrstd), _lib.ptr(ws), _lib.stream_ptr(dev))
+    return y, count, mean, var, cummean, cumrstd
+
+
+def group_timestep_norm_bwd(
+    y_grad: torch.Tensor,
+    mean_grad: torch.Tensor,
+    var_grad: torch.Tensor,
+    x: torch.Tensor,
+    prev_mean: torch.Tensor,
+    count: torch.Tensor,
+    cummean: torch.Tensor,
+    cumrstd: torch.Tensor,
+    gamma: torch.Tensor,
+    padding_mask: Optional[torch.Tensor],
+    num_groups: int,
+):
+    """(dx, dprev_mean, dprev_var, dgamma, dbeta)."""
+    dev = _require_cuda(y_grad, mean_grad, var_grad, x, prev_mean, count, cummean, cumrstd, gamma, padding_mask)
+    B, L, D = x.shape
+    G = int(num_groups)
+    for name, t in (("y_grad", y_grad), ("mean_grad", mean_grad), ("var_grad", var_grad),
+                    ("prev_mean", prev_mean), ("gamma", gamma)):
+        if t.dtype != x.dtype:
+            raise RuntimeError(f"{name} must have x's dtype {x.dtype} (got {t.dtype})")
+    xc, dy = x.contiguous(), y_grad.contiguous()
+    dx = torch.empty_like(xc)
+    dpm = torch.empty((B, G), dtype=x.dtype, device=dev)
+    dpv = torch.empty((B, G), dtype=x.dtype, device=dev)
+    dg = torch.empty((D,), dtype=x.dtype, device=dev)
+    db = torch.empty((D,), dtype=x.dtype, device=dev)
+    mask = _mask_bytes(padding_mask)
+    ws = _tsn_workspace(B, L, D, G, True, dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_group_timestep_norm_bwd", _lib.ptr(dy), _lib.ptr(mean_grad.contiguous()),
+                  _lib.ptr(var_grad.contiguous()), _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
+                  _lib.ptr(prev_mean.contiguous()), _lib.ptr(count.contiguous()),
+                  _lib.ptr(cummean.contiguous()), _lib.ptr(cumrstd.contiguous()), _lib.ptr(gamma.contiguous()),
+                  _lib.ptr(mask), _lib.i64(B), _lib.i64(L), _lib.i64(D), _lib.i64(G), _lib.ptr(dx),
+                  _lib.ptr(dpm), _lib.ptr(dpv), _lib.ptr(dg), _lib.ptr(db), _lib.ptr(ws),
+                  _lib.stream_ptr(dev))
+    return dx, dpm, dpv, dg, db
