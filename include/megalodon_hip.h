@@ -149,6 +149,42 @@ int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, const void* 
                                  void* dprev_var, void* dgamma, void* dbeta,
                                  void* workspace, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Chunk attention (causal inside each chunk), fused fp32 softmax.
+ *
+ * Replaces attention_fwd(q, k, v, scale, dropout=0, use_causal_mask) -> (y, w)
+ *   reference: megalodon/csrc/ops/attention_kernel.cu:40-133,261-281,
+ *              megalodon/csrc/softmax.cuh:86-131, binding attention.cc:28.
+ *   q (B, L1, NH, H1), k (B, L2, NH, H1), v (B, L2, NH, H2), y (B, L1, NH, H2),
+ *   w (B, NH, L1, L2), all of `dtype` (MEGA_BF16 or MEGA_F16), contiguous; B
+ *   counts chunks (the module views (batch, L) as (batch*L/chunk, chunk)).
+ *   S = scale * q k^T rounded to `dtype`; row r keeps columns 0..r when
+ *   `causal` (L1 == L2 required), all columns otherwise; P = softmax in fp32,
+ *   stored in `dtype` into w; y = P v.  With `causal`, w is written only up to
+ *   the end of the 256-column block holding the diagonal of each row (zeros
+ *   above the diagonal inside that block); the blocks to the right are never
+ *   read by the backward and are left untouched.  DropKey dropout is not
+ *   implemented (dropout must be 0).
+ *   `workspace`: mega_attention_workspace_bytes(B, L1, L2, NH, H1, H2, 0) bytes.
+ * ---------------------------------------------------------------------- */
+int64_t mega_attention_workspace_bytes(int64_t B, int64_t L1, int64_t L2, int64_t NH,
+                                       int64_t H1, int64_t H2, int backward);
+int mega_attention_fwd(const void* q, const void* k, const void* v, int dtype,
+                       int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1,
+                       int64_t H2, double scale, int causal, void* y, void* w,
+                       void* workspace, void* stream);
+
+/* Replaces attention_bwd(dy, q, k, v, w, scale, use_causal_mask) -> (dq, dk, dv)
+ *   reference: attention_kernel.cu:135-257,283-303, softmax.cuh:198-234,
+ *              binding attention.cc:29.
+ *   dv = P^T dy; dP = dy v^T; dS = P o (dP - rowsum(P o dP)); dq = scale dS k;
+ *   dk = scale dS^T q.  `w` is the forward's output.
+ *   `workspace`: mega_attention_workspace_bytes(B, L1, L2, NH, H1, H2, 1) bytes. */
+int mega_attention_bwd(const void* dy, const void* q, const void* k, const void* v,
+                       const void* w, int dtype, int64_t B, int64_t L1, int64_t L2,
+                       int64_t NH, int64_t H1, int64_t H2, double scale, int causal,
+                       void* dq, void* dk, void* dv, void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

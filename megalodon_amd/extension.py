@@ -246,3 +246,63 @@ def group_timestep_norm_bwd(
                   _lib.ptr(dpm), _lib.ptr(dpv), _lib.ptr(dg), _lib.ptr(db), _lib.ptr(ws),
                   _lib.stream_ptr(dev))
     return dx, dpm, dpv, dg, db
+
+
+# --------------------------------------------------------------------------
+# attention (reference: csrc/ops/attention.cc:28-29, attention_kernel.cu:261-303)
+# --------------------------------------------------------------------------
+def _attn_workspace(B, L1, L2, NH, H1, H2, backward, dev):
+    fn = _lib.load().mega_attention_workspace_bytes
+    fn.restype = _lib.ctypes.c_int64
+    nbytes = int(fn(_lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH), _lib.i64(H1), _lib.i64(H2),
+                    _lib.i32(1 if backward else 0)))
+    return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+
+def _attn_dims(q, k, v):
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise RuntimeError("q, k, v must be (B, L, N, H)")
+    B, L1, NH, H1 = q.shape
+    L2, H2 = k.shape[1], v.shape[3]
+    if k.shape != (B, L2, NH, H1) or v.shape != (B, L2, NH, H2):
+        raise RuntimeError(f"attention: inconsistent shapes q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError("q, k, v must share one dtype")
+    return B, L1, L2, NH, H1, H2
+
+
+def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, dropout: float,
+                  use_causal_mask: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(y, w): y (B, L1, N, H2), w = softmax probabilities (B, N, L1, L2)."""
+    dev = _require_cuda(q, k, v)
+    if dropout != 0.0:
+        raise NotImplementedError("DropKey dropout is not implemented (dropout must be 0)")
+    B, L1, L2, NH, H1, H2 = _attn_dims(q, k, v)
+    qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
+    y = torch.empty((B, L1, NH, H2), dtype=v.dtype, device=dev)
+    w = torch.empty((B, NH, L1, L2), dtype=v.dtype, device=dev)
+    ws = _attn_workspace(B, L1, L2, NH, H1, H2, False, dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_attention_fwd", _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc),
+                  _lib.i32(_lib.dtype_code(q.dtype)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH),
+                  _lib.i64(H1), _lib.i64(H2), _lib.f64(scale), _lib.i32(1 if use_causal_mask else 0),
+                  _lib.ptr(y), _lib.ptr(w), _lib.ptr(ws), _lib.stream_ptr(dev))
+    return y, w
+
+
+def attention_bwd(y_grad: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w: torch.Tensor,
+                  scale: float, use_causal_mask: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dq, dk, dv)."""
+    dev = _require_cuda(y_grad, q, k, v, w)
+    B, L1, L2, NH, H1, H2 = _attn_dims(q, k, v)
+    if w.shape != (B, NH, L1, L2) or y_grad.shape != (B, L1, NH, H2):
+        raise RuntimeError("attention_bwd: w / y_grad shapes do not match q, k, v")
+    qc, kc, vc, dy, wc = q.contiguous(), k.contiguous(), v.contiguous(), y_grad.contiguous(), w.contiguous()
+    dq, dk, dv = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc)
+    ws = _attn_workspace(B, L1, L2, NH, H1, H2, True, dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_attention_bwd", _lib.ptr(dy), _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc), _lib.ptr(wc),
+                  _lib.i32(_lib.dtype_code(q.dtype)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH),
+                  _lib.i64(H1), _lib.i64(H2), _lib.f64(scale), _lib.i32(1 if use_causal_mask else 0),
+                  _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(ws), _lib.stream_ptr(dev))
+    return dq, dk, dv

@@ -1,5 +1,8 @@
 """Fused ops with the reference's names (megalodon/modules/fused_ops/__init__.py:1-14)."""
+from .attention import (swift_efficient_attention, swift_efficient_attention_bwd,
+                        swift_efficient_attention_fwd)
 from .ema_parameters import ema_parameters
 from .fftconv import fftconv
 
-__all__ = ["ema_parameters", "fftconv"]
+__all__ = ["ema_parameters", "fftconv", "swift_efficient_attention", "swift_efficient_attention_fwd",
+           "swift_efficient_attention_bwd"]

@@ -1,5 +1,7 @@
 """Modules with the reference's names (megalodon/modules/__init__.py:1-15) for the hot path."""
+from .chunk_attention import _InnerAttention, apply_rotary_emb
 from .complex_exponential_moving_average import MultiHeadComplexEMA
 from .timestep_norm import TimestepNorm, TimestepNormFunc, timestep_norm
 
-__all__ = ["MultiHeadComplexEMA", "TimestepNorm", "TimestepNormFunc", "timestep_norm"]
+__all__ = ["MultiHeadComplexEMA", "TimestepNorm", "TimestepNormFunc", "timestep_norm", "_InnerAttention",
+           "apply_rotary_emb"]

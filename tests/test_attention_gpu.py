@@ -1,0 +1,114 @@
+"""Parity of the HIP chunk attention with the float64 oracle.  Tolerance:
+rel err (max|a-b|/max|b|) <= 2e-2 for bfloat16 / float16 tensors (forward
+values and the gradients of q, k, v)."""
+import pytest
+import torch
+
+from conftest import rel_err
+from megalodon_amd import extension as ops
+from megalodon_amd import synthetic
+from megalodon_amd.fused_ops import swift_efficient_attention
+from megalodon_amd.modules import _InnerAttention
+from oracle import attention as oa
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def _run(B, L1, L2, NH, H1, H2, causal, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(B, L1, NH, H1, generator=g) / H1 ** 0.5).to(dtype)
+    k = (torch.randn(B, L2, NH, H1, generator=g) / H1 ** 0.5).to(dtype)
+    v = (torch.randn(B, L2, NH, H2, generator=g) / H2 ** 0.5).to(dtype)
+    dy = torch.randn(B, L1, NH, H2, generator=g).to(dtype)
+    y, w = ops.attention_fwd(q.cuda(), k.cuda(), v.cuda(), scale, 0.0, causal)
+    wy, wp = oa.chunk_attention_fwd(q, k, v, scale, causal)
+    assert y.shape == (B, L1, NH, H2) and w.shape == (B, NH, L1, L2) and y.dtype == dtype
+    assert rel_err(y, wy) <= TOL
+    if causal:
+        # compare the probabilities on and below the diagonal (blocks right of the diagonal block are not written)
+        assert rel_err(torch.tril(w.float()), wp) <= TOL
+    else:
+        assert rel_err(w, wp) <= TOL
+    dq, dk, dv = ops.attention_bwd(dy.cuda(), q.cuda(), k.cuda(), v.cuda(), w, scale, causal)
+    wdq, wdk, wdv = oa.chunk_attention_bwd(dy, q, k, v, scale, causal)
+    assert rel_err(dq, wdq) <= TOL and rel_err(dk, wdk) <= TOL and rel_err(dv, wdv) <= TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,NH,H1,H2", [
+    (2, 256, 2, 64, 128),     # exactly one tile
+    (1, 512, 1, 256, 256),    # 2x2 tiles: off-diagonal tile skipping
+    (2, 300, 3, 32, 72),      # ragged edges in every dimension
+    (1, 1024, 2, 256, 512),   # config-3 head dims (qk 256), shorter chunk
+    (3, 50, 2, 16, 24),       # tiny, rows not multiples of 8 (unaligned operand path)
+    (1, 1, 1, 8, 8),          # single query
+])
+def test_causal_fwd_bwd(B, L, NH, H1, H2, dtype):
+    _run(B, L, L, NH, H1, H2, True, dtype, seed=L + H2)
+
+
+@pytest.mark.parametrize("B,L1,L2,NH,H1,H2", [(2, 1, 77, 2, 32, 64), (1, 130, 260, 1, 64, 64)])
+def test_non_causal_rectangular(B, L1, L2, NH, H1, H2):
+    _run(B, L1, L2, NH, H1, H2, False, torch.bfloat16, seed=7, scale=0.5)
+
+
+def test_config3_shape_one_chunk():
+    """BASELINE config 3 shape (chunk 4096, 4 heads, qk 256, value 2048), one chunk."""
+    io = synthetic.attention_inputs(1, 4096, 4, 256, 2048, 1003)
+    y, w = ops.attention_fwd(io["q"].cuda(), io["k"].cuda(), io["v"].cuda(), 1.0, 0.0, True)
+    wy, _ = oa.chunk_attention_fwd(io["q"], io["k"], io["v"], 1.0, True)
+    assert rel_err(y, wy) <= TOL
+    dq, dk, dv = ops.attention_bwd(io["dy"].cuda(), io["q"].cuda(), io["k"].cuda(), io["v"].cuda(), w, 1.0, True)
+    wdq, wdk, wdv = oa.chunk_attention_bwd(io["dy"], io["q"], io["k"], io["v"], 1.0, True)
+    assert rel_err(dq, wdq) <= TOL and rel_err(dk, wdk) <= TOL and rel_err(dv, wdv) <= TOL
+
+
+def test_full_config3_properties():
+    """Size-independent checks on all 8 chunks x 4 heads of config 3: chunks are
+    independent (a permutation of chunks permutes the output), row 0 of every
+    chunk returns v[0], and y stays inside the convex hull of the values."""
+    io = synthetic.attention_inputs(8, 4096, 4, 256, 2048, 1003)
+    q, k, v = io["q"].cuda(), io["k"].cuda(), io["v"].cuda()
+    y, _ = ops.attention_fwd(q, k, v, 1.0, 0.0, True)
+    perm = torch.tensor([3, 0, 7, 1, 6, 2, 5, 4], device="cuda")
+    yp, _ = ops.attention_fwd(q[perm].contiguous(), k[perm].contiguous(), v[perm].contiguous(), 1.0, 0.0, True)
+    assert torch.equal(yp, y[perm])
+    assert rel_err(y[:, 0], v[:, 0]) <= 1e-2
+    assert y.float().abs().max() <= v.float().abs().max() * 1.01
+
+
+def test_autograd_function_and_module():
+    torch.manual_seed(0)
+    bs, slen, NH, zd, vd, chunk = 2, 512, 2, 32, 64, 256
+    attn = _InnerAttention(zd, vd, NH, chunk, 0.0, "fused").cuda()
+    g = torch.Generator().manual_seed(3)
+    xq = (torch.randn(bs, slen, NH * zd, generator=g) / zd ** 0.5).bfloat16()
+    xk = (torch.randn(bs, slen, NH * zd, generator=g) / zd ** 0.5).bfloat16()
+    xv = torch.randn(bs, slen, NH * vd, generator=g).bfloat16()
+    dy = torch.randn(bs, slen, NH * vd, generator=g).bfloat16()
+    cq, ck, cv = [t.cuda().requires_grad_(True) for t in (xq, xk, xv)]
+    out, cache = attn(cq, ck, cv, None, None)
+    assert cache is None and out.shape == (bs, slen, NH * vd)
+    out.backward(dy.cuda())
+    nc = slen // chunk
+    oq = xq.view(bs * nc, chunk, NH, zd)
+    okk = xk.view(bs * nc, chunk, NH, zd)
+    ov = xv.view(bs * nc, chunk, NH, vd)
+    wy, _ = oa.chunk_attention_fwd(oq, okk, ov, 1.0, True)
+    assert rel_err(out, wy.reshape(bs, slen, -1)) <= TOL
+    wdq, wdk, wdv = oa.chunk_attention_bwd(dy.view(bs * nc, chunk, NH, vd), oq, okk, ov, 1.0, True)
+    assert rel_err(cq.grad, wdq.reshape(bs, slen, -1)) <= TOL
+    assert rel_err(ck.grad, wdk.reshape(bs, slen, -1)) <= TOL
+    assert rel_err(cv.grad, wdv.reshape(bs, slen, -1)) <= TOL
+
+
+def test_unsupported_cases_fail_loudly():
+    q = torch.zeros(1, 8, 1, 8, device="cuda", dtype=torch.bfloat16)
+    k = torch.zeros(1, 16, 1, 8, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="not implemented"):
+        ops.attention_fwd(q, k, k, 1.0, 0.0, True)   # causal with a key prefix
+    with pytest.raises(NotImplementedError):
+        ops.attention_fwd(q, q, q, 1.0, 0.1, True)   # DropKey
+    with pytest.raises(RuntimeError, match="bfloat16"):
+        ops.attention_fwd(q.float(), q.float(), q.float(), 1.0, 0.0, True)
