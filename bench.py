@@ -36,7 +36,7 @@ def cpu_baseline(B, D, N, L, seed, budget_s=25.0):
     torch.set_num_threads(cores)
     os.environ.setdefault("OMP_NUM_THREADS", str(cores))
     lib = native.port()
-    Ds = 64
+    Ds = 512
     prm = synthetic.cema_params(D, N, seed)
     io = synthetic.cema_inputs(B, Ds, L, seed, torch.bfloat16)
     p, lq, g = prm["p"][:Ds], prm["q"][:Ds].log(), prm["gamma"][:Ds]
@@ -147,6 +147,43 @@ def main():
     kernels["ema_weight_fwd_GBps"] = 4 * E / (kernels["ema_weight_fwd_ms"] * 1e-3) / 1e9
     kernels["ema_weight_bwd_GBps"] = 4 * E / (kernels["ema_weight_bwd_ms"] * 1e-3) / 1e9
 
+    # the other hot-path operators at their BASELINE shapes (configs 2 and 3), device events
+    def dev_ms(fn, n):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    from megalodon_amd import extension as ops
+    other = {}
+    tB, tL, tD, tG = 4, 8192, 4096, 32
+    tio = {k_: v_.to(dev) for k_, v_ in synthetic.timestep_norm_inputs(tB, tL, tD, tG, 1002).items()}
+    tE = tB * tL * tD
+    fwd = lambda: ops.group_timestep_norm_fwd(tio["x"], tio["prev_count"], tio["prev_mean"], tio["prev_var"],
+                                              tio["gamma"], tio["beta"], tio["mask"], tG, 1e-5)
+    ty, tcount, tmean, tvar, tcm, tcr = fwd()
+    ms = dev_ms(fwd, 10)
+    other["timestep_norm_fwd"] = {"ms": ms, "GBps": 4 * tE / ms / 1e6, "frac_hbm": 4 * tE / ms / 1e6 / HBM_PEAK_GBS}
+    ms = dev_ms(lambda: ops.group_timestep_norm_bwd(tio["dy"], tio["dmean"], tio["dvar"], tio["x"], tio["prev_mean"],
+                                                    tcount, tcm, tcr, tio["gamma"], tio["mask"], tG), 10)
+    other["timestep_norm_bwd"] = {"ms": ms, "GBps": 6 * tE / ms / 1e6, "frac_hbm": 6 * tE / ms / 1e6 / HBM_PEAK_GBS}
+    del tio, ty, tcm, tcr
+    aio = {k_: v_.to(dev) for k_, v_ in synthetic.attention_inputs(8, 4096, 4, 256, 2048, 1003).items()}
+    pairs = 4096 * 4097 // 2
+    f_fwd, f_bwd = 2 * pairs * (256 + 2048) * 32, 2 * pairs * (2 * 256 + 2 * 2048) * 32
+    ay, aw = ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True)
+    ms = dev_ms(lambda: ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True), 3)
+    other["attention_fwd"] = {"ms": ms, "TFLOPs": f_fwd / ms / 1e9, "frac_mfma_bf16": f_fwd / ms / 1e9 / 2516.6}
+    ms = dev_ms(lambda: ops.attention_bwd(aio["dy"], aio["q"], aio["k"], aio["v"], aw, 1.0, True), 3)
+    other["attention_bwd"] = {"ms": ms, "TFLOPs": f_bwd / ms / 1e9, "frac_mfma_bf16": f_bwd / ms / 1e9 / 2516.6}
+    del aio, ay, aw
+    torch.cuda.empty_cache()
+
     result = {
         "metric": "Megalodon layer fwd+bwd tokens/s at L=32K, 1 GPU; CEMA+FFT-conv HBM GB/s (% peak)",
         "value": B * L / (dt / args.steps),
@@ -169,6 +206,7 @@ def main():
             "frac": achieved / HBM_PEAK_GBS, "traffic": None,
         },
         "kernels": kernels,
+        "other_ops": other,
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(B, D, N, L, seed)
