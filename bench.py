@@ -184,6 +184,33 @@ def main():
     del aio, ay, aw
     torch.cuda.empty_cache()
 
+    # config 4: one full 7B-style block forward+backward (random init std 0.02, bf16)
+    from megalodon_amd.modules import MegaBlock
+    torch.manual_seed(1004)
+    blk = MegaBlock(model_dim=4096, z_dim=1024, value_dim=8192, num_heads=4, cema_ndim=16, chunk_size=4096,
+                    ffn_hidden_dim=11008, norm_num_groups=32).to(dev).bfloat16()
+    gb = torch.Generator().manual_seed(1004)
+    bx = (torch.rand(1, 32768, 4096, generator=gb) * 2 - 1).bfloat16().to(dev).requires_grad_(True)
+    bdy = torch.randn(1, 32768, 4096, generator=gb).bfloat16().to(dev)
+
+    def block_step():
+        bx.grad = None
+        for prm in blk.parameters():
+            prm.grad = None
+        o, _ = blk(bx)
+        o.backward(bdy)
+
+    block_step()
+    torch.cuda.synchronize()
+    tb0 = time.perf_counter()
+    for _ in range(3):
+        block_step()
+    torch.cuda.synchronize()
+    bms = (time.perf_counter() - tb0) / 3 * 1e3
+    other["block_config4_fwd_bwd"] = {"ms": bms, "tokens_per_s": 32768 / (bms * 1e-3)}
+    del blk, bx, bdy
+    torch.cuda.empty_cache()
+
     result = {
         "metric": "Megalodon layer fwd+bwd tokens/s at L=32K, 1 GPU; CEMA+FFT-conv HBM GB/s (% peak)",
         "value": B * L / (dt / args.steps),

@@ -1,0 +1,121 @@
+"""`MovingAverageGatedAttention` and `MegaBlock` for one device
+(megalodon/modules/moving_average_gated_attention.py:145-353,
+megalodon/model/mega.py:43-88): TimestepNorm -> CEMA -> RMSNorm -> z/q/k, v, r
+projections -> chunk attention -> gate -> wh1 + wh2 -> residual, then the
+normalised feed-forward network.  World size 1: the Column/RowParallelLinear
+layers are `nn.Linear`, the chunk-parallel send/recv and the key/value cache
+branches are not part of this path, dropout is 0."""
+import math
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+from torch.nn import Parameter
+
+from .chunk_attention import _InnerAttention
+from .complex_exponential_moving_average import MultiHeadComplexEMA
+from .layer_norm import FusedRMSNorm
+from .normalized_feedforward_network import NormalizedFeedForwardNetwork
+from .timestep_norm import TimestepNorm
+
+
+class MovingAverageGatedAttention(nn.Module):
+    """Exponential Moving Average Gated Attention."""
+
+    def __init__(self, mdim: int, zdim: int, hdim: int, ndim: int, num_heads: int, dropout: float = 0.0,
+                 attention_dropout: float = 0.0, hidden_dropout: float = 0.0, chunk_size: int = 2048,
+                 efficient_attn: Optional[str] = "fused", norm_num_groups: Optional[int] = None,
+                 norm_affine: bool = True, norm_eps: float = 1e-5, init_std: float = 0.02):
+        super().__init__()
+        assert dropout == 0.0 and attention_dropout == 0.0 and hidden_dropout == 0.0, \
+            "dropout is outside the path built here"
+        self.mdim, self.hdim, self.zdim, self.ndim = mdim, hdim, zdim, ndim
+        self.num_heads = num_heads
+        assert zdim % num_heads == 0 and hdim % num_heads == 0
+        self.z_head_dim = zdim // num_heads
+        self.v_head_dim = hdim // num_heads
+        self.local_heads = num_heads
+        self.chunk_size = chunk_size
+        self.efficient_attn = efficient_attn
+
+        self.timenorm = TimestepNorm(mdim, norm_num_groups, eps=norm_eps)
+        self.cema = MultiHeadComplexEMA(mdim, ndim)
+        self.rmsnorm = FusedRMSNorm(mdim, elementwise_affine=norm_affine, eps=norm_eps)
+        self.znorm = FusedRMSNorm(self.z_head_dim, elementwise_affine=False, eps=norm_eps)
+
+        self.wv = nn.Linear(mdim, hdim, bias=True)
+        self.wz = nn.Linear(mdim, zdim, bias=True)
+        self.wr = nn.Linear(mdim, hdim, bias=True)
+        self.wh1 = nn.Linear(mdim, mdim, bias=True)
+        self.wh2 = nn.Linear(hdim, mdim, bias=False)
+        for lin in (self.wv, self.wz, self.wr, self.wh1, self.wh2):
+            nn.init.normal_(lin.weight, mean=0.0, std=init_std)
+            if lin.bias is not None:
+                nn.init.zeros_(lin.bias)
+        self.inner_attention = _InnerAttention(self.z_head_dim, self.v_head_dim, self.local_heads,
+                                               self.chunk_size, attention_dropout, efficient_attn)
+        self.gamma = Parameter(torch.zeros(2, self.z_head_dim * self.local_heads))
+        self.beta = Parameter(torch.zeros(2, self.z_head_dim * self.local_heads))
+
+    def forward(self, x: Tensor, freqs_cis: Optional[Tensor] = None, mask: Optional[Tensor] = None, cache=None):
+        if cache is not None:
+            raise NotImplementedError("cached inference is not implemented")
+        bsz, seq_len, _ = x.size()
+        residual = x
+
+        # B x L x D
+        out_tsn, prev_count, prev_mean, prev_var = self.timenorm(x, None, None, None)
+        # B x D x L
+        out_cema, _ = self.cema(out_tsn.transpose(1, 2), None, compute_last_state=False)
+        # B x L x D
+        out_cema = out_cema.transpose(1, 2)
+        mx = self.rmsnorm(out_cema)
+
+        # B x L x S -> B x L x H x S/H -> B x L x S
+        z = self.wz(mx).view(bsz, seq_len, self.local_heads, self.z_head_dim)
+        z = self.znorm(z).view(bsz, seq_len, -1)
+        # B x L x 1 x S -> B x L x 2 x S
+        gamma = (self.gamma + 1.0) / math.sqrt(self.z_head_dim)
+        z = z.unsqueeze(2) * gamma + self.beta
+        q, k = torch.unbind(z, dim=2)
+
+        # B x L x E
+        v = F.silu(self.wv(out_tsn))
+        r = F.silu(self.wr(mx))
+
+        attn, _ = self.inner_attention(q.contiguous(), k.contiguous(), v, mask, freqs_cis, None)
+        attn = attn * r
+
+        # B x L x E -> B x L x D
+        h = self.wh1(mx) + self.wh2(attn)
+        out = h + residual
+        return out, None
+
+    def extra_repr(self) -> str:
+        return 'edim={}, zdim={}, hdim={}, heads={}, chunk={}, eff_attn={}'.format(
+            self.mdim, self.zdim, self.hdim, self.num_heads, self.chunk_size, self.efficient_attn)
+
+
+class MegaBlock(nn.Module):
+    """One Megalodon layer: gated attention + normalised FFN (model/mega.py:43-88)."""
+
+    def __init__(self, model_dim: int, z_dim: int, value_dim: int, num_heads: int, cema_ndim: int,
+                 chunk_size: int, ffn_hidden_dim: int, norm_num_groups: int, swiglu: bool = True,
+                 efficient_attn: Optional[str] = "fused", norm_affine: bool = True, norm_eps: float = 1e-5,
+                 rescale_nffn: bool = False, layer_id: int = 0, init_std: float = 0.02):
+        super().__init__()
+        self.layer_id = layer_id
+        self.mega = MovingAverageGatedAttention(
+            mdim=model_dim, zdim=z_dim, hdim=value_dim, num_heads=num_heads, ndim=cema_ndim,
+            chunk_size=chunk_size, efficient_attn=efficient_attn, norm_num_groups=norm_num_groups,
+            norm_affine=norm_affine, norm_eps=norm_eps, init_std=init_std)
+        rescale = 0.1 * (0.5 ** layer_id) if rescale_nffn else None
+        self.nffn = NormalizedFeedForwardNetwork(
+            model_dim=model_dim, ffn_hidden_dim=ffn_hidden_dim, swiglu=swiglu, norm_affine=norm_affine,
+            norm_eps=norm_eps, rescale=rescale, init_std=init_std)
+
+    def forward(self, x: Tensor, freqs_cis: Optional[Tensor] = None, mask: Optional[Tensor] = None, cache=None):
+        y, cache = self.mega(x, freqs_cis, mask, cache)
+        out = self.nffn(y, x)
+        return out, cache

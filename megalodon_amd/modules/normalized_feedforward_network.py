@@ -1,0 +1,47 @@
+"""`NormalizedFeedForwardNetwork` (megalodon/modules/normalized_feedforward_network.py:15-98)
+for model-parallel world size 1: Column/RowParallelLinear are plain `nn.Linear`
+(megalodon/modules/model_parallel/layers.py:222-235,321-341), dropout 0."""
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from .layer_norm import FusedLayerNorm
+
+
+class NormalizedFeedForwardNetwork(nn.Module):
+    def __init__(self, model_dim, ffn_hidden_dim, dropout=0.0, hidden_dropout=0.0, swiglu=False,
+                 norm_affine=True, norm_eps=1e-5, rescale=None, init_std=0.02):
+        super().__init__()
+        assert dropout == 0.0 and hidden_dropout == 0.0, "dropout is outside the path built here"
+        self.model_dim = model_dim
+        self.hidden_dim = ffn_hidden_dim
+        self.swiglu = swiglu
+        self.rescale_init = rescale
+        self.norm = FusedLayerNorm(model_dim, elementwise_affine=norm_affine, eps=norm_eps)
+        self.fc1 = nn.Linear(model_dim, ffn_hidden_dim, bias=False)
+        self.fc2 = nn.Linear(ffn_hidden_dim, model_dim, bias=False)
+        self.fc3 = nn.Linear(model_dim, ffn_hidden_dim, bias=False) if swiglu else None
+        for lin in (self.fc1, self.fc2, self.fc3):
+            if lin is not None:
+                nn.init.normal_(lin.weight, mean=0.0, std=init_std)
+        if rescale is None:
+            self.register_parameter('alpha', None)
+        else:
+            assert rescale > 0., 'Layer scale init value should be positive.'
+            self.alpha = nn.Parameter(torch.full((model_dim,), rescale))
+
+    def rescale(self, x: torch.Tensor) -> torch.Tensor:
+        return x if self.alpha is None else (self.alpha * x)
+
+    def forward(self, x, residual):
+        x = self.norm(x)
+        if self.swiglu:
+            hidden = F.silu(self.fc1(x)) * self.fc3(x)
+        else:
+            hidden = F.silu(self.fc1(x))
+        x = self.fc2(hidden)
+        return self.rescale(x) + residual
+
+    def extra_repr(self) -> str:
+        return 'dim={}, hdim={}, swiglu={}, rescale={}'.format(self.model_dim, self.hidden_dim, self.swiglu,
+                                                             self.rescale_init)

@@ -104,8 +104,10 @@ class TimestepNorm(nn.Module):
         if prev_var is None:
             prev_var = self.prior_logv.exp().expand(batch_size, -1).contiguous()
 
-        output = timestep_norm(x, prev_count, prev_mean, prev_var,
-                               self.weight + 1.0, self.bias, padding_mask,
+        # the operator wants statistics and affine parameters in x's dtype
+        # (timestep_norm_kernel.cu:1270-1273 reads them as data_ptr<T>())
+        output = timestep_norm(x, prev_count, prev_mean.to(x), prev_var.to(x),
+                               (self.weight + 1.0).to(x), self.bias.to(x), padding_mask,
                                self.groups_per_partition, self.eps)
         return output
 
