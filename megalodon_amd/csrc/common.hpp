@@ -38,11 +38,14 @@ int set_error(int code, const char* fmt, ...);
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t v) {
   return __uint_as_float(static_cast<uint32_t>(v) << 16);
 }
+// gfx950 converts in hardware (v_cvt_pk_bf16_f32, round to nearest even)
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);  // NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const bf16x2_t v = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+  return __builtin_bit_cast(uint32_t, v);
 }
 __device__ __forceinline__ float f16_bits_to_float(uint16_t v) {
   return __half2float(__ushort_as_half(v));
@@ -84,6 +87,27 @@ __device__ __forceinline__ cf cmulc(cf a, cf b) {  // a * conj(b)
 }
 __device__ __forceinline__ cf cadd(cf a, cf b) { return {a.x + b.x, a.y + b.y}; }
 __device__ __forceinline__ cf csub(cf a, cf b) { return {a.x - b.x, a.y - b.y}; }
+
+// ---- DPP row reductions --------------------------------------------------------
+// v + (v moved by a DPP pattern inside the 16-lane row); folds into one
+// v_add_f32_dpp.  0xB1 / 0x4E = quad_perm [1,0,3,2] / [2,3,0,1], 0x141 =
+// row_half_mirror, 0x140 = row_mirror.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v),
+                                                                    CTRL, 0xf, 0xf, true));
+}
+// sum over aligned groups of W lanes (W = 2..64), result in every lane of the group
+template <int W>
+__device__ __forceinline__ float group_sum(float v) {
+  if (W >= 2) v = dpp_add<0xB1>(v);
+  if (W >= 4) v = dpp_add<0x4E>(v);
+  if (W >= 8) v = dpp_add<0x141>(v);
+  if (W >= 16) v = dpp_add<0x140>(v);
+  if (W >= 32) v += __shfl_xor(v, 16, 64);
+  if (W >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
 
 // ---- wave64 reductions ------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {

@@ -105,10 +105,7 @@ template <> struct Pair<MEGA_BF16> {
     lo = __uint_as_float(v << 16);
     hi = __uint_as_float(v & 0xffff0000u);
   }
-  static __device__ __forceinline__ type pack(float lo, float hi) {
-    return static_cast<uint32_t>(float_to_bf16_bits(lo)) |
-           (static_cast<uint32_t>(float_to_bf16_bits(hi)) << 16);
-  }
+  static __device__ __forceinline__ type pack(float lo, float hi) { return pack_bf16x2(lo, hi); }
 };
 template <> struct Pair<MEGA_F16> {
   using type = uint32_t;

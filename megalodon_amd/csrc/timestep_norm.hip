@@ -131,12 +131,8 @@ template <> struct Vec<MEGA_BF16> {
     }
   }
   static __device__ __forceinline__ uint4 pack(const float* f) {
-    uint32_t w[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      w[i] = static_cast<uint32_t>(float_to_bf16_bits(f[2 * i])) |
-             (static_cast<uint32_t>(float_to_bf16_bits(f[2 * i + 1])) << 16);
-    return make_uint4(w[0], w[1], w[2], w[3]);
+    return make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                      pack_bf16x2(f[6], f[7]));
   }
 };
 template <> struct Vec<MEGA_F16> {
@@ -170,6 +166,7 @@ __device__ __forceinline__ void stT(void* p, int64_t i, float v) {
 
 template <int LPR>
 __device__ __forceinline__ float row_sum(float v) {  // sum over the LPR lanes of a row
+  if (LPR <= 16) return group_sum<LPR>(v);  // inside one 16-lane DPP row
 #pragma unroll
   for (int off = LPR / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
   return v;
@@ -746,25 +743,35 @@ __global__ __launch_bounds__(kWave) void tsn_bwd_serial_kernel(const TsnParams p
   }
 }
 
-// dgamma[h] = sum_rows part_g[row][h] (same for dbeta), rows = B*NT
+// dgamma[h] = sum_rows part_g[row][h] (same for dbeta), rows = B*NT.  A workgroup
+// owns 64 columns; its 4 waves split the rows (Kahan-compensated partial sums in
+// a fixed order: deterministic), then combine through LDS.
 template <int DT>
-__global__ void tsn_param_grad_kernel(const float* part_g, const float* part_b, int rows, int D,
-                                      void* dgamma, void* dbeta) {
-  const int h = blockIdx.x * blockDim.x + threadIdx.x;
-  if (h >= D) return;
-  float a = 0.f, c = 0.f, ca = 0.f, cc = 0.f;  // Kahan-compensated column sums
-  for (int r = 0; r < rows; ++r) {
-    const float ya = part_g[static_cast<int64_t>(r) * D + h] - ca;
-    const float ta = a + ya;
-    ca = (ta - a) - ya;
-    a = ta;
-    const float yc = part_b[static_cast<int64_t>(r) * D + h] - cc;
-    const float tc = c + yc;
-    cc = (tc - c) - yc;
-    c = tc;
+__global__ __launch_bounds__(256) void tsn_param_grad_kernel(const float* part_g, const float* part_b,
+                                                            int rows, int D, void* dgamma, void* dbeta) {
+  __shared__ float sg[4][64], sb[4][64];
+  const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
+  const int h = blockIdx.x * 64 + lane;
+  float a = 0.f, c = 0.f, ca = 0.f, cc = 0.f;
+  if (h < D) {
+    for (int r = w; r < rows; r += 4) {
+      const float ya = part_g[static_cast<int64_t>(r) * D + h] - ca;
+      const float ta = a + ya;
+      ca = (ta - a) - ya;
+      a = ta;
+      const float yc = part_b[static_cast<int64_t>(r) * D + h] - cc;
+      const float tc = c + yc;
+      cc = (tc - c) - yc;
+      c = tc;
+    }
   }
-  stT<DT>(dgamma, h, a);
-  stT<DT>(dbeta, h, c);
+  sg[w][lane] = a;
+  sb[w][lane] = c;
+  __syncthreads();
+  if (w == 0 && h < D) {
+    stT<DT>(dgamma, h, (sg[0][lane] + sg[1][lane]) + (sg[2][lane] + sg[3][lane]));
+    stT<DT>(dbeta, h, (sb[0][lane] + sb[1][lane]) + (sb[2][lane] + sb[3][lane]));
+  }
 }
 
 // ------------------------------ host side --------------------------------------
@@ -857,7 +864,7 @@ int tsn_bwd_impl(TsnParams p, void* dgamma, void* dbeta, void* workspace, hipStr
     MEGA_CHECK_LAUNCH();
     rows = p.B;
   }
-  tsn_param_grad_kernel<DT><<<(p.D + 255) / 256, 256, 0, s>>>(p.part_g, p.part_b, rows, p.D, dgamma, dbeta);
+  tsn_param_grad_kernel<DT><<<(p.D + 63) / 64, 256, 0, s>>>(p.part_g, p.part_b, rows, p.D, dgamma, dbeta);
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
 }
