@@ -32,8 +32,12 @@ def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
 
-def _compile(src: Path, obj_dir: Path, extra: list[str]) -> Path:
+def _compile(src: Path, obj_dir: Path, extra: list[str], force: bool = True) -> Path:
     obj = obj_dir / (src.stem + ".o")
+    if not force and obj.exists():
+        deps = [src, *CSRC.glob("*.hpp"), PKG_DIR.parent / "include" / "megalodon_hip.h"]
+        if all(obj.stat().st_mtime > d.stat().st_mtime for d in deps):
+            return obj
     cmd = [HIPCC, *FLAGS, *extra, "-c", str(src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -41,8 +45,11 @@ def _compile(src: Path, obj_dir: Path, extra: list[str]) -> Path:
     return obj
 
 
-def build_library(verbose: bool = True, extra: list[str] | None = None, jobs: int = 8) -> Path:
-    """Compile every ``csrc/*.hip`` and link ``libmegalodon_hip.so``."""
+def build_library(verbose: bool = True, extra: list[str] | None = None, jobs: int = 8,
+                  force: bool = True) -> Path:
+    """Compile every ``csrc/*.hip`` and link ``libmegalodon_hip.so``.  With
+    ``force=False`` objects newer than their source and the shared headers are
+    reused (developer iterations only)."""
     extra = list(extra or [])
     obj_dir = PKG_DIR / "build"
     obj_dir.mkdir(exist_ok=True)
@@ -51,7 +58,7 @@ def build_library(verbose: bool = True, extra: list[str] | None = None, jobs: in
     if verbose:
         print(f"[megalodon_amd] hipcc {ARCH}: {', '.join(s.name for s in srcs)}", flush=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(lambda s: _compile(s, obj_dir, extra), srcs))
+        objs = list(ex.map(lambda s: _compile(s, obj_dir, extra, force), srcs))
     tmp = LIB_PATH.with_suffix(".so.tmp")
     cmd = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -64,4 +71,6 @@ def build_library(verbose: bool = True, extra: list[str] | None = None, jobs: in
 
 
 if __name__ == "__main__":
-    build_library(extra=sys.argv[1:])
+    args = sys.argv[1:]
+    incremental = "--incremental" in args
+    build_library(extra=[a for a in args if a != "--incremental"], force=not incremental)
