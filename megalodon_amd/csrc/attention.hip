@@ -25,23 +25,38 @@ namespace mega {
 namespace {
 
 constexpr int kTile = 256;     // workgroup tile (M and N)
-constexpr int kSlab = 64;      // k elements staged per iteration
-constexpr int kPitch = kSlab + 8;  // LDS row pitch in elements (144 B: conflict-free 16 B reads)
+constexpr int kSlab = 32;      // k elements staged per iteration
+// LDS slab layout: 16-byte chunks (8 k values of one row), chunk (c, row) at
+// index c * kChunkPitch + row.  A fragment read then has consecutive lanes on
+// consecutive chunks, and the 4 (c) x 4 (row) chunks a group of 16 lanes writes
+// land on 16 different bank groups (260 = 4 mod 16).
+constexpr int kChunkPitch = kTile + 4;
+constexpr int kOperandElems = (kSlab / 8) * kChunkPitch * 8;  // elements per operand slab
 constexpr int kThreads = 256;
+constexpr int kXcds = 8;       // accelerator dies, each with a private L2
+constexpr int kRing = 3;       // slabs in flight in registers (prefetch distance)
+constexpr int kEpiPitch = 128 + 8;  // epilogue staging pitch (elements) of a wave's 128x128 tile
+constexpr size_t kGemmLds =
+    sizeof(uint16_t) * (4 * 128 * kEpiPitch > 2 * 2 * kOperandElems ? 4 * 128 * kEpiPitch
+                                                                     : 2 * 2 * kOperandElems);
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
+// native 16-byte vector: loads and stores of it are typed, so register arrays
+// of it are promoted out of memory
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
 template <int DT> struct Mma;
 template <> struct Mma<MEGA_BF16> {
-  static __device__ __forceinline__ floatx16 run(uint4 a, uint4 b, floatx16 c) {
+  static __device__ __forceinline__ floatx16 run(u32x4 a, u32x4 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
 };
 template <> struct Mma<MEGA_F16> {
-  static __device__ __forceinline__ floatx16 run(uint4 a, uint4 b, floatx16 c) {
+  static __device__ __forceinline__ floatx16 run(u32x4 a, u32x4 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
@@ -62,13 +77,13 @@ struct GemmParams {
 };
 
 template <bool ALIGNED>
-__device__ __forceinline__ uint4 load_chunk(const uint16_t* base, int64_t ld, int row, int rows,
+__device__ __forceinline__ u32x4 load_chunk(const uint16_t* base, int64_t ld, int row, int rows,
                                             int k, int kend) {
-  uint4 v = make_uint4(0, 0, 0, 0);
+  u32x4 v = {0u, 0u, 0u, 0u};
   if (row < rows && k < kend) {
     const uint16_t* p = base + static_cast<int64_t>(row) * ld + k;
     if (ALIGNED && k + 8 <= kend) {
-      v = *reinterpret_cast<const uint4*>(p);
+      v = *reinterpret_cast<const u32x4*>(p);
     } else {
       uint16_t t[8];
 #pragma unroll
@@ -82,14 +97,29 @@ __device__ __forceinline__ uint4 load_chunk(const uint16_t* base, int64_t ld, in
   return v;
 }
 
+// Workgroup barrier that waits for this wave's LDS traffic only, so global
+// loads of later slabs stay in flight across it.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <int DT, bool ALIGNED>
 __global__ __launch_bounds__(kThreads) void gemm_tn_kernel(const GemmParams p) {
   extern __shared__ __align__(16) uint16_t smem[];
-  // [buf][A|B][256][kPitch]
-  constexpr int kOperand = kTile * kPitch;
-  const int mt = blockIdx.y, nt = blockIdx.x;
+  // main loop: [buf][A|B][256][kPitch]; epilogue: [wave][128][kEpiPitch]
+  constexpr int kOperand = kOperandElems;
+  // Workgroups are handed to the 8 XCDs round-robin by linear index, and each
+  // XCD has its own L2.  Renumber so that one XCD runs a contiguous run of
+  // tiles (n fastest, then m, then batch): neighbours that share an A row
+  // block or the B matrix of a head then hit the same L2.
+  const unsigned total = gridDim.x * gridDim.y * gridDim.z;
+  const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const unsigned xcd = lin % kXcds, slot = lin / kXcds;
+  const unsigned id = xcd * (total / kXcds) + min(xcd, total % kXcds) + slot;
+  const int nt = id % gridDim.x, mt = (id / gridDim.x) % gridDim.y;
+  const int zz = id / (gridDim.x * gridDim.y);
   if (p.tri_out && nt > mt) return;
-  const int z0 = blockIdx.z / p.nh, z1 = blockIdx.z % p.nh;
+  const int z0 = zz / p.nh, z1 = zz % p.nh;
   const uint16_t* A = p.A + z0 * p.sa0 + z1 * p.sa1;
   const uint16_t* B = p.B + z0 * p.sb0 + z1 * p.sb1;
   uint16_t* C = p.C + z0 * p.sc0 + z1 * p.sc1;
@@ -97,6 +127,7 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_kernel(const GemmParams p) {
   int kb = 0, ke = p.K;
   if (p.k_mode == 1) ke = min(p.K, (mt + 1) * kTile);
   if (p.k_mode == 2) kb = min(p.K, mt * kTile);
+  const int nslab = (ke - kb + kSlab - 1) / kSlab;
 
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int wm = wave >> 1, wn = wave & 1;
@@ -109,72 +140,159 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_kernel(const GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  uint4 ra[8], rb[8];
-  auto gload = [&](int k0) {
+  // register ring: slab s lives in ring[s % kRing] from its issue (three
+  // iterations before use) until it is written to LDS
+  u32x4 ra0[4], ra1[4], ra2[4], rb0[4], rb1[4], rb2[4];
+  // ALIGNED (16-byte aligned rows, K % 32 == 0, operand extents below 2 GiB):
+  // branch-free loads from a uniform base plus 32-bit byte offsets, rows and
+  // slab index clamped into the matrix, so nothing forces a wait on the loads
+  // in flight.  Otherwise: bounds-checked element loads.
+  uint32_t offa[4], offb[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int c = tid + kThreads * i;
-      const int row = c >> 3, kc = (c & 7) * 8;
-      ra[i] = load_chunk<ALIGNED>(A, p.lda, m0 + row, p.M, k0 + kc, ke);
-      rb[i] = load_chunk<ALIGNED>(B, p.ldb, n0 + row, p.N, k0 + kc, ke);
-    }
-  };
-  auto sstore = [&](int buf) {
-    uint16_t* sa = smem + buf * 2 * kOperand;
-    uint16_t* sb = sa + kOperand;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int c = tid + kThreads * i;
-      const int row = c >> 3, kc = (c & 7) * 8;
-      *reinterpret_cast<uint4*>(sa + row * kPitch + kc) = ra[i];
-      *reinterpret_cast<uint4*>(sb + row * kPitch + kc) = rb[i];
-    }
-  };
-
-  if (kb < ke) {
-    gload(kb);
-    sstore(0);
+  for (int i = 0; i < 4; ++i) {
+    const int c = tid + kThreads * i;
+    const int row = c >> 2, kc = (c & 3) * 8;
+    offa[i] = static_cast<uint32_t>((static_cast<int64_t>(min(m0 + row, p.M - 1)) * p.lda + kb + kc) * 2);
+    offb[i] = static_cast<uint32_t>((static_cast<int64_t>(min(n0 + row, p.N - 1)) * p.ldb + kb + kc) * 2);
   }
-  __syncthreads();
-  int buf = 0;
-  for (int k0 = kb; k0 < ke; k0 += kSlab) {
-    const bool more = k0 + kSlab < ke;
-    if (more) gload(k0 + kSlab);
-    const uint16_t* sa = smem + buf * 2 * kOperand + (wm * 128 + (lane & 31)) * kPitch + 8 * (lane >> 5);
-    const uint16_t* sb = smem + buf * 2 * kOperand + kOperand + (wn * 128 + (lane & 31)) * kPitch + 8 * (lane >> 5);
-#pragma unroll
-    for (int ks = 0; ks < kSlab / 16; ++ks) {
-      uint4 fa[4], fb[4];
+  auto gload = [&](u32x4* qa, u32x4* qb, int s) {
+    if (ALIGNED) {
+      const uint32_t kbyte = static_cast<uint32_t>(min(s, nslab - 1)) * (kSlab * 2);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        fa[i] = *reinterpret_cast<const uint4*>(sa + i * 32 * kPitch + ks * 16);
-        fb[i] = *reinterpret_cast<const uint4*>(sb + i * 32 * kPitch + ks * 16);
+        qa[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(A) + (offa[i] + kbyte));
+        qb[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(B) + (offb[i] + kbyte));
       }
+    } else {
+      const int k0 = kb + s * kSlab;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = Mma<DT>::run(fa[i], fb[j], acc[i][j]);
+      for (int i = 0; i < 4; ++i) {
+        const int c = tid + kThreads * i;
+        const int row = c >> 2, kc = (c & 3) * 8;
+        qa[i] = load_chunk<false>(A, p.lda, m0 + row, p.M, k0 + kc, ke);
+        qb[i] = load_chunk<false>(B, p.ldb, n0 + row, p.N, k0 + kc, ke);
+      }
     }
-    if (more) sstore(buf ^ 1);
-    __syncthreads();
-    buf ^= 1;
-  }
+  };
+  const int st_off = ((tid & 3) * kChunkPitch + (tid >> 2)) * 8;  // + 64 rows per chunk i
+  auto sstore = [&](const u32x4* qa, const u32x4* qb, int s) {
+    uint16_t* sa = smem + (s & 1) * 2 * kOperand + st_off;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<u32x4*>(sa + i * 64 * 8) = qa[i];
+      *reinterpret_cast<u32x4*>(sa + kOperand + i * 64 * 8) = qb[i];
+    }
+  };
+  // MFMA fragments: set ks holds the k-step ks (16 k values) of a slab
+  static_assert(kSlab == 32, "the pipeline below is written for two k-steps per slab");
+  u32x4 fa0[4], fb0[4], fa1[4], fb1[4];
+  const int frag_a = ((lane >> 5) * kChunkPitch + wm * 128 + (lane & 31)) * 8;
+  const int frag_b = kOperand + ((lane >> 5) * kChunkPitch + wn * 128 + (lane & 31)) * 8;
+  auto fread = [&](u32x4* fa, u32x4* fb, int set, int buf) {
+    const uint16_t* base = smem + buf * 2 * kOperand + set * 2 * kChunkPitch * 8;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      fa[i] = *reinterpret_cast<const u32x4*>(base + frag_a + i * 32 * 8);
+      fb[i] = *reinterpret_cast<const u32x4*>(base + frag_b + i * 32 * 8);
+    }
+  };
+  auto mma = [&](const u32x4* fa, const u32x4* fb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = Mma<DT>::run(fb[j], fa[i], acc[i][j]);
+  };
 
-  // epilogue: D[i][j] of a 32x32 tile sits in lane (j = lane % 32), register
-  // r -> i = 8 (r / 4) + 4 (lane / 32) + r % 4
+  // One step per slab, one barrier per step, placed between the two k-steps:
+  //   write slab cur+1 to the other LDS buffer, request slab cur+3,
+  //   read the second fragment set of slab cur, first 16 MFMAs,
+  //   barrier,
+  //   read the first fragment set of slab cur+1, last 16 MFMAs.
+  // Each wait (LDS writes, barrier skew, fragment reads) then has 16 MFMAs
+  // already issued behind it.  Loads and LDS stores are unconditional
+  // (addresses clamped, chunks past the k range stored as zeros), so every
+  // path has the same number of loads in flight and the waits can count.
+#define MEGA_GEMM_STEP(R, CA, CB, NA, NB)                                                \
+  {                                                                        \
+    const int cur = it + (R);                                              \
+    sstore(NA, NB, cur + 1);                                               \
+    gload(CA, CB, cur + kRing);                                            \
+    fread(fa1, fb1, 1, cur & 1);                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                     \
+    mma(fa0, fb0);                                                                \
+    __builtin_amdgcn_sched_barrier(0);                                     \
+    lds_barrier();                                                         \
+    fread(fa0, fb0, 0, (cur + 1) & 1);                                               \
+    __builtin_amdgcn_sched_barrier(0);                                     \
+    mma(fa1, fb1);                                                                \
+    __builtin_amdgcn_sched_barrier(0);                                     \
+  }
+  if (nslab > 0) {
+    gload(ra0, rb0, 0);
+    gload(ra1, rb1, 1);
+    gload(ra2, rb2, 2);
+    sstore(ra0, rb0, 0);
+    lds_barrier();
+    fread(fa0, fb0, 0, 0);
+    // ring slot R held slab cur, already written to LDS, so it is free for
+    // slab cur + kRing
+    int it = 0;
+    for (; it + kRing <= nslab; it += kRing) {
+      MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
+      MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
+      MEGA_GEMM_STEP(2, ra2, rb2, ra0, rb0)
+    }
+    if (it < nslab) MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
+    if (it + 1 < nslab) MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
+    lds_barrier();  // every wave is done with the slab buffers before they are reused
+  }
+#undef MEGA_GEMM_STEP
+
+  // epilogue: stage the wave's 128x128 tile in LDS ([row][col], element type),
+  // then write it with 16-byte row segments.  The products are issued as
+  // B-fragment x A-fragment, so a 32x32 MFMA tile holds C transposed: lane l has
+  // row m = l % 32 and register r the column n = 8 (r / 4) + 4 (l / 32) + r % 4,
+  // i.e. four consecutive columns per register quad -> one 8-byte LDS write.
+  uint16_t* stage = smem + wave * 128 * kEpiPitch;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int col = n0 + wn * 128 + j * 32 + (lane & 31);
+      const int row = i * 32 + (lane & 31);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (row < p.M && col < p.N) {
-          const float v = p.alpha * acc[i][j][r];
-          C[static_cast<int64_t>(row) * p.ldc + col] =
-              DT == MEGA_BF16 ? float_to_bf16_bits(v) : float_to_f16_bits(v);
+      for (int g = 0; g < 4; ++g) {
+        const int col = j * 32 + 8 * g + 4 * (lane >> 5);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[i][j][4 * g + e];
+        uint2 w;
+        if (DT == MEGA_BF16) {
+          w.x = pack_bf16x2(v[0], v[1]);
+          w.y = pack_bf16x2(v[2], v[3]);
+        } else {
+          w.x = static_cast<uint32_t>(float_to_f16_bits(v[0])) | (static_cast<uint32_t>(float_to_f16_bits(v[1])) << 16);
+          w.y = static_cast<uint32_t>(float_to_f16_bits(v[2])) | (static_cast<uint32_t>(float_to_f16_bits(v[3])) << 16);
         }
+        *reinterpret_cast<uint2*>(stage + row * kEpiPitch + col) = w;
+      }
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave reads back only its own region
+  const bool vec_ok = (p.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+#pragma unroll 4
+  for (int i = 0; i < 32; ++i) {
+    const int c = lane + kWave * i;
+    const int row = c >> 4, kc = (c & 15) * 8;
+    const int grow = m0 + wm * 128 + row, gcol = n0 + wn * 128 + kc;
+    if (grow < p.M && gcol < p.N) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * kEpiPitch + kc);
+      uint16_t* dst = C + static_cast<int64_t>(grow) * p.ldc + gcol;
+      if (vec_ok && gcol + 8 <= p.N) {
+        *reinterpret_cast<u32x4*>(dst) = v;
+      } else {
+        const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+        for (int q = 0; q < 8; ++q)
+          if (gcol + q < p.N) dst[q] = e[q];
       }
     }
   }
@@ -207,6 +325,85 @@ __global__ __launch_bounds__(kThreads) void softmax_fwd_kernel(uint16_t* w, int 
   }
 }
 
+template <int DT>
+__device__ __forceinline__ void unpack8(const uint4& q, float* v) {
+  const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (DT == MEGA_BF16) {
+      v[2 * e] = __uint_as_float(u[e] << 16);
+      v[2 * e + 1] = __uint_as_float(u[e] & 0xffff0000u);
+    } else {
+      v[2 * e] = f16_bits_to_float(static_cast<uint16_t>(u[e] & 0xffffu));
+      v[2 * e + 1] = f16_bits_to_float(static_cast<uint16_t>(u[e] >> 16));
+    }
+  }
+}
+template <int DT>
+__device__ __forceinline__ uint4 pack8(const float* v) {
+  uint32_t u[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (DT == MEGA_BF16) {
+      u[e] = pack_bf16x2(v[2 * e], v[2 * e + 1]);
+    } else {
+      u[e] = static_cast<uint32_t>(float_to_f16_bits(v[2 * e])) |
+             (static_cast<uint32_t>(float_to_f16_bits(v[2 * e + 1])) << 16);
+    }
+  }
+  return make_uint4(u[0], u[1], u[2], u[3]);
+}
+
+// Same contract with the row held in registers: needs L2 % 8 == 0, a 16-byte
+// aligned base and L2 <= 64 * 8 * NCH; one read and one write of the row.
+template <int DT, int NCH>
+__global__ __launch_bounds__(kThreads) void softmax_fwd_vec_kernel(uint16_t* w, int L1, int L2,
+                                                                  int causal) {
+  const int lane = threadIdx.x % kWave;
+  const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
+  if (r >= L1) return;
+  uint16_t* x = w + (static_cast<int64_t>(blockIdx.y) * L1 + r) * L2;
+  const int n = causal ? min(r + 1, L2) : L2;
+  const int nz = causal ? min(L2, (r / kTile + 1) * kTile) : L2;
+  float v[NCH][8];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c8 = (lane + kWave * i) * 8;
+    if (c8 < n) {
+      unpack8<DT>(*reinterpret_cast<const uint4*>(x + c8), v[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (c8 + e >= n) v[i][e] = -INFINITY;
+        m = fmaxf(m, v[i][e]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[i][e] = -INFINITY;
+    }
+  }
+  m = wave_max(m);
+  float d = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[i][e] = __expf(v[i][e] - m);  // exp(-inf) = 0 outside the kept prefix
+      d += v[i][e];
+    }
+  d = wave_sum(d);
+  const float c = d == 0.f ? 0.f : 1.f / d;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c8 = (lane + kWave * i) * 8;
+    if (c8 < nz) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[i][e] *= c;
+      *reinterpret_cast<uint4*>(x + c8) = pack8<DT>(v[i]);
+    }
+  }
+}
+
 // dS = P o (dP - sum_j P_j dP_j), written over dP.  softmax.cuh:198-234.
 template <int DT>
 __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const uint16_t* w, uint16_t* dw,
@@ -228,6 +425,78 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const uint16_t* w
   }
 }
 
+template <int DT, int NCH>
+__global__ __launch_bounds__(kThreads) void softmax_bwd_vec_kernel(const uint16_t* w, uint16_t* dw,
+                                                                  int L1, int L2, int causal) {
+  const int lane = threadIdx.x % kWave;
+  const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
+  if (r >= L1) return;
+  const int64_t o = (static_cast<int64_t>(blockIdx.y) * L1 + r) * L2;
+  const uint16_t* pw = w + o;
+  uint16_t* pd = dw + o;
+  const int n = causal ? min(r + 1, L2) : L2;
+  const int nz = causal ? min(L2, (r / kTile + 1) * kTile) : L2;
+  float pv[NCH][8], dv[NCH][8];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c8 = (lane + kWave * i) * 8;
+    if (c8 < n) {
+      unpack8<DT>(*reinterpret_cast<const uint4*>(pw + c8), pv[i]);
+      unpack8<DT>(*reinterpret_cast<const uint4*>(pd + c8), dv[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (c8 + e >= n) pv[i][e] = 0.f, dv[i][e] = 0.f;
+        s += pv[i][e] * dv[i][e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pv[i][e] = 0.f, dv[i][e] = 0.f;
+    }
+  }
+  s = wave_sum(s);
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c8 = (lane + kWave * i) * 8;
+    if (c8 < nz) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dv[i][e] = pv[i][e] * (dv[i][e] - s);
+      *reinterpret_cast<uint4*>(pd + c8) = pack8<DT>(dv[i]);
+    }
+  }
+}
+
+template <int DT>
+int launch_softmax(const uint16_t* p, uint16_t* x, int64_t Z, int64_t L1, int64_t L2, int causal,
+                   hipStream_t s) {
+  // p == nullptr: forward over x in place; else backward with probabilities p
+  if (Z == 0 || L1 == 0 || L2 == 0) return MEGA_OK;
+  const dim3 grid((unsigned)((L1 + 3) / 4), (unsigned)Z);
+  const bool vec = L2 % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(p) % 16 == 0;
+#define MEGA_SOFTMAX(NCH)                                                                   \
+  if (p == nullptr)                                                                         \
+    softmax_fwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, causal); \
+  else                                                                                      \
+    softmax_bwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, causal);
+  if (vec && L2 <= 512) {
+    MEGA_SOFTMAX(1)
+  } else if (vec && L2 <= 1024) {
+    MEGA_SOFTMAX(2)
+  } else if (vec && L2 <= 2048) {
+    MEGA_SOFTMAX(4)
+  } else if (vec && L2 <= 4096) {
+    MEGA_SOFTMAX(8)
+  } else if (p == nullptr) {
+    softmax_fwd_kernel<DT><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, causal);
+  } else {
+    softmax_bwd_kernel<DT><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, causal);
+  }
+#undef MEGA_SOFTMAX
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
+}
+
 // ---- batched transpose of 16-bit matrices: out[z][c][r] = in[z][r][c] ----------
 struct TransParams {
   const uint16_t* in;
@@ -238,22 +507,58 @@ struct TransParams {
   int nh;
   int tri;  // 1: only 256-blocks with column block <= row block are copied
 };
-__global__ __launch_bounds__(256) void transpose_kernel(const TransParams p) {
-  __shared__ uint16_t tile[64][66];
+// 64x64 tiles through LDS; 16-byte global accesses on both sides wherever the
+// leading dimension, the batch offsets and the base allow them.
+__global__ __launch_bounds__(256) void transpose_kernel(const TransParams p, int vec_in, int vec_out) {
+  constexpr int kTp = 66;  // tile pitch in elements (33 dwords)
+  __shared__ __align__(16) uint16_t tile[64 * kTp];
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
   if (p.tri && (c0 / kTile) > (r0 / kTile)) return;
   const int z0 = blockIdx.z / p.nh, z1 = blockIdx.z % p.nh;
   const uint16_t* in = p.in + z0 * p.si0 + z1 * p.si1;
   uint16_t* out = p.out + z0 * p.so0 + z1 * p.so1;
-  const int tx = threadIdx.x % 64, ty = threadIdx.x / 64;
-  for (int i = ty; i < 64; i += 4) {
-    const int r = r0 + i, c = c0 + tx;
-    tile[i][tx] = (r < p.R && c < p.Cc) ? in[static_cast<int64_t>(r) * p.ldi + c] : static_cast<uint16_t>(0);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = threadIdx.x + 256 * i;
+    const int rr = q >> 3, cc = (q & 7) * 8;
+    const int r = r0 + rr, c = c0 + cc;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (r < p.R && c < p.Cc) {
+      const uint16_t* src = in + static_cast<int64_t>(r) * p.ldi + c;
+      if (vec_in && c + 8 <= p.Cc) {
+        v = *reinterpret_cast<const uint4*>(src);
+      } else {
+        uint16_t t[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] = c + e < p.Cc ? src[e] : static_cast<uint16_t>(0);
+        v = make_uint4(t[0] | (uint32_t)t[1] << 16, t[2] | (uint32_t)t[3] << 16,
+                       t[4] | (uint32_t)t[5] << 16, t[6] | (uint32_t)t[7] << 16);
+      }
+    }
+    uint32_t* dst = reinterpret_cast<uint32_t*>(tile + rr * kTp + cc);
+    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
   }
   __syncthreads();
-  for (int i = ty; i < 64; i += 4) {
-    const int c = c0 + i, r = r0 + tx;
-    if (c < p.Cc && r < p.R) out[static_cast<int64_t>(c) * p.ldo + r] = tile[tx][i];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = threadIdx.x + 256 * i;
+    const int cc = q >> 3, rr = (q & 7) * 8;  // output row cc, output columns rr .. rr+7
+    const int c = c0 + cc, r = r0 + rr;
+    if (c < p.Cc && r < p.R) {
+      uint16_t t[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) t[e] = tile[(rr + e) * kTp + cc];
+      uint16_t* dst = out + static_cast<int64_t>(c) * p.ldo + r;
+      if (vec_out && r + 8 <= p.R) {
+        *reinterpret_cast<uint4*>(dst) =
+            make_uint4(t[0] | (uint32_t)t[1] << 16, t[2] | (uint32_t)t[3] << 16,
+                       t[4] | (uint32_t)t[5] << 16, t[6] | (uint32_t)t[7] << 16);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (r + e < p.R) dst[e] = t[e];
+      }
+    }
   }
 }
 
@@ -263,9 +568,10 @@ int launch_gemm(const GemmParams& p, int batch, hipStream_t s) {
   if (p.M == 0 || p.N == 0 || batch == 0) return MEGA_OK;
   const auto a16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
   const bool aligned = a16(p.A) && a16(p.B) && p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa0 % 8 == 0 &&
-                       p.sa1 % 8 == 0 && p.sb0 % 8 == 0 && p.sb1 % 8 == 0;
+                       p.sa1 % 8 == 0 && p.sb0 % 8 == 0 && p.sb1 % 8 == 0 && p.K % kSlab == 0 &&
+                       p.K >= kSlab && p.M * p.lda < (1ll << 30) && p.N * p.ldb < (1ll << 30);
   const dim3 grid((p.N + kTile - 1) / kTile, (p.M + kTile - 1) / kTile, batch);
-  const size_t lds = sizeof(uint16_t) * 2 * 2 * kTile * kPitch;
+  const size_t lds = kGemmLds;
   if (aligned) {
     MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tn_kernel<DT, true>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -282,7 +588,10 @@ int launch_gemm(const GemmParams& p, int batch, hipStream_t s) {
 int launch_transpose(const TransParams& p, int batch, hipStream_t s) {
   if (p.R == 0 || p.Cc == 0 || batch == 0) return MEGA_OK;
   const dim3 grid((p.Cc + 63) / 64, (p.R + 63) / 64, batch);
-  transpose_kernel<<<grid, 256, 0, s>>>(p);
+  const auto a16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  const int vec_in = a16(p.in) && p.ldi % 8 == 0 && p.si0 % 8 == 0 && p.si1 % 8 == 0;
+  const int vec_out = a16(p.out) && p.ldo % 8 == 0 && p.so0 % 8 == 0 && p.so1 % 8 == 0;
+  transpose_kernel<<<grid, 256, 0, s>>>(p, vec_in, vec_out);
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
 }
@@ -339,11 +648,7 @@ int attn_fwd_impl(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64
   int rc = launch_gemm<DT>(g, Z, s);
   if (rc != MEGA_OK) return rc;
   // P = softmax(S) in place
-  {
-    const dim3 grid((unsigned)((L1 + 3) / 4), (unsigned)Z);
-    softmax_fwd_kernel<DT><<<grid, kThreads, 0, s>>>(w, (int)L1, (int)L2, causal);
-    MEGA_CHECK_LAUNCH();
-  }
+  if ((rc = launch_softmax<DT>(nullptr, w, Z, L1, L2, causal, s)) != MEGA_OK) return rc;
   // Vt[z][c][key]
   uint16_t* vt = ws + l.vt;
   TransParams t{};
@@ -384,11 +689,7 @@ int attn_bwd_impl(const uint16_t* dy, const uint16_t* q, const uint16_t* k, cons
   g.tri_out = causal; g.k_mode = 0;
   if ((rc = launch_gemm<DT>(g, Z, s)) != MEGA_OK) return rc;
   // dS = P o (dP - rowsum(P o dP)) in place
-  {
-    const dim3 grid((unsigned)((L1 + 3) / 4), (unsigned)Z);
-    softmax_bwd_kernel<DT><<<grid, kThreads, 0, s>>>(w, dp, (int)L1, (int)L2, causal);
-    MEGA_CHECK_LAUNCH();
-  }
+  if ((rc = launch_softmax<DT>(w, dp, Z, L1, L2, causal, s)) != MEGA_OK) return rc;
   // transposes: Kt[z][h][key], Qt[z][h][q], dYt[z][c][q], Pt[z][key][q], dSt[z][key][q]
   TransParams t{};
   t.nh = (int)NH;
