@@ -31,7 +31,11 @@ constexpr int kSlab = 32;      // k elements staged per iteration
 // consecutive chunks, and the 4 (c) x 4 (row) chunks a group of 16 lanes writes
 // land on 16 different bank groups (260 = 4 mod 16).
 constexpr int kChunkPitch = kTile + 4;
-constexpr int kOperandElems = (kSlab / 8) * kChunkPitch * 8;  // elements per operand slab
+// k-major operands keep their rows of k: 256 + 32 elements per row, so that the
+// four rows a transposing read touches start 16 banks apart.
+constexpr int kPitchT = kTile + 32;
+constexpr int kOperandElems = kSlab * kPitchT;  // elements per operand slab (either layout fits)
+static_assert((kSlab / 8) * kChunkPitch * 8 <= kOperandElems, "chunk layout must fit");
 constexpr int kThreads = 256;
 constexpr int kXcds = 8;       // accelerator dies, each with a private L2
 constexpr int kRing = 3;       // slabs in flight in registers (prefetch distance)
@@ -62,7 +66,8 @@ template <> struct Mma<MEGA_F16> {
   }
 };
 
-// C[m][n] = alpha * sum_k A[m][k] B[n][k]   (both operands k-contiguous)
+// C[m][n] = alpha * sum_k A(m, k) B(n, k); element (m, k) of an operand sits at
+// [m * ld + k], or at [k * ld + m] when the operand is flagged k-major
 struct GemmParams {
   const uint16_t* A;
   const uint16_t* B;
@@ -74,6 +79,7 @@ struct GemmParams {
   float alpha;
   int tri_out;  // 1: tiles with nt > mt are skipped (left unwritten)
   int k_mode;   // 0: all k; 1: k < (mt+1)*256; 2: k >= mt*256
+  int ta, tb;   // operand is k-major: element (m, k) at [k * ld + m]
 };
 
 template <bool ALIGNED>
@@ -103,10 +109,25 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <int DT, bool ALIGNED>
-__global__ __launch_bounds__(kThreads) void gemm_tn_kernel(const GemmParams p) {
+// Transposing LDS read (gfx950 ds_read_b64_tr_b16).  Inside each group of 16
+// lanes, source lane 4a + b supplies 4 consecutive 16-bit elements s[4a+b][0..3]
+// from its own address; destination lane 4b + c receives {s[4e + b][c]}, e =
+// 0..3.  Pointing source lane 4a + b at row k0 + a, columns m0 + 4b .. + 3 of a
+// k-major tile therefore hands lane t the column m0 + t at rows k0 .. k0 + 3:
+// the k-contiguous quad an MFMA operand wants.
+typedef short short4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint2 lds_read_tr(const uint16_t* q) {
+  const short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) short4v*)(q));
+  return __builtin_bit_cast(uint2, v);
+}
+
+// C[m][n] = alpha * sum_k A(m, k) B(n, k).  An operand is either k-contiguous
+// (rows m, `ld` between rows) or, with TA / TB, k-major (rows k, m contiguous).
+template <int DT, bool FAST, bool TA, bool TB>
+__global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
   extern __shared__ __align__(16) uint16_t smem[];
-  // main loop: [buf][A|B][256][kPitch]; epilogue: [wave][128][kEpiPitch]
+  // main loop: [buf][A|B] operand slabs; epilogue: [wave][128][kEpiPitch]
   constexpr int kOperand = kOperandElems;
   // Workgroups are handed to the 8 XCDs round-robin by linear index, and each
   // XCD has its own L2.  Renumber so that one XCD runs a contiguous run of
@@ -116,7 +137,11 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_kernel(const GemmParams p) {
   const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
   const unsigned xcd = lin % kXcds, slot = lin / kXcds;
   const unsigned id = xcd * (total / kXcds) + min(xcd, total % kXcds) + slot;
-  const int nt = id % gridDim.x, mt = (id / gridDim.x) % gridDim.y;
+  // with a triangular k range or output the work of a tile grows with mt:
+  // start the heavy rows first so the light ones fill the tail
+  const int nt = id % gridDim.x;
+  const int mt_raw = (id / gridDim.x) % gridDim.y;
+  const int mt = (p.tri_out || p.k_mode) ? static_cast<int>(gridDim.y) - 1 - mt_raw : mt_raw;
   const int zz = id / (gridDim.x * gridDim.y);
   if (p.tri_out && nt > mt) return;
   const int z0 = zz / p.nh, z1 = zz % p.nh;
@@ -140,60 +165,85 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_kernel(const GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // register ring: slab s lives in ring[s % kRing] from its issue (three
-  // iterations before use) until it is written to LDS
+  // register ring: slab s lives in ring slot s % 3 from its issue (three steps
+  // before use) until it is written to LDS
   u32x4 ra0[4], ra1[4], ra2[4], rb0[4], rb1[4], rb2[4];
-  // ALIGNED (16-byte aligned rows, K % 32 == 0, operand extents below 2 GiB):
-  // branch-free loads from a uniform base plus 32-bit byte offsets, rows and
-  // slab index clamped into the matrix, so nothing forces a wait on the loads
-  // in flight.  Otherwise: bounds-checked element loads.
+
+  // Global -> register chunk i of a thread (16 bytes):
+  //   k-contiguous operand: row (tid >> 2) + 64 i, k chunk tid & 3
+  //   k-major operand:      k row (tid >> 5) + 8 i, m chunk tid & 31
+  // FAST (16-byte aligned rows, K % 32 == 0, extents % 8 == 0 and below 1 GiB):
+  // branch-free loads from a uniform base plus 32-bit byte offsets with rows,
+  // columns and slab index clamped into the matrix, so nothing forces a wait
+  // on the loads in flight.  Otherwise: bounds-checked element loads.
   uint32_t offa[4], offb[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int c = tid + kThreads * i;
-    const int row = c >> 2, kc = (c & 3) * 8;
-    offa[i] = static_cast<uint32_t>((static_cast<int64_t>(min(m0 + row, p.M - 1)) * p.lda + kb + kc) * 2);
-    offb[i] = static_cast<uint32_t>((static_cast<int64_t>(min(n0 + row, p.N - 1)) * p.ldb + kb + kc) * 2);
+    if (TA) offa[i] = static_cast<uint32_t>(((kb + (tid >> 5) + 8 * i) * p.lda + min(m0 + (tid & 31) * 8, p.M - 8)) * 2);
+    else offa[i] = static_cast<uint32_t>((static_cast<int64_t>(min(m0 + (tid >> 2) + 64 * i, p.M - 1)) * p.lda + kb + (tid & 3) * 8) * 2);
+    if (TB) offb[i] = static_cast<uint32_t>(((kb + (tid >> 5) + 8 * i) * p.ldb + min(n0 + (tid & 31) * 8, p.N - 8)) * 2);
+    else offb[i] = static_cast<uint32_t>((static_cast<int64_t>(min(n0 + (tid >> 2) + 64 * i, p.N - 1)) * p.ldb + kb + (tid & 3) * 8) * 2);
   }
+  const uint32_t stepa = static_cast<uint32_t>((TA ? p.lda : 1) * kSlab * 2);
+  const uint32_t stepb = static_cast<uint32_t>((TB ? p.ldb : 1) * kSlab * 2);
   auto gload = [&](u32x4* qa, u32x4* qb, int s) {
-    if (ALIGNED) {
-      const uint32_t kbyte = static_cast<uint32_t>(min(s, nslab - 1)) * (kSlab * 2);
+    if (FAST) {
+      const uint32_t sc = static_cast<uint32_t>(min(s, nslab - 1));
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        qa[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(A) + (offa[i] + kbyte));
-        qb[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(B) + (offb[i] + kbyte));
+        qa[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(A) + (offa[i] + sc * stepa));
+        qb[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(B) + (offb[i] + sc * stepb));
       }
     } else {
       const int k0 = kb + s * kSlab;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int c = tid + kThreads * i;
-        const int row = c >> 2, kc = (c & 3) * 8;
-        qa[i] = load_chunk<false>(A, p.lda, m0 + row, p.M, k0 + kc, ke);
-        qb[i] = load_chunk<false>(B, p.ldb, n0 + row, p.N, k0 + kc, ke);
+        if (TA) qa[i] = load_chunk<false>(A, p.lda, k0 + (tid >> 5) + 8 * i, ke, m0 + (tid & 31) * 8, p.M);
+        else qa[i] = load_chunk<false>(A, p.lda, m0 + (tid >> 2) + 64 * i, p.M, k0 + (tid & 3) * 8, ke);
+        if (TB) qb[i] = load_chunk<false>(B, p.ldb, k0 + (tid >> 5) + 8 * i, ke, n0 + (tid & 31) * 8, p.N);
+        else qb[i] = load_chunk<false>(B, p.ldb, n0 + (tid >> 2) + 64 * i, p.N, k0 + (tid & 3) * 8, ke);
       }
     }
   };
-  const int st_off = ((tid & 3) * kChunkPitch + (tid >> 2)) * 8;  // + 64 rows per chunk i
+  // register -> LDS: chunk layout for k-contiguous operands, padded rows of k
+  // for k-major ones
+  const int st_a = TA ? (tid >> 5) * kPitchT + (tid & 31) * 8 : ((tid & 3) * kChunkPitch + (tid >> 2)) * 8;
+  const int st_b = TB ? (tid >> 5) * kPitchT + (tid & 31) * 8 : ((tid & 3) * kChunkPitch + (tid >> 2)) * 8;
   auto sstore = [&](const u32x4* qa, const u32x4* qb, int s) {
-    uint16_t* sa = smem + (s & 1) * 2 * kOperand + st_off;
+    uint16_t* sa = smem + (s & 1) * 2 * kOperand + st_a;
+    uint16_t* sb = smem + (s & 1) * 2 * kOperand + kOperand + st_b;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<u32x4*>(sa + i * 64 * 8) = qa[i];
-      *reinterpret_cast<u32x4*>(sa + kOperand + i * 64 * 8) = qb[i];
+      *reinterpret_cast<u32x4*>(sa + i * (TA ? 8 * kPitchT : 64 * 8)) = qa[i];
+      *reinterpret_cast<u32x4*>(sb + i * (TB ? 8 * kPitchT : 64 * 8)) = qb[i];
     }
   };
-  // MFMA fragments: set ks holds the k-step ks (16 k values) of a slab
+
+  // MFMA fragments: set ks holds the k-step ks (16 k values) of a slab; lane l
+  // owns row l % 32 of a 32-row tile and k values 8 (l / 32) .. + 7
   static_assert(kSlab == 32, "the pipeline below is written for two k-steps per slab");
   u32x4 fa0[4], fb0[4], fa1[4], fb1[4];
-  const int frag_a = ((lane >> 5) * kChunkPitch + wm * 128 + (lane & 31)) * 8;
-  const int frag_b = kOperand + ((lane >> 5) * kChunkPitch + wn * 128 + (lane & 31)) * 8;
+  const int tr_lane = (8 * (lane >> 5) + ((lane & 15) >> 2)) * kPitchT + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const int frag_a = TA ? tr_lane + wm * 128 : ((lane >> 5) * kChunkPitch + wm * 128 + (lane & 31)) * 8;
+  const int frag_b = kOperand + (TB ? tr_lane + wn * 128 : ((lane >> 5) * kChunkPitch + wn * 128 + (lane & 31)) * 8);
   auto fread = [&](u32x4* fa, u32x4* fb, int set, int buf) {
-    const uint16_t* base = smem + buf * 2 * kOperand + set * 2 * kChunkPitch * 8;
+    const uint16_t* base = smem + buf * 2 * kOperand;
+    const uint16_t* qa = base + frag_a + set * (TA ? 16 * kPitchT : 2 * kChunkPitch * 8);
+    const uint16_t* qb = base + frag_b + set * (TB ? 16 * kPitchT : 2 * kChunkPitch * 8);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      fa[i] = *reinterpret_cast<const u32x4*>(base + frag_a + i * 32 * 8);
-      fb[i] = *reinterpret_cast<const u32x4*>(base + frag_b + i * 32 * 8);
+      if (TA) {
+        const uint2 lo = lds_read_tr(qa + i * 32), hi = lds_read_tr(qa + i * 32 + 4 * kPitchT);
+        fa[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+      } else {
+        fa[i] = *reinterpret_cast<const u32x4*>(qa + i * 32 * 8);
+      }
+      if (TB) {
+        const uint2 lo = lds_read_tr(qb + i * 32), hi = lds_read_tr(qb + i * 32 + 4 * kPitchT);
+        fb[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+      } else {
+        fb[i] = *reinterpret_cast<const u32x4*>(qb + i * 32 * 8);
+      }
     }
   };
   auto mma = [&](const u32x4* fa, const u32x4* fb) {
@@ -209,22 +259,21 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_kernel(const GemmParams p) {
   //   barrier,
   //   read the first fragment set of slab cur+1, last 16 MFMAs.
   // Each wait (LDS writes, barrier skew, fragment reads) then has 16 MFMAs
-  // already issued behind it.  Loads and LDS stores are unconditional
-  // (addresses clamped, chunks past the k range stored as zeros), so every
+  // already issued behind it.  Loads and LDS stores are unconditional, so every
   // path has the same number of loads in flight and the waits can count.
-#define MEGA_GEMM_STEP(R, CA, CB, NA, NB)                                                \
+#define MEGA_GEMM_STEP(R, CA, CB, NA, NB)                                  \
   {                                                                        \
     const int cur = it + (R);                                              \
     sstore(NA, NB, cur + 1);                                               \
     gload(CA, CB, cur + kRing);                                            \
-    fread(fa1, fb1, 1, cur & 1);                                                     \
+    fread(fa1, fb1, 1, cur & 1);                                           \
     __builtin_amdgcn_sched_barrier(0);                                     \
-    mma(fa0, fb0);                                                                \
+    mma(fa0, fb0);                                                         \
     __builtin_amdgcn_sched_barrier(0);                                     \
     lds_barrier();                                                         \
-    fread(fa0, fb0, 0, (cur + 1) & 1);                                               \
+    fread(fa0, fb0, 0, (cur + 1) & 1);                                     \
     __builtin_amdgcn_sched_barrier(0);                                     \
-    mma(fa1, fb1);                                                                \
+    mma(fa1, fb1);                                                         \
     __builtin_amdgcn_sched_barrier(0);                                     \
   }
   if (nslab > 0) {
@@ -497,125 +546,45 @@ int launch_softmax(const uint16_t* p, uint16_t* x, int64_t Z, int64_t L1, int64_
   return MEGA_OK;
 }
 
-// ---- batched transpose of 16-bit matrices: out[z][c][r] = in[z][r][c] ----------
-struct TransParams {
-  const uint16_t* in;
-  uint16_t* out;
-  int R, Cc;
-  int64_t ldi, ldo;
-  int64_t si0, si1, so0, so1;
-  int nh;
-  int tri;  // 1: only 256-blocks with column block <= row block are copied
-};
-// 64x64 tiles through LDS; 16-byte global accesses on both sides wherever the
-// leading dimension, the batch offsets and the base allow them.
-__global__ __launch_bounds__(256) void transpose_kernel(const TransParams p, int vec_in, int vec_out) {
-  constexpr int kTp = 66;  // tile pitch in elements (33 dwords)
-  __shared__ __align__(16) uint16_t tile[64 * kTp];
-  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-  if (p.tri && (c0 / kTile) > (r0 / kTile)) return;
-  const int z0 = blockIdx.z / p.nh, z1 = blockIdx.z % p.nh;
-  const uint16_t* in = p.in + z0 * p.si0 + z1 * p.si1;
-  uint16_t* out = p.out + z0 * p.so0 + z1 * p.so1;
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int q = threadIdx.x + 256 * i;
-    const int rr = q >> 3, cc = (q & 7) * 8;
-    const int r = r0 + rr, c = c0 + cc;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (r < p.R && c < p.Cc) {
-      const uint16_t* src = in + static_cast<int64_t>(r) * p.ldi + c;
-      if (vec_in && c + 8 <= p.Cc) {
-        v = *reinterpret_cast<const uint4*>(src);
-      } else {
-        uint16_t t[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) t[e] = c + e < p.Cc ? src[e] : static_cast<uint16_t>(0);
-        v = make_uint4(t[0] | (uint32_t)t[1] << 16, t[2] | (uint32_t)t[3] << 16,
-                       t[4] | (uint32_t)t[5] << 16, t[6] | (uint32_t)t[7] << 16);
-      }
-    }
-    uint32_t* dst = reinterpret_cast<uint32_t*>(tile + rr * kTp + cc);
-    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+// ------------------------------ host side --------------------------------------
+template <int DT, bool TA, bool TB>
+int launch_gemm_t(const GemmParams& p, int batch, hipStream_t s) {
+  const auto a16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  const int64_t lim = 1ll << 30;  // elements: byte offsets stay below 2^31
+  const bool fast_a = a16(p.A) && p.lda % 8 == 0 && p.sa0 % 8 == 0 && p.sa1 % 8 == 0 &&
+                      (TA ? (p.M % 8 == 0 && p.M >= 8 && p.K * p.lda < lim) : p.M * p.lda < lim);
+  const bool fast_b = a16(p.B) && p.ldb % 8 == 0 && p.sb0 % 8 == 0 && p.sb1 % 8 == 0 &&
+                      (TB ? (p.N % 8 == 0 && p.N >= 8 && p.K * p.ldb < lim) : p.N * p.ldb < lim);
+  const bool fast = fast_a && fast_b && p.K % kSlab == 0 && p.K >= kSlab;
+  const dim3 grid((p.N + kTile - 1) / kTile, (p.M + kTile - 1) / kTile, batch);
+  const size_t lds = kGemmLds;
+  if (fast) {
+    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, true, TA, TB>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    gemm_kernel<DT, true, TA, TB><<<grid, kThreads, lds, s>>>(p);
+  } else {
+    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, false, TA, TB>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    gemm_kernel<DT, false, TA, TB><<<grid, kThreads, lds, s>>>(p);
   }
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int q = threadIdx.x + 256 * i;
-    const int cc = q >> 3, rr = (q & 7) * 8;  // output row cc, output columns rr .. rr+7
-    const int c = c0 + cc, r = r0 + rr;
-    if (c < p.Cc && r < p.R) {
-      uint16_t t[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) t[e] = tile[(rr + e) * kTp + cc];
-      uint16_t* dst = out + static_cast<int64_t>(c) * p.ldo + r;
-      if (vec_out && r + 8 <= p.R) {
-        *reinterpret_cast<uint4*>(dst) =
-            make_uint4(t[0] | (uint32_t)t[1] << 16, t[2] | (uint32_t)t[3] << 16,
-                       t[4] | (uint32_t)t[5] << 16, t[6] | (uint32_t)t[7] << 16);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (r + e < p.R) dst[e] = t[e];
-      }
-    }
-  }
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
 }
 
-// ------------------------------ host side --------------------------------------
 template <int DT>
 int launch_gemm(const GemmParams& p, int batch, hipStream_t s) {
   if (p.M == 0 || p.N == 0 || batch == 0) return MEGA_OK;
-  const auto a16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
-  const bool aligned = a16(p.A) && a16(p.B) && p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa0 % 8 == 0 &&
-                       p.sa1 % 8 == 0 && p.sb0 % 8 == 0 && p.sb1 % 8 == 0 && p.K % kSlab == 0 &&
-                       p.K >= kSlab && p.M * p.lda < (1ll << 30) && p.N * p.ldb < (1ll << 30);
-  const dim3 grid((p.N + kTile - 1) / kTile, (p.M + kTile - 1) / kTile, batch);
-  const size_t lds = kGemmLds;
-  if (aligned) {
-    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tn_kernel<DT, true>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    gemm_tn_kernel<DT, true><<<grid, kThreads, lds, s>>>(p);
-  } else {
-    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tn_kernel<DT, false>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    gemm_tn_kernel<DT, false><<<grid, kThreads, lds, s>>>(p);
-  }
-  MEGA_CHECK_LAUNCH();
-  return MEGA_OK;
+  if (p.ta) return p.tb ? launch_gemm_t<DT, true, true>(p, batch, s) : launch_gemm_t<DT, true, false>(p, batch, s);
+  return p.tb ? launch_gemm_t<DT, false, true>(p, batch, s) : launch_gemm_t<DT, false, false>(p, batch, s);
 }
-
-int launch_transpose(const TransParams& p, int batch, hipStream_t s) {
-  if (p.R == 0 || p.Cc == 0 || batch == 0) return MEGA_OK;
-  const dim3 grid((p.Cc + 63) / 64, (p.R + 63) / 64, batch);
-  const auto a16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
-  const int vec_in = a16(p.in) && p.ldi % 8 == 0 && p.si0 % 8 == 0 && p.si1 % 8 == 0;
-  const int vec_out = a16(p.out) && p.ldo % 8 == 0 && p.so0 % 8 == 0 && p.so1 % 8 == 0;
-  transpose_kernel<<<grid, 256, 0, s>>>(p, vec_in, vec_out);
-  MEGA_CHECK_LAUNCH();
-  return MEGA_OK;
-}
-
-inline int64_t up8(int64_t v) { return (v + 7) / 8 * 8; }
 
 struct AttnWs {
-  int64_t ld1, ld2;  // padded leading dimensions of transposed buffers (>= L1, L2)
-  int64_t vt, dp, kt, qt, dot, pt, dst, total;  // element offsets
+  int64_t dp, total;  // element offset of dP / dS, total bytes
 };
 AttnWs attn_ws(int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1, int64_t H2, bool bwd) {
   AttnWs w;
-  w.ld1 = up8(L1);
-  w.ld2 = up8(L2);
-  int64_t o = 0;
-  const int64_t Z = B * NH;
-  w.vt = o; o += bwd ? 0 : Z * H2 * w.ld2;
-  w.dp = o; o += bwd ? Z * L1 * L2 : 0;
-  w.kt = o; o += bwd ? Z * H1 * w.ld2 : 0;
-  w.qt = o; o += bwd ? Z * H1 * w.ld1 : 0;
-  w.dot = o; o += bwd ? Z * H2 * w.ld1 : 0;
-  w.pt = o; o += bwd ? Z * L2 * w.ld1 : 0;
-  w.dst = o; o += bwd ? Z * L2 * w.ld1 : 0;
-  w.total = (o + 8) * 2;
+  w.dp = 0;
+  w.total = ((bwd ? B * NH * L1 * L2 : 0) + 8) * 2;
   return w;
 }
 
@@ -636,7 +605,7 @@ template <int DT>
 int attn_fwd_impl(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64_t B, int64_t L1,
                   int64_t L2, int64_t NH, int64_t H1, int64_t H2, float scale, int causal,
                   uint16_t* y, uint16_t* w, uint16_t* ws, hipStream_t s) {
-  const AttnWs l = attn_ws(B, L1, L2, NH, H1, H2, false);
+  (void)ws;
   const int Z = static_cast<int>(B * NH);
   // S = scale Q K^T  -> w
   GemmParams g{};
@@ -649,18 +618,11 @@ int attn_fwd_impl(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64
   if (rc != MEGA_OK) return rc;
   // P = softmax(S) in place
   if ((rc = launch_softmax<DT>(nullptr, w, Z, L1, L2, causal, s)) != MEGA_OK) return rc;
-  // Vt[z][c][key]
-  uint16_t* vt = ws + l.vt;
-  TransParams t{};
-  t.in = v; t.out = vt; t.R = (int)L2; t.Cc = (int)H2; t.ldi = NH * H2; t.ldo = l.ld2;
-  t.si0 = L2 * NH * H2; t.si1 = H2; t.so0 = NH * H2 * l.ld2; t.so1 = H2 * l.ld2; t.nh = (int)NH;
-  rc = launch_transpose(t, Z, s);
-  if (rc != MEGA_OK) return rc;
-  // Y = P Vt^T
+  // Y = P V: V[key][c] is the k-major B operand
   GemmParams o{};
-  o.A = w; o.B = vt; o.C = y; o.M = (int)L1; o.N = (int)H2; o.K = (int)L2;
-  o.lda = L2; o.ldb = l.ld2; o.ldc = NH * H2;
-  o.sa0 = NH * L1 * L2; o.sa1 = L1 * L2; o.sb0 = NH * H2 * l.ld2; o.sb1 = H2 * l.ld2;
+  o.A = w; o.B = v; o.C = y; o.M = (int)L1; o.N = (int)H2; o.K = (int)L2;
+  o.lda = L2; o.ldb = NH * H2; o.ldc = NH * H2; o.tb = 1;
+  o.sa0 = NH * L1 * L2; o.sa1 = L1 * L2; o.sb0 = L2 * NH * H2; o.sb1 = H2;
   o.sc0 = L1 * NH * H2; o.sc1 = H2; o.nh = (int)NH; o.alpha = 1.f;
   o.tri_out = 0; o.k_mode = causal ? 1 : 0;
   return launch_gemm<DT>(o, Z, s);
@@ -674,11 +636,6 @@ int attn_bwd_impl(const uint16_t* dy, const uint16_t* q, const uint16_t* k, cons
   const AttnWs l = attn_ws(B, L1, L2, NH, H1, H2, true);
   const int Z = static_cast<int>(B * NH);
   uint16_t* dp = ws + l.dp;
-  uint16_t* kt = ws + l.kt;
-  uint16_t* qt = ws + l.qt;
-  uint16_t* dot = ws + l.dot;
-  uint16_t* pt = ws + l.pt;
-  uint16_t* dst = ws + l.dst;
   int rc;
   // dP = dY V^T
   GemmParams g{};
@@ -690,42 +647,25 @@ int attn_bwd_impl(const uint16_t* dy, const uint16_t* q, const uint16_t* k, cons
   if ((rc = launch_gemm<DT>(g, Z, s)) != MEGA_OK) return rc;
   // dS = P o (dP - rowsum(P o dP)) in place
   if ((rc = launch_softmax<DT>(w, dp, Z, L1, L2, causal, s)) != MEGA_OK) return rc;
-  // transposes: Kt[z][h][key], Qt[z][h][q], dYt[z][c][q], Pt[z][key][q], dSt[z][key][q]
-  TransParams t{};
-  t.nh = (int)NH;
-  t.in = k; t.out = kt; t.R = (int)L2; t.Cc = (int)H1; t.ldi = NH * H1; t.ldo = l.ld2;
-  t.si0 = L2 * NH * H1; t.si1 = H1; t.so0 = NH * H1 * l.ld2; t.so1 = H1 * l.ld2; t.tri = 0;
-  if ((rc = launch_transpose(t, Z, s)) != MEGA_OK) return rc;
-  t.in = q; t.out = qt; t.R = (int)L1; t.Cc = (int)H1; t.ldi = NH * H1; t.ldo = l.ld1;
-  t.si0 = L1 * NH * H1; t.si1 = H1; t.so0 = NH * H1 * l.ld1; t.so1 = H1 * l.ld1;
-  if ((rc = launch_transpose(t, Z, s)) != MEGA_OK) return rc;
-  t.in = dy; t.out = dot; t.R = (int)L1; t.Cc = (int)H2; t.ldi = NH * H2; t.ldo = l.ld1;
-  t.si0 = L1 * NH * H2; t.si1 = H2; t.so0 = NH * H2 * l.ld1; t.so1 = H2 * l.ld1;
-  if ((rc = launch_transpose(t, Z, s)) != MEGA_OK) return rc;
-  t.in = w; t.out = pt; t.R = (int)L1; t.Cc = (int)L2; t.ldi = L2; t.ldo = l.ld1;
-  t.si0 = NH * L1 * L2; t.si1 = L1 * L2; t.so0 = NH * L2 * l.ld1; t.so1 = L2 * l.ld1; t.tri = causal;
-  if ((rc = launch_transpose(t, Z, s)) != MEGA_OK) return rc;
-  t.in = dp; t.out = dst;
-  if ((rc = launch_transpose(t, Z, s)) != MEGA_OK) return rc;
-  // dQ = scale dS Kt^T
+  // dQ = scale dS K: K[key][h] is the k-major B operand
   GemmParams a{};
-  a.A = dp; a.B = kt; a.C = dq; a.M = (int)L1; a.N = (int)H1; a.K = (int)L2;
-  a.lda = L2; a.ldb = l.ld2; a.ldc = NH * H1;
-  a.sa0 = NH * L1 * L2; a.sa1 = L1 * L2; a.sb0 = NH * H1 * l.ld2; a.sb1 = H1 * l.ld2;
+  a.A = dp; a.B = k; a.C = dq; a.M = (int)L1; a.N = (int)H1; a.K = (int)L2;
+  a.lda = L2; a.ldb = NH * H1; a.ldc = NH * H1; a.tb = 1;
+  a.sa0 = NH * L1 * L2; a.sa1 = L1 * L2; a.sb0 = L2 * NH * H1; a.sb1 = H1;
   a.sc0 = L1 * NH * H1; a.sc1 = H1; a.nh = (int)NH; a.alpha = scale; a.k_mode = causal ? 1 : 0;
   if ((rc = launch_gemm<DT>(a, Z, s)) != MEGA_OK) return rc;
-  // dK = scale dSt Qt^T
+  // dK = scale dS^T Q: dS[q][key] and Q[q][h] are both k-major (k = q)
   GemmParams b{};
-  b.A = dst; b.B = qt; b.C = dk; b.M = (int)L2; b.N = (int)H1; b.K = (int)L1;
-  b.lda = l.ld1; b.ldb = l.ld1; b.ldc = NH * H1;
-  b.sa0 = NH * L2 * l.ld1; b.sa1 = L2 * l.ld1; b.sb0 = NH * H1 * l.ld1; b.sb1 = H1 * l.ld1;
+  b.A = dp; b.B = q; b.C = dk; b.M = (int)L2; b.N = (int)H1; b.K = (int)L1;
+  b.lda = L2; b.ldb = NH * H1; b.ldc = NH * H1; b.ta = 1; b.tb = 1;
+  b.sa0 = NH * L1 * L2; b.sa1 = L1 * L2; b.sb0 = L1 * NH * H1; b.sb1 = H1;
   b.sc0 = L2 * NH * H1; b.sc1 = H1; b.nh = (int)NH; b.alpha = scale; b.k_mode = causal ? 2 : 0;
   if ((rc = launch_gemm<DT>(b, Z, s)) != MEGA_OK) return rc;
-  // dV = Pt dYt^T
+  // dV = P^T dY: P[q][key] and dY[q][c] are both k-major (k = q)
   GemmParams c{};
-  c.A = pt; c.B = dot; c.C = dv; c.M = (int)L2; c.N = (int)H2; c.K = (int)L1;
-  c.lda = l.ld1; c.ldb = l.ld1; c.ldc = NH * H2;
-  c.sa0 = NH * L2 * l.ld1; c.sa1 = L2 * l.ld1; c.sb0 = NH * H2 * l.ld1; c.sb1 = H2 * l.ld1;
+  c.A = w; c.B = dy; c.C = dv; c.M = (int)L2; c.N = (int)H2; c.K = (int)L1;
+  c.lda = L2; c.ldb = NH * H2; c.ldc = NH * H2; c.ta = 1; c.tb = 1;
+  c.sa0 = NH * L1 * L2; c.sa1 = L1 * L2; c.sb0 = L1 * NH * H2; c.sb1 = H2;
   c.sc0 = L2 * NH * H2; c.sc1 = H2; c.nh = (int)NH; c.alpha = 1.f; c.k_mode = causal ? 2 : 0;
   return launch_gemm<DT>(c, Z, s);
 }
