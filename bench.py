@@ -118,7 +118,8 @@ def main():
         step()
     torch.cuda.synchronize()
 
-    log = {"mega_fftconv_fwd": [], "mega_fftconv_bwd": [], "mega_ema_weight_fwd": [], "mega_ema_weight_bwd": []}
+    log = {"mega_fftconv_residual_fwd": [], "mega_fftconv_residual_bwd": [], "mega_ema_weight_fwd": [],
+           "mega_ema_weight_bwd": []}
     _lib.set_event_log(log)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -134,12 +135,12 @@ def main():
 
     E = B * D * L
     ms_step = dt / args.steps * 1e3
-    conv_ms = avg_ms("mega_fftconv_fwd")  # one launch of the convolution kernel
+    conv_ms = avg_ms("mega_fftconv_residual_fwd")  # one launch of the convolution kernel
     conv_bytes = 8 * E  # x 2E + k 4E in, y 2E out (bf16 rows, fp32 kernel)
     achieved = conv_bytes / (conv_ms * 1e-3) / 1e9
     kernels = {
         "fftconv_fwd_ms": conv_ms,
-        "fftconv_bwd_ms": avg_ms("mega_fftconv_bwd"),
+        "fftconv_bwd_ms": avg_ms("mega_fftconv_residual_bwd"),
         "ema_weight_fwd_ms": avg_ms("mega_ema_weight_fwd"),
         "ema_weight_bwd_ms": avg_ms("mega_ema_weight_bwd"),
     }

@@ -106,6 +106,23 @@ int mega_fftconv_bwd(const void* dy, const void* x, int dtype, const float* k,
                      int64_t B, int64_t D, int64_t L, void* dx, float* dk,
                      void* stream);
 
+/* The convolution and the per-channel skip term of MultiHeadComplexEMA in one
+ * pass: y = fftconv(x, k) + omega[d] * x.
+ *   Replaces the pair `fftconv(x, k) + x * self.omega` of
+ *   megalodon/modules/complex_exponential_moving_average.py:129-141 (forward of
+ *   MultiHeadComplexEMA); omega (D) float32, the rest as mega_fftconv_fwd/bwd.
+ *   Backward: dx = (dx of the convolution) + omega[d] * dy; dk as in
+ *   mega_fftconv_bwd.  The gradient of omega is dk[:, 0]
+ *   (sum_b sum_t dy[b,d,t] x[b,d,t], the lag-0 correlation), so it has no
+ *   output of its own. */
+int mega_fftconv_residual_fwd(const void* x, int dtype, const float* k,
+                              const float* omega, int64_t B, int64_t D,
+                              int64_t L, void* y, void* stream);
+int mega_fftconv_residual_bwd(const void* dy, const void* x, int dtype,
+                              const float* k, const float* omega, int64_t B,
+                              int64_t D, int64_t L, void* dx, float* dk,
+                              void* stream);
+
 /* ------------------------------------------------------------------------
  * Group TimestepNorm (cumulative group mean / variance over time).
  *

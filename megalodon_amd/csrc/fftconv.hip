@@ -152,10 +152,12 @@ __device__ __forceinline__ void load_row(float* re, float* im, const void* row, 
 }
 
 // out[2n] = re[j], out[2n+1] = im[j] for n = t + T j (reversed when flip);
-// ACC adds to what is there (fp32 rows only).
+// ACC adds to what is there (fp32 rows only).  With `res` non-null the stored
+// value is out[m] + w * res[m] (res has the dtype and layout of the output row).
 template <int LOGM, int DT, bool VEC, bool ACC>
 __device__ __forceinline__ void store_row(const float* re, const float* im, void* row, int L,
-                                          bool flip, int t) {
+                                          bool flip, int t, const void* res = nullptr,
+                                          float w = 0.f) {
   using C = Cfg<LOGM>;
   if (VEC) {
     using P = typename Pair<DT>::type;
@@ -172,6 +174,12 @@ __device__ __forceinline__ void store_row(const float* re, const float* im, void
           lo += plo;
           hi += phi;
         }
+        if (res != nullptr) {
+          float rlo, rhi;
+          Pair<DT>::unpack(gld<P>(res, off), rlo, rhi);
+          lo = fmaf(w, rlo, lo);
+          hi = fmaf(w, rhi, hi);
+        }
         gst<P>(row, off, Pair<DT>::pack(lo, hi));
       }
     }
@@ -181,11 +189,13 @@ __device__ __forceinline__ void store_row(const float* re, const float* im, void
       const int m0 = 2 * (t + C::T * j), m1 = m0 + 1;
       if (m0 < L) {
         const int o = flip ? L - 1 - m0 : m0;
-        st<DT>(row, o, ACC ? ld<DT>(row, o) + re[j] : re[j]);
+        const float r = res != nullptr ? w * ld<DT>(res, o) : 0.f;
+        st<DT>(row, o, (ACC ? ld<DT>(row, o) + re[j] : re[j]) + r);
       }
       if (m1 < L) {
         const int o = flip ? L - 1 - m1 : m1;
-        st<DT>(row, o, ACC ? ld<DT>(row, o) + im[j] : im[j]);
+        const float r = res != nullptr ? w * ld<DT>(res, o) : 0.f;
+        st<DT>(row, o, (ACC ? ld<DT>(row, o) + im[j] : im[j]) + r);
       }
     }
   }
@@ -271,8 +281,9 @@ __device__ __forceinline__ void conv_half(const void* arow, bool flip_a, const v
   }
 }
 
-// MODE 0: out[b,d,:] = conv(a[b,d,:], k[d,:]); `flip` reverses a on load and
-//         the result on store (backward dx).  a, out have dtype DT; k is fp32.
+// MODE 0: out[b,d,:] = conv(a[b,d,:], k[d,:]) (+ omega[d] a[b,d,:] when omega is
+//         given); `flip` reverses a on load and the result on store (backward
+//         dx).  a, out have dtype DT; k is fp32.
 // MODE 1: out[d,:] (+)= reverse(conv(reverse(a[b0,d,:]), x[b0,d,:])), fp32
 //         (backward dk, one batch index per launch; `flip` != 0 accumulates).
 // Persistent: workgroup g handles rows g, g + gridDim.x, ... and owns scratch
@@ -280,7 +291,8 @@ __device__ __forceinline__ void conv_half(const void* arow, bool flip_a, const v
 template <int LOGM, int DT, int MODE, bool VEC>
 __global__ __launch_bounds__(Cfg<LOGM>::T) void fftconv_kernel(
     const void* __restrict__ a, const void* __restrict__ b, void* __restrict__ out, int rows,
-    int D, int L, int flip, const c32* __restrict__ tab, float* __restrict__ scratch_all) {
+    int D, int L, int flip, const c32* __restrict__ tab, float* __restrict__ scratch_all,
+    const float* __restrict__ omega) {
   using C = Cfg<LOGM>;
   extern __shared__ float lds[];
   float* lre = lds;
@@ -303,7 +315,10 @@ __global__ __launch_bounds__(Cfg<LOGM>::T) void fftconv_kernel(
       char* orow = static_cast<char*>(out) + row * L * esz;
       conv_half<LOGM, DT, MEGA_F32, VEC, 0>(arow, flip != 0, krow, L, t, tb, lre, lim, scratch, ore, oim);
       conv_half<LOGM, DT, MEGA_F32, VEC, 1>(arow, flip != 0, krow, L, t, tb, lre, lim, scratch, ore, oim);
-      store_row<LOGM, DT, VEC, false>(ore, oim, orow, L, flip != 0, t);
+      // optional residual: out += omega[d] * a (MODE 0 only)
+      store_row<LOGM, DT, VEC, false>(ore, oim, orow, L, flip != 0, t,
+                                      omega != nullptr ? arow : nullptr,
+                                      omega != nullptr ? omega[d] : 0.f);
     } else {
       const char* arow = static_cast<const char*>(a) + row * L * esz;
       const char* xrow = static_cast<const char*>(b) + row * L * esz;
@@ -320,7 +335,7 @@ __global__ __launch_bounds__(Cfg<LOGM>::T) void fftconv_kernel(
 
 template <int LOGM, int DT, int MODE, bool VEC>
 int launch_fft_v(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_t L,
-                 int flip, hipStream_t stream) {
+                 int flip, const float* omega, hipStream_t stream) {
   using C = Cfg<LOGM>;
   const c32* tab = nullptr;
   float* scratch = nullptr;
@@ -338,7 +353,7 @@ int launch_fft_v(const void* a, const void* b, void* out, int64_t B, int64_t D, 
     const unsigned grid = static_cast<unsigned>(rows < slots ? rows : slots);
     fftconv_kernel<LOGM, DT, MODE, VEC><<<dim3(grid), C::T, lds_bytes, stream>>>(
         a, b, out, static_cast<int>(rows), static_cast<int>(D), static_cast<int>(L), flip, tab,
-        scratch);
+        scratch, omega);
     MEGA_CHECK_LAUNCH();
   } else {
     const unsigned grid = static_cast<unsigned>(D < slots ? D : slots);
@@ -347,7 +362,7 @@ int launch_fft_v(const void* a, const void* b, void* out, int64_t B, int64_t D, 
       const char* xb = static_cast<const char*>(b) + bb * D * L * esz;
       fftconv_kernel<LOGM, DT, MODE, VEC><<<dim3(grid), C::T, lds_bytes, stream>>>(
           ab, xb, out, static_cast<int>(D), static_cast<int>(D), static_cast<int>(L),
-          bb > 0 ? 1 : 0, tab, scratch);
+          bb > 0 ? 1 : 0, tab, scratch, nullptr);
       MEGA_CHECK_LAUNCH();
     }
   }
@@ -356,14 +371,14 @@ int launch_fft_v(const void* a, const void* b, void* out, int64_t B, int64_t D, 
 
 template <int LOGM, int DT, int MODE>
 int launch_fft(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_t L, int flip,
-               hipStream_t stream) {
+               const float* omega, hipStream_t stream) {
   const auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 8 == 0; };
   const bool vec = (L % 2 == 0) && al(a) && al(b) && al(out);
-  if (vec) return launch_fft_v<LOGM, DT, MODE, true>(a, b, out, B, D, L, flip, stream);
+  if (vec) return launch_fft_v<LOGM, DT, MODE, true>(a, b, out, B, D, L, flip, omega, stream);
 #ifdef MEGA_FFTCONV_SINGLE
   return MEGA_ERR_UNSUPPORTED;
 #else
-  return launch_fft_v<LOGM, DT, MODE, false>(a, b, out, B, D, L, flip, stream);
+  return launch_fft_v<LOGM, DT, MODE, false>(a, b, out, B, D, L, flip, omega, stream);
 #endif
 }
 
@@ -375,7 +390,7 @@ constexpr int kDirectThreads = 256;
 template <int DT, int MODE>
 __global__ __launch_bounds__(kDirectThreads) void direct_conv_kernel(
     const void* __restrict__ a, const void* __restrict__ b, void* __restrict__ out, int B, int D,
-    int L, int flip) {
+    int L, int flip, const float* __restrict__ omega) {
   __shared__ float sa[kDirectMaxL];
   __shared__ float sb[kDirectMaxL];
   const int64_t esz = DT == MEGA_F32 ? 4 : 2;
@@ -399,6 +414,7 @@ __global__ __launch_bounds__(kDirectThreads) void direct_conv_kernel(
       for (int s = 0; s <= i; ++s) acc = fmaf(sb[i - s], sa[s], acc);
       const int o = fl ? L - 1 - i : i;
       if (MODE == 0) {
+        if (omega != nullptr) acc = fmaf(omega[d], sa[i], acc);  // sa[i] is a[o]
         st<DT>(static_cast<char*>(out) + row * L * esz, o, acc);
       } else {
         float* orow = static_cast<float*>(out) + d * L;
@@ -410,33 +426,33 @@ __global__ __launch_bounds__(kDirectThreads) void direct_conv_kernel(
 
 template <int DT, int MODE>
 int launch_conv(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_t L, int flip,
-                hipStream_t stream) {
+                const float* omega, hipStream_t stream) {
 #ifdef MEGA_FFTCONV_SINGLE  // development switch: one instantiation, fast compile
-  if (DT == MEGA_BF16 && MODE == 0) return launch_fft<14, MEGA_BF16, 0>(a, b, out, B, D, L, flip, stream);
+  if (DT == MEGA_BF16 && MODE == 0) return launch_fft<14, MEGA_BF16, 0>(a, b, out, B, D, L, flip, omega, stream);
   return MEGA_ERR_UNSUPPORTED;
 #else
   if (L <= kDirectMaxL) {
     const int64_t rows = MODE == 0 ? B * D : D;
     MEGA_CHECK_ARG(rows <= 0x7fffffff, "fftconv: too many rows");
     direct_conv_kernel<DT, MODE><<<dim3(static_cast<unsigned>(rows)), kDirectThreads, 0, stream>>>(
-        a, b, out, static_cast<int>(B), static_cast<int>(D), static_cast<int>(L), flip);
+        a, b, out, static_cast<int>(B), static_cast<int>(D), static_cast<int>(L), flip, omega);
     MEGA_CHECK_LAUNCH();
     return MEGA_OK;
   }
-  if (L <= 4096) return launch_fft<11, DT, MODE>(a, b, out, B, D, L, flip, stream);
-  if (L <= 8192) return launch_fft<12, DT, MODE>(a, b, out, B, D, L, flip, stream);
-  if (L <= 16384) return launch_fft<13, DT, MODE>(a, b, out, B, D, L, flip, stream);
-  return launch_fft<14, DT, MODE>(a, b, out, B, D, L, flip, stream);
+  if (L <= 4096) return launch_fft<11, DT, MODE>(a, b, out, B, D, L, flip, omega, stream);
+  if (L <= 8192) return launch_fft<12, DT, MODE>(a, b, out, B, D, L, flip, omega, stream);
+  if (L <= 16384) return launch_fft<13, DT, MODE>(a, b, out, B, D, L, flip, omega, stream);
+  return launch_fft<14, DT, MODE>(a, b, out, B, D, L, flip, omega, stream);
 #endif
 }
 
 template <int MODE>
 int dispatch_conv(int dtype, const void* a, const void* b, void* out, int64_t B, int64_t D,
-                  int64_t L, int flip, hipStream_t stream) {
+                  int64_t L, int flip, const float* omega, hipStream_t stream) {
   switch (dtype) {
-    case MEGA_F32: return launch_conv<MEGA_F32, MODE>(a, b, out, B, D, L, flip, stream);
-    case MEGA_BF16: return launch_conv<MEGA_BF16, MODE>(a, b, out, B, D, L, flip, stream);
-    case MEGA_F16: return launch_conv<MEGA_F16, MODE>(a, b, out, B, D, L, flip, stream);
+    case MEGA_F32: return launch_conv<MEGA_F32, MODE>(a, b, out, B, D, L, flip, omega, stream);
+    case MEGA_BF16: return launch_conv<MEGA_BF16, MODE>(a, b, out, B, D, L, flip, omega, stream);
+    case MEGA_F16: return launch_conv<MEGA_F16, MODE>(a, b, out, B, D, L, flip, omega, stream);
   }
   return set_error(MEGA_ERR_INVALID_ARG, "fftconv: bad dtype %d", dtype);
 }
@@ -455,26 +471,27 @@ using namespace mega;
 
 extern "C" int mega_fftconv_max_length(void) { return static_cast<int>(kMaxL); }
 
-extern "C" int mega_fftconv_fwd(const void* x, int dtype, const float* k, int64_t B, int64_t D,
-                                int64_t L, void* y, void* stream) {
-  MEGA_CHECK_ARG(x && k && y, "mega_fftconv_fwd: null pointer");
-  MEGA_CHECK_ARG(valid_dtype(dtype), "mega_fftconv_fwd: bad dtype %d", dtype);
-  MEGA_CHECK_ARG(B >= 0 && D >= 0 && L >= 0, "mega_fftconv_fwd: negative size");
+namespace {
+int fftconv_fwd_impl(const char* who, const void* x, int dtype, const float* k, const float* omega,
+                     int64_t B, int64_t D, int64_t L, void* y, void* stream) {
+  MEGA_CHECK_ARG(x && k && y, "%s: null pointer", who);
+  MEGA_CHECK_ARG(valid_dtype(dtype), "%s: bad dtype %d", who, dtype);
+  MEGA_CHECK_ARG(B >= 0 && D >= 0 && L >= 0, "%s: negative size", who);
   if (L > kMaxL)
-    return set_error(MEGA_ERR_UNSUPPORTED, "mega_fftconv_fwd: L=%lld exceeds the supported %lld",
+    return set_error(MEGA_ERR_UNSUPPORTED, "%s: L=%lld exceeds the supported %lld", who,
                      (long long)L, (long long)kMaxL);
   if (B == 0 || D == 0 || L == 0) return MEGA_OK;
-  return dispatch_conv<0>(dtype, x, k, y, B, D, L, 0, static_cast<hipStream_t>(stream));
+  return dispatch_conv<0>(dtype, x, k, y, B, D, L, 0, omega, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int mega_fftconv_bwd(const void* dy, const void* x, int dtype, const float* k,
-                                int64_t B, int64_t D, int64_t L, void* dx, float* dk,
-                                void* stream) {
-  MEGA_CHECK_ARG(dy && x && k && dx && dk, "mega_fftconv_bwd: null pointer");
-  MEGA_CHECK_ARG(valid_dtype(dtype), "mega_fftconv_bwd: bad dtype %d", dtype);
-  MEGA_CHECK_ARG(B >= 0 && D >= 0 && L >= 0, "mega_fftconv_bwd: negative size");
+int fftconv_bwd_impl(const char* who, const void* dy, const void* x, int dtype, const float* k,
+                     const float* omega, int64_t B, int64_t D, int64_t L, void* dx, float* dk,
+                     void* stream) {
+  MEGA_CHECK_ARG(dy && x && k && dx && dk, "%s: null pointer", who);
+  MEGA_CHECK_ARG(valid_dtype(dtype), "%s: bad dtype %d", who, dtype);
+  MEGA_CHECK_ARG(B >= 0 && D >= 0 && L >= 0, "%s: negative size", who);
   if (L > kMaxL)
-    return set_error(MEGA_ERR_UNSUPPORTED, "mega_fftconv_bwd: L=%lld exceeds the supported %lld",
+    return set_error(MEGA_ERR_UNSUPPORTED, "%s: L=%lld exceeds the supported %lld", who,
                      (long long)L, (long long)kMaxL);
   if (D == 0 || L == 0) return MEGA_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -484,7 +501,34 @@ extern "C" int mega_fftconv_bwd(const void* dy, const void* x, int dtype, const 
     MEGA_CHECK_LAUNCH();
     return MEGA_OK;
   }
-  int rc = dispatch_conv<0>(dtype, dy, k, dx, B, D, L, 1, s);
+  int rc = dispatch_conv<0>(dtype, dy, k, dx, B, D, L, 1, omega, s);
   if (rc != MEGA_OK) return rc;
-  return dispatch_conv<1>(dtype, dy, x, dk, B, D, L, 1, s);
+  return dispatch_conv<1>(dtype, dy, x, dk, B, D, L, 1, nullptr, s);
+}
+}  // namespace
+
+extern "C" int mega_fftconv_fwd(const void* x, int dtype, const float* k, int64_t B, int64_t D,
+                                int64_t L, void* y, void* stream) {
+  return fftconv_fwd_impl("mega_fftconv_fwd", x, dtype, k, nullptr, B, D, L, y, stream);
+}
+
+extern "C" int mega_fftconv_bwd(const void* dy, const void* x, int dtype, const float* k,
+                                int64_t B, int64_t D, int64_t L, void* dx, float* dk,
+                                void* stream) {
+  return fftconv_bwd_impl("mega_fftconv_bwd", dy, x, dtype, k, nullptr, B, D, L, dx, dk, stream);
+}
+
+extern "C" int mega_fftconv_residual_fwd(const void* x, int dtype, const float* k,
+                                         const float* omega, int64_t B, int64_t D, int64_t L,
+                                         void* y, void* stream) {
+  MEGA_CHECK_ARG(omega, "mega_fftconv_residual_fwd: null omega");
+  return fftconv_fwd_impl("mega_fftconv_residual_fwd", x, dtype, k, omega, B, D, L, y, stream);
+}
+
+extern "C" int mega_fftconv_residual_bwd(const void* dy, const void* x, int dtype, const float* k,
+                                         const float* omega, int64_t B, int64_t D, int64_t L,
+                                         void* dx, float* dk, void* stream) {
+  MEGA_CHECK_ARG(omega, "mega_fftconv_residual_bwd: null omega");
+  return fftconv_bwd_impl("mega_fftconv_residual_bwd", dy, x, dtype, k, omega, B, D, L, dx, dk,
+                          stream);
 }

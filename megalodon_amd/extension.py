@@ -147,6 +147,48 @@ def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
     return dx, dk.to(k_dtype)
 
 
+def fftconv_residual_fwd(x: torch.Tensor, k: torch.Tensor, omega: torch.Tensor) -> torch.Tensor:
+    """y = causal_conv(x, k) + omega[d] * x in one kernel: the convolution and the
+    skip term of MultiHeadComplexEMA.forward
+    (complex_exponential_moving_average.py:136-146).  omega (D,) or (D, 1)."""
+    dev = _require_cuda(x, k, omega)
+    if x.dim() != 3 or k.dim() != 2 or k.shape[0] != x.shape[1] or k.shape[1] != x.shape[2]:
+        raise RuntimeError(f"fftconv: x {tuple(x.shape)} and k {tuple(k.shape)} do not match (B,D,L)/(D,L)")
+    if omega.numel() != x.shape[1]:
+        raise RuntimeError(f"fftconv: omega has {omega.numel()} elements for D={x.shape[1]}")
+    B, D, L = x.shape
+    xc = x.contiguous()
+    kc = k.contiguous().float()
+    wc = omega.reshape(-1).contiguous().float()
+    y = torch.empty_like(xc)
+    with torch.cuda.device(dev):
+        _lib.call("mega_fftconv_residual_fwd", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
+                  _lib.ptr(kc), _lib.ptr(wc), _lib.i64(B), _lib.i64(D), _lib.i64(L), _lib.ptr(y),
+                  _lib.stream_ptr(dev))
+    return y
+
+
+def fftconv_residual_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
+                         omega: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dx, dk, domega) of ``fftconv_residual_fwd``; dk and domega are float32.
+    domega is the lag-0 column of dk: sum_b sum_t dy[b,d,t] x[b,d,t]."""
+    dev = _require_cuda(y_grad, x, k, omega)
+    B, D, L = x.shape
+    if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
+        raise RuntimeError("fftconv_bwd: y_grad must match x in shape and dtype")
+    dy = y_grad.contiguous()
+    xc = x.contiguous()
+    kc = k.contiguous().float()
+    wc = omega.reshape(-1).contiguous().float()
+    dx = torch.empty_like(xc)
+    dk = torch.empty((D, L), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_fftconv_residual_bwd", _lib.ptr(dy), _lib.ptr(xc),
+                  _lib.i32(_lib.dtype_code(x.dtype)), _lib.ptr(kc), _lib.ptr(wc), _lib.i64(B),
+                  _lib.i64(D), _lib.i64(L), _lib.ptr(dx), _lib.ptr(dk), _lib.stream_ptr(dev))
+    return dx, dk, dk[:, 0].clone()
+
+
 # --------------------------------------------------------------------------
 # group_timestep_norm (reference: csrc/ops/timestep_norm.cc:621-705)
 # --------------------------------------------------------------------------

@@ -2,7 +2,7 @@
 from .attention import (swift_efficient_attention, swift_efficient_attention_bwd,
                         swift_efficient_attention_fwd)
 from .ema_parameters import ema_parameters
-from .fftconv import fftconv
+from .fftconv import fftconv, fftconv_residual
 
-__all__ = ["ema_parameters", "fftconv", "swift_efficient_attention", "swift_efficient_attention_fwd",
+__all__ = ["ema_parameters", "fftconv", "fftconv_residual", "swift_efficient_attention", "swift_efficient_attention_fwd",
            "swift_efficient_attention_bwd"]

@@ -7,7 +7,7 @@ from typing import Tuple
 import torch
 from torch.autograd.function import FunctionCtx
 
-from ..extension import fftconv_bwd, fftconv_fwd
+from ..extension import fftconv_bwd, fftconv_fwd, fftconv_residual_bwd, fftconv_residual_fwd
 
 
 class FFTConvFunc(torch.autograd.Function):
@@ -26,3 +26,25 @@ class FFTConvFunc(torch.autograd.Function):
 
 
 fftconv = FFTConvFunc.apply
+
+
+class FFTConvResidualFunc(torch.autograd.Function):
+    """``fftconv(x, k) + x * omega`` as one op: the two lines around the
+    convolution in MultiHeadComplexEMA.forward
+    (megalodon/modules/complex_exponential_moving_average.py:136-146) without the
+    two extra passes over the activations.  The result has the dtype of x."""
+
+    @staticmethod
+    def forward(ctx: FunctionCtx, x: torch.Tensor, k: torch.Tensor, omega: torch.Tensor) -> torch.Tensor:
+        y = fftconv_residual_fwd(x, k, omega)
+        ctx.save_for_backward(x, k, omega)
+        return y
+
+    @staticmethod
+    def backward(ctx: FunctionCtx, y_grad: torch.Tensor):
+        x, k, omega = ctx.saved_tensors
+        dx, dk, dw = fftconv_residual_bwd(y_grad, x, k, omega)
+        return dx, dk.to(k.dtype), dw.to(omega.dtype).view_as(omega)
+
+
+fftconv_residual = FFTConvResidualFunc.apply

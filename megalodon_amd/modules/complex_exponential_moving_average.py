@@ -9,7 +9,7 @@ import math
 import torch
 from torch import nn
 
-from ..fused_ops import ema_parameters, fftconv
+from ..fused_ops import ema_parameters, fftconv_residual
 
 _r2c = torch.view_as_complex
 
@@ -88,12 +88,11 @@ class MultiHeadComplexEMA(nn.Module):
             raise NotImplementedError(
                 "carried EMA state (hx / compute_last_state) is outside the single-sequence training path")
         bsz, _, seq_len = x.size()
-        residual = x * self.omega
-
         p, q, gamma = self.coeffs()
         k, b = ema_parameters(p, q, gamma, hx, seq_len)
-        output = fftconv(x, k)
-        output = output + residual
+        # fftconv(x, k) + x * omega, the skip term folded into the convolution's
+        # output pass (the reference adds `residual = x * self.omega` afterwards)
+        output = fftconv_residual(x, k, self.omega)
         return output, None
 
     def extra_repr(self) -> str:

@@ -7,7 +7,7 @@ import torch
 from conftest import rel_err
 from megalodon_amd import extension as ops
 from megalodon_amd import synthetic
-from megalodon_amd.fused_ops import ema_parameters, fftconv as fftconv_op
+from megalodon_amd.fused_ops import ema_parameters, fftconv as fftconv_op, fftconv_residual
 from oracle import cema, fftconv
 
 pytestmark = pytest.mark.gpu
@@ -48,6 +48,39 @@ def test_bwd_matches_oracle(B, D, L, dtype):
     wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
     assert rel_err(dx, wdx) <= TOL[dtype]
     assert rel_err(dk, wdk) <= TOL[dtype]
+
+
+RES_SHAPES = [(2, 3, 50), (1, 4, 2048), (2, 3, 4097), (1, 3, 8192), (2, 2, 12345), (2, 3, 32768), (1, 2, 32767)]
+
+
+@pytest.mark.parametrize("B,D,L", RES_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_residual_variant_matches_oracle(B, D, L, dtype):
+    """y = fftconv(x, k) + omega x and its three gradients; the expected values
+    are the float64 oracle convolution plus the skip term written out."""
+    x, k, dy = _data(B, D, L, dtype, 7 * L + B)
+    omega = torch.randn(D, 1, generator=torch.Generator().manual_seed(L)) * 0.5
+    y = ops.fftconv_residual_fwd(x.cuda(), k.cuda(), omega.cuda())
+    assert y.dtype == dtype and y.shape == x.shape
+    w64 = omega.double().view(1, D, 1)
+    want = fftconv.fftconv_fwd(x, k).double() + w64 * x.double()
+    assert rel_err(y, want) <= TOL[dtype]
+    dx, dk, dw = ops.fftconv_residual_bwd(dy.cuda(), x.cuda(), k.cuda(), omega.cuda())
+    wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
+    assert rel_err(dx, wdx.double() + w64 * dy.double()) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= TOL[dtype]
+    assert dw.shape == (D,) and rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= TOL[dtype]
+
+
+def test_residual_autograd_function():
+    x, k, dy = _data(2, 3, 3000, torch.float32, 3)
+    omega = torch.randn(3, 1)
+    xg, kg, wg = (t.cuda().requires_grad_() for t in (x, k, omega))
+    fftconv_residual(xg, kg, wg).backward(dy.cuda())
+    xr, kr, wr = (t.cuda().requires_grad_() for t in (x, k, omega))
+    (fftconv_op(xr, kr) + xr * wr).backward(dy.cuda())
+    assert rel_err(xg.grad, xr.grad) <= 1e-4 and rel_err(kg.grad, kr.grad) <= 1e-4
+    assert wg.grad.shape == omega.shape and rel_err(wg.grad, wr.grad) <= 1e-4
 
 
 def test_float16_rows():
