@@ -19,6 +19,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+# HBM bytes one forward convolution launch moves at config 1: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from
+# two rocprofv3 --pmc passes of this script, the factors being what the same counters read for a plain
+# copy of 2^30 bytes (--copy-calibration).  A measured constant: counters cannot be read from in here.
+FFTCONV_TRAFFIC_BYTES = 4.62e9
 
 
 def cpu_baseline(B, D, N, L, seed, budget_s=25.0):
@@ -76,12 +80,85 @@ def cpu_baseline(B, D, N, L, seed, budget_s=25.0):
     }
 
 
+def other_ops(torch, dev, synthetic):
+    """TimestepNorm (config 2), chunk attention (config 3) and one block (config 4),
+    timed with device events; reported beside the config-1 step."""
+    def dev_ms(fn, n):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    from megalodon_amd import extension as ops
+    other = {}
+    tB, tL, tD, tG = 4, 8192, 4096, 32
+    tio = {k_: v_.to(dev) for k_, v_ in synthetic.timestep_norm_inputs(tB, tL, tD, tG, 1002).items()}
+    tE = tB * tL * tD
+    fwd = lambda: ops.group_timestep_norm_fwd(tio["x"], tio["prev_count"], tio["prev_mean"], tio["prev_var"],
+                                              tio["gamma"], tio["beta"], tio["mask"], tG, 1e-5)
+    ty, tcount, tmean, tvar, tcm, tcr = fwd()
+    ms = dev_ms(fwd, 10)
+    other["timestep_norm_fwd"] = {"ms": ms, "GBps": 4 * tE / ms / 1e6, "frac_hbm": 4 * tE / ms / 1e6 / HBM_PEAK_GBS}
+    ms = dev_ms(lambda: ops.group_timestep_norm_bwd(tio["dy"], tio["dmean"], tio["dvar"], tio["x"], tio["prev_mean"],
+                                                    tcount, tcm, tcr, tio["gamma"], tio["mask"], tG), 10)
+    other["timestep_norm_bwd"] = {"ms": ms, "GBps": 6 * tE / ms / 1e6, "frac_hbm": 6 * tE / ms / 1e6 / HBM_PEAK_GBS}
+    del tio, ty, tcm, tcr
+    aio = {k_: v_.to(dev) for k_, v_ in synthetic.attention_inputs(8, 4096, 4, 256, 2048, 1003).items()}
+    pairs = 4096 * 4097 // 2
+    f_fwd, f_bwd = 2 * pairs * (256 + 2048) * 32, 2 * pairs * (2 * 256 + 2 * 2048) * 32
+    ay, aw = ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True)
+    ms = dev_ms(lambda: ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True), 3)
+    other["attention_fwd"] = {"ms": ms, "TFLOPs": f_fwd / ms / 1e9, "frac_mfma_bf16": f_fwd / ms / 1e9 / 2516.6}
+    ms = dev_ms(lambda: ops.attention_bwd(aio["dy"], aio["q"], aio["k"], aio["v"], aw, 1.0, True), 3)
+    other["attention_bwd"] = {"ms": ms, "TFLOPs": f_bwd / ms / 1e9, "frac_mfma_bf16": f_bwd / ms / 1e9 / 2516.6}
+    del aio, ay, aw
+    torch.cuda.empty_cache()
+
+    # config 4: one full 7B-style block forward+backward (random init std 0.02, bf16)
+    from megalodon_amd.modules import MegaBlock
+    torch.manual_seed(1004)
+    blk = MegaBlock(model_dim=4096, z_dim=1024, value_dim=8192, num_heads=4, cema_ndim=16, chunk_size=4096,
+                    ffn_hidden_dim=11008, norm_num_groups=32).to(dev).bfloat16()
+    gb = torch.Generator().manual_seed(1004)
+    bx = (torch.rand(1, 32768, 4096, generator=gb) * 2 - 1).bfloat16().to(dev).requires_grad_(True)
+    bdy = torch.randn(1, 32768, 4096, generator=gb).bfloat16().to(dev)
+
+    def block_step():
+        bx.grad = None
+        for prm in blk.parameters():
+            prm.grad = None
+        o, _ = blk(bx)
+        o.backward(bdy)
+
+    block_step()
+    torch.cuda.synchronize()
+    tb0 = time.perf_counter()
+    for _ in range(3):
+        block_step()
+    torch.cuda.synchronize()
+    bms = (time.perf_counter() - tb0) / 3 * 1e3
+    other["block_config4_fwd_bwd"] = {"ms": bms, "tokens_per_s": 32768 / (bms * 1e-3)}
+    del blk, bx, bdy
+    torch.cuda.empty_cache()
+    return other
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--skip-other-ops", action="store_true",
+                    help="time only the config-1 step (short runs under a profiler)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one plain elementwise copy of 1 GiB in, 1 GiB out "
+                         "(reference point for scaling FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (every op shards "
@@ -148,70 +225,16 @@ def main():
     kernels["ema_weight_fwd_GBps"] = 4 * E / (kernels["ema_weight_fwd_ms"] * 1e-3) / 1e9
     kernels["ema_weight_bwd_GBps"] = 4 * E / (kernels["ema_weight_bwd_ms"] * 1e-3) / 1e9
 
-    # the other hot-path operators at their BASELINE shapes (configs 2 and 3), device events
-    def dev_ms(fn, n):
-        fn()
+    if args.copy_calibration:
+        src = torch.ones(1 << 29, dtype=torch.bfloat16, device=dev)
+        dst = torch.empty_like(src)
+        torch.mul(src, 1.0, out=dst)  # reads 2^30 bytes, writes 2^30 bytes
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(n):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / n
+        del src, dst
 
-    from megalodon_amd import extension as ops
     other = {}
-    tB, tL, tD, tG = 4, 8192, 4096, 32
-    tio = {k_: v_.to(dev) for k_, v_ in synthetic.timestep_norm_inputs(tB, tL, tD, tG, 1002).items()}
-    tE = tB * tL * tD
-    fwd = lambda: ops.group_timestep_norm_fwd(tio["x"], tio["prev_count"], tio["prev_mean"], tio["prev_var"],
-                                              tio["gamma"], tio["beta"], tio["mask"], tG, 1e-5)
-    ty, tcount, tmean, tvar, tcm, tcr = fwd()
-    ms = dev_ms(fwd, 10)
-    other["timestep_norm_fwd"] = {"ms": ms, "GBps": 4 * tE / ms / 1e6, "frac_hbm": 4 * tE / ms / 1e6 / HBM_PEAK_GBS}
-    ms = dev_ms(lambda: ops.group_timestep_norm_bwd(tio["dy"], tio["dmean"], tio["dvar"], tio["x"], tio["prev_mean"],
-                                                    tcount, tcm, tcr, tio["gamma"], tio["mask"], tG), 10)
-    other["timestep_norm_bwd"] = {"ms": ms, "GBps": 6 * tE / ms / 1e6, "frac_hbm": 6 * tE / ms / 1e6 / HBM_PEAK_GBS}
-    del tio, ty, tcm, tcr
-    aio = {k_: v_.to(dev) for k_, v_ in synthetic.attention_inputs(8, 4096, 4, 256, 2048, 1003).items()}
-    pairs = 4096 * 4097 // 2
-    f_fwd, f_bwd = 2 * pairs * (256 + 2048) * 32, 2 * pairs * (2 * 256 + 2 * 2048) * 32
-    ay, aw = ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True)
-    ms = dev_ms(lambda: ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True), 3)
-    other["attention_fwd"] = {"ms": ms, "TFLOPs": f_fwd / ms / 1e9, "frac_mfma_bf16": f_fwd / ms / 1e9 / 2516.6}
-    ms = dev_ms(lambda: ops.attention_bwd(aio["dy"], aio["q"], aio["k"], aio["v"], aw, 1.0, True), 3)
-    other["attention_bwd"] = {"ms": ms, "TFLOPs": f_bwd / ms / 1e9, "frac_mfma_bf16": f_bwd / ms / 1e9 / 2516.6}
-    del aio, ay, aw
-    torch.cuda.empty_cache()
-
-    # config 4: one full 7B-style block forward+backward (random init std 0.02, bf16)
-    from megalodon_amd.modules import MegaBlock
-    torch.manual_seed(1004)
-    blk = MegaBlock(model_dim=4096, z_dim=1024, value_dim=8192, num_heads=4, cema_ndim=16, chunk_size=4096,
-                    ffn_hidden_dim=11008, norm_num_groups=32).to(dev).bfloat16()
-    gb = torch.Generator().manual_seed(1004)
-    bx = (torch.rand(1, 32768, 4096, generator=gb) * 2 - 1).bfloat16().to(dev).requires_grad_(True)
-    bdy = torch.randn(1, 32768, 4096, generator=gb).bfloat16().to(dev)
-
-    def block_step():
-        bx.grad = None
-        for prm in blk.parameters():
-            prm.grad = None
-        o, _ = blk(bx)
-        o.backward(bdy)
-
-    block_step()
-    torch.cuda.synchronize()
-    tb0 = time.perf_counter()
-    for _ in range(3):
-        block_step()
-    torch.cuda.synchronize()
-    bms = (time.perf_counter() - tb0) / 3 * 1e3
-    other["block_config4_fwd_bwd"] = {"ms": bms, "tokens_per_s": 32768 / (bms * 1e-3)}
-    del blk, bx, bdy
-    torch.cuda.empty_cache()
-
+    if not args.skip_other_ops:
+        other = other_ops(torch, dev, synthetic)
     result = {
         "metric": "Megalodon layer fwd+bwd tokens/s at L=32K, 1 GPU; CEMA+FFT-conv HBM GB/s (% peak)",
         "value": B * L / (dt / args.steps),
@@ -231,7 +254,7 @@ def main():
         "roofline": {
             "bound": "hbm", "kernel": "fftconv_kernel<LOGM=14, bf16, MODE=0> (one launch = forward conv of all rows)",
             "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBS, "traffic": FFTCONV_TRAFFIC_BYTES,
         },
         "kernels": kernels,
         "other_ops": other,
