@@ -14,6 +14,7 @@
 // Rows with L <= 2048 use a direct time-domain kernel (exact, O(L^2) per row).
 #include "common.hpp"
 #include "fftconv_core.hpp"
+#include "fftconv_mfma.hpp"
 
 #include <mutex>
 #include <vector>
@@ -439,6 +440,9 @@ int launch_conv(const void* a, const void* b, void* out, int64_t B, int64_t D, i
     MEGA_CHECK_LAUNCH();
     return MEGA_OK;
   }
+  // 16-bit rows of 16385..32768 samples run their DFT stages on the matrix cores
+  if (fftm::applicable(DT, L, a, b, out) && getenv("MEGA_FFTCONV_VALU") == nullptr)
+    return fftm::launch_conv(DT, MODE, a, b, out, B, D, L, flip, omega, stream);
   if (L <= 4096) return launch_fft<11, DT, MODE>(a, b, out, B, D, L, flip, omega, stream);
   if (L <= 8192) return launch_fft<12, DT, MODE>(a, b, out, B, D, L, flip, omega, stream);
   if (L <= 16384) return launch_fft<13, DT, MODE>(a, b, out, B, D, L, flip, omega, stream);
