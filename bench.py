@@ -22,7 +22,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes one forward convolution launch moves at config 1: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from
 # two rocprofv3 --pmc passes of this script, the factors being what the same counters read for a plain
 # copy of 2^30 bytes (--copy-calibration).  A measured constant: counters cannot be read from in here.
-FFTCONV_TRAFFIC_BYTES = 4.62e9
+FFTCONV_TRAFFIC_BYTES = 1.40e9
 
 
 def cpu_baseline(B, D, N, L, seed, budget_s=25.0):
@@ -252,7 +252,7 @@ def main():
                                "B=1 L=32768 D=4096 ndim=16, x/dy bf16, fp32 arithmetic",
                    "global_batch": B, "seq_len": L},
         "roofline": {
-            "bound": "hbm", "kernel": "fftconv_kernel<LOGM=14, bf16, MODE=0> (one launch = forward conv of all rows)",
+            "bound": "hbm", "kernel": "fftconv_mfma_kernel<bf16, MODE=0> (one launch = forward conv of all rows, skip term included)",
             "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS, "traffic": FFTCONV_TRAFFIC_BYTES,
         },
