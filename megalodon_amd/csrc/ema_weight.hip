@@ -230,6 +230,158 @@ __global__ __launch_bounds__(kThreads) void ema_weight_bwd_kernel(
   }
 }
 
+
+// ---- backward on the matrix cores (N <= 16) -----------------------------------
+// With j = 64 lo + h the two sums over the row become one small GEMM per channel,
+//   C[lo][.] = sum_h dw[64 lo + h] * Q[h][.],  Q[h] = (q_n^h, h q_n^h) for the 16 modes,
+// followed by a weighted column sum with q_n^(64 lo):
+//   S2 = sum_lo q^(64 lo) A[lo],   sum_j j dw_j q^j = sum_lo q^(64 lo) (64 lo A[lo] + B[lo]).
+// The products run as bf16 MFMAs with both operands split into high and low
+// halves (hi*hi + hi*lo + lo*hi): 16 significant bits per factor, fp32
+// accumulation, which keeps the fp32 tolerance of the operator.
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ floatx16 mfma_bf16(u32x4 a, u32x4 b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+// 8 floats -> packed bf16 high parts and packed bf16 residuals
+__device__ __forceinline__ void split8(const float* v, u32x4& hi, u32x4& lo) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint32_t h = pack_bf16x2(v[2 * e], v[2 * e + 1]);
+    const float r0 = v[2 * e] - __uint_as_float(h << 16);
+    const float r1 = v[2 * e + 1] - __uint_as_float(h & 0xffff0000u);
+    hi[e] = h;
+    lo[e] = pack_bf16x2(r0, r1);
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void ema_weight_bwd_mfma_kernel(
+    const float* __restrict__ dw, const float* __restrict__ p, const cf* __restrict__ log_q,
+    const cf* __restrict__ gamma, int N, int64_t L, float* __restrict__ dp, cf* __restrict__ dq,
+    cf* __restrict__ dgamma) {
+  __shared__ float red[kThreads][4];
+  const int64_t d = blockIdx.x;
+  const cf* lq = log_q + d * N;
+  const float* drow = dw + d * L;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int g = lane >> 5, col = lane & 31;
+  const int n = col & 15, kind = col >> 4;  // kind 0: q^h, kind 1: h q^h
+  const bool live = n < N;
+  const float la = live ? lq[n].x : 0.f, lphi = live ? lq[n].y : 0.f;
+
+  // B operand: lane <-> column (kind, n), k = h = 16 s + 8 g + e; real and
+  // imaginary parts are the two 32-column tiles
+  u32x4 qre_hi[4], qre_lo[4], qim_hi[4], qim_lo[4];
+  const cf q1 = qpow(la, lphi, 1);
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    float vr[8], vi[8];
+    cf v = qpow(la, lphi, 16 * s + 8 * g);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float sc = !live ? 0.f : (kind ? static_cast<float>(16 * s + 8 * g + e) : 1.f);
+      vr[e] = v.x * sc;
+      vi[e] = v.y * sc;
+      v = cmul(v, q1);
+    }
+    split8(vr, qre_hi[s], qre_lo[s]);
+    split8(vi, qim_hi[s], qim_lo[s]);
+  }
+  // q^(64 lo) for the rows a lane meets: lo = 32 mt + 8 qd + 4 g + e
+  const cf st1 = qpow(la, lphi, 64), st2 = cmul(st1, st1), st3 = cmul(st2, st1);
+  const cf st8 = qpow(la, lphi, 512);
+
+  const int64_t rows = (L + 63) / 64;
+  const int64_t mtiles = (rows + 31) / 32;
+  cf s2{0.f, 0.f}, s1{0.f, 0.f};
+
+  auto load_tile = [&](int64_t mt, float (*raw)[8]) {
+    const int64_t j0 = (32 * mt + col) * 64 + 8 * g;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int64_t j = j0 + 16 * s;
+      if (j + 8 <= L) {
+        const float4 u = *reinterpret_cast<const float4*>(drow + j);
+        const float4 v = *reinterpret_cast<const float4*>(drow + j + 4);
+        raw[s][0] = u.x; raw[s][1] = u.y; raw[s][2] = u.z; raw[s][3] = u.w;
+        raw[s][4] = v.x; raw[s][5] = v.y; raw[s][6] = v.z; raw[s][7] = v.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) raw[s][e] = j + e < L ? drow[j + e] : 0.f;
+      }
+    }
+  };
+
+  float raw[4][8];
+  if (wave < mtiles) load_tile(wave, raw);
+  for (int64_t mt = wave; mt < mtiles; mt += kThreads / kWave) {
+    u32x4 ahi[4], alo[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) split8(raw[s], ahi[s], alo[s]);
+    if (mt + kThreads / kWave < mtiles) load_tile(mt + kThreads / kWave, raw);  // next tile in flight
+    floatx16 cr, ci;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) cr[r] = ci[r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      cr = mfma_bf16(ahi[s], qre_hi[s], cr);
+      ci = mfma_bf16(ahi[s], qim_hi[s], ci);
+      cr = mfma_bf16(ahi[s], qre_lo[s], cr);
+      ci = mfma_bf16(ahi[s], qim_lo[s], ci);
+      cr = mfma_bf16(alo[s], qre_hi[s], cr);
+      ci = mfma_bf16(alo[s], qim_hi[s], ci);
+    }
+    // result: lane <-> column, register r <-> row lo = 32 mt + 8 (r / 4) + 4 g + r % 4
+    const int64_t lo0 = 32 * mt + 4 * g;
+    cf qq = qpow(la, lphi, 64 * lo0);
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      const cf w4[4] = {qq, cmul(qq, st1), cmul(qq, st2), cmul(qq, st3)};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int r = 4 * qd + e;
+        const cf t = cmul(w4[e], cf{cr[r], ci[r]});
+        const float jlo = static_cast<float>(64 * (lo0 + 8 * qd + e));
+        const float c2 = kind ? 0.f : 1.f, c1 = kind ? 1.f : jlo;
+        s2.x = fmaf(c2, t.x, s2.x);
+        s2.y = fmaf(c2, t.y, s2.y);
+        s1.x = fmaf(c1, t.x, s1.x);
+        s1.y = fmaf(c1, t.y, s1.y);
+      }
+      qq = cmul(qq, st8);
+    }
+  }
+  red[threadIdx.x][0] = s2.x;
+  red[threadIdx.x][1] = s2.y;
+  red[threadIdx.x][2] = s1.x;
+  red[threadIdx.x][3] = s1.y;
+  __syncthreads();
+  if (threadIdx.x < N) {
+    const int m = threadIdx.x;
+    cf t2{0.f, 0.f}, s1q{0.f, 0.f};
+    for (int wv = 0; wv < kThreads / kWave; ++wv)
+      for (int c = 0; c < 4; ++c) {
+        const float* r = red[wv * kWave + m + 16 * c];
+        t2.x += r[0];
+        t2.y += r[1];
+        s1q.x += r[2];
+        s1q.y += r[3];
+      }
+    // S1 = sum_j j dw_j q^(j-1) = (sum_j j dw_j q^j) / q
+    const cf sq = cmul(s1q, qpow(lq[m].x, lq[m].y, -1));
+    const cf gm = gamma[d * N + m];
+    const float pp = p[d * N + m];
+    dp[d * N + m] = t2.x * gm.x - t2.y * gm.y;
+    const cf t = cmul(sq, cf{pp * gm.x, pp * gm.y});
+    dq[d * N + m] = cf{t.x, -t.y};
+    dgamma[d * N + m] = cf{t2.x * pp, -t2.y * pp};
+  }
+}
+
 }  // namespace
 }  // namespace mega
 
@@ -286,7 +438,10 @@ extern "C" int mega_ema_weight_bwd(const float* dw, const float* p,
   cf* dgc = reinterpret_cast<cf*>(dgamma);
   const bool vec = (L % 2 == 0) && (reinterpret_cast<uintptr_t>(dw) % 8 == 0);
   dim3 grid(static_cast<unsigned>(D));
-  if (N <= 16) {
+  if (N <= 16 && L >= 1 && reinterpret_cast<uintptr_t>(dw) % 16 == 0 && L % 4 == 0 &&
+      getenv("MEGA_EMA_BWD_VALU") == nullptr) {
+    ema_weight_bwd_mfma_kernel<<<grid, kThreads, 0, s>>>(dw, p, lq, gm, (int)N, L, dp, dqc, dgc);
+  } else if (N <= 16) {
     if (vec)
       ema_weight_bwd_kernel<16, 2, true><<<grid, kThreads, 0, s>>>(dw, p, lq, gm, (int)N, L, dp, dqc, dgc);
     else
