@@ -505,6 +505,10 @@ int fftconv_bwd_impl(const char* who, const void* dy, const void* x, int dtype, 
     MEGA_CHECK_LAUNCH();
     return MEGA_OK;
   }
+  if (fftm::applicable(dtype, L, dy, x, dx) && reinterpret_cast<uintptr_t>(k) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(dk) % 16 == 0 && getenv("MEGA_FFTCONV_VALU") == nullptr &&
+      getenv("MEGA_FFTCONV_SPLIT_BWD") == nullptr)
+    return fftm::launch_backward(dtype, dy, x, k, dx, dk, B, D, L, omega, s);
   int rc = dispatch_conv<0>(dtype, dy, k, dx, B, D, L, 1, omega, s);
   if (rc != MEGA_OK) return rc;
   return dispatch_conv<1>(dtype, dy, x, dk, B, D, L, 1, nullptr, s);

@@ -755,6 +755,91 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_kernel(
   }
 }
 
+// Backward of one channel in one pass: dy is transformed once and its spectrum
+// parked; then k (-> dx) and x (-> dk) are each transformed, multiplied with
+// it and transformed back.
+//   dx[b,d,:] = reverse(conv(reverse(dy[b,d,:]), k[d,:])) (+ omega[d] dy[b,d,:])
+//   dk[d,:]   = sum_b reverse(conv(reverse(dy[b,d,:]), x[b,d,:]))
+// A workgroup owns channels d = blockIdx.x, + gridDim.x, ... and walks the batch
+// itself, so dk accumulates in order without atomics.
+template <int DT>
+__global__ __launch_bounds__(kThreads) void fftconv_mfma_bwd_kernel(
+    const void* __restrict__ dy, const void* __restrict__ x, const float* __restrict__ k,
+    void* __restrict__ dx, float* __restrict__ dk, int B, int D, int L,
+    const float* __restrict__ omega) {
+  extern __shared__ __align__(16) uint16_t lds[];
+  uint16_t* pre = lds;
+  uint16_t* pim = lds + kPlane;
+  float* red = reinterpret_cast<float*>(lds + 2 * kPlane);
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const Dft w = make_dft(lane);
+  const int64_t rows = static_cast<int64_t>(B) * D;  // visited as (d, b), b fastest
+  const int64_t total = (static_cast<int64_t>(D) - blockIdx.x + gridDim.x - 1) / gridDim.x * B;
+  auto row_of = [&](int64_t it) -> int64_t {  // it-th row of this workgroup
+    const int64_t d = blockIdx.x + (it / B) * gridDim.x, bb = it % B;
+    return bb * D + d;
+  };
+  (void)rows;
+  RowRegs<DT> rdy;
+  if (total > 0) fetch_row(rdy, static_cast<const char*>(dy) + row_of(0) * L * 2, L, true, tid);
+  for (int64_t it = 0; it < total; ++it) {
+    const int64_t row = row_of(it), d = row % D;
+    const bool first = it % B == 0;
+    const char* dyrow = static_cast<const char*>(dy) + row * L * 2;
+    const float sdy = place_row(pre, pim, red, rdy, true, tid);
+    transform<false>(pre, pim, w, wave, lane);
+    RowRegs<MEGA_F32> rk;
+    fetch_row(rk, k + d * L, L, false, tid);
+    Spectrum sp;
+    capture_spectrum(pre, pim, sp, tid);
+    lds_barrier();
+    // dx
+    const float sk = place_row(pre, pim, red, rk, false, tid);
+    transform<false>(pre, pim, w, wave, lane);
+    pointwise(pre, pim, sp, tid);
+    lds_barrier();
+    RowRegs<DT> rx;
+    fetch_row(rx, static_cast<const char*>(x) + row * L * 2, L, false, tid);
+    transform<true>(pre, pim, w, wave, lane);
+    store_row<DT, false>(pre, pim, static_cast<char*>(dx) + row * L * 2, L, true,
+                         181.01933598375618f / (sdy * sk), omega != nullptr ? dyrow : nullptr,
+                         omega != nullptr ? omega[d] : 0.f, tid);
+    lds_barrier();
+    // dk
+    const float sx = place_row(pre, pim, red, rx, false, tid);
+    transform<false>(pre, pim, w, wave, lane);
+    pointwise(pre, pim, sp, tid);
+    lds_barrier();
+    if (it + 1 < total)
+      fetch_row(rdy, static_cast<const char*>(dy) + row_of(it + 1) * L * 2, L, true, tid);
+    transform<true>(pre, pim, w, wave, lane);
+    float* krow = dk + d * L;
+    const float sc = 181.01933598375618f / (sdy * sx);
+    if (first)
+      store_row<MEGA_F32, false>(pre, pim, krow, L, true, sc, nullptr, 0.f, tid);
+    else
+      store_row<MEGA_F32, true>(pre, pim, krow, L, true, sc, nullptr, 0.f, tid);
+    lds_barrier();
+  }
+}
+
+template <int DT>
+int launch_bwd(const void* dy, const void* x, const float* k, void* dx, float* dk, int64_t B,
+               int64_t D, int64_t L, const float* omega, hipStream_t stream) {
+  int dev = 0, cus = 0;
+  MEGA_CHECK_HIP(hipGetDevice(&dev));
+  MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&fftconv_mfma_bwd_kernel<DT>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     static_cast<int>(kLdsBytes)));
+  MEGA_CHECK_ARG(B * D <= 0x7fffffff, "fftconv: too many rows");
+  const unsigned grid = static_cast<unsigned>(D < cus ? D : cus);
+  fftconv_mfma_bwd_kernel<DT><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
+      dy, x, k, dx, dk, static_cast<int>(B), static_cast<int>(D), static_cast<int>(L), omega);
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
+}
+
 template <int DT, int MODE>
 int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_t L, int flip,
            const float* omega, hipStream_t stream, uint16_t* dbg, int dbg_stage) {
@@ -802,6 +887,12 @@ int launch_conv(int dtype, int mode, const void* a, const void* b, void* out, in
                      : launch<MEGA_BF16, 1>(a, b, out, B, D, L, flip, omega, stream, dbg, dbg_stage);
   return mode == 0 ? launch<MEGA_F16, 0>(a, b, out, B, D, L, flip, omega, stream, dbg, dbg_stage)
                    : launch<MEGA_F16, 1>(a, b, out, B, D, L, flip, omega, stream, dbg, dbg_stage);
+}
+
+int launch_backward(int dtype, const void* dy, const void* x, const float* k, void* dx, float* dk,
+                    int64_t B, int64_t D, int64_t L, const float* omega, hipStream_t stream) {
+  if (dtype == MEGA_BF16) return launch_bwd<MEGA_BF16>(dy, x, k, dx, dk, B, D, L, omega, stream);
+  return launch_bwd<MEGA_F16>(dy, x, k, dx, dk, B, D, L, omega, stream);
 }
 
 }  // namespace fftm

@@ -17,5 +17,10 @@ int launch_conv(int dtype, int mode, const void* a, const void* b, void* out, in
                 int64_t L, int flip, const float* omega, hipStream_t stream,
                 uint16_t* dbg = nullptr, int dbg_stage = -1);
 
+// dx (+ omega dy) and dk of the convolution in one launch (dy is transformed once);
+// dk (D, L) fp32 is overwritten.  Same applicability as launch_conv; B >= 1.
+int launch_backward(int dtype, const void* dy, const void* x, const float* k, void* dx, float* dk,
+                    int64_t B, int64_t D, int64_t L, const float* omega, hipStream_t stream);
+
 }  // namespace fftm
 }  // namespace mega
