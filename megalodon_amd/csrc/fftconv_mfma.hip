@@ -2,7 +2,7 @@
 //
 // One workgroup (8 waves) owns one row at a time.  The zero-padded real row of
 // 2N = 65536 samples is packed as z[n] = s[2n] + i s[2n+1], n < N = 32768, and
-// kept in LDS as two planes (re, im) of fp16.  The N-point transform is three
+// kept in LDS as fp16 re and im values (rows of a, re half then im half).  The N-point transform is three
 // radix-32 stages over the digits of n = 1024 a + 32 b + c:
 //     forward  F1 over a, F2 over b, F3 over c  -> Z[k1 + 32 k2 + 1024 k3] at (k1, k2, k3)
 //     inverse  I1 over c, I2 over b, I3 over a  -> z[n] back at (a, b, c)
@@ -27,8 +27,13 @@ namespace fftm {
 namespace {
 
 constexpr int kN = 32768;             // complex points per transform
-constexpr int kRS = 1024 + 32;        // elements between consecutive a (rows of the LDS planes)
-constexpr int kPlane = 32 * kRS;      // elements per plane
+// LDS: row a holds its 1024 re values, 16 elements of padding, then its 1024 im
+// values and padding.  The a-stride of 1040 dwords is 16 mod 64 banks, and the
+// im value of an element sits a constant 2080 bytes after its re value, which
+// every access folds into the instruction's immediate offset.
+constexpr int kIm = 1024 + 16;        // elements from a re value to its im value
+constexpr int kRS = 2 * kIm;          // elements between consecutive a
+constexpr int kPlane = 16 * kRS;      // half of the LDS elements (two "planes" of 32 half rows)
 constexpr int kThreads = 512;         // 8 waves, two per SIMD
 constexpr int kWaves = kThreads / kWave;
 constexpr size_t kLdsBytes = sizeof(uint16_t) * 2 * kPlane + 64;
@@ -154,21 +159,6 @@ __device__ __forceinline__ void dft_xb(const u32x4* xr, const u32x4* xi, const D
   }
 }
 
-// write a result tile: register quad qd of a lane holds 4 consecutive c
-// starting at 8 qd + 4 (lane / 32); `at(c0)` gives the element offset
-template <typename At>
-__device__ __forceinline__ void write_tile(uint16_t* pre, uint16_t* pim, const floatx16& dr,
-                                           const floatx16& di, int g, At at) {
-#pragma unroll
-  for (int qd = 0; qd < 4; ++qd) {
-    const int o = at(8 * qd + 4 * g);
-    *reinterpret_cast<uint2*>(pre + o) =
-        make_uint2(pack_h2(dr[4 * qd], dr[4 * qd + 1]), pack_h2(dr[4 * qd + 2], dr[4 * qd + 3]));
-    *reinterpret_cast<uint2*>(pim + o) =
-        make_uint2(pack_h2(di[4 * qd], di[4 * qd + 1]), pack_h2(di[4 * qd + 2], di[4 * qd + 3]));
-  }
-}
-
 // exp(+i 2 pi c m / N) for the 16 values c = 8 qd + 4 g + e a lane holds after a
 // stage (register 4 qd + e), from three sin/cos pairs and complex products:
 // W^(c m) = W^(4 g m) (W^(8 m))^qd (W^m)^e.
@@ -215,26 +205,55 @@ __device__ __forceinline__ void apply_tw(floatx16& dr, floatx16& di, const Tw16&
   }
 }
 
-// ---- stages over a (F1 / I3): tile = fixed b, rows a, bystander c -------------
-// F1: only a < 16 holds data (zero padding) -> one k-step; twiddle W_1024^(b k1).
-// I3: all 32 rows; no twiddle.
-template <bool INV>
-__device__ __forceinline__ void stage_a(uint16_t* pre, uint16_t* pim, const Dft& w, int wave,
-                                        int lane) {
-  for (int b = wave; b < 32; b += kWaves) {
-    lane = opaque(lane) & 63;
-    const int g = lane >> 5, f = lane & 31;
-    const int rsrc = 8 * g + ((lane & 15) >> 2);          // + 16 s + 4 h
-    const int csrc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    u32x4 xr[2], xi[2];
+// Per-lane pieces of the LDS offsets (elements), computed once per stage call.
+// A tile adds its own digit (wave-uniform, scalar) and XORs its swizzle bits.
+struct LaneGeo {
+  int g, f;         // lane / 32, lane % 32
+  int rd[2];        // transposing read, h = 0, 1: row part + swizzled source column
+  int wr;           // tile write: lane part
+};
+// quad slot q of a tile write lands at 8 (q ^ x): x = swizzle bits of (tile digit, lane digit)
+__device__ __forceinline__ void write_tile_x(uint16_t* pre, const floatx16& dr, const floatx16& di,
+                                             int base, int x) {
 #pragma unroll
-    for (int s = 0; s < (INV ? 2 : 1); ++s) {
-      const int o0 = pos(16 * s + rsrc, b, csrc), o1 = pos(16 * s + rsrc + 4, b, csrc);
-      const uint2 r0 = lds_read_tr(pre + o0), r1 = lds_read_tr(pre + o1);
-      const uint2 i0 = lds_read_tr(pim + o0), i1 = lds_read_tr(pim + o1);
-      xr[s] = u32x4{r0.x, r0.y, r1.x, r1.y};
-      xi[s] = u32x4{i0.x, i0.y, i1.x, i1.y};
-    }
+  for (int qd = 0; qd < 4; ++qd) {
+    uint16_t* q = pre + base + ((qd ^ x) << 3);
+    *reinterpret_cast<uint2*>(q) =
+        make_uint2(pack_h2(dr[4 * qd], dr[4 * qd + 1]), pack_h2(dr[4 * qd + 2], dr[4 * qd + 3]));
+    *reinterpret_cast<uint2*>(q + kIm) =
+        make_uint2(pack_h2(di[4 * qd], di[4 * qd + 1]), pack_h2(di[4 * qd + 2], di[4 * qd + 3]));
+  }
+}
+template <int KSTEPS, int SSTRIDE>
+__device__ __forceinline__ void read_tile_tr(const uint16_t* pre, int o0, int o1, u32x4* xr,
+                                             u32x4* xi) {
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    const uint2 r0 = lds_read_tr(pre + o0 + s * SSTRIDE), r1 = lds_read_tr(pre + o1 + s * SSTRIDE);
+    const uint2 i0 = lds_read_tr(pre + o0 + s * SSTRIDE + kIm);
+    const uint2 i1 = lds_read_tr(pre + o1 + s * SSTRIDE + kIm);
+    xr[s] = u32x4{r0.x, r0.y, r1.x, r1.y};
+    xi[s] = u32x4{i0.x, i0.y, i1.x, i1.y};
+  }
+}
+
+// ---- stages over a (F1 / I3): tile = fixed b, rows a, bystander c -------------
+// F1 (a -> k1): only a < 16 holds data (zero padding) -> one k-step; then
+// twiddle W_1024^(b k1), one factor per lane.  I3 (k1 -> a): all 32 rows, no twiddle.
+template <bool INV>
+__device__ __forceinline__ void stage_a(uint16_t* pre, const Dft& w, int wave, int lane) {
+  lane = opaque(lane) & 63;
+  const int g = lane >> 5, f = lane & 31;
+  const int rsrc = 8 * g + ((lane & 15) >> 2), csrc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  // pos(16 s + rsrc + 4 h, b, csrc): the row's swizzle bits are (2 g + h) & 3
+  const int rd0 = rsrc * kRS + (csrc ^ (((2 * g) & 3) << 3));
+  const int rd1 = (rsrc + 4) * kRS + (csrc ^ (((2 * g + 1) & 3) << 3));
+  const int wr = f * kRS + 4 * g, fx = (f >> 2) & 3;
+  const int wv = __builtin_amdgcn_readfirstlane(wave);
+  for (int b = wv; b < 32; b += kWaves) {
+    const int bx = ((b >> 2) & 3) << 3;
+    u32x4 xr[2], xi[2];
+    read_tile_tr<INV ? 2 : 1, 16 * kRS>(pre, (rd0 ^ bx) + 32 * b, (rd1 ^ bx) + 32 * b, xr, xi);
     floatx16 dr, di;
     dft_xa<INV, INV ? 2 : 1>(xr, xi, w, dr, di);
     if (!INV) {
@@ -247,7 +266,7 @@ __device__ __forceinline__ void stage_a(uint16_t* pre, uint16_t* pim, const Dft&
         di[r] = vi * tc - vr * ts;
       }
     }
-    write_tile(pre, pim, dr, di, g, [&](int c0) { return pos(f, b, c0); });
+    write_tile_x(pre, dr, di, wr + 32 * b, fx ^ (bx >> 3));
   }
 }
 
@@ -255,22 +274,18 @@ __device__ __forceinline__ void stage_a(uint16_t* pre, uint16_t* pim, const Dft&
 // F2 (b -> k2): then twiddle W_N^(c (a + 32 k2)).  I2 (k2 -> n2): undoes F1's
 // twiddle, conj W_1024^(n2 a), one factor per lane.
 template <bool INV>
-__device__ __forceinline__ void stage_b(uint16_t* pre, uint16_t* pim, const Dft& w, int wave,
-                                        int lane) {
-  for (int a = wave; a < 32; a += kWaves) {
-    lane = opaque(lane) & 63;
-    const int g = lane >> 5, f = lane & 31;
-    const int rsrc = 8 * g + ((lane & 15) >> 2);
-    const int csrc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+__device__ __forceinline__ void stage_b(uint16_t* pre, const Dft& w, int wave, int lane) {
+  lane = opaque(lane) & 63;
+  const int g = lane >> 5, f = lane & 31;
+  const int rsrc = 8 * g + ((lane & 15) >> 2), csrc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const int rd0 = 32 * rsrc + (csrc ^ (((2 * g) & 3) << 3));
+  const int rd1 = 32 * (rsrc + 4) + (csrc ^ (((2 * g + 1) & 3) << 3));
+  const int wr = 32 * f + 4 * g, fx = (f >> 2) & 3;
+  const int wv = __builtin_amdgcn_readfirstlane(wave);
+  for (int a = wv; a < 32; a += kWaves) {
+    const int ax = ((a >> 2) & 3) << 3;
     u32x4 xr[2], xi[2];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const int o0 = pos(a, 16 * s + rsrc, csrc), o1 = pos(a, 16 * s + rsrc + 4, csrc);
-      const uint2 r0 = lds_read_tr(pre + o0), r1 = lds_read_tr(pre + o1);
-      const uint2 i0 = lds_read_tr(pim + o0), i1 = lds_read_tr(pim + o1);
-      xr[s] = u32x4{r0.x, r0.y, r1.x, r1.y};
-      xi[s] = u32x4{i0.x, i0.y, i1.x, i1.y};
-    }
+    read_tile_tr<2, 512>(pre, (rd0 ^ ax) + a * kRS, (rd1 ^ ax) + a * kRS, xr, xi);
     floatx16 dr, di;
     dft_xa<INV, 2>(xr, xi, w, dr, di);
     if (!INV) {
@@ -286,7 +301,7 @@ __device__ __forceinline__ void stage_b(uint16_t* pre, uint16_t* pim, const Dft&
         di[r] = vi * tc + vr * ts;
       }
     }
-    write_tile(pre, pim, dr, di, g, [&](int c0) { return pos(a, f, c0); });
+    write_tile_x(pre, dr, di, wr + a * kRS, fx ^ (ax >> 3));
   }
 }
 
@@ -294,17 +309,21 @@ __device__ __forceinline__ void stage_b(uint16_t* pre, uint16_t* pim, const Dft&
 // F3 (c -> k3): no twiddle.  I1 (k3 -> n3): then undoes F2's twiddle,
 // conj W_N^(n3 (a + 32 b)).
 template <bool INV>
-__device__ __forceinline__ void stage_c(uint16_t* pre, uint16_t* pim, const Dft& w, int wave,
-                                        int lane) {
-  for (int a = wave; a < 32; a += kWaves) {
-    lane = opaque(lane) & 63;
-    const int g = lane >> 5, b = lane & 31;
+__device__ __forceinline__ void stage_c(uint16_t* pre, const Dft& w, int wave, int lane) {
+  lane = opaque(lane) & 63;
+  const int g = lane >> 5, b = lane & 31;
+  const int bx = (b >> 2) & 3, row = 32 * b;
+  const int wv = __builtin_amdgcn_readfirstlane(wave);
+  for (int a = wv; a < 32; a += kWaves) {
+    const int x = bx ^ ((a >> 2) & 3);
+    // pos(a, b, 16 s + 8 g) = row part + 8 ((2 s + g) ^ x)
+    const int base = a * kRS + row;
     u32x4 xr[2], xi[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const int o = pos(a, b, 16 * s + 8 * g);
-      xr[s] = *reinterpret_cast<const u32x4*>(pre + o);
-      xi[s] = *reinterpret_cast<const u32x4*>(pim + o);
+      const uint16_t* q = pre + base + (((2 * s + g) ^ x) << 3);
+      xr[s] = *reinterpret_cast<const u32x4*>(q);
+      xi[s] = *reinterpret_cast<const u32x4*>(q + kIm);
     }
     floatx16 dr, di;
     dft_xb<INV>(xr, xi, w, dr, di);
@@ -312,7 +331,7 @@ __device__ __forceinline__ void stage_c(uint16_t* pre, uint16_t* pim, const Dft&
       const Tw16 t = twiddles16(a + 32 * b, g);
       apply_tw<true>(dr, di, t);
     }
-    write_tile(pre, pim, dr, di, g, [&](int c0) { return pos(a, b, c0); });
+    write_tile_x(pre, dr, di, base + 4 * g, x);
   }
 }
 
@@ -320,18 +339,18 @@ template <bool INV>
 __device__ __forceinline__ void transform(uint16_t* pre, uint16_t* pim, const Dft& w, int wave,
                                           int lane) {
   if (!INV) {
-    stage_a<false>(pre, pim, w, wave, lane);
+    stage_a<false>(pre, w, wave, lane);
     lds_barrier();
-    stage_b<false>(pre, pim, w, wave, lane);
+    stage_b<false>(pre, w, wave, lane);
     lds_barrier();
-    stage_c<false>(pre, pim, w, wave, lane);
+    stage_c<false>(pre, w, wave, lane);
     lds_barrier();
   } else {
-    stage_c<true>(pre, pim, w, wave, lane);
+    stage_c<true>(pre, w, wave, lane);
     lds_barrier();
-    stage_b<true>(pre, pim, w, wave, lane);
+    stage_b<true>(pre, w, wave, lane);
     lds_barrier();
-    stage_a<true>(pre, pim, w, wave, lane);
+    stage_a<true>(pre, w, wave, lane);
     lds_barrier();
   }
 }
@@ -685,7 +704,7 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_kernel(
     int dbg_stage) {
   extern __shared__ __align__(16) uint16_t lds[];
   uint16_t* pre = lds;
-  uint16_t* pim = lds + kPlane;
+  uint16_t* pim = lds + kIm;
   float* red = reinterpret_cast<float*>(lds + 2 * kPlane);
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const Dft w = make_dft(lane);
@@ -769,7 +788,7 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_bwd_kernel(
     const float* __restrict__ omega) {
   extern __shared__ __align__(16) uint16_t lds[];
   uint16_t* pre = lds;
-  uint16_t* pim = lds + kPlane;
+  uint16_t* pim = lds + kIm;
   float* red = reinterpret_cast<float*>(lds + 2 * kPlane);
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const Dft w = make_dft(lane);
