@@ -231,14 +231,17 @@ __device__ __forceinline__ Wel fwd_lookback(const TsnParams& p, int b, int g, in
     if (idx >= 0) {
       const unsigned long long* r = rec + static_cast<int64_t>(idx) * kFwdWords;
       while (true) {
+        // all four words in one round trip: the aggregate is checked only if
+        // the inclusive prefix is not there yet
         float iu, iv, au, av;
-        const bool fi = get_word(r + 2, iu) & get_word(r + 3, iv);
+        const bool f2 = get_word(r + 2, iu), f3 = get_word(r + 3, iv);
+        const bool f0 = get_word(r + 0, au), f1 = get_word(r + 1, av);
+        const bool fi = f2 & f3, fa = f0 & f1;
         if (fi) {
           kind = 2;
           val = Wel{prior.n + static_cast<float>(nb[idx + 1]), iu, iv};
           break;
         }
-        const bool fa = get_word(r + 0, au) & get_word(r + 1, av);
         if (fa) {
           kind = 1;
           val = Wel{static_cast<float>(nb[idx + 1] - nb[idx]), au, av};
@@ -284,6 +287,8 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
   const bool col_ok = col * VEC < p.Dg;
   const float inv_dg = 1.f / static_cast<float>(p.Dg);
 
+  // everything the tile needs from memory is requested up front: the rows, the
+  // affine parameters of the last phase and the chain's prior state
   uint4 xv[P];
 #pragma unroll
   for (int q = 0; q < P; ++q) {
@@ -294,6 +299,18 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
       const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
       xv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.x) + off);
     }
+  }
+  uint4 gmv = make_uint4(0, 0, 0, 0), btv = make_uint4(0, 0, 0, 0);
+  if (col_ok) {
+    gmv = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.gamma) + g * p.Dg + col * VEC);
+    btv = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.beta) + g * p.Dg + col * VEC);
+  }
+  const int64_t chain64 = static_cast<int64_t>(b) * p.G + g;
+  const Wel prior{static_cast<float>(p.prev_count[b]), ldT<DT>(p.prev_mean, chain64),
+                  ldT<DT>(p.prev_var, chain64)};
+#pragma unroll
+  for (int q = 0; q < P; ++q) {
+    const int r = q * RPP + wave * RPW + lane / LPR;
     float f[VEC];
     Vec<DT>::unpack(xv[q], f);
     float s = 0.f;
@@ -322,15 +339,12 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
       const Wel o = wel_shfl_up(me, d);
       if (lane >= d) me = wel_merge(o, me);
     }
-    const int64_t chain64 = static_cast<int64_t>(b) * p.G + g;
     unsigned long long* rec = p.rec + (chain64 * p.NT + j) * kFwdWords;
     const Wel agg{__shfl(me.n, 63, 64), __shfl(me.u, 63, 64), __shfl(me.v, 63, 64)};
     if (lane == 0 && j + 1 < p.NT) {
       put_word(rec + 0, agg.u);
       put_word(rec + 1, agg.v);
     }
-    const Wel prior{static_cast<float>(p.prev_count[b]), ldT<DT>(p.prev_mean, chain64),
-                    ldT<DT>(p.prev_var, chain64)};
     const Wel prefix = j == 0 ? prior : fwd_lookback(p, b, g, j, lane, prior);
     if (lane == 0 && j + 1 < p.NT) {
       const Wel inc = wel_merge(prefix, agg);
@@ -350,7 +364,9 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
       stT<DT>(p.var, chain64, st.v);
       if (g == 0) p.count[b] = p.prev_count[b] + p.nbefore[b * (p.NT + 1) + p.NT];
     }
-    __builtin_amdgcn_s_waitcnt(0);  // s_a/s_b reads retired before they are overwritten
+    // s_a/s_b reads retired before they are overwritten (LDS only: the stores
+    // above need not have landed)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
     s_a[lane] = st.u;
     s_b[lane] = rstd;
@@ -358,11 +374,8 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
   __syncthreads();
 
   float gm[VEC], bt[VEC];
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) {
-    gm[e] = col_ok ? ldT<DT>(p.gamma, g * p.Dg + col * VEC + e) : 0.f;
-    bt[e] = col_ok ? ldT<DT>(p.beta, g * p.Dg + col * VEC + e) : 0.f;
-  }
+  Vec<DT>::unpack(gmv, gm);
+  Vec<DT>::unpack(btv, bt);
 #pragma unroll
   for (int q = 0; q < P; ++q) {
     const int r = q * RPP + wave * RPW + lane / LPR;
@@ -450,14 +463,17 @@ __device__ __forceinline__ State2 bwd_lookahead(const TsnParams& p, int64_t chai
     if (idx < p.NT) {
       const unsigned long long* r = rec + static_cast<int64_t>(idx) * kBwdWords;
       while (true) {
+        // all six words in one round trip
         float a, e, bu, bv, ug, vg;
-        const bool fs = get_word(r + 4, ug) & get_word(r + 5, vg);
+        const bool f4 = get_word(r + 4, ug), f5 = get_word(r + 5, vg);
+        const bool f0 = get_word(r + 0, a), f1 = get_word(r + 1, e);
+        const bool f2 = get_word(r + 2, bu), f3 = get_word(r + 3, bv);
+        const bool fs = f4 & f5, fa = f0 & f1 & f2 & f3;
         if (fs) {
           kind = 2;
           sv = State2{ug, vg};
           break;
         }
-        const bool fa = get_word(r + 0, a) & get_word(r + 1, e) & get_word(r + 2, bu) & get_word(r + 3, bv);
         if (fa) {
           kind = 1;
           val = Aff{a, e, bu, bv};
@@ -490,7 +506,9 @@ __device__ __forceinline__ State2 bwd_lookahead(const TsnParams& p, int64_t chai
 }
 
 template <int DT, int LPR>
-__global__ __launch_bounds__(kThreads) void tsn_bwd_kernel(const TsnParams p) {
+__global__ __launch_bounds__(kThreads)
+__attribute__((amdgpu_waves_per_eu(LPR <= 16 ? 4 : (LPR == 32 ? 2 : 1))))  // 132 -> 128 registers at LPR 16: one more wave per SIMD
+void tsn_bwd_kernel(const TsnParams p) {
   constexpr int VEC = Vec<DT>::N;
   constexpr int RPW = kWave / LPR;
   constexpr int RPP = RPW * kWaves;
@@ -513,23 +531,8 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_kernel(const TsnParams p) {
   const bool col_ok = col * VEC < p.Dg;
   const float inv_dg = 1.f / static_cast<float>(p.Dg);
 
-  float gm[VEC];
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) gm[e] = col_ok ? ldT<DT>(p.gamma, g * p.Dg + col * VEC + e) : 0.f;
-
-  // statistics saved by the forward pass, one row per lane of every wave
-  {
-    const int t = t0 + lane;
-    if (wave == 0) {
-      const bool in = t < p.L;
-      const int64_t o = (static_cast<int64_t>(b) * p.L + (in ? t : 0)) * p.G + g;
-      s_u[lane] = in ? p.cummean_in[o] : 0.f;
-      s_r[lane] = in ? p.cumrstd_in[o] : 0.f;
-      s_valid[lane] = (in && (p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0)) ? 1 : 0;
-    }
-  }
-  __syncthreads();
-
+  // everything the tile needs from memory is requested up front: the rows of x
+  // and dy, gamma, the saved statistics and the chain's boundary values
   uint4 xv[P], dv[P];
 #pragma unroll
   for (int q = 0; q < P; ++q) {
@@ -542,6 +545,37 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_kernel(const TsnParams p) {
       xv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.x) + off);
       dv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.dy) + off);
     }
+  }
+  uint4 gmv = make_uint4(0, 0, 0, 0);
+  if (col_ok)
+    gmv = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.gamma) + g * p.Dg + col * VEC);
+  const int64_t chain64 = static_cast<int64_t>(b) * p.G + g;
+  // wave 0 only uses these; loading them in every wave keeps the code uniform
+  const float before_u = t0 == 0 ? ldT<DT>(p.prev_mean, chain64)
+                                 : p.cummean_in[(static_cast<int64_t>(b) * p.L + t0 - 1) * p.G + g];
+  const State2 init{ldT<DT>(p.dmean, chain64), ldT<DT>(p.dvar, chain64)};
+  const int* nb = p.nbefore + b * (p.NT + 1);
+  const int64_t n0 = p.prev_count[b] - nb[p.NT];  // prior count
+  const int nbj = nb[j];
+
+  // statistics saved by the forward pass, one row per lane
+  {
+    const int t = t0 + lane;
+    if (wave == 0) {
+      const bool in = t < p.L;
+      const int64_t o = (static_cast<int64_t>(b) * p.L + (in ? t : 0)) * p.G + g;
+      s_u[lane] = in ? p.cummean_in[o] : 0.f;
+      s_r[lane] = in ? p.cumrstd_in[o] : 0.f;
+      s_valid[lane] = (in && (p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0)) ? 1 : 0;
+    }
+  }
+  __syncthreads();
+  float gm[VEC];
+  Vec<DT>::unpack(gmv, gm);
+
+#pragma unroll
+  for (int q = 0; q < P; ++q) {
+    const int r = q * RPP + wave * RPW + lane / LPR;
     float f[VEC], d[VEC];
     Vec<DT>::unpack(xv[q], f);
     Vec<DT>::unpack(dv[q], d);
@@ -567,26 +601,15 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_kernel(const TsnParams p) {
   __syncthreads();
 
   if (wave == 0) {
-    const int64_t chain64 = static_cast<int64_t>(b) * p.G + g;
-    const int t = t0 + lane;
     const bool valid = s_valid[lane] != 0;
-    const int* nb = p.nbefore + b * (p.NT + 1);
     // n_t = number of valid steps up to and including t, prior included
     const unsigned long long vm = __ballot(valid);
     const int incl = __popcll(vm & ((lane == 63) ? ~0ull : ((1ull << (lane + 1)) - 1ull)));
-    const int64_t n0 = p.prev_count[b] - nb[p.NT];  // prior count
-    const float nt = static_cast<float>(n0 + nb[j] + incl);
+    const float nt = static_cast<float>(n0 + nbj + incl);
     const float c1 = valid ? (nt - 1.f) / nt : 0.f;
     const float c2 = valid ? 1.f / nt : 0.f;
     const float r = s_r[lane], ux = s_ux[lane];
-    float prev_u;
-    if (t == 0) {
-      prev_u = ldT<DT>(p.prev_mean, chain64);
-    } else if (lane == 0) {
-      prev_u = p.cummean_in[(static_cast<int64_t>(b) * p.L + t - 1) * p.G + g];
-    } else {
-      prev_u = s_u[lane - 1];
-    }
+    const float prev_u = lane == 0 ? before_u : s_u[lane - 1];
     const float delta = ux - prev_u;
     const float pu = -r * s_db[lane];
     const float pv = -0.5f * r * r * r * s_ds[lane];
@@ -606,7 +629,6 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_kernel(const TsnParams p) {
       put_word(rec + 2, inc.bu);
       put_word(rec + 3, inc.bv);
     }
-    const State2 init{ldT<DT>(p.dmean, chain64), ldT<DT>(p.dvar, chain64)};
     const State2 sin = j == p.NT - 1 ? init : bwd_lookahead(p, chain64, j, lane, init);
     // state entering row i = (X_(i+1) o ... o X_63)(sin)
     Aff exc = aff_shfl_down(inc, 1);
@@ -626,7 +648,7 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_kernel(const TsnParams p) {
     const float dvv = si.vg + pv;
     const float dux = c2 * du + 2.f * c1 * c2 * dvv * delta;
     const float dvx = c2 * dvv;
-    __builtin_amdgcn_s_waitcnt(0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // LDS reads above retired
     __builtin_amdgcn_wave_barrier();
     s_ds[lane] = dux;
     s_db[lane] = dvx;
@@ -795,7 +817,8 @@ WsLayout ws_layout(int64_t B, int64_t L, int64_t D, int64_t G, int words, bool p
 bool fast_path_ok(int dtype, int64_t D, int64_t Dg, const void* a, const void* b, const void* c) {
   const int vec = dtype == MEGA_F32 ? 4 : 8;
   const auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  return Dg % vec == 0 && D % vec == 0 && Dg / vec <= 64 && al(a) && al(b) && (c == nullptr || al(c));
+  return Dg % vec == 0 && D % vec == 0 && Dg / vec <= 64 && al(a) && (b == nullptr || al(b)) &&
+         (c == nullptr || al(c));
 }
 
 template <int DT, bool FWD>
@@ -821,7 +844,7 @@ int launch_fast(const TsnParams& p, int64_t tiles, hipStream_t s) {
 template <int DT>
 int tsn_fwd_impl(TsnParams p, void* workspace, hipStream_t s) {
   const int64_t NT = p.NT;
-  if (fast_path_ok(DT, p.D, p.Dg, p.x, p.y, nullptr)) {
+  if (fast_path_ok(DT, p.D, p.Dg, p.x, p.y, nullptr) && fast_path_ok(DT, p.D, p.Dg, p.gamma, p.beta, nullptr)) {
     const WsLayout w = ws_layout(p.B, p.L, p.D, p.G, kFwdWords, false);
     char* ws = static_cast<char*>(workspace);
     p.ticket = reinterpret_cast<int*>(ws + w.ticket_off);
@@ -847,7 +870,7 @@ int tsn_bwd_impl(TsnParams p, void* dgamma, void* dbeta, void* workspace, hipStr
   p.part_g = reinterpret_cast<float*>(ws + w.part_off);
   p.part_b = p.part_g + static_cast<int64_t>(p.B) * NT * p.D;
   int rows;
-  if (fast_path_ok(DT, p.D, p.Dg, p.x, p.y, p.dy)) {
+  if (fast_path_ok(DT, p.D, p.Dg, p.x, p.y, p.dy) && fast_path_ok(DT, p.D, p.Dg, p.gamma, nullptr, nullptr)) {
     p.ticket = reinterpret_cast<int*>(ws + w.ticket_off);
     int* nbefore = reinterpret_cast<int*>(ws + w.nbefore_off);
     p.nbefore = nbefore;
