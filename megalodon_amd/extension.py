@@ -41,6 +41,45 @@ def _as_c64(t: torch.Tensor, name: str) -> torch.Tensor:
 # --------------------------------------------------------------------------
 # ema_parameters (reference: csrc/ops/ema_parameters.cc:195-290)
 # --------------------------------------------------------------------------
+def _weight_rows(coef: torch.Tensor, log_q_rows: torch.Tensor, L: int) -> torch.Tensor:
+    """rows[r, j] = sum_n Re(coef[r, n] q[r, n]^j), j < L: the weight kernel with
+    one complex coefficient per (row, mode) (p = 1, gamma = coef)."""
+    R, N = coef.shape
+    dev = coef.device
+    ones = torch.ones((R, N), dtype=torch.float32, device=dev)
+    out = torch.empty((R, L), dtype=torch.float32, device=dev)
+    cf, lq = coef.contiguous(), log_q_rows.contiguous()
+    with torch.cuda.device(dev):
+        _lib.call("mega_ema_weight_fwd", _lib.ptr(ones), _lib.ptr(lq), _lib.ptr(cf), _lib.i64(R),
+                  _lib.i64(N), _lib.i64(L), _lib.ptr(out), _lib.stream_ptr(dev))
+    return out
+
+
+def _row_moments(rows: torch.Tensor, log_q_rows: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(S2, S1)[r, n] = (sum_j rows[r, j] q^j, sum_j j rows[r, j] q^(j-1)): the
+    weight-backward kernel with p = gamma = 1, whose dgamma = conj(S2) and
+    dq = conj(S1) (ema_parameters.cc:80-98)."""
+    R, L = rows.shape
+    N = log_q_rows.shape[1]
+    dev = rows.device
+    ones = torch.ones((R, N), dtype=torch.float32, device=dev)
+    onec = torch.ones((R, N), dtype=torch.complex64, device=dev)
+    dp = torch.empty((R, N), dtype=torch.float32, device=dev)
+    dq = torch.empty((R, N), dtype=torch.complex64, device=dev)
+    dg = torch.empty((R, N), dtype=torch.complex64, device=dev)
+    rw, lq = rows.contiguous(), log_q_rows.contiguous()
+    with torch.cuda.device(dev):
+        _lib.call("mega_ema_weight_bwd", _lib.ptr(rw), _lib.ptr(ones), _lib.ptr(lq), _lib.ptr(onec),
+                  _lib.i64(R), _lib.i64(N), _lib.i64(L), _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg),
+                  _lib.stream_ptr(dev))
+    return dg.conj().resolve_conj(), dq.conj().resolve_conj()
+
+
+def _qpow(log_q: torch.Tensor, k: int) -> torch.Tensor:
+    """q^k in complex64, evaluated in complex128 (k * arg q loses bits in float32)."""
+    return torch.exp(log_q.to(torch.complex128) * float(k)).to(torch.complex64)
+
+
 def ema_parameters_fwd(
     p: torch.Tensor,
     log_q: torch.Tensor,
@@ -48,15 +87,16 @@ def ema_parameters_fwd(
     h: Optional[torch.Tensor],
     L: int,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
-    """(w, b, v) = ema_parameters_fwd(p, log_q, gamma, h, L); weight path only.
+    """(w, b, v) = ema_parameters_fwd(p, log_q, gamma, h, L).
 
-    p (D,N[,1]) float32, log_q/gamma complex64 -> w (D, L) float32.  With
-    ``h`` given the reference also returns the bias of the carried state
-    (ema_parameters.cc:56-77); that branch is not part of this library yet.
+    p (D,N[,1]) float32, log_q/gamma complex64 -> w (D, L) float32.  With the
+    carried state ``h`` (B, D, N) complex64 also the bias
+    ``b[b,d,j] = sum_n Re(q^(j+1) gamma h[b,d,n])`` (B, D, L)
+    (ema_parameters.cc:56-77): the weight kernel run on the B*D rows with the
+    coefficient q*gamma*h.  ``v`` (the reference's Vandermonde scratch for B > 8)
+    is never needed and stays ``None``.
     """
     dev = _require_cuda(p, log_q, gamma, h)
-    if h is not None:
-        raise NotImplementedError("ema_parameters with a carried state (h) is not implemented")
     if p.dtype != torch.float32:
         raise RuntimeError(f"p must be float32 (got {p.dtype})")
     D, N = p.shape[0], p.shape[1]
@@ -67,7 +107,17 @@ def ema_parameters_fwd(
     with torch.cuda.device(dev):
         _lib.call("mega_ema_weight_fwd", _lib.ptr(p_c), _lib.ptr(lq), _lib.ptr(gm),
                   _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(w), _lib.stream_ptr(dev))
-    return w, None, None
+    if h is None:
+        return w, None, None
+    hc = _as_c64(h, "h")
+    if hc.dim() != 3 or hc.shape[1] != D or hc.shape[2] != N:
+        raise RuntimeError(f"h must be (B, {D}, {N}) (got {tuple(hc.shape)})")
+    B = hc.shape[0]
+    lq2, gm2 = lq.reshape(D, N), gm.reshape(D, N)
+    coef = (torch.exp(lq2) * gm2).unsqueeze(0) * hc
+    lq_rows = lq2.unsqueeze(0).expand(B, D, N).reshape(B * D, N)
+    b = _weight_rows(coef.reshape(B * D, N), lq_rows, L).view(B, D, L)
+    return w, b, None
 
 
 def ema_parameters_bwd(
@@ -80,10 +130,8 @@ def ema_parameters_bwd(
     v: Optional[torch.Tensor],
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     """(dp, dq, dgamma, dh); gradients w.r.t. q (not log q), PyTorch conjugate
-    convention (ema_parameters.cc:80-98)."""
+    convention (ema_parameters.cc:80-98; bias part :100-117,158-188)."""
     dev = _require_cuda(w_grad, p, log_q, gamma, h, b_grad)
-    if h is not None or b_grad is not None:
-        raise NotImplementedError("ema_parameters with a carried state (h) is not implemented")
     if p.dtype != torch.float32 or w_grad.dtype != torch.float32:
         raise RuntimeError("p and w_grad must be float32")
     D, N = p.shape[0], p.shape[1]
@@ -99,7 +147,84 @@ def ema_parameters_bwd(
         _lib.call("mega_ema_weight_bwd", _lib.ptr(dw), _lib.ptr(p_c), _lib.ptr(lq), _lib.ptr(gm),
                   _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg),
                   _lib.stream_ptr(dev))
-    return dp, dq, dg, None
+    if b_grad is None:
+        return dp, dq, dg, (torch.zeros_like(h) if h is not None else None)
+    if h is None:
+        raise RuntimeError("ema_parameters_bwd: a bias gradient needs the carried state h")
+    hc = _as_c64(h, "h")
+    B = hc.shape[0]
+    lq2, gm2 = lq.reshape(D, N), gm.reshape(D, N)
+    lq_rows = lq2.unsqueeze(0).expand(B, D, N).reshape(B * D, N)
+    s2, s1 = _row_moments(b_grad.reshape(B * D, L).float(), lq_rows)
+    s2, s1 = s2.view(B, D, N), s1.view(B, D, N)
+    q = torch.exp(lq2)
+    sum2 = q * s2               # sum_i db_i q^(i+1)
+    sum1 = q * s1 + s2          # sum_i (i+1) db_i q^i
+    dq = dq + torch.conj(sum1 * gm2 * hc).sum(dim=0).reshape(dq.shape)
+    dg = dg + torch.conj(sum2 * hc).sum(dim=0).reshape(dg.shape)
+    dh = torch.conj(sum2 * gm2)
+    return dp, dq, dg, dh
+
+
+# --------------------------------------------------------------------------
+# ema_hidden (reference: csrc/ops/ema_hidden.cc:16-159, fused_ops/ema_hidden.py)
+# --------------------------------------------------------------------------
+def ema_hidden_fwd(
+    x: torch.Tensor,
+    p: torch.Tensor,
+    log_q: torch.Tensor,
+    h: Optional[torch.Tensor],
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Last EMA state ``y[b,d,n] = p sum_j q^(L-1-j) x[b,d,j] (+ q^L h)``
+    (ema_hidden.cc:16-62) and the saved moments ``v`` for backward.
+
+    The time-reversed rows go through the weight-backward kernel, whose two sums
+    over a row are exactly ``sum_i q^i x'[i]`` and ``sum_i i q^(i-1) x'[i]``;
+    ``v`` stacks them (2, B, D, N) in place of the reference's Vandermonde tensor.
+    x (B, D, L) any float dtype; p (D,N[,1]) float32; log_q complex64."""
+    dev = _require_cuda(x, p, log_q, h)
+    if p.dtype != torch.float32:
+        raise RuntimeError(f"p must be float32 (got {p.dtype})")
+    B, D, L = x.shape
+    N = p.shape[1]
+    lq2 = _as_c64(log_q, "log_q").reshape(D, N)
+    lq_rows = lq2.unsqueeze(0).expand(B, D, N).reshape(B * D, N)
+    s2, s1 = _row_moments(x.flip(-1).reshape(B * D, L).float(), lq_rows)
+    s2, s1 = s2.view(B, D, N), s1.view(B, D, N)
+    y = p.reshape(D, N) * s2
+    if h is not None:
+        y = y + _qpow(lq2, L) * _as_c64(h, "h")
+    return y, torch.stack([s2, s1])
+
+
+def ema_hidden_bwd(
+    y_grad: torch.Tensor,
+    x: torch.Tensor,
+    p: torch.Tensor,
+    log_q: torch.Tensor,
+    h: Optional[torch.Tensor],
+    v: torch.Tensor,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """(dx, dp, dq, dh) of ``ema_hidden_fwd`` (ema_hidden.cc:64-159)."""
+    dev = _require_cuda(y_grad, x, p, log_q, h, v)
+    B, D, L = x.shape
+    N = p.shape[1]
+    lq2 = _as_c64(log_q, "log_q").reshape(D, N)
+    lq_rows = lq2.unsqueeze(0).expand(B, D, N).reshape(B * D, N)
+    p2 = p.reshape(D, N)
+    dyc = torch.conj(_as_c64(y_grad, "y_grad")).resolve_conj()
+    s2, s1 = v[0], v[1]
+    # dx[j] = sum_n Re(conj(dy) p q^(L-1-j)): the weight kernel, then reversed in time
+    dx = _weight_rows((dyc * p2).reshape(B * D, N), lq_rows, L).view(B, D, L).flip(-1).to(x.dtype)
+    dp = (dyc * s2).real.sum(dim=0).reshape(p.shape)
+    dq_sum = (dyc * p2 * s1).sum(dim=0)
+    dh = None
+    if h is not None:
+        hc = _as_c64(h, "h")
+        dq_sum = dq_sum + (dyc * hc).sum(dim=0) * _qpow(lq2, L - 1) * float(L)
+        dh = torch.conj(dyc * _qpow(lq2, L))
+    dq = torch.conj(dq_sum).reshape(log_q.shape)
+    return dx, dp, dq, dh
 
 
 # --------------------------------------------------------------------------

@@ -9,7 +9,7 @@ import math
 import torch
 from torch import nn
 
-from ..fused_ops import ema_parameters, fftconv_residual
+from ..fused_ops import ema_hidden, ema_parameters, fftconv_residual
 
 _r2c = torch.view_as_complex
 
@@ -84,16 +84,17 @@ class MultiHeadComplexEMA(nn.Module):
         compute_last_state: bool = False,
     ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
         # B x D x L
-        if hx is not None or compute_last_state:
-            raise NotImplementedError(
-                "carried EMA state (hx / compute_last_state) is outside the single-sequence training path")
         bsz, _, seq_len = x.size()
         p, q, gamma = self.coeffs()
         k, b = ema_parameters(p, q, gamma, hx, seq_len)
         # fftconv(x, k) + x * omega, the skip term folded into the convolution's
         # output pass (the reference adds `residual = x * self.omega` afterwards)
         output = fftconv_residual(x, k, self.omega)
-        return output, None
+        if b is not None:
+            output = output + b.to(output)
+        # compute the last hidden state
+        h = ema_hidden(x, p, q, hx) if compute_last_state else None
+        return output, h
 
     def extra_repr(self) -> str:
         return 'edim={} ({}), ndim={}'.format(self.embed_dim, self.dim_per_partition, self.ndim)

@@ -13,6 +13,11 @@ Pinning status (what independently fixes each function; see tests/test_oracle_*.
   invariance), torch autograd over the complex128 closed form, central finite
   differences, and -- where ``oracle/_ref`` is built -- the reference's own
   C++ CPU path compiled from /root/reference.
+* ``cema.ema_bias_fwd/bwd``, ``cema.ema_hidden_fwd/bwd`` (carried state):
+  pinned by the EMA recurrence h_t = q h_(t-1) + p x_t run step by step,
+  by splitting a sequence in two with the state handed over, by autograd over
+  the complex128 closed forms and by the reference's EMAParametersCPU* /
+  EMAHiddenCPU* operators (``oracle/_ref``).
 * ``fftconv.fftconv_fwd/bwd``: pinned by brute-force O(L^2) causal sums,
   ``numpy.convolve``, the EMA recurrence (no FFT involved) and autograd.
 * ``timestep_norm.group_timestep_norm_fwd/bwd``: pinned by brute-force

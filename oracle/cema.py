@@ -116,3 +116,77 @@ def cema_forward(x, p, q, gamma, omega):
         ys.append((gamma * h).real.sum(-1))
     y = torch.stack(ys, dim=-1)
     return y + x * omega.double().reshape(1, D, 1)
+
+
+# ---- carried state: bias of ema_parameters and the last hidden state ---------------
+def _c128(t, *shape):
+    return t.reshape(*shape).to(torch.complex128)
+
+
+def ema_bias_fwd(log_q, gamma, h, L):
+    """b[b, d, j] = sum_n Re(exp(log_q (j + 1)) gamma h[b, d, n]) (ema_parameters.cc:56-77).
+    h: (B, D, N) complex.  Returns float64 (B, D, L)."""
+    B, D, N = h.shape
+    lq, g, hh = _c128(log_q, D, N), _c128(gamma, D, N), h.to(torch.complex128)
+    j = torch.arange(1, L + 1, dtype=torch.float64)
+    qw = torch.exp(lq.unsqueeze(-1) * j)  # (D, N, L): q^(j+1)
+    return ((g.unsqueeze(-1) * qw).unsqueeze(0) * hh.unsqueeze(-1)).real.sum(dim=2)
+
+
+def ema_bias_bwd(db, log_q, gamma, h):
+    """(dq, dgamma, dh) contributions of the bias, restating RowwiseEMABiasCPUBwd
+    and its caller (ema_parameters.cc:100-117, 158-188):
+      sum1 = sum_i db[i] (i + 1) q^i,  sum2 = sum_i db[i] q^(i + 1)
+      dq += conj(sum1 gamma h), dgamma += conj(sum2 h) (summed over the batch), dh = conj(sum2 gamma)."""
+    B, D, N = h.shape
+    L = db.shape[-1]
+    lq, g, hh = _c128(log_q, D, N), _c128(gamma, D, N), h.to(torch.complex128)
+    i = torch.arange(L, dtype=torch.float64)
+    qw1 = torch.exp(lq.unsqueeze(-1) * i)          # q^i
+    qw2 = qw1 * torch.exp(lq).unsqueeze(-1)        # q^(i+1)
+    dbc = db.to(torch.float64).to(torch.complex128).unsqueeze(2)  # (B, D, 1, L)
+    sum1 = (dbc * qw1 * (i + 1.0)).sum(-1)         # (B, D, N)
+    sum2 = (dbc * qw2).sum(-1)
+    return torch.conj(sum1 * g * hh).sum(0), torch.conj(sum2 * hh).sum(0), torch.conj(sum2 * g)
+
+
+def ema_hidden_fwd(x, p, log_q, h):
+    """y[b, d, n] = p sum_j exp(log_q (L - 1 - j)) x[b, d, j] (+ exp(log_q L) h)
+    (ema_hidden.cc:16-62).  Returns complex128 (B, D, N)."""
+    B, D, L = x.shape
+    pp = p.reshape(D, -1).to(torch.float64)
+    N = pp.shape[1]
+    lq = _c128(log_q, D, N)
+    e = torch.arange(L - 1, -1, -1, dtype=torch.float64)       # L - 1 - j
+    qw = torch.exp(lq.unsqueeze(-1) * e)                       # (D, N, L)
+    y = (qw.unsqueeze(0) * x.to(torch.float64).unsqueeze(2)).sum(-1) * pp
+    if h is not None:
+        y = y + torch.exp(lq * float(L)) * h.to(torch.complex128)
+    return y
+
+
+def ema_hidden_bwd(dy, x, p, log_q, h):
+    """(dx, dp, dq, dh) restating ema_hidden.cc:64-159 (PyTorch conjugate convention)."""
+    B, D, L = x.shape
+    pp = p.reshape(D, -1).to(torch.float64)
+    N = pp.shape[1]
+    lq = _c128(log_q, D, N)
+    q = torch.exp(lq)
+    dyc = torch.conj(dy.to(torch.complex128))                   # (B, D, N)
+    xx = x.to(torch.float64)
+    e = torch.arange(L - 1, -1, -1, dtype=torch.float64)       # L - 1 - j
+    qw2 = torch.exp(lq.unsqueeze(-1) * e)                      # q^(L-1-j)
+    qw1 = torch.exp(lq.unsqueeze(-1) * (e - 1.0))              # q^(L-j-2), unused at j = L-1
+    qw1[..., L - 1] = 0.0
+    dx = ((dyc * pp).unsqueeze(-1) * qw2.unsqueeze(0)).real.sum(dim=2)
+    xq2 = (qw2.unsqueeze(0) * xx.unsqueeze(2)).sum(-1)         # sum_j x q^(L-1-j)
+    xq1 = (qw1.unsqueeze(0) * (xx * e).unsqueeze(2)).sum(-1)   # sum_j x (L-1-j) q^(L-j-2)
+    dp = (dyc * xq2).real.sum(0)
+    sum2 = (dyc * pp * xq1).sum(0)
+    dh = None
+    if h is not None:
+        hh = h.to(torch.complex128)
+        qw = torch.exp(lq * float(L - 1))
+        sum2 = sum2 + (dyc * hh).sum(0) * qw * float(L)
+        dh = torch.conj(dyc * qw * q)
+    return dx, dp, torch.conj(sum2), dh

@@ -122,3 +122,50 @@ def group_timestep_norm_bwd(lib, prefix, dy, dmean, dvar, x, prev_mean, count, c
         _p(dyf), _p(dm), _p(dv), _p(xf), _p(pm), _p(cnt), _p(cm), _p(cr), _p(gm), _p(mk),
         _i(B), _i(L), _i(H), _i(G), _p(dx), _p(dpm), _p(dpv), _p(dg), _p(db))
     return dx, dpm, dpv, dg, db
+
+
+# ---- carried state (reference build only) ---------------------------------------
+def ema_bias_fwd(lib, p, log_q, gamma, h, L):
+    B, D, N = h.shape
+    pf = p.reshape(D, N).float().contiguous()
+    b = torch.empty(B, D, L, dtype=torch.float32)
+    lib.ref_ema_bias_fwd(_p(pf), _p(_c64_as_f32(log_q.reshape(D, N))), _p(_c64_as_f32(gamma.reshape(D, N))),
+                         _p(_c64_as_f32(h)), _i(B), _i(D), _i(N), _i(L), _p(b))
+    return b
+
+
+def ema_bias_bwd(lib, db, p, log_q, gamma, h):
+    B, D, N = h.shape
+    L = db.shape[-1]
+    pf = p.reshape(D, N).float().contiguous()
+    dq = torch.empty(D, N, 2, dtype=torch.float32)
+    dg = torch.empty(D, N, 2, dtype=torch.float32)
+    dh = torch.empty(B, D, N, 2, dtype=torch.float32)
+    lib.ref_ema_bias_bwd(_p(db.float().contiguous()), _p(pf), _p(_c64_as_f32(log_q.reshape(D, N))),
+                         _p(_c64_as_f32(gamma.reshape(D, N))), _p(_c64_as_f32(h)), _i(B), _i(D), _i(N),
+                         _i(L), _p(dq), _p(dg), _p(dh))
+    return torch.view_as_complex(dq), torch.view_as_complex(dg), torch.view_as_complex(dh)
+
+
+def ema_hidden_fwd(lib, x, p, log_q, h):
+    B, D, L = x.shape
+    pf = p.reshape(D, -1).float().contiguous()
+    N = pf.shape[1]
+    y = torch.empty(B, D, N, 2, dtype=torch.float32)
+    lib.ref_ema_hidden_fwd(_p(x.float().contiguous()), _p(pf), _p(_c64_as_f32(log_q.reshape(D, N))),
+                           _p(None if h is None else _c64_as_f32(h)), _i(B), _i(D), _i(N), _i(L), _p(y))
+    return torch.view_as_complex(y)
+
+
+def ema_hidden_bwd(lib, dy, x, p, log_q, h):
+    B, D, L = x.shape
+    pf = p.reshape(D, -1).float().contiguous()
+    N = pf.shape[1]
+    dx = torch.empty(B, D, L, dtype=torch.float32)
+    dp = torch.empty(D, N, dtype=torch.float32)
+    dq = torch.empty(D, N, 2, dtype=torch.float32)
+    dh = torch.empty(B, D, N, 2, dtype=torch.float32)
+    lib.ref_ema_hidden_bwd(_p(_c64_as_f32(dy)), _p(x.float().contiguous()), _p(pf),
+                           _p(_c64_as_f32(log_q.reshape(D, N))), _p(None if h is None else _c64_as_f32(h)),
+                           _i(B), _i(D), _i(N), _i(L), _p(dx), _p(dp), _p(dq), _p(dh))
+    return dx, dp, torch.view_as_complex(dq), (None if h is None else torch.view_as_complex(dh))

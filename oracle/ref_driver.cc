@@ -2,10 +2,11 @@
 // from the sources where they lie under /root/reference (see oracle/Makefile).
 // TEST INFRASTRUCTURE ONLY: used to validate the oracle restatements and,
 // optionally, as the timed CPU baseline.  Only the reference's *CPU* entry
-// points are called (EMAParametersCPUFwd/Bwd, GroupTimestepNormCPUFwd/Bwd,
+// points are called (EMAParametersCPUFwd/Bwd, EMAHiddenCPUFwd/Bwd, GroupTimestepNormCPUFwd/Bwd,
 // declared in megalodon/csrc/ops/ema_parameters.h:19-49 and timestep_norm.h).
 #include <torch/torch.h>
 
+#include "ops/ema_hidden.h"
 #include "ops/ema_parameters.h"
 #include "ops/timestep_norm.h"
 
@@ -80,5 +81,54 @@ extern "C" __attribute__((visibility("default"))) int ref_group_timestep_norm_bw
   std::memcpy(dprev_var, std::get<2>(out).data_ptr<float>(), sizeof(float) * B * G);
   std::memcpy(dgamma, std::get<3>(out).data_ptr<float>(), sizeof(float) * H);
   std::memcpy(dbeta, std::get<4>(out).data_ptr<float>(), sizeof(float) * H);
+  return 0;
+}
+
+// ---- carried state: bias branch of ema_parameters and ema_hidden (float32) -------
+// h (B, D, N) complex; b, b_grad (B, D, L).  w_grad is taken as zeros so that the
+// returned gradients are the bias contributions alone.
+extern "C" __attribute__((visibility("default"))) int ref_ema_bias_fwd(
+    const float* p, const float* log_q, const float* gamma, const float* h, int64_t B, int64_t D,
+    int64_t N, int64_t L, float* b) {
+  auto out = mo::EMAParametersCPUFwd(f32(p, {D, N}), c64(log_q, {D, N}), c64(gamma, {D, N}),
+                                     c10::make_optional(c64(h, {B, D, N})), L);
+  std::memcpy(b, std::get<1>(out)->data_ptr<float>(), sizeof(float) * B * D * L);
+  return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int ref_ema_bias_bwd(
+    const float* b_grad, const float* p, const float* log_q, const float* gamma, const float* h,
+    int64_t B, int64_t D, int64_t N, int64_t L, float* dq, float* dgamma, float* dh) {
+  auto out = mo::EMAParametersCPUBwd(torch::zeros({D, L}, torch::kFloat32),
+                                     c10::make_optional(f32(b_grad, {B, D, L})), f32(p, {D, N}),
+                                     c64(log_q, {D, N}), c64(gamma, {D, N}),
+                                     c10::make_optional(c64(h, {B, D, N})), c10::nullopt);
+  std::memcpy(dq, std::get<1>(out).data_ptr(), sizeof(float) * 2 * D * N);
+  std::memcpy(dgamma, std::get<2>(out).data_ptr(), sizeof(float) * 2 * D * N);
+  std::memcpy(dh, std::get<3>(out)->data_ptr(), sizeof(float) * 2 * B * D * N);
+  return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int ref_ema_hidden_fwd(
+    const float* x, const float* p, const float* log_q, const float* h, int64_t B, int64_t D,
+    int64_t N, int64_t L, float* y) {
+  c10::optional<torch::Tensor> hh = c10::nullopt;
+  if (h) hh = c64(h, {B, D, N});
+  auto out = mo::EMAHiddenCPUFwd(f32(x, {B, D, L}), f32(p, {D, N}), c64(log_q, {D, N}), hh);
+  std::memcpy(y, std::get<0>(out).data_ptr(), sizeof(float) * 2 * B * D * N);
+  return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int ref_ema_hidden_bwd(
+    const float* y_grad, const float* x, const float* p, const float* log_q, const float* h,
+    int64_t B, int64_t D, int64_t N, int64_t L, float* dx, float* dp, float* dq, float* dh) {
+  c10::optional<torch::Tensor> hh = c10::nullopt;
+  if (h) hh = c64(h, {B, D, N});
+  auto out = mo::EMAHiddenCPUBwd(c64(y_grad, {B, D, N}), f32(x, {B, D, L}), f32(p, {D, N}),
+                                 c64(log_q, {D, N}), hh, c10::nullopt);
+  std::memcpy(dx, std::get<0>(out).data_ptr<float>(), sizeof(float) * B * D * L);
+  std::memcpy(dp, std::get<1>(out).data_ptr<float>(), sizeof(float) * D * N);
+  std::memcpy(dq, std::get<2>(out).data_ptr(), sizeof(float) * 2 * D * N);
+  if (h) std::memcpy(dh, std::get<3>(out)->data_ptr(), sizeof(float) * 2 * B * D * N);
   return 0;
 }

@@ -1,0 +1,125 @@
+"""Carried EMA state on the GPU: the bias branch of `ema_parameters`, `ema_hidden`
+and `MultiHeadComplexEMA` with `hx` / `compute_last_state`, against the float64
+oracle.  Tolerance: rel err (max|a-b|/max|b|) <= 1e-4 for float32 tensors,
+<= 2e-2 for bfloat16 rows."""
+import math
+
+import pytest
+import torch
+
+from conftest import rel_err
+from megalodon_amd import extension as ops
+from megalodon_amd.fused_ops import ema_hidden, ema_parameters
+from megalodon_amd.modules import MultiHeadComplexEMA
+from oracle import cema
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def _close(got, want, tol):
+    """rel_err <= tol; quantities that are below float32 range in the oracle
+    (|q|^L for long rows) must simply vanish."""
+    if want.abs().max() < 1e-30:
+        return bool(got.abs().max() < 1e-30)
+    return rel_err(got, want) <= tol
+
+
+def _case(B, D, N, L, seed):
+    g = torch.Generator().manual_seed(seed)
+    p = torch.sigmoid(torch.randn(D, N, 1, generator=g))
+    rho = 1.0 - p * torch.sigmoid(torch.randn(D, N, 1, generator=g))
+    q = torch.polar(rho, torch.rand(D, N, 1, generator=g) * 2 * math.pi)
+    gamma = torch.randn(D, N, dtype=torch.complex64, generator=g)
+    h = torch.randn(B, D, N, dtype=torch.complex64, generator=g)
+    x = torch.randn(B, D, L, generator=g)
+    return p, q, gamma, h, x
+
+
+@pytest.mark.parametrize("B,D,N,L", [(2, 5, 16, 300), (1, 3, 4, 1), (3, 2, 16, 4099), (9, 2, 2, 64)])
+def test_bias_fwd_bwd_match_oracle(B, D, N, L):
+    p, q, gamma, h, _ = _case(B, D, N, L, 3 * L + B)
+    lq = q.log()
+    w, b, v = ops.ema_parameters_fwd(p.cuda(), lq.cuda(), gamma.cuda(), h.cuda(), L)
+    assert b.shape == (B, D, L) and b.dtype == torch.float32 and v is None
+    assert rel_err(w, cema.ema_weight_fwd(p, lq, gamma, L)) <= TOL
+    assert rel_err(b, cema.ema_bias_fwd(lq, gamma, h, L)) <= TOL
+    g = torch.Generator().manual_seed(L)
+    dw, db = torch.randn(D, L, generator=g), torch.randn(B, D, L, generator=g)
+    dp, dq, dg, dh = ops.ema_parameters_bwd(dw.cuda(), db.cuda(), p.cuda(), lq.cuda(), gamma.cuda(), h.cuda(), None)
+    wp, wq, wg = cema.ema_weight_bwd(dw, p, lq, gamma)
+    bq, bg, bh = cema.ema_bias_bwd(db, lq, gamma, h)
+    assert dq.shape == q.shape and dh.shape == h.shape
+    assert rel_err(dp.reshape(D, N), wp) <= TOL
+    assert rel_err(dq.reshape(D, N), wq + bq) <= TOL
+    assert rel_err(dg.reshape(D, N), wg + bg) <= TOL
+    assert _close(dh, bh, TOL)
+
+
+@pytest.mark.parametrize("B,D,N,L", [(2, 5, 16, 300), (1, 3, 4, 1), (2, 2, 16, 4099)])
+@pytest.mark.parametrize("with_h", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_hidden_fwd_bwd_match_oracle(B, D, N, L, with_h, dtype):
+    p, q, gamma, h, x = _case(B, D, N, L, 5 * L + B)
+    x = x.to(dtype)
+    lq = q.log()
+    hh = h if with_h else None
+    tol = TOL if dtype == torch.float32 else 2e-2
+    y, v = ops.ema_hidden_fwd(x.cuda(), p.cuda(), lq.cuda(), None if hh is None else hh.cuda())
+    assert y.shape == (B, D, N) and y.dtype == torch.complex64
+    assert rel_err(y, cema.ema_hidden_fwd(x, p, lq, hh)) <= TOL
+    dy = torch.randn(B, D, N, dtype=torch.complex64, generator=torch.Generator().manual_seed(L))
+    dx, dp, dq, dh = ops.ema_hidden_bwd(dy.cuda(), x.cuda(), p.cuda(), lq.cuda(),
+                                        None if hh is None else hh.cuda(), v)
+    wx, wp, wq, wh = cema.ema_hidden_bwd(dy, x, p, lq, hh)
+    assert dx.dtype == dtype and dp.shape == p.shape and dq.shape == q.shape
+    assert rel_err(dx, wx) <= tol
+    assert rel_err(dp.reshape(D, N), wp) <= TOL
+    assert rel_err(dq.reshape(D, N), wq) <= TOL
+    assert (dh is None) == (wh is None)
+    if dh is not None:
+        assert _close(dh, wh, TOL)
+
+
+def test_autograd_functions_with_state():
+    B, D, N, L = 2, 4, 16, 257
+    p, q, gamma, h, x = _case(B, D, N, L, 11)
+    pc, qc, gc, hc, xc = (t.cuda().requires_grad_() for t in (p, q, gamma, h, x))
+    w, b = ema_parameters(pc, qc, gc, hc, L)
+    hl = ema_hidden(xc, pc, qc, hc)
+    g = torch.Generator().manual_seed(1)
+    dw, db = torch.randn(D, L, generator=g), torch.randn(B, D, L, generator=g)
+    dh = torch.randn(B, D, N, dtype=torch.complex64, generator=g)
+    ((w * dw.cuda()).sum() + (b * db.cuda()).sum() + (hl * dh.cuda().conj()).real.sum()).backward()
+    p64, q64, g64, h64, x64 = (t.detach().clone().to(torch.complex128 if t.is_complex() else torch.float64).requires_grad_()
+                               for t in (p, q, gamma, h, x))
+    ow = cema.ema_weight_fwd(p64, q64.log(), g64, L)
+    ob = cema.ema_bias_fwd(q64.log(), g64, h64, L)
+    oh = cema.ema_hidden_fwd(x64, p64, q64.log(), h64)
+    ((ow * dw.double()).sum() + (ob * db.double()).sum() + (oh * dh.to(torch.complex128).conj()).real.sum()).backward()
+    for got, want in ((pc.grad, p64.grad), (qc.grad, q64.grad), (gc.grad, g64.grad), (hc.grad, h64.grad),
+                      (xc.grad, x64.grad)):
+        assert got.shape == want.shape and rel_err(got, want) <= TOL
+
+
+@pytest.mark.parametrize("dtype,L1,L2", [(torch.float32, 1000, 1500), (torch.bfloat16, 20000, 12768)])
+def test_layer_split_sequence_equals_whole(dtype, L1, L2):
+    """MultiHeadComplexEMA over [x1 | x2] in two calls with the state handed over
+    (hx, compute_last_state) equals one call over the whole sequence."""
+    torch.manual_seed(5)
+    D, N, B = 6, 16, 2
+    layer = MultiHeadComplexEMA(D, N).cuda()
+    x = torch.randn(B, D, L1 + L2).to(dtype).cuda()
+    with torch.no_grad():
+        whole, hw = layer(x, None, True)
+        y1, h1 = layer(x[:, :, :L1].contiguous(), None, True)
+        y2, h2 = layer(x[:, :, L1:].contiguous(), h1, True)
+    tol = TOL if dtype == torch.float32 else 2e-2
+    assert h1.shape == (B, D, N) and h1.dtype == torch.complex64
+    assert rel_err(y1, whole[:, :, :L1]) <= tol
+    assert rel_err(y2, whole[:, :, L1:]) <= tol
+    assert rel_err(h2, hw) <= (TOL if dtype == torch.float32 else 1e-3)
+    # and against the oracle's recurrence-equivalent closed form
+    p, q, gamma = layer.coeffs()
+    want = cema.ema_hidden_fwd(x.cpu(), p.cpu(), q.cpu().log(), None)
+    assert rel_err(hw, want) <= TOL
