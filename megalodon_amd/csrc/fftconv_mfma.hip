@@ -700,8 +700,7 @@ __device__ __forceinline__ void pointwise(uint16_t* pre, uint16_t* pim, const Sp
 template <int DT, int MODE>
 __global__ __launch_bounds__(kThreads) void fftconv_mfma_kernel(
     const void* __restrict__ a, const void* __restrict__ b, void* __restrict__ out, int rows,
-    int D, int L, int flip, const float* __restrict__ omega, uint16_t* __restrict__ dbg,
-    int dbg_stage) {
+    int D, int L, int flip, const float* __restrict__ omega) {
   extern __shared__ __align__(16) uint16_t lds[];
   uint16_t* pre = lds;
   uint16_t* pim = lds + kIm;
@@ -720,40 +719,23 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_kernel(
   };
   RegsB rb;
   if (blockIdx.x < rows) fetch_row(rb, brow_of(blockIdx.x), L, false, tid);
-  int tick = 0;
-  auto stamp = [&]() {
-    if (dbg != nullptr && dbg_stage == 200 && blockIdx.x == 0 && tid == 0 && tick < 256)
-      reinterpret_cast<unsigned long long*>(dbg)[tick++] = __builtin_readcyclecounter();
-  };
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const int64_t d = row % D;
     const char* arow = static_cast<const char*>(a) + row * L * esz;
     const bool flip_a = MODE == 1 || flip != 0;
-    stamp();
     const float sb = place_row(pre, pim, red, rb, false, tid);
-    stamp();
     RowRegs<DT> ra;
     fetch_row(ra, arow, L, flip_a, tid);
     transform<false>(pre, pim, w, wave, lane);
-    stamp();
     Spectrum sp;
     capture_spectrum(pre, pim, sp, tid);
     lds_barrier();
-    stamp();
     const float sa = place_row(pre, pim, red, ra, flip_a, tid);
-    stamp();
-    if (dbg != nullptr && dbg_stage == 0) break;
     transform<false>(pre, pim, w, wave, lane);
-    if (dbg != nullptr && dbg_stage == 1) break;
-    stamp();
     pointwise(pre, pim, sp, tid);
     lds_barrier();
-    stamp();
-    if (dbg != nullptr && dbg_stage == 2) break;
     if (row + gridDim.x < rows) fetch_row(rb, brow_of(row + gridDim.x), L, false, tid);
     transform<true>(pre, pim, w, wave, lane);
-    if (dbg != nullptr && dbg_stage == 3) break;
-    stamp();
     const float scale = 181.01933598375618f / (sa * sb);  // sqrt(N) / (row scales)
     if (MODE == 0) {
       store_row<DT, false>(pre, pim, static_cast<char*>(out) + row * L * esz, L, flip != 0, scale,
@@ -766,11 +748,6 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_kernel(
         store_row<MEGA_F32, false>(pre, pim, orow, L, true, scale, nullptr, 0.f, tid);
     }
     lds_barrier();  // the planes are rewritten by the next row's operand
-    stamp();
-  }
-  if (dbg != nullptr && dbg_stage != 200 && blockIdx.x == 0) {
-    lds_barrier();
-    for (int i = tid; i < 2 * kPlane; i += kThreads) dbg[i] = lds[i];
   }
 }
 
@@ -861,7 +838,7 @@ int launch_bwd(const void* dy, const void* x, const float* k, void* dx, float* d
 
 template <int DT, int MODE>
 int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_t L, int flip,
-           const float* omega, hipStream_t stream, uint16_t* dbg, int dbg_stage) {
+           const float* omega, hipStream_t stream) {
   int dev = 0, cus = 0;
   MEGA_CHECK_HIP(hipGetDevice(&dev));
   MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
@@ -873,8 +850,7 @@ int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_
     MEGA_CHECK_ARG(rows <= 0x7fffffff, "fftconv: too many rows");
     const unsigned grid = static_cast<unsigned>(rows < cus ? rows : cus);
     fftconv_mfma_kernel<DT, MODE><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
-        a, b, out, static_cast<int>(rows), static_cast<int>(D), static_cast<int>(L), flip, omega,
-        dbg, dbg_stage);
+        a, b, out, static_cast<int>(rows), static_cast<int>(D), static_cast<int>(L), flip, omega);
     MEGA_CHECK_LAUNCH();
   } else {
     const unsigned grid = static_cast<unsigned>(D < cus ? D : cus);
@@ -883,7 +859,7 @@ int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_
       const char* xb = static_cast<const char*>(b) + bb * D * L * 2;
       fftconv_mfma_kernel<DT, MODE><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
           ab, xb, out, static_cast<int>(D), static_cast<int>(D), static_cast<int>(L),
-          bb > 0 ? 1 : 0, nullptr, dbg, dbg_stage);
+          bb > 0 ? 1 : 0, nullptr);
       MEGA_CHECK_LAUNCH();
     }
   }
@@ -899,13 +875,12 @@ bool applicable(int dtype, int64_t L, const void* a, const void* b, const void* 
 }
 
 int launch_conv(int dtype, int mode, const void* a, const void* b, void* out, int64_t B,
-                int64_t D, int64_t L, int flip, const float* omega, hipStream_t stream,
-                uint16_t* dbg, int dbg_stage) {
+                int64_t D, int64_t L, int flip, const float* omega, hipStream_t stream) {
   if (dtype == MEGA_BF16)
-    return mode == 0 ? launch<MEGA_BF16, 0>(a, b, out, B, D, L, flip, omega, stream, dbg, dbg_stage)
-                     : launch<MEGA_BF16, 1>(a, b, out, B, D, L, flip, omega, stream, dbg, dbg_stage);
-  return mode == 0 ? launch<MEGA_F16, 0>(a, b, out, B, D, L, flip, omega, stream, dbg, dbg_stage)
-                   : launch<MEGA_F16, 1>(a, b, out, B, D, L, flip, omega, stream, dbg, dbg_stage);
+    return mode == 0 ? launch<MEGA_BF16, 0>(a, b, out, B, D, L, flip, omega, stream)
+                     : launch<MEGA_BF16, 1>(a, b, out, B, D, L, flip, omega, stream);
+  return mode == 0 ? launch<MEGA_F16, 0>(a, b, out, B, D, L, flip, omega, stream)
+                   : launch<MEGA_F16, 1>(a, b, out, B, D, L, flip, omega, stream);
 }
 
 int launch_backward(int dtype, const void* dy, const void* x, const float* k, void* dx, float* dk,

@@ -12,10 +12,8 @@ bool applicable(int dtype, int64_t L, const void* a, const void* b, const void* 
 
 // mode 0: out[b,d,:] = conv(a[b,d,:], k[d,:]) (+ omega[d] a), k fp32, `flip` = backward dx form;
 // mode 1: out[d,:] = sum_b reverse(conv(reverse(a[b,d,:]), x[b,d,:])), fp32 out.
-// dbg / dbg_stage: development hook (LDS dump of workgroup 0 after a stage), nullptr in production.
 int launch_conv(int dtype, int mode, const void* a, const void* b, void* out, int64_t B, int64_t D,
-                int64_t L, int flip, const float* omega, hipStream_t stream,
-                uint16_t* dbg = nullptr, int dbg_stage = -1);
+                int64_t L, int flip, const float* omega, hipStream_t stream);
 
 // dx (+ omega dy) and dk of the convolution in one launch (dy is transformed once);
 // dk (D, L) fp32 is overwritten.  Same applicability as launch_conv; B >= 1.
