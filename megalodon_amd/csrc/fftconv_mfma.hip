@@ -1,9 +1,10 @@
 // Causal convolution of 16-bit rows with the DFT stages on the matrix cores.
 //
-// One workgroup (8 waves) owns one row at a time.  The zero-padded real row of
+// One workgroup (8 waves) owns one row at a time (the longest rows; shorter
+// rows go 2, 4 or 8 to a pass, see Geo below).  The zero-padded real row of
 // 2N = 65536 samples is packed as z[n] = s[2n] + i s[2n+1], n < N = 32768, and
-// kept in LDS as fp16 re and im values (rows of a, re half then im half).  The N-point transform is three
-// radix-32 stages over the digits of n = 1024 a + 32 b + c:
+// kept in LDS as fp16 re and im values (rows of a, re half then im half).  The
+// N-point transform is three radix-32 stages over the digits of n = 1024 a + 32 b + c:
 //     forward  F1 over a, F2 over b, F3 over c  -> Z[k1 + 32 k2 + 1024 k3] at (k1, k2, k3)
 //     inverse  I1 over c, I2 over b, I3 over a  -> z[n] back at (a, b, c)
 // (the inverse undoes the forward steps in reverse order, conjugated)
@@ -17,8 +18,10 @@
 // (the kernel row) waits in registers while the first operand is transformed;
 // the real-signal product is formed on conjugate bin pairs (k, N - k).
 //
-// Used for bf16 / fp16 rows with 16384 < L <= 32768 and L % 8 == 0; everything else
-// stays with the fp32 VALU engine of fftconv.hip.
+// Used for bf16 / fp16 rows with 2048 < L <= 32768 and L % 8 == 0; everything else
+// stays with the fp32 VALU engine of fftconv.hip.  Rows that share a pass are
+// independent for finite data; a NaN or Inf in one of them spreads to the
+// others of its pass (0 x NaN in the block-diagonal stage).
 #include "common.hpp"
 #include "fftconv_mfma.hpp"
 
@@ -26,7 +29,21 @@ namespace mega {
 namespace fftm {
 namespace {
 
-constexpr int kN = 32768;             // complex points per transform
+// Row lengths: a row of L samples needs N' = 1024 A complex points with
+// A = 32, 16, 8 or 4 digits a (L <= N').  The LDS always holds 32 values of a:
+// a workgroup pass takes R = 32 / A rows side by side, row r owning a = r A ..
+// r A + A - 1; the stage over a multiplies by the block-diagonal matrix of R
+// DFT-A blocks, every other stage is unchanged (the row index rides along as a
+// bystander).
+template <int LOGA>
+struct Geo {
+  static constexpr int A = 1 << LOGA;       // digits a per row
+  static constexpr int R = 32 / A;          // rows per workgroup pass
+  static constexpr int NP = A * 1024;       // complex points of a row's transform
+  static constexpr int HALF = NP / 2;       // packed points a row can fill (the rest is padding)
+  static constexpr int JSH = LOGA - 2;      // quad j of a thread belongs to row j >> JSH
+  static __device__ __forceinline__ int row_of_quad(int j) { return LOGA == 5 ? 0 : (j >> JSH); }
+};
 // LDS: row a holds its 1024 re values, 16 elements of padding, then its 1024 im
 // values and padding.  The a-stride of 1040 dwords is 16 mod 64 banks, and the
 // im value of an element sits a constant 2080 bytes after its re value, which
@@ -36,7 +53,7 @@ constexpr int kRS = 2 * kIm;          // elements between consecutive a
 constexpr int kPlane = 16 * kRS;      // half of the LDS elements (two "planes" of 32 half rows)
 constexpr int kThreads = 512;         // 8 waves, two per SIMD
 constexpr int kWaves = kThreads / kWave;
-constexpr size_t kLdsBytes = sizeof(uint16_t) * 2 * kPlane + 64;
+constexpr size_t kLdsBytes = sizeof(uint16_t) * 2 * kPlane + 256;  // + 8 x 8 floats for row maxima
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -159,7 +176,7 @@ __device__ __forceinline__ void dft_xb(const u32x4* xr, const u32x4* xi, const D
   }
 }
 
-// exp(+i 2 pi c m / N) for the 16 values c = 8 qd + 4 g + e a lane holds after a
+// exp(+i 2 pi c m / N') for the 16 values c = 8 qd + 4 g + e a lane holds after a
 // stage (register 4 qd + e), from three sin/cos pairs and complex products:
 // W^(c m) = W^(4 g m) (W^(8 m))^qd (W^m)^e.
 struct Tw16 {
@@ -169,7 +186,9 @@ __device__ __forceinline__ void cmul(float ar, float ai, float br, float bi, flo
   cr = ar * br - ai * bi;
   ci = ar * bi + ai * br;
 }
+template <int LOGA>
 __device__ __forceinline__ Tw16 twiddles16(int m, int g) {
+  constexpr int kN = Geo<LOGA>::NP;
   Tw16 t;
   float t1c, t1s, t2c, t2s, t3c, t3s, bc, bs, s8c, s8s;
   cis(m & (kN - 1), 1.f / kN, t1c, t1s);
@@ -237,12 +256,46 @@ __device__ __forceinline__ void read_tile_tr(const uint16_t* pre, int o0, int o1
   }
 }
 
+// The block-diagonal matrix of 32 / A DFT-A blocks in MFMA operand form (lane l:
+// j = l % 32 the output digit, k = 16 s + 8 (l / 32) + e the input digit),
+// scaled by 1 / sqrt(A).
+template <int LOGA>
+__device__ __forceinline__ Dft make_dft_a(int lane) {
+  constexpr int A = Geo<LOGA>::A;
+  Dft w;
+  const int j = lane & 31, g = lane >> 5;
+  const float sc = LOGA == 4 ? 0.25f : (LOGA == 3 ? 0.35355339059327379f : 0.5f);
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    float c[8], sn[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int k = 16 * s + 8 * g + e;
+      const bool on = (k >> LOGA) == (j >> LOGA);
+      cis(((k & (A - 1)) * (j & (A - 1))) & (A - 1), 1.f / A, c[e], sn[e]);
+      c[e] = on ? c[e] * sc : 0.f;
+      sn[e] = on ? sn[e] * sc : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      w.re[s][e] = pack_h2(c[2 * e], c[2 * e + 1]);
+      w.im[s][e] = pack_h2(-sn[2 * e], -sn[2 * e + 1]);
+      w.nim[s][e] = pack_h2(sn[2 * e], sn[2 * e + 1]);
+    }
+  }
+  return w;
+}
+
 // ---- stages over a (F1 / I3): tile = fixed b, rows a, bystander c -------------
-// F1 (a -> k1): only a < 16 holds data (zero padding) -> one k-step; then
-// twiddle W_1024^(b k1), one factor per lane.  I3 (k1 -> a): all 32 rows, no twiddle.
-template <bool INV>
-__device__ __forceinline__ void stage_a(uint16_t* pre, const Dft& w, int wave, int lane) {
+// F1 (a -> k1): then twiddle W_(32 A)^(b k1), one factor per lane.  With A = 32
+// only a < 16 holds data (zero padding) -> one k-step; shorter rows have their
+// padding written as zeros and take both.  I3 (k1 -> a): no twiddle.
+template <int LOGA, bool INV>
+__device__ __forceinline__ void stage_a(uint16_t* pre, const Dft& w32, int wave, int lane) {
+  constexpr int A = Geo<LOGA>::A;
+  constexpr int KS = (INV || LOGA < 5) ? 2 : 1;
   lane = opaque(lane) & 63;
+  const Dft w = LOGA == 5 ? w32 : make_dft_a<LOGA>(lane);
   const int g = lane >> 5, f = lane & 31;
   const int rsrc = 8 * g + ((lane & 15) >> 2), csrc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
   // pos(16 s + rsrc + 4 h, b, csrc): the row's swizzle bits are (2 g + h) & 3
@@ -253,12 +306,12 @@ __device__ __forceinline__ void stage_a(uint16_t* pre, const Dft& w, int wave, i
   for (int b = wv; b < 32; b += kWaves) {
     const int bx = ((b >> 2) & 3) << 3;
     u32x4 xr[2], xi[2];
-    read_tile_tr<INV ? 2 : 1, 16 * kRS>(pre, (rd0 ^ bx) + 32 * b, (rd1 ^ bx) + 32 * b, xr, xi);
+    read_tile_tr<KS, 16 * kRS>(pre, (rd0 ^ bx) + 32 * b, (rd1 ^ bx) + 32 * b, xr, xi);
     floatx16 dr, di;
-    dft_xa<INV, INV ? 2 : 1>(xr, xi, w, dr, di);
+    dft_xa<INV, KS>(xr, xi, w, dr, di);
     if (!INV) {
       float tc, ts;
-      cis((b * f) & 1023, 1.f / 1024.f, tc, ts);
+      cis((b * (f & (A - 1))) & (32 * A - 1), 1.f / (32 * A), tc, ts);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float vr = dr[r], vi = di[r];
@@ -271,10 +324,11 @@ __device__ __forceinline__ void stage_a(uint16_t* pre, const Dft& w, int wave, i
 }
 
 // ---- stages over b (F2 / I2): tile = fixed a, rows b, bystander c -------------
-// F2 (b -> k2): then twiddle W_N^(c (a + 32 k2)).  I2 (k2 -> n2): undoes F1's
-// twiddle, conj W_1024^(n2 a), one factor per lane.
-template <bool INV>
+// With k1 = a % A: F2 (b -> k2): then twiddle W_N'^(c (k1 + A k2)).  I2 (k2 ->
+// n2): undoes F1's twiddle, conj W_(32 A)^(n2 k1), one factor per lane.
+template <int LOGA, bool INV>
 __device__ __forceinline__ void stage_b(uint16_t* pre, const Dft& w, int wave, int lane) {
+  constexpr int A = Geo<LOGA>::A;
   lane = opaque(lane) & 63;
   const int g = lane >> 5, f = lane & 31;
   const int rsrc = 8 * g + ((lane & 15) >> 2), csrc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
@@ -283,17 +337,17 @@ __device__ __forceinline__ void stage_b(uint16_t* pre, const Dft& w, int wave, i
   const int wr = 32 * f + 4 * g, fx = (f >> 2) & 3;
   const int wv = __builtin_amdgcn_readfirstlane(wave);
   for (int a = wv; a < 32; a += kWaves) {
-    const int ax = ((a >> 2) & 3) << 3;
+    const int ax = ((a >> 2) & 3) << 3, k1 = a & (A - 1);
     u32x4 xr[2], xi[2];
     read_tile_tr<2, 512>(pre, (rd0 ^ ax) + a * kRS, (rd1 ^ ax) + a * kRS, xr, xi);
     floatx16 dr, di;
     dft_xa<INV, 2>(xr, xi, w, dr, di);
     if (!INV) {
-      const Tw16 t = twiddles16(a + 32 * f, g);
+      const Tw16 t = twiddles16<LOGA>(k1 + A * f, g);
       apply_tw<false>(dr, di, t);
     } else {
       float tc, ts;
-      cis((a * f) & 1023, 1.f / 1024.f, tc, ts);
+      cis((k1 * f) & (32 * A - 1), 1.f / (32 * A), tc, ts);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float vr = dr[r], vi = di[r];
@@ -307,9 +361,10 @@ __device__ __forceinline__ void stage_b(uint16_t* pre, const Dft& w, int wave, i
 
 // ---- stages over c (F3 / I1): tile = fixed a, lanes b, rows c (contiguous) ----
 // F3 (c -> k3): no twiddle.  I1 (k3 -> n3): then undoes F2's twiddle,
-// conj W_N^(n3 (a + 32 b)).
-template <bool INV>
+// conj W_N'^(n3 (k1 + A b)).
+template <int LOGA, bool INV>
 __device__ __forceinline__ void stage_c(uint16_t* pre, const Dft& w, int wave, int lane) {
+  constexpr int A = Geo<LOGA>::A;
   lane = opaque(lane) & 63;
   const int g = lane >> 5, b = lane & 31;
   const int bx = (b >> 2) & 3, row = 32 * b;
@@ -328,29 +383,28 @@ __device__ __forceinline__ void stage_c(uint16_t* pre, const Dft& w, int wave, i
     floatx16 dr, di;
     dft_xb<INV>(xr, xi, w, dr, di);
     if (INV) {
-      const Tw16 t = twiddles16(a + 32 * b, g);
+      const Tw16 t = twiddles16<LOGA>((a & (A - 1)) + A * b, g);
       apply_tw<true>(dr, di, t);
     }
     write_tile_x(pre, dr, di, base + 4 * g, x);
   }
 }
 
-template <bool INV>
-__device__ __forceinline__ void transform(uint16_t* pre, uint16_t* pim, const Dft& w, int wave,
-                                          int lane) {
+template <int LOGA, bool INV>
+__device__ __forceinline__ void transform(uint16_t* pre, const Dft& w, int wave, int lane) {
   if (!INV) {
-    stage_a<false>(pre, w, wave, lane);
+    stage_a<LOGA, false>(pre, w, wave, lane);
     lds_barrier();
-    stage_b<false>(pre, w, wave, lane);
+    stage_b<LOGA, false>(pre, w, wave, lane);
     lds_barrier();
-    stage_c<false>(pre, w, wave, lane);
+    stage_c<LOGA, false>(pre, w, wave, lane);
     lds_barrier();
   } else {
-    stage_c<true>(pre, w, wave, lane);
+    stage_c<LOGA, true>(pre, w, wave, lane);
     lds_barrier();
-    stage_b<true>(pre, w, wave, lane);
+    stage_b<LOGA, true>(pre, w, wave, lane);
     lds_barrier();
-    stage_a<true>(pre, w, wave, lane);
+    stage_a<LOGA, true>(pre, w, wave, lane);
     lds_barrier();
   }
 }
@@ -420,33 +474,49 @@ template <> struct QuadIo<MEGA_F16> {
   }
 };
 
-// A row in flight: a thread's 8 quads n0 = 4 (tid + 512 j) of sample pairs
-// (reversed order when flip), as loaded.  L % 8 == 0 keeps quads whole.
+// The rows of a pass in flight: a thread's 8 quads of sample pairs, as loaded.
+// Quad j belongs to row j >> JSH of the pass and covers the packed points
+// n0 .. n0 + 3, n0 = 4 (tid + 512 j) mod (N' / 2) (reversed order when flip).
+// L % 8 == 0 keeps quads whole.  Absent rows (null pointer) read as zeros.
 template <int DT>
 struct RowRegs {
   typename QuadIo<DT>::Raw q[8];
 };
-template <int DT>
-__device__ __forceinline__ void fetch_row(RowRegs<DT>& r, const void* row, int L, bool flip,
-                                          int tid) {
+template <int LOGA>
+struct RowPtrs {
+  const char* p[Geo<LOGA>::R];
+};
+template <int LOGA>
+__device__ __forceinline__ unsigned quad_n0(int tid, int j) {
+  return (4u * (static_cast<unsigned>(tid) + kThreads * j)) & (Geo<LOGA>::HALF - 1);
+}
+template <int LOGA, int DT>
+__device__ __forceinline__ void fetch_rows(RowRegs<DT>& r, const RowPtrs<LOGA>& rows, int L,
+                                           bool flip, int tid) {
   const unsigned half = static_cast<unsigned>(L) >> 1;
   tid = opaque(tid) & (kThreads - 1);
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const unsigned n0 = 4u * (static_cast<unsigned>(tid) + kThreads * j);
+    const unsigned n0 = quad_n0<LOGA>(tid, j);
+    const char* row = rows.p[Geo<LOGA>::row_of_quad(j)];
     r.q[j] = QuadIo<DT>::zero();
-    if (n0 < half) r.q[j] = QuadIo<DT>::fetch(row, flip ? half - 4u - n0 : n0);
+    if (n0 < half && row != nullptr) r.q[j] = QuadIo<DT>::fetch(row, flip ? half - 4u - n0 : n0);
   }
 }
-// Writes the fetched row to the planes as z[n] = s[2n] + i s[2n+1], n < 16384
-// (zeros beyond the row), scaled by a power of two so that max |s| lands in
-// [1/8, 1/4).  Returns the scale.  `red` is 8 floats of LDS.  Ends with a barrier.
-template <int DT>
-__device__ __forceinline__ float place_row(uint16_t* pre, uint16_t* pim, float* red,
-                                           const RowRegs<DT>& r, bool flip, int tid) {
+// Writes the fetched rows to the LDS as z[n] = s[2n] + i s[2n+1], n < N' / 2
+// (zeros beyond the row), each row scaled by a power of two so that its max |s|
+// lands in [1/8, 1/4); `scale` receives the R scales.  Rows of fewer than 32
+// digits a also have their padding half written as zeros (A = 32 never reads
+// it).  `red` is 8 R floats of LDS.  Ends with a barrier.
+template <int LOGA, int DT>
+__device__ __forceinline__ void place_rows(uint16_t* pre, float* red, const RowRegs<DT>& r,
+                                           bool flip, int tid, float* scale) {
+  constexpr int A = Geo<LOGA>::A, R = Geo<LOGA>::R;
   tid = opaque(tid) & (kThreads - 1);
   float re[8][4], im[8][4];
-  float m = 0.f;
+  float m[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) m[i] = 0.f;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     float lo[4], hi[4];
@@ -455,50 +525,67 @@ __device__ __forceinline__ float place_row(uint16_t* pre, uint16_t* pim, float* 
     for (int e = 0; e < 4; ++e) {
       re[j][e] = flip ? hi[3 - e] : lo[e];
       im[j][e] = flip ? lo[3 - e] : hi[e];
-      m = fmaxf(m, fmaxf(fabsf(re[j][e]), fabsf(im[j][e])));
+      m[Geo<LOGA>::row_of_quad(j)] = fmaxf(m[Geo<LOGA>::row_of_quad(j)], fmaxf(fabsf(re[j][e]), fabsf(im[j][e])));
     }
   }
-  m = wave_max(m);
-  if ((tid & (kWave - 1)) == 0) red[tid / kWave] = m;
-  lds_barrier();
-  m = red[0];
 #pragma unroll
-  for (int i = 1; i < kWaves; ++i) m = fmaxf(m, red[i]);
-  // 2^-(e+2) with m = f 2^e, f in [0.5, 1); finite non-zero m only
-  float scale = 1.f;
-  if (m > 0.f && m < 3.0e38f) {
-    int e;
-    (void)frexpf(m, &e);
-    scale = ldexpf(1.f, -(e + 2));
+  for (int i = 0; i < R; ++i) {
+    m[i] = wave_max(m[i]);
+    if ((tid & (kWave - 1)) == 0) red[(tid / kWave) * R + i] = m[i];
+  }
+  lds_barrier();
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    float v = red[i];
+#pragma unroll
+    for (int wv = 1; wv < kWaves; ++wv) v = fmaxf(v, red[wv * R + i]);
+    // 2^-(e+2) with v = f 2^e, f in [0.5, 1); finite non-zero v only
+    float sc = 1.f;
+    if (v > 0.f && v < 3.0e38f) {
+      int e;
+      (void)frexpf(v, &e);
+      sc = ldexpf(1.f, -(e + 2));
+    }
+    scale[i] = sc;
   }
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const int n0 = 4 * (tid + kThreads * j);
-    const int o = pos(n0 >> 10, (n0 >> 5) & 31, n0 & 31);
-    *reinterpret_cast<uint2*>(pre + o) = make_uint2(pack_h2(re[j][0] * scale, re[j][1] * scale),
-                                                    pack_h2(re[j][2] * scale, re[j][3] * scale));
-    *reinterpret_cast<uint2*>(pim + o) = make_uint2(pack_h2(im[j][0] * scale, im[j][1] * scale),
-                                                    pack_h2(im[j][2] * scale, im[j][3] * scale));
+    const int n0 = static_cast<int>(quad_n0<LOGA>(tid, j));
+    const float sc = scale[Geo<LOGA>::row_of_quad(j)];
+    const int a = Geo<LOGA>::row_of_quad(j) * A + (n0 >> 10);
+    const int o = pos(a, (n0 >> 5) & 31, n0 & 31);
+    *reinterpret_cast<uint2*>(pre + o) =
+        make_uint2(pack_h2(re[j][0] * sc, re[j][1] * sc), pack_h2(re[j][2] * sc, re[j][3] * sc));
+    *reinterpret_cast<uint2*>(pre + o + kIm) =
+        make_uint2(pack_h2(im[j][0] * sc, im[j][1] * sc), pack_h2(im[j][2] * sc, im[j][3] * sc));
+    if (LOGA < 5) {
+      const int oz = pos(a + A / 2, (n0 >> 5) & 31, n0 & 31);
+      *reinterpret_cast<uint2*>(pre + oz) = make_uint2(0u, 0u);
+      *reinterpret_cast<uint2*>(pre + oz + kIm) = make_uint2(0u, 0u);
+    }
   }
   lds_barrier();
-  return scale;
 }
 
-// out[2n] = re z[n] * scale (+ w res[2n]), out[2n+1] likewise, n < L/2
-// (reversed when flip); ACC adds to what is there (fp32 rows).
-template <int DT, bool ACC>
-__device__ __forceinline__ void store_row(const uint16_t* pre, const uint16_t* pim, void* row,
-                                          int L, bool flip, float scale, const void* res, float w,
-                                          int tid) {
+// Row r of the pass: out[2n] = re z[n] * scale[r] (+ w[r] res[r][2n]), out[2n+1]
+// likewise, n < L/2 (reversed when flip); ACC adds to what is there (fp32 rows).
+// Absent rows (null pointer) are skipped.
+template <int LOGA, int DT, bool ACC>
+__device__ __forceinline__ void store_rows(const uint16_t* pre, const RowPtrs<LOGA>& rows, int L,
+                                           bool flip, const float* scale,
+                                           const RowPtrs<LOGA>* res, const float* w, int tid) {
+  constexpr int A = Geo<LOGA>::A;
   const unsigned half = static_cast<unsigned>(L) >> 1;
   tid = opaque(tid) & (kThreads - 1);
-#pragma unroll 2
+#pragma unroll(LOGA == 5 ? 2 : 8)
   for (int j = 0; j < 8; ++j) {
-    const unsigned n0 = 4u * (static_cast<unsigned>(tid) + kThreads * j);
-    if (n0 < half) {
-      const int o = pos(n0 >> 10, (n0 >> 5) & 31, n0 & 31);
+    const unsigned n0 = quad_n0<LOGA>(tid, j);
+    char* row = const_cast<char*>(rows.p[Geo<LOGA>::row_of_quad(j)]);
+    if (n0 < half && row != nullptr) {
+      const float sc = scale[Geo<LOGA>::row_of_quad(j)];
+      const int o = pos(Geo<LOGA>::row_of_quad(j) * A + static_cast<int>(n0 >> 10), (n0 >> 5) & 31, n0 & 31);
       const uint2 ur = *reinterpret_cast<const uint2*>(pre + o);
-      const uint2 ui = *reinterpret_cast<const uint2*>(pim + o);
+      const uint2 ui = *reinterpret_cast<const uint2*>(pre + o + kIm);
       float zr[4], zi[4], lo[4], hi[4];
       unpack_h2(ur.x, zr[0], zr[1]);
       unpack_h2(ur.y, zr[2], zr[3]);
@@ -506,8 +593,8 @@ __device__ __forceinline__ void store_row(const uint16_t* pre, const uint16_t* p
       unpack_h2(ui.y, zi[2], zi[3]);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        lo[e] = (flip ? zi[3 - e] : zr[e]) * scale;
-        hi[e] = (flip ? zr[3 - e] : zi[e]) * scale;
+        lo[e] = (flip ? zi[3 - e] : zr[e]) * sc;
+        hi[e] = (flip ? zr[3 - e] : zi[e]) * sc;
       }
       const unsigned m0 = flip ? half - 4u - n0 : n0;
       if (ACC) {
@@ -521,11 +608,12 @@ __device__ __forceinline__ void store_row(const uint16_t* pre, const uint16_t* p
       }
       if (res != nullptr) {
         float rlo[4], rhi[4];
-        QuadIo<DT>::load(res, m0, rlo, rhi);
+        QuadIo<DT>::load(res->p[Geo<LOGA>::row_of_quad(j)], m0, rlo, rhi);
+        const float wt = w[Geo<LOGA>::row_of_quad(j)];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          lo[e] = fmaf(w, rlo[e], lo[e]);
-          hi[e] = fmaf(w, rhi[e], hi[e]);
+          lo[e] = fmaf(wt, rlo[e], lo[e]);
+          hi[e] = fmaf(wt, rhi[e], hi[e]);
         }
       }
       QuadIo<DT>::store(row, m0, lo, hi);
@@ -534,43 +622,47 @@ __device__ __forceinline__ void store_row(const uint16_t* pre, const uint16_t* p
 }
 
 // ---- conjugate bin pairs ------------------------------------------------------
-// Bin k = k1 + 32 k2 + 1024 k3 sits at (k1, k2, k3); its partner N - k at the
-// mirrored row (k1', k2') = (32 - k1, 31 - k2) (k1 != 0) or (0, 32 - k2), with
-// k3' = 31 - k3.  Row (0, 0) is its own mirror with k3' = (32 - k3) % 32 and is
-// handled apart.  The other 1023 rows form 511 pairs plus the self-mirrored row
-// (0, 16): row pair q of 512 is
-//   q < 480: (1 + q / 32, q % 32);  480..495: (16, q - 480);  496..510: (0, q - 495);  511: (0, 16).
-// A lane takes one quad of a row pair: bins k3 = 4u .. 4u+3 of the row and the
-// reversed quad 7 - u of the mirror row; task T = tid + 512 i -> q = T / 8, u = T % 8.
+// Bin k = k1 + A k2 + 32 A k3 of row r sits at (r A + k1, k2, k3); its partner
+// N' - k at the mirrored LDS row (k1', k2') = (A - k1, 31 - k2) (k1 != 0) or
+// (0, 32 - k2), with k3' = 31 - k3.  LDS row (0, 0) is its own mirror with
+// k3' = (32 - k3) % 32 and is handled apart.  The other 32 A - 1 LDS rows of a
+// row form 16 A - 1 pairs plus the self-mirrored (0, 16): pair q of 16 A is
+//   q < 32 (A/2 - 1): (1 + q / 32, q % 32);  the next 16: (A/2, 0..15);
+//   the next 15: (0, 1..15);  the last: (0, 16).
+// A lane takes one quad of a pair: bins k3 = 4u .. 4u+3 and the reversed quad
+// 7 - u of the mirror; task T = tid + 512 i -> row T / (128 A), q = T / 8 % (16 A), u = T % 8.
 struct RowPair {
   int ok, om;   // LDS offsets of the two quads
-  int k0;       // bin index of the quad's first element: k1 + 32 k2 + 4096 u
+  int k0;       // bin index of the quad's first element: k1 + A k2 + 128 A u
   bool writes;  // false for the duplicate lanes of the self-mirrored row
 };
+template <int LOGA>
 __device__ __forceinline__ RowPair row_pair(int task) {
-  const int q = task >> 3, u = task & 7;
+  constexpr int A = Geo<LOGA>::A;
+  const int r = task >> (LOGA + 7), q = (task >> 3) & (16 * A - 1), u = task & 7;
+  constexpr int kBulk = 32 * (A / 2 - 1);
   int k1, k2;
-  if (q < 480) {
+  if (q < kBulk) {
     k1 = 1 + (q >> 5);
     k2 = q & 31;
-  } else if (q < 496) {
-    k1 = 16;
-    k2 = q - 480;
-  } else if (q < 511) {
+  } else if (q < kBulk + 16) {
+    k1 = A / 2;
+    k2 = q - kBulk;
+  } else if (q < kBulk + 31) {
     k1 = 0;
-    k2 = q - 495;
+    k2 = q - (kBulk + 15);
   } else {
     k1 = 0;
     k2 = 16;
   }
-  const int m1 = k1 != 0 ? 32 - k1 : 0;
+  const int m1 = k1 != 0 ? A - k1 : 0;
   const int m2 = k1 != 0 ? 31 - k2 : 32 - k2;
-  RowPair r;
-  r.ok = pos(k1, k2, 4 * u);
-  r.om = pos(m1, m2, 4 * (7 - u));
-  r.k0 = k1 + 32 * k2 + 4096 * u;
-  r.writes = q != 511 || u < 4;
-  return r;
+  RowPair rp;
+  rp.ok = pos(r * A + k1, k2, 4 * u);
+  rp.om = pos(r * A + m1, m2, 4 * (7 - u));
+  rp.k0 = k1 + A * k2 + 128 * A * u;
+  rp.writes = q != 16 * A - 1 || u < 4;
+  return rp;
 }
 __device__ __forceinline__ void read_quad(const uint16_t* p, float* v) {
   const uint2 u = *reinterpret_cast<const uint2*>(p);
@@ -610,12 +702,14 @@ struct Spectrum {
   uint32_t e0, o0;            // row (0, 0), lane = k3 (threads 0..31)
 };
 
-__device__ __forceinline__ void capture_spectrum(const uint16_t* pre, const uint16_t* pim,
-                                                 Spectrum& sp, int tid) {
+template <int LOGA>
+__device__ __forceinline__ void capture_spectrum(const uint16_t* pre, Spectrum& sp, int tid) {
+  constexpr int A = Geo<LOGA>::A, R = Geo<LOGA>::R;
+  const uint16_t* pim = pre + kIm;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     tid = opaque(tid) & (kThreads - 1);
-    const RowPair rp = row_pair(tid + kThreads * i);
+    const RowPair rp = row_pair<LOGA>(tid + kThreads * i);
     float kr[4], ki[4], mr[4], mi[4];
     read_quad(pre + rp.ok, kr);
     read_quad(pim + rp.ok, ki);
@@ -631,8 +725,9 @@ __device__ __forceinline__ void capture_spectrum(const uint16_t* pre, const uint
   }
   sp.e0 = sp.o0 = 0u;
   tid = opaque(tid) & (kThreads - 1);
-  if (tid < 32) {
-    const int ok = pos(0, 0, tid), om = pos(0, 0, (32 - tid) & 31);
+  if (tid < 32 * R) {
+    const int a0 = (tid >> 5) * A, k3 = tid & 31;
+    const int ok = pos(a0, 0, k3), om = pos(a0, 0, (32 - k3) & 31);
     float er, ei, orr, oi;
     untangle(h2f(pre[ok]), h2f(pim[ok]), h2f(pre[om]), h2f(pim[om]), er, ei, orr, oi);
     sp.e0 = pack_h2(er, ei);
@@ -641,20 +736,22 @@ __device__ __forceinline__ void capture_spectrum(const uint16_t* pre, const uint
 }
 
 // the product of the two real signals' spectra, written over Za
-__device__ __forceinline__ void pointwise(uint16_t* pre, uint16_t* pim, const Spectrum& sp,
-                                          int tid) {
+template <int LOGA>
+__device__ __forceinline__ void pointwise(uint16_t* pre, const Spectrum& sp, int tid) {
+  constexpr int A = Geo<LOGA>::A, R = Geo<LOGA>::R, NP = Geo<LOGA>::NP;
+  uint16_t* pim = pre + kIm;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     tid = opaque(tid) & (kThreads - 1);
-    const RowPair rp = row_pair(tid + kThreads * i);
+    const RowPair rp = row_pair<LOGA>(tid + kThreads * i);
     float kr[4], ki[4], mr[4], mi[4];
     read_quad(pre + rp.ok, kr);
     read_quad(pim + rp.ok, ki);
     read_quad(pre + rp.om, mr);
     read_quad(pim + rp.om, mi);
     float w0c, w0s;
-    cis(rp.k0, 1.f / kN, w0c, w0s);
-    // W_N^(k0 + 1024 e) = W_N^k0 W_32^e
+    cis(rp.k0, 1.f / NP, w0c, w0s);
+    // W_N'^(k0 + 32 A e) = W_N'^k0 W_32^e
     const float c32[4] = {1.f, 0.98078528040323043f, 0.92387953251128674f, 0.83146961230254524f};
     const float s32[4] = {0.f, 0.19509032201612825f, 0.38268343236508978f, 0.55557023301960218f};
     float okr[4], oki[4], omr[4], omi[4];
@@ -675,16 +772,16 @@ __device__ __forceinline__ void pointwise(uint16_t* pre, uint16_t* pim, const Sp
     }
   }
   tid = opaque(tid) & (kThreads - 1);
-  if (tid < 32) {
-    const int m3 = (32 - tid) & 31;
-    const int ok = pos(0, 0, tid), om = pos(0, 0, m3);
+  if (tid < 32 * R) {
+    const int a0 = (tid >> 5) * A, k3 = tid & 31, m3 = (32 - k3) & 31;
+    const int ok = pos(a0, 0, k3), om = pos(a0, 0, m3);
     float ar, ai, pr, pi, br, bi, qr, qi, wc, ws, zkr, zki, zmr, zmi;
     untangle(h2f(pre[ok]), h2f(pim[ok]), h2f(pre[om]), h2f(pim[om]), ar, ai, pr, pi);
     unpack_h2(sp.e0, br, bi);
     unpack_h2(sp.o0, qr, qi);
-    cis(1024 * tid, 1.f / kN, wc, ws);
+    cis(k3, 1.f / 32.f, wc, ws);
     bin_product(ar, ai, pr, pi, br, bi, qr, qi, wc, ws, zkr, zki, zmr, zmi);
-    if (tid <= m3) {
+    if (k3 <= m3) {
       pre[ok] = f2h(zkr);
       pim[ok] = f2h(zki);
       pre[om] = f2h(zmr);
@@ -693,171 +790,216 @@ __device__ __forceinline__ void pointwise(uint16_t* pre, uint16_t* pim, const Sp
   }
 }
 
+// sqrt(N') / (the two operands' row scales): undoes the three unitary transforms
+template <int LOGA>
+__device__ __forceinline__ void final_scales(const float* sa, const float* sb, float* out) {
+  constexpr float root = LOGA == 5 ? 181.01933598375618f
+                                   : (LOGA == 4 ? 128.f : (LOGA == 3 ? 90.509667991878086f : 64.f));
+#pragma unroll
+  for (int i = 0; i < Geo<LOGA>::R; ++i) out[i] = root / (sa[i] * sb[i]);
+}
+
+// A pass takes R consecutive rows (R = 1 for the longest rows).
 // MODE 0: out[b,d,:] = conv(a[b,d,:], k[d,:]) (+ omega[d] a[b,d,:]); `flip`
 //         reverses a on load and the result on store (backward dx); k fp32.
 // MODE 1: out[d,:] (+)= reverse(conv(reverse(a[b0,d,:]), x[b0,d,:])), fp32 out,
 //         `flip` != 0 accumulates (backward dk, one batch index per launch).
-template <int DT, int MODE>
+template <int DT, int MODE, int LOGA>
 __global__ __launch_bounds__(kThreads) void fftconv_mfma_kernel(
     const void* __restrict__ a, const void* __restrict__ b, void* __restrict__ out, int rows,
     int D, int L, int flip, const float* __restrict__ omega) {
+  constexpr int R = Geo<LOGA>::R;
   extern __shared__ __align__(16) uint16_t lds[];
   uint16_t* pre = lds;
-  uint16_t* pim = lds + kIm;
   float* red = reinterpret_cast<float*>(lds + 2 * kPlane);
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const Dft w = make_dft(lane);
   const int64_t esz = 2;
+  const int passes = (rows + R - 1) / R;
 
-  // Software pipeline over the rows of this workgroup: the first-operand row is
-  // fetched while the second operand is transformed, and the next row's second
-  // operand while the inverse transform runs.
+  // Software pipeline over the passes of this workgroup: the first-operand rows
+  // are fetched while the second operand is transformed, and the next pass's
+  // second operand while the inverse transform runs.
   typedef RowRegs<MODE == 0 ? MEGA_F32 : DT> RegsB;
-  auto brow_of = [&](int64_t row) -> const void* {
-    if (MODE == 0) return static_cast<const float*>(b) + (row % D) * L;
-    return static_cast<const char*>(b) + row * L * esz;
+  auto brows_of = [&](int pass) {
+    RowPtrs<LOGA> p;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int64_t row = static_cast<int64_t>(pass) * R + i;
+      p.p[i] = row >= rows ? nullptr
+               : MODE == 0 ? reinterpret_cast<const char*>(static_cast<const float*>(b) + (row % D) * L)
+                           : static_cast<const char*>(b) + row * L * esz;
+    }
+    return p;
   };
   RegsB rb;
-  if (blockIdx.x < rows) fetch_row(rb, brow_of(blockIdx.x), L, false, tid);
-  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-    const int64_t d = row % D;
-    const char* arow = static_cast<const char*>(a) + row * L * esz;
-    const bool flip_a = MODE == 1 || flip != 0;
-    const float sb = place_row(pre, pim, red, rb, false, tid);
-    RowRegs<DT> ra;
-    fetch_row(ra, arow, L, flip_a, tid);
-    transform<false>(pre, pim, w, wave, lane);
-    Spectrum sp;
-    capture_spectrum(pre, pim, sp, tid);
-    lds_barrier();
-    const float sa = place_row(pre, pim, red, ra, flip_a, tid);
-    transform<false>(pre, pim, w, wave, lane);
-    pointwise(pre, pim, sp, tid);
-    lds_barrier();
-    if (row + gridDim.x < rows) fetch_row(rb, brow_of(row + gridDim.x), L, false, tid);
-    transform<true>(pre, pim, w, wave, lane);
-    const float scale = 181.01933598375618f / (sa * sb);  // sqrt(N) / (row scales)
-    if (MODE == 0) {
-      store_row<DT, false>(pre, pim, static_cast<char*>(out) + row * L * esz, L, flip != 0, scale,
-                           omega != nullptr ? arow : nullptr, omega != nullptr ? omega[d] : 0.f, tid);
-    } else {
-      float* orow = static_cast<float*>(out) + row * L;
-      if (flip)
-        store_row<MEGA_F32, true>(pre, pim, orow, L, true, scale, nullptr, 0.f, tid);
-      else
-        store_row<MEGA_F32, false>(pre, pim, orow, L, true, scale, nullptr, 0.f, tid);
+  if (static_cast<int>(blockIdx.x) < passes)
+    fetch_rows<LOGA>(rb, brows_of(blockIdx.x), L, false, tid);
+  for (int pass = blockIdx.x; pass < passes; pass += gridDim.x) {
+    RowPtrs<LOGA> arows, orows;
+    float wres[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int64_t row = static_cast<int64_t>(pass) * R + i;
+      const bool on = row < rows;
+      arows.p[i] = on ? static_cast<const char*>(a) + row * L * esz : nullptr;
+      orows.p[i] = !on ? nullptr
+                   : MODE == 0 ? static_cast<const char*>(out) + row * L * esz
+                               : reinterpret_cast<const char*>(static_cast<float*>(out) + row * L);
+      wres[i] = (MODE == 0 && omega != nullptr && on) ? omega[row % D] : 0.f;
     }
-    lds_barrier();  // the planes are rewritten by the next row's operand
+    const bool flip_a = MODE == 1 || flip != 0;
+    float sb[R], sa[R], scale[R];
+    place_rows<LOGA>(pre, red, rb, false, tid, sb);
+    RowRegs<DT> ra;
+    fetch_rows<LOGA>(ra, arows, L, flip_a, tid);
+    transform<LOGA, false>(pre, w, wave, lane);
+    Spectrum sp;
+    capture_spectrum<LOGA>(pre, sp, tid);
+    lds_barrier();
+    place_rows<LOGA>(pre, red, ra, flip_a, tid, sa);
+    transform<LOGA, false>(pre, w, wave, lane);
+    pointwise<LOGA>(pre, sp, tid);
+    lds_barrier();
+    if (pass + static_cast<int>(gridDim.x) < passes)
+      fetch_rows<LOGA>(rb, brows_of(pass + gridDim.x), L, false, tid);
+    transform<LOGA, true>(pre, w, wave, lane);
+    final_scales<LOGA>(sa, sb, scale);
+    if (MODE == 0) {
+      store_rows<LOGA, DT, false>(pre, orows, L, flip != 0, scale,
+                                  omega != nullptr ? &arows : nullptr, wres, tid);
+    } else {
+      if (flip)
+        store_rows<LOGA, MEGA_F32, true>(pre, orows, L, true, scale, nullptr, wres, tid);
+      else
+        store_rows<LOGA, MEGA_F32, false>(pre, orows, L, true, scale, nullptr, wres, tid);
+    }
+    lds_barrier();  // the planes are rewritten by the next pass's operand
   }
 }
 
-// Backward of one channel in one pass: dy is transformed once and its spectrum
+// Backward of R channels in one pass: dy is transformed once and its spectrum
 // parked; then k (-> dx) and x (-> dk) are each transformed, multiplied with
 // it and transformed back.
 //   dx[b,d,:] = reverse(conv(reverse(dy[b,d,:]), k[d,:])) (+ omega[d] dy[b,d,:])
 //   dk[d,:]   = sum_b reverse(conv(reverse(dy[b,d,:]), x[b,d,:]))
-// A workgroup owns channels d = blockIdx.x, + gridDim.x, ... and walks the batch
-// itself, so dk accumulates in order without atomics.
-template <int DT>
+// A workgroup owns the channel groups blockIdx.x, + gridDim.x, ... (R channels
+// each) and walks the batch itself, so dk accumulates in order without atomics.
+template <int DT, int LOGA>
 __global__ __launch_bounds__(kThreads) void fftconv_mfma_bwd_kernel(
     const void* __restrict__ dy, const void* __restrict__ x, const float* __restrict__ k,
     void* __restrict__ dx, float* __restrict__ dk, int B, int D, int L,
     const float* __restrict__ omega) {
+  constexpr int R = Geo<LOGA>::R;
   extern __shared__ __align__(16) uint16_t lds[];
   uint16_t* pre = lds;
-  uint16_t* pim = lds + kIm;
   float* red = reinterpret_cast<float*>(lds + 2 * kPlane);
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const Dft w = make_dft(lane);
-  const int64_t rows = static_cast<int64_t>(B) * D;  // visited as (d, b), b fastest
-  const int64_t total = (static_cast<int64_t>(D) - blockIdx.x + gridDim.x - 1) / gridDim.x * B;
-  auto row_of = [&](int64_t it) -> int64_t {  // it-th row of this workgroup
-    const int64_t d = blockIdx.x + (it / B) * gridDim.x, bb = it % B;
-    return bb * D + d;
+  const int64_t groups = (static_cast<int64_t>(D) + R - 1) / R;
+  const int64_t total = (groups - blockIdx.x + gridDim.x - 1) / gridDim.x * B;
+  // rows of this workgroup's it-th pass: channels d0 .. d0 + R - 1 of batch index bb
+  auto rows_of = [&](int64_t it, const void* base, int64_t esz, bool batched) {
+    const int64_t d0 = (blockIdx.x + (it / B) * gridDim.x) * R, bb = it % B;
+    RowPtrs<LOGA> p;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      p.p[i] = d0 + i < D ? static_cast<const char*>(base) + ((batched ? bb * D : 0) + d0 + i) * L * esz
+                          : nullptr;
+    return p;
   };
-  (void)rows;
   RowRegs<DT> rdy;
-  if (total > 0) fetch_row(rdy, static_cast<const char*>(dy) + row_of(0) * L * 2, L, true, tid);
+  if (total > 0) fetch_rows<LOGA>(rdy, rows_of(0, dy, 2, true), L, true, tid);
   for (int64_t it = 0; it < total; ++it) {
-    const int64_t row = row_of(it), d = row % D;
+    const int64_t d0 = (blockIdx.x + (it / B) * gridDim.x) * R;
     const bool first = it % B == 0;
-    const char* dyrow = static_cast<const char*>(dy) + row * L * 2;
-    const float sdy = place_row(pre, pim, red, rdy, true, tid);
-    transform<false>(pre, pim, w, wave, lane);
+    const RowPtrs<LOGA> dyrows = rows_of(it, dy, 2, true);
+    float wres[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) wres[i] = (omega != nullptr && d0 + i < D) ? omega[d0 + i] : 0.f;
+    float sdy[R], sk[R], sx[R], scale[R];
+    place_rows<LOGA>(pre, red, rdy, true, tid, sdy);
+    transform<LOGA, false>(pre, w, wave, lane);
     RowRegs<MEGA_F32> rk;
-    fetch_row(rk, k + d * L, L, false, tid);
+    fetch_rows<LOGA>(rk, rows_of(it, k, 4, false), L, false, tid);
     Spectrum sp;
-    capture_spectrum(pre, pim, sp, tid);
+    capture_spectrum<LOGA>(pre, sp, tid);
     lds_barrier();
     // dx
-    const float sk = place_row(pre, pim, red, rk, false, tid);
-    transform<false>(pre, pim, w, wave, lane);
-    pointwise(pre, pim, sp, tid);
+    place_rows<LOGA>(pre, red, rk, false, tid, sk);
+    transform<LOGA, false>(pre, w, wave, lane);
+    pointwise<LOGA>(pre, sp, tid);
     lds_barrier();
     RowRegs<DT> rx;
-    fetch_row(rx, static_cast<const char*>(x) + row * L * 2, L, false, tid);
-    transform<true>(pre, pim, w, wave, lane);
-    store_row<DT, false>(pre, pim, static_cast<char*>(dx) + row * L * 2, L, true,
-                         181.01933598375618f / (sdy * sk), omega != nullptr ? dyrow : nullptr,
-                         omega != nullptr ? omega[d] : 0.f, tid);
+    fetch_rows<LOGA>(rx, rows_of(it, x, 2, true), L, false, tid);
+    transform<LOGA, true>(pre, w, wave, lane);
+    final_scales<LOGA>(sdy, sk, scale);
+    store_rows<LOGA, DT, false>(pre, rows_of(it, dx, 2, true), L, true, scale,
+                                omega != nullptr ? &dyrows : nullptr, wres, tid);
     lds_barrier();
     // dk
-    const float sx = place_row(pre, pim, red, rx, false, tid);
-    transform<false>(pre, pim, w, wave, lane);
-    pointwise(pre, pim, sp, tid);
+    place_rows<LOGA>(pre, red, rx, false, tid, sx);
+    transform<LOGA, false>(pre, w, wave, lane);
+    pointwise<LOGA>(pre, sp, tid);
     lds_barrier();
-    if (it + 1 < total)
-      fetch_row(rdy, static_cast<const char*>(dy) + row_of(it + 1) * L * 2, L, true, tid);
-    transform<true>(pre, pim, w, wave, lane);
-    float* krow = dk + d * L;
-    const float sc = 181.01933598375618f / (sdy * sx);
+    if (it + 1 < total) fetch_rows<LOGA>(rdy, rows_of(it + 1, dy, 2, true), L, true, tid);
+    transform<LOGA, true>(pre, w, wave, lane);
+    final_scales<LOGA>(sdy, sx, scale);
+    const RowPtrs<LOGA> krows = rows_of(it, dk, 4, false);
     if (first)
-      store_row<MEGA_F32, false>(pre, pim, krow, L, true, sc, nullptr, 0.f, tid);
+      store_rows<LOGA, MEGA_F32, false>(pre, krows, L, true, scale, nullptr, wres, tid);
     else
-      store_row<MEGA_F32, true>(pre, pim, krow, L, true, sc, nullptr, 0.f, tid);
+      store_rows<LOGA, MEGA_F32, true>(pre, krows, L, true, scale, nullptr, wres, tid);
     lds_barrier();
   }
 }
 
-template <int DT>
+// digits a per row for a row of L samples: the smallest of 4, 8, 16, 32 with L <= 1024 A
+inline int loga_of(int64_t L) { return L > 16384 ? 5 : (L > 8192 ? 4 : (L > 4096 ? 3 : 2)); }
+
+template <int DT, int LOGA>
 int launch_bwd(const void* dy, const void* x, const float* k, void* dx, float* dk, int64_t B,
                int64_t D, int64_t L, const float* omega, hipStream_t stream) {
   int dev = 0, cus = 0;
   MEGA_CHECK_HIP(hipGetDevice(&dev));
   MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&fftconv_mfma_bwd_kernel<DT>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     static_cast<int>(kLdsBytes)));
+  MEGA_CHECK_HIP(hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&fftconv_mfma_bwd_kernel<DT, LOGA>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBytes)));
   MEGA_CHECK_ARG(B * D <= 0x7fffffff, "fftconv: too many rows");
-  const unsigned grid = static_cast<unsigned>(D < cus ? D : cus);
-  fftconv_mfma_bwd_kernel<DT><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
+  const int64_t groups = (D + Geo<LOGA>::R - 1) / Geo<LOGA>::R;
+  const unsigned grid = static_cast<unsigned>(groups < cus ? groups : cus);
+  fftconv_mfma_bwd_kernel<DT, LOGA><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
       dy, x, k, dx, dk, static_cast<int>(B), static_cast<int>(D), static_cast<int>(L), omega);
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
 }
 
-template <int DT, int MODE>
+template <int DT, int MODE, int LOGA>
 int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_t L, int flip,
            const float* omega, hipStream_t stream) {
   int dev = 0, cus = 0;
   MEGA_CHECK_HIP(hipGetDevice(&dev));
   MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&fftconv_mfma_kernel<DT, MODE>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     static_cast<int>(kLdsBytes)));
+  MEGA_CHECK_HIP(hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&fftconv_mfma_kernel<DT, MODE, LOGA>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBytes)));
+  constexpr int R = Geo<LOGA>::R;
   if (MODE == 0) {
     const int64_t rows = B * D;
     MEGA_CHECK_ARG(rows <= 0x7fffffff, "fftconv: too many rows");
-    const unsigned grid = static_cast<unsigned>(rows < cus ? rows : cus);
-    fftconv_mfma_kernel<DT, MODE><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
+    const int64_t passes = (rows + R - 1) / R;
+    const unsigned grid = static_cast<unsigned>(passes < cus ? passes : cus);
+    fftconv_mfma_kernel<DT, MODE, LOGA><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
         a, b, out, static_cast<int>(rows), static_cast<int>(D), static_cast<int>(L), flip, omega);
     MEGA_CHECK_LAUNCH();
   } else {
-    const unsigned grid = static_cast<unsigned>(D < cus ? D : cus);
+    const int64_t passes = (D + R - 1) / R;
+    const unsigned grid = static_cast<unsigned>(passes < cus ? passes : cus);
     for (int64_t bb = 0; bb < B; ++bb) {
       const char* ab = static_cast<const char*>(a) + bb * D * L * 2;
       const char* xb = static_cast<const char*>(b) + bb * D * L * 2;
-      fftconv_mfma_kernel<DT, MODE><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
+      fftconv_mfma_kernel<DT, MODE, LOGA><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
           ab, xb, out, static_cast<int>(D), static_cast<int>(D), static_cast<int>(L),
           bb > 0 ? 1 : 0, nullptr);
       MEGA_CHECK_LAUNCH();
@@ -866,27 +1008,49 @@ int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_
   return MEGA_OK;
 }
 
+template <int DT, int MODE>
+int launch_len(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_t L, int flip,
+               const float* omega, hipStream_t stream) {
+  switch (loga_of(L)) {
+    case 5: return launch<DT, MODE, 5>(a, b, out, B, D, L, flip, omega, stream);
+    case 4: return launch<DT, MODE, 4>(a, b, out, B, D, L, flip, omega, stream);
+    case 3: return launch<DT, MODE, 3>(a, b, out, B, D, L, flip, omega, stream);
+    default: return launch<DT, MODE, 2>(a, b, out, B, D, L, flip, omega, stream);
+  }
+}
+template <int DT>
+int launch_bwd_len(const void* dy, const void* x, const float* k, void* dx, float* dk, int64_t B,
+                   int64_t D, int64_t L, const float* omega, hipStream_t stream) {
+  switch (loga_of(L)) {
+    case 5: return launch_bwd<DT, 5>(dy, x, k, dx, dk, B, D, L, omega, stream);
+    case 4: return launch_bwd<DT, 4>(dy, x, k, dx, dk, B, D, L, omega, stream);
+    case 3: return launch_bwd<DT, 3>(dy, x, k, dx, dk, B, D, L, omega, stream);
+    default: return launch_bwd<DT, 2>(dy, x, k, dx, dk, B, D, L, omega, stream);
+  }
+}
+
 }  // namespace
 
 bool applicable(int dtype, int64_t L, const void* a, const void* b, const void* out) {
   const auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  return (dtype == MEGA_BF16 || dtype == MEGA_F16) && L > 16384 && L <= 32768 && L % 8 == 0 &&
+  return (dtype == MEGA_BF16 || dtype == MEGA_F16) && L > 2048 && L <= 32768 && L % 8 == 0 &&
          al(a) && al(b) && al(out);
 }
 
 int launch_conv(int dtype, int mode, const void* a, const void* b, void* out, int64_t B,
                 int64_t D, int64_t L, int flip, const float* omega, hipStream_t stream) {
   if (dtype == MEGA_BF16)
-    return mode == 0 ? launch<MEGA_BF16, 0>(a, b, out, B, D, L, flip, omega, stream)
-                     : launch<MEGA_BF16, 1>(a, b, out, B, D, L, flip, omega, stream);
-  return mode == 0 ? launch<MEGA_F16, 0>(a, b, out, B, D, L, flip, omega, stream)
-                   : launch<MEGA_F16, 1>(a, b, out, B, D, L, flip, omega, stream);
+    return mode == 0 ? launch_len<MEGA_BF16, 0>(a, b, out, B, D, L, flip, omega, stream)
+                     : launch_len<MEGA_BF16, 1>(a, b, out, B, D, L, flip, omega, stream);
+  return mode == 0 ? launch_len<MEGA_F16, 0>(a, b, out, B, D, L, flip, omega, stream)
+                   : launch_len<MEGA_F16, 1>(a, b, out, B, D, L, flip, omega, stream);
 }
 
 int launch_backward(int dtype, const void* dy, const void* x, const float* k, void* dx, float* dk,
                     int64_t B, int64_t D, int64_t L, const float* omega, hipStream_t stream) {
-  if (dtype == MEGA_BF16) return launch_bwd<MEGA_BF16>(dy, x, k, dx, dk, B, D, L, omega, stream);
-  return launch_bwd<MEGA_F16>(dy, x, k, dx, dk, B, D, L, omega, stream);
+  if (dtype == MEGA_BF16)
+    return launch_bwd_len<MEGA_BF16>(dy, x, k, dx, dk, B, D, L, omega, stream);
+  return launch_bwd_len<MEGA_F16>(dy, x, k, dx, dk, B, D, L, omega, stream);
 }
 
 }  // namespace fftm

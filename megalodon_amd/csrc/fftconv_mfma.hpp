@@ -7,7 +7,7 @@
 namespace mega {
 namespace fftm {
 
-// bf16 / fp16 rows, 16384 < L <= 32768, L % 8 == 0, 16-byte aligned operands
+// bf16 / fp16 rows, 2048 < L <= 32768, L % 8 == 0, 16-byte aligned operands
 bool applicable(int dtype, int64_t L, const void* a, const void* b, const void* out);
 
 // mode 0: out[b,d,:] = conv(a[b,d,:], k[d,:]) (+ omega[d] a), k fp32, `flip` = backward dx form;

@@ -18,6 +18,8 @@ SHAPES = [
     (1, 3, 2049), (2, 2, 4096), (1, 3, 4097), (2, 2, 6001),            # M = 2048, 4096
     (1, 3, 8192), (1, 2, 8193), (2, 2, 16384), (1, 2, 12345),          # M = 4096, 8192
     (1, 3, 16385), (2, 3, 32768), (1, 2, 32767), (1, 2, 20001),        # M = 16384 (even and odd L)
+    # several 16-bit rows per workgroup pass (8, 4 or 2), full and ragged last passes
+    (3, 5, 2056), (1, 16, 4096), (2, 9, 6000), (1, 11, 8192), (2, 5, 12344), (3, 3, 16384),
 ]
 
 
@@ -50,7 +52,8 @@ def test_bwd_matches_oracle(B, D, L, dtype):
     assert rel_err(dk, wdk) <= TOL[dtype]
 
 
-RES_SHAPES = [(2, 3, 50), (1, 4, 2048), (2, 3, 4097), (1, 3, 8192), (2, 2, 12345), (2, 3, 32768), (1, 2, 32767)]
+RES_SHAPES = [(2, 3, 50), (1, 4, 2048), (2, 3, 4097), (1, 3, 8192), (2, 2, 12345), (2, 3, 32768), (1, 2, 32767),
+              (2, 9, 3000), (1, 7, 8200), (3, 3, 16384)]
 
 
 @pytest.mark.parametrize("B,D,L", RES_SHAPES)
@@ -83,10 +86,27 @@ def test_residual_autograd_function():
     assert wg.grad.shape == omega.shape and rel_err(wg.grad, wr.grad) <= 1e-4
 
 
-def test_float16_rows():
-    x, k, dy = _data(2, 3, 5000, torch.float16, 5)
+@pytest.mark.parametrize("B,D,L", [(2, 3, 5000), (1, 5, 2400), (2, 3, 10000), (1, 2, 30000)])
+def test_float16_rows(B, D, L):
+    x, k, dy = _data(B, D, L, torch.float16, 5)
     y = ops.fftconv_fwd(x.cuda(), k.cuda())
     assert rel_err(y, fftconv.fftconv_fwd(x, k)) <= TOL[torch.float16]
+    dx, dk = ops.fftconv_bwd(dy.cuda(), x.cuda(), k.cuda(), torch.float32)
+    wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
+    assert rel_err(dx, wdx) <= TOL[torch.float16] and rel_err(dk, wdk) <= TOL[torch.float16]
+
+
+def test_rows_of_a_pass_do_not_mix():
+    """Short 16-bit rows share a workgroup pass: a row of zeros between busy
+    rows stays exactly zero, and every row equals its single-row result."""
+    B, D, L = 1, 8, 4096
+    x, k, _ = _data(B, D, L, torch.bfloat16, 11)
+    x[:, 3] = 0
+    y = ops.fftconv_fwd(x.cuda(), k.cuda())
+    assert y[:, 3].abs().max().item() == 0.0
+    for d in (0, 5):
+        yd = ops.fftconv_fwd(x[:, d:d + 1].contiguous().cuda(), k[d:d + 1].contiguous().cuda())
+        assert torch.equal(yd[:, 0], y[:, d])
 
 
 def test_config0_cema_forward_fp32():
