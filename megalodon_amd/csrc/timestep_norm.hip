@@ -13,8 +13,11 @@
 // registers, reduces every row to its moments, scans the 64 rows inside one
 // wavefront (lane = timestep) and obtains the carry of all earlier tiles by a
 // decoupled look-back over per-tile records in device memory (aggregate /
-// inclusive-prefix words published with relaxed device-scope atomics, value and
-// ready-flag in one 64-bit word).  The tile is then normalised from registers:
+// inclusive-prefix words published with relaxed device-scope atomics, two
+// floats per 64-bit word, all ones meaning "not written yet").  Groups of at
+// most 16 lanes per row (128 bf16 features) give every wavefront a tile of its
+// own in the forward pass, with no workgroup barrier after the ticket.
+// The tile is then normalised from registers:
 // x is read once and y written once.  The backward pass runs the same scheme
 // in reverse time with 2x2 upper-triangular affine maps as the carried
 // quantity (the reverse recurrence on (dmean, dvar) is affine in the state).
@@ -59,16 +62,26 @@ struct TsnParams {
   float eps;
 };
 
-// ---- 64-bit (value, flag) words -------------------------------------------
-__device__ __forceinline__ void put_word(unsigned long long* p, float v) {
-  const unsigned long long w = (static_cast<unsigned long long>(1u) << 32) | __float_as_uint(v);
+// ---- 64-bit record words: two floats published together -------------------------
+// A word that nobody has written yet holds kEmpty (all ones).  A published word
+// never does: a float whose bits are all ones (one of the NaN encodings) is
+// stored as the default NaN instead.
+constexpr unsigned long long kEmpty = ~0ull;
+constexpr int kWin = 32;  // records polled per look-back round (lanes 0 .. kWin-1)
+__device__ __forceinline__ uint32_t word_bits(float v) {
+  const uint32_t b = __float_as_uint(v);
+  return b == 0xffffffffu ? 0x7fc00000u : b;
+}
+__device__ __forceinline__ void put_pair(unsigned long long* p, float lo, float hi) {
+  const unsigned long long w = (static_cast<unsigned long long>(word_bits(hi)) << 32) | word_bits(lo);
   __hip_atomic_store(p, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ bool get_word(const unsigned long long* p, float& v) {
+__device__ __forceinline__ bool get_pair(const unsigned long long* p, float& lo, float& hi) {
   const unsigned long long w =
       __hip_atomic_load(const_cast<unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  v = __uint_as_float(static_cast<uint32_t>(w));
-  return (w >> 32) != 0;
+  lo = __uint_as_float(static_cast<uint32_t>(w));
+  hi = __uint_as_float(static_cast<uint32_t>(w >> 32));
+  return w != kEmpty;
 }
 
 // ---- Welford triple ----------------------------------------------------------
@@ -164,6 +177,13 @@ __device__ __forceinline__ void stT(void* p, int64_t i, float v) {
   Elem<DT>::store(static_cast<typename Elem<DT>::type*>(p) + i, v);
 }
 
+// Hides a loaded vector from common-subexpression elimination: the unpacked
+// floats of an earlier phase are recomputed instead of being kept in registers.
+__device__ __forceinline__ uint4 reload(uint4 v) {
+  asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
+  return v;
+}
+
 template <int LPR>
 __device__ __forceinline__ float row_sum(float v) {  // sum over the LPR lanes of a row
   if (LPR <= 16) return group_sum<LPR>(v);  // inside one 16-lane DPP row
@@ -177,44 +197,60 @@ __global__ void tsn_prep_kernel(int* ticket, unsigned long long* rec, int64_t re
                                 const uint8_t* mask, int* nbefore, int B, int L, int NT) {
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  for (int64_t i = gid; i < rec_words; i += stride) rec[i] = 0ull;
+  for (int64_t i = gid; i < rec_words; i += stride) rec[i] = kEmpty;
   if (gid == 0) *ticket = 0;
-  // block b (< B) also builds nbefore[b][0..NT]
+  // block b (< B) also builds nbefore[b][0..NT]: thread i counts the unmasked
+  // steps of tiles i per .. i per + per - 1, a block-wide exclusive scan turns
+  // the counts into starting values
   if (blockIdx.x < static_cast<unsigned>(B)) {
-    __shared__ int sums[256];
+    __shared__ int wsum[4];
     const int b = blockIdx.x;
+    const uint8_t* mrow = mask == nullptr ? nullptr : mask + static_cast<int64_t>(b) * L;
+    const bool vec_ok = mrow != nullptr && reinterpret_cast<uintptr_t>(mrow) % 16 == 0;
+    auto tile_count = [&](int j) -> int {
+      const int tb = j * kTL, te = min(tb + kTL, L);
+      if (mrow == nullptr) return te - tb;
+      int c = 0;
+      if (vec_ok && te - tb == kTL) {
+#pragma unroll
+        for (int i = 0; i < kTL / 16; ++i) {
+          const uint4 v = *reinterpret_cast<const uint4*>(mrow + tb + 16 * i);
+          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int sh = 0; sh < 32; sh += 8) c += ((w[k] >> sh) & 0xffu) == 0u ? 1 : 0;
+        }
+      } else {
+        for (int t = tb; t < te; ++t) c += mrow[t] == 0 ? 1 : 0;
+      }
+      return c;
+    };
     const int per = (NT + 255) / 256;  // tiles per thread
     const int j0 = threadIdx.x * per;
     int local = 0;
-    for (int j = j0; j < j0 + per && j < NT; ++j) {
-      int c = 0;
-      for (int t = j * kTL; t < (j + 1) * kTL && t < L; ++t)
-        c += (mask == nullptr || mask[static_cast<int64_t>(b) * L + t] == 0) ? 1 : 0;
-      local += c;
+    for (int j = j0; j < j0 + per && j < NT; ++j) local += tile_count(j);
+    const int lane = threadIdx.x % kWave, wv = threadIdx.x / kWave;
+    int inc = local;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int o = __shfl_up(inc, d, kWave);
+      if (lane >= d) inc += o;
     }
-    sums[threadIdx.x] = local;
+    if (lane == kWave - 1) wsum[wv] = inc;
     __syncthreads();
-    if (threadIdx.x == 0) {
-      int run = 0;
-      for (int i = 0; i < 256; ++i) {
-        const int v = sums[i];
-        sums[i] = run;
-        run += v;
-      }
-    }
-    __syncthreads();
-    int run = sums[threadIdx.x];
+    int run = inc - local;
+    for (int i = 0; i < wv; ++i) run += wsum[i];
     for (int j = j0; j < j0 + per && j < NT; ++j) {
       nbefore[b * (NT + 1) + j] = run;
-      for (int t = j * kTL; t < (j + 1) * kTL && t < L; ++t)
-        run += (mask == nullptr || mask[static_cast<int64_t>(b) * L + t] == 0) ? 1 : 0;
+      run += per == 1 ? local : tile_count(j);
       if (j == NT - 1) nbefore[b * (NT + 1) + NT] = run;
     }
   }
 }
 
 // ------------------------------ forward ---------------------------------------
-constexpr int kFwdWords = 4;  // aggregate (u, v), inclusive (u, v)
+constexpr int kFwdWords = 2;  // aggregate (u, v), inclusive prefix (u, v)
 
 // carry of all tiles before tile j of this chain (wave 0 only)
 __device__ __forceinline__ Wel fwd_lookback(const TsnParams& p, int b, int g, int j, int lane,
@@ -226,41 +262,43 @@ __device__ __forceinline__ Wel fwd_lookback(const TsnParams& p, int b, int g, in
   int base = j - 1;
   while (true) {
     const int idx = base - lane;
-    int kind = 3;  // 1 aggregate, 2 inclusive prefix, 3 beyond the chain start
+    int kind = 3;  // 1 aggregate, 2 inclusive prefix, 3 beyond the chain start or outside the window
     Wel val{0.f, 0.f, 0.f};
-    if (idx >= 0) {
-      const unsigned long long* r = rec + static_cast<int64_t>(idx) * kFwdWords;
-      while (true) {
-        // all four words in one round trip: the aggregate is checked only if
-        // the inclusive prefix is not there yet
-        float iu, iv, au, av;
-        const bool f2 = get_word(r + 2, iu), f3 = get_word(r + 3, iv);
-        const bool f0 = get_word(r + 0, au), f1 = get_word(r + 1, av);
-        const bool fi = f2 & f3, fa = f0 & f1;
-        if (fi) {
-          kind = 2;
-          val = Wel{prior.n + static_cast<float>(nb[idx + 1]), iu, iv};
-          break;
+    if (lane < kWin) {
+      if (idx >= 0) {
+        const unsigned long long* r = rec + static_cast<int64_t>(idx) * kFwdWords;
+        while (true) {
+          // both words in one round trip: the aggregate counts only if the
+          // inclusive prefix is not there yet
+          float iu, iv, au, av;
+          const bool fi = get_pair(r + 1, iu, iv);
+          const bool fa = get_pair(r + 0, au, av);
+          if (fi) {
+            kind = 2;
+            val = Wel{prior.n + static_cast<float>(nb[idx + 1]), iu, iv};
+            break;
+          }
+          if (fa) {
+            kind = 1;
+            val = Wel{static_cast<float>(nb[idx + 1] - nb[idx]), au, av};
+            break;
+          }
+          __builtin_amdgcn_s_sleep(2);
         }
-        if (fa) {
-          kind = 1;
-          val = Wel{static_cast<float>(nb[idx + 1] - nb[idx]), au, av};
-          break;
-        }
-        __builtin_amdgcn_s_sleep(2);
+      } else if (idx == -1) {
+        kind = 2;
+        val = prior;
       }
-    } else if (idx == -1) {
-      kind = 2;
-      val = prior;
     }
     const unsigned long long m2 = __ballot(kind == 2);
     const int k = m2 ? __ffsll(static_cast<long long>(m2)) - 1 : 64;
     if (lane > k || kind == 3) val = Wel{0.f, 0.f, 0.f};
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) val = wel_merge(val, wel_shfl_xor(val, off));
+    for (int off = kWin / 2; off > 0; off >>= 1) val = wel_merge(val, wel_shfl_xor(val, off));
+    val = Wel{__shfl(val.n, 0, 64), __shfl(val.u, 0, 64), __shfl(val.v, 0, 64)};
     total = wel_merge(val, total);
     if (m2) break;
-    base -= 64;
+    base -= kWin;
   }
   return total;
 }
@@ -342,14 +380,12 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
     unsigned long long* rec = p.rec + (chain64 * p.NT + j) * kFwdWords;
     const Wel agg{__shfl(me.n, 63, 64), __shfl(me.u, 63, 64), __shfl(me.v, 63, 64)};
     if (lane == 0 && j + 1 < p.NT) {
-      put_word(rec + 0, agg.u);
-      put_word(rec + 1, agg.v);
+      put_pair(rec + 0, agg.u, agg.v);
     }
     const Wel prefix = j == 0 ? prior : fwd_lookback(p, b, g, j, lane, prior);
     if (lane == 0 && j + 1 < p.NT) {
       const Wel inc = wel_merge(prefix, agg);
-      put_word(rec + 2, inc.u);
-      put_word(rec + 3, inc.v);
+      put_pair(rec + 1, inc.u, inc.v);
     }
     const Wel st = wel_merge(prefix, me);
     const float rstd = 1.f / sqrtf(st.v + p.eps);
@@ -388,6 +424,138 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
 #pragma unroll
       for (int e = 0; e < VEC; ++e) o[e] = valid ? (f[e] - u) * rs * gm[e] + bt[e] : 0.f;
       const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
+      *reinterpret_cast<uint4*>(static_cast<typename Elem<DT>::type*>(p.y) + off) = Vec<DT>::pack(o);
+    }
+  }
+}
+
+// Narrow groups (at most 32 lanes per row): every wavefront owns a tile of its
+// own -- it loads the 64 rows, reduces, scans, looks back and normalises
+// without a workgroup barrier, so a slow tile holds up nobody else and each
+// wave keeps a whole tile's loads in flight.  The workgroup's four waves share
+// one ticket: tiles 4 ticket .. 4 ticket + 3 in time order, which only ever
+// wait for tiles of smaller or equal ticket.
+template <int DT, int LPR>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4)))
+void tsn_fwd_wave_kernel(const TsnParams p, int tiles) {
+  constexpr int VEC = Vec<DT>::N;
+  constexpr int RPW = kWave / LPR;  // rows per pass
+  constexpr int P = LPR;            // passes: kTL / RPW
+  __shared__ float s_a[kWaves][kTL], s_b[kWaves][kTL];
+  __shared__ int s_valid[kWaves][kTL];
+  __shared__ int s_ticket;
+
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  if (threadIdx.x == 0) s_ticket = atomicAdd(p.ticket, 1);
+  __syncthreads();
+  const int tile = s_ticket * kWaves + wave;
+  if (tile >= tiles) return;  // no workgroup barrier below
+  const int NC = p.B * p.G;
+  const int j = tile / NC;
+  const int chain = tile % NC;
+  const int b = chain / p.G, g = chain % p.G;
+  const int t0 = j * kTL;
+  const int col = lane % LPR;
+  const bool col_ok = col * VEC < p.Dg;
+  const float inv_dg = 1.f / static_cast<float>(p.Dg);
+  float* sa = s_a[wave];
+  float* sb = s_b[wave];
+  int* sv = s_valid[wave];
+
+  uint4 xv[P];
+#pragma unroll
+  for (int q = 0; q < P; ++q) {
+    const int t = t0 + q * RPW + lane / LPR;
+    xv[q] = make_uint4(0, 0, 0, 0);
+    if (t < p.L && col_ok) {
+      const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
+      xv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.x) + off);
+    }
+  }
+  uint4 gmv = make_uint4(0, 0, 0, 0), btv = make_uint4(0, 0, 0, 0);
+  if (col_ok) {
+    gmv = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.gamma) + g * p.Dg + col * VEC);
+    btv = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.beta) + g * p.Dg + col * VEC);
+  }
+  const int64_t chain64 = static_cast<int64_t>(b) * p.G + g;
+  const Wel prior{static_cast<float>(p.prev_count[b]), ldT<DT>(p.prev_mean, chain64),
+                  ldT<DT>(p.prev_var, chain64)};
+  const int t = t0 + lane;
+  const bool valid = t < p.L && (p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0);
+#pragma unroll
+  for (int q = 0; q < P; ++q) {
+    const int r = q * RPW + lane / LPR;
+    float f[VEC];
+    Vec<DT>::unpack(xv[q], f);
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) s += f[e];
+    const float mu = row_sum<LPR>(s) * inv_dg;
+    float s2 = 0.f;
+    if (col_ok) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) s2 += (f[e] - mu) * (f[e] - mu);
+    }
+    const float var = row_sum<LPR>(s2) * inv_dg;
+    if (col == 0) {
+      sa[r] = mu;
+      sb[r] = var;
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+
+  Wel me{valid ? 1.f : 0.f, valid ? sa[lane] : 0.f, valid ? sb[lane] : 0.f};
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const Wel o = wel_shfl_up(me, d);
+    if (lane >= d) me = wel_merge(o, me);
+  }
+  unsigned long long* rec = p.rec + (chain64 * p.NT + j) * kFwdWords;
+  const Wel agg{__shfl(me.n, 63, 64), __shfl(me.u, 63, 64), __shfl(me.v, 63, 64)};
+  if (lane == 0 && j + 1 < p.NT) {
+    put_pair(rec + 0, agg.u, agg.v);
+  }
+  const Wel prefix = j == 0 ? prior : fwd_lookback(p, b, g, j, lane, prior);
+  if (lane == 0 && j + 1 < p.NT) {
+    const Wel inc = wel_merge(prefix, agg);
+    put_pair(rec + 1, inc.u, inc.v);
+  }
+  const Wel st = wel_merge(prefix, me);
+  const float rstd = 1.f / sqrtf(st.v + p.eps);
+  if (t < p.L) {
+    const int64_t o = (static_cast<int64_t>(b) * p.L + t) * p.G + g;
+    p.cummean[o] = st.u;
+    p.cumrstd[o] = rstd;
+  }
+  if (j == p.NT - 1 && lane == 63) {
+    stT<DT>(p.mean, chain64, st.u);
+    stT<DT>(p.var, chain64, st.v);
+    if (g == 0) p.count[b] = p.prev_count[b] + p.nbefore[b * (p.NT + 1) + p.NT];
+  }
+  // the row moments were read before the scan (the shuffles above depend on
+  // them); a wave runs in program order, so they can be overwritten now
+  sa[lane] = st.u;
+  sb[lane] = rstd;
+  sv[lane] = valid ? 1 : 0;
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+
+  float gm[VEC], bt[VEC];
+  Vec<DT>::unpack(gmv, gm);
+  Vec<DT>::unpack(btv, bt);
+#pragma unroll
+  for (int q = 0; q < P; ++q) {
+    const int r = q * RPW + lane / LPR;
+    const int tr = t0 + r;
+    if (tr < p.L && col_ok) {
+      float f[VEC], o[VEC];
+      Vec<DT>::unpack(reload(xv[q]), f);
+      const float u = sa[r], rs = sb[r];
+      const bool ok = sv[r] != 0;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) o[e] = ok ? (f[e] - u) * rs * gm[e] + bt[e] : 0.f;
+      const int64_t off = (static_cast<int64_t>(b) * p.L + tr) * p.D + g * p.Dg + col * VEC;
       *reinterpret_cast<uint4*>(static_cast<typename Elem<DT>::type*>(p.y) + off) = Vec<DT>::pack(o);
     }
   }
@@ -440,7 +608,7 @@ __global__ __launch_bounds__(kWave) void tsn_fwd_serial_kernel(const TsnParams p
 }
 
 // ------------------------------ backward --------------------------------------
-constexpr int kBwdWords = 6;  // aggregate (a, e, bu, bv), outgoing state (ug, vg)
+constexpr int kBwdWords = 3;  // aggregate (a, e), (bu, bv), outgoing state (ug, vg)
 
 struct State2 {
   float ug, vg;
@@ -460,48 +628,48 @@ __device__ __forceinline__ State2 bwd_lookahead(const TsnParams& p, int64_t chai
     int kind = 3;
     Aff val{1.f, 0.f, 0.f, 0.f};
     State2 sv{0.f, 0.f};
-    if (idx < p.NT) {
-      const unsigned long long* r = rec + static_cast<int64_t>(idx) * kBwdWords;
-      while (true) {
-        // all six words in one round trip
-        float a, e, bu, bv, ug, vg;
-        const bool f4 = get_word(r + 4, ug), f5 = get_word(r + 5, vg);
-        const bool f0 = get_word(r + 0, a), f1 = get_word(r + 1, e);
-        const bool f2 = get_word(r + 2, bu), f3 = get_word(r + 3, bv);
-        const bool fs = f4 & f5, fa = f0 & f1 & f2 & f3;
-        if (fs) {
-          kind = 2;
-          sv = State2{ug, vg};
-          break;
+    if (lane < kWin) {
+      if (idx < p.NT) {
+        const unsigned long long* r = rec + static_cast<int64_t>(idx) * kBwdWords;
+        while (true) {
+          // all three words in one round trip
+          float a, e, bu, bv, ug, vg;
+          const bool fs = get_pair(r + 2, ug, vg);
+          const bool f0 = get_pair(r + 0, a, e), f1 = get_pair(r + 1, bu, bv);
+          if (fs) {
+            kind = 2;
+            sv = State2{ug, vg};
+            break;
+          }
+          if (f0 & f1) {
+            kind = 1;
+            val = Aff{a, e, bu, bv};
+            break;
+          }
+          __builtin_amdgcn_s_sleep(2);
         }
-        if (fa) {
-          kind = 1;
-          val = Aff{a, e, bu, bv};
-          break;
-        }
-        __builtin_amdgcn_s_sleep(2);
+      } else if (idx == p.NT) {
+        kind = 2;
+        sv = init;
       }
-    } else if (idx == p.NT) {
-      kind = 2;
-      sv = init;
     }
     const unsigned long long m2 = __ballot(kind == 2);
     const int k = m2 ? __ffsll(static_cast<long long>(m2)) - 1 : 64;
     if (lane >= k || kind != 1) val = Aff{1.f, 0.f, 0.f, 0.f};
     // ordered prefix composition: lane l holds A_base o ... o A_(base+l)
 #pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
+    for (int d = 1; d < kWin; d <<= 1) {
       const Aff o = aff_shfl_up(val, d);
       if (lane >= d) val = aff_compose(o, val);
     }
-    const Aff win{__shfl(val.a, 63, 64), __shfl(val.e, 63, 64), __shfl(val.bu, 63, 64),
-                  __shfl(val.bv, 63, 64)};
+    const Aff win{__shfl(val.a, kWin - 1, 64), __shfl(val.e, kWin - 1, 64),
+                  __shfl(val.bu, kWin - 1, 64), __shfl(val.bv, kWin - 1, 64)};
     total = aff_compose(total, win);
     if (m2) {
       const State2 s{__shfl(sv.ug, k, 64), __shfl(sv.vg, k, 64)};
       return aff_apply(total, s);
     }
-    base += 64;
+    base += kWin;
   }
 }
 
@@ -624,10 +792,8 @@ void tsn_bwd_kernel(const TsnParams p) {
     }
     unsigned long long* rec = p.rec + (chain64 * p.NT + j) * kBwdWords;
     if (lane == 0 && j > 0) {
-      put_word(rec + 0, inc.a);
-      put_word(rec + 1, inc.e);
-      put_word(rec + 2, inc.bu);
-      put_word(rec + 3, inc.bv);
+      put_pair(rec + 0, inc.a, inc.e);
+      put_pair(rec + 1, inc.bu, inc.bv);
     }
     const State2 sin = j == p.NT - 1 ? init : bwd_lookahead(p, chain64, j, lane, init);
     // state entering row i = (X_(i+1) o ... o X_63)(sin)
@@ -637,8 +803,7 @@ void tsn_bwd_kernel(const TsnParams p) {
     if (lane == 0) {
       const State2 sout = aff_apply(inc, sin);
       if (j > 0) {
-        put_word(rec + 4, sout.ug);
-        put_word(rec + 5, sout.vg);
+        put_pair(rec + 2, sout.ug, sout.vg);
       } else {
         stT<DT>(p.mean, chain64, sout.ug);
         stT<DT>(p.var, chain64, sout.vg);
@@ -766,17 +931,39 @@ __global__ __launch_bounds__(kWave) void tsn_bwd_serial_kernel(const TsnParams p
 }
 
 // dgamma[h] = sum_rows part_g[row][h] (same for dbeta), rows = B*NT.  A workgroup
-// owns 64 columns; its 4 waves split the rows (Kahan-compensated partial sums in
-// a fixed order: deterministic), then combine through LDS.
+// owns 64 columns; its 16 waves split the rows (Kahan-compensated partial sums
+// in a fixed order: deterministic), then combine through LDS.
+constexpr int kPgWaves = 16;
 template <int DT>
-__global__ __launch_bounds__(256) void tsn_param_grad_kernel(const float* part_g, const float* part_b,
-                                                            int rows, int D, void* dgamma, void* dbeta) {
-  __shared__ float sg[4][64], sb[4][64];
+__global__ __launch_bounds__(kPgWaves * 64) void tsn_param_grad_kernel(
+    const float* part_g, const float* part_b, int rows, int D, void* dgamma, void* dbeta) {
+  __shared__ float sg[kPgWaves][64], sb[kPgWaves][64];
   const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
   const int h = blockIdx.x * 64 + lane;
   float a = 0.f, c = 0.f, ca = 0.f, cc = 0.f;
   if (h < D) {
-    for (int r = w; r < rows; r += 4) {
+    constexpr int U = 8;  // rows in flight per wave
+    int r = w;
+    for (; r + (U - 1) * kPgWaves < rows; r += U * kPgWaves) {
+      float va[U], vc[U];
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        va[i] = part_g[static_cast<int64_t>(r + i * kPgWaves) * D + h];
+        vc[i] = part_b[static_cast<int64_t>(r + i * kPgWaves) * D + h];
+      }
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        const float ya = va[i] - ca;
+        const float ta = a + ya;
+        ca = (ta - a) - ya;
+        a = ta;
+        const float yc = vc[i] - cc;
+        const float tc = c + yc;
+        cc = (tc - c) - yc;
+        c = tc;
+      }
+    }
+    for (; r < rows; r += kPgWaves) {
       const float ya = part_g[static_cast<int64_t>(r) * D + h] - ca;
       const float ta = a + ya;
       ca = (ta - a) - ya;
@@ -791,8 +978,14 @@ __global__ __launch_bounds__(256) void tsn_param_grad_kernel(const float* part_g
   sb[w][lane] = c;
   __syncthreads();
   if (w == 0 && h < D) {
-    stT<DT>(dgamma, h, (sg[0][lane] + sg[1][lane]) + (sg[2][lane] + sg[3][lane]));
-    stT<DT>(dbeta, h, (sb[0][lane] + sb[1][lane]) + (sb[2][lane] + sb[3][lane]));
+    float ta = 0.f, tc = 0.f;
+#pragma unroll
+    for (int i = 0; i < kPgWaves; ++i) {
+      ta += sg[i][lane];
+      tc += sb[i][lane];
+    }
+    stT<DT>(dgamma, h, ta);
+    stT<DT>(dbeta, h, tc);
   }
 }
 
@@ -826,17 +1019,29 @@ int launch_fast(const TsnParams& p, int64_t tiles, hipStream_t s) {
   const int vec = DT == MEGA_F32 ? 4 : 8;
   const int lanes = p.Dg / vec;
   const dim3 grid(static_cast<unsigned>(tiles));
+  // forward, narrow groups: one tile per wavefront
+  const dim3 wgrid(static_cast<unsigned>((tiles + kWaves - 1) / kWaves));
+  const int nt = static_cast<int>(tiles);
 #define MEGA_TSN_LAUNCH(LPR)                                              \
   do {                                                                    \
     if (FWD) tsn_fwd_kernel<DT, LPR><<<grid, kThreads, 0, s>>>(p);        \
     else tsn_bwd_kernel<DT, LPR><<<grid, kThreads, 0, s>>>(p);            \
   } while (0)
-  if (lanes <= 4) MEGA_TSN_LAUNCH(4);
-  else if (lanes <= 8) MEGA_TSN_LAUNCH(8);
-  else if (lanes <= 16) MEGA_TSN_LAUNCH(16);
+#define MEGA_TSN_LAUNCH_WAVE(LPR) tsn_fwd_wave_kernel<DT, LPR><<<wgrid, kThreads, 0, s>>>(p, nt)
+  if (!FWD) {  // two operand tiles per wave leave too few waves resident
+    if (lanes <= 4) MEGA_TSN_LAUNCH(4);
+    else if (lanes <= 8) MEGA_TSN_LAUNCH(8);
+    else if (lanes <= 16) MEGA_TSN_LAUNCH(16);
+    else if (lanes <= 32) MEGA_TSN_LAUNCH(32);
+    else MEGA_TSN_LAUNCH(64);
+  } else
+  if (lanes <= 4) MEGA_TSN_LAUNCH_WAVE(4);
+  else if (lanes <= 8) MEGA_TSN_LAUNCH_WAVE(8);
+  else if (lanes <= 16) MEGA_TSN_LAUNCH_WAVE(16);
   else if (lanes <= 32) MEGA_TSN_LAUNCH(32);
   else MEGA_TSN_LAUNCH(64);
 #undef MEGA_TSN_LAUNCH
+#undef MEGA_TSN_LAUNCH_WAVE
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
 }
@@ -887,7 +1092,7 @@ int tsn_bwd_impl(TsnParams p, void* dgamma, void* dbeta, void* workspace, hipStr
     MEGA_CHECK_LAUNCH();
     rows = p.B;
   }
-  tsn_param_grad_kernel<DT><<<(p.D + 63) / 64, 256, 0, s>>>(p.part_g, p.part_b, rows, p.D, dgamma, dbeta);
+  tsn_param_grad_kernel<DT><<<(p.D + 63) / 64, kPgWaves * 64, 0, s>>>(p.part_g, p.part_b, rows, p.D, dgamma, dbeta);
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
 }
