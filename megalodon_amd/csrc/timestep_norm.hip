@@ -88,12 +88,15 @@ __device__ __forceinline__ bool get_pair(const unsigned long long* p, float& lo,
 struct Wel {
   float n, u, v;
 };
+// Two empty operands (a prior of count zero and masked steps, or the identity)
+// keep the prior's mean and variance: at most one of them is not all zeros.
 __device__ __forceinline__ Wel wel_merge(Wel a, Wel b) {  // utils.h:154-164
   const float n = a.n + b.n;
   const float inv = n > 0.f ? 1.f / n : 0.f;
   const float c1 = a.n * inv, c2 = b.n * inv;
   const float d = b.u - a.u;
-  return Wel{n, c1 * a.u + c2 * b.u, c1 * a.v + c2 * b.v + (c1 * d) * (c2 * d)};
+  const float u = c1 * a.u + c2 * b.u, v = c1 * a.v + c2 * b.v + (c1 * d) * (c2 * d);
+  return Wel{n, n > 0.f ? u : a.u + b.u, n > 0.f ? v : a.v + b.v};
 }
 __device__ __forceinline__ Wel wel_shfl_up(Wel a, int d) {
   return Wel{__shfl_up(a.n, d, 64), __shfl_up(a.u, d, 64), __shfl_up(a.v, d, 64)};
@@ -135,6 +138,20 @@ template <> struct Vec<MEGA_F32> {
 };
 template <> struct Vec<MEGA_BF16> {
   static constexpr int N = 8;
+  // sum and sum of squares of the 8 elements, products exact, fp32 accumulation
+  // (v_dot2c_f32_bf16: no unpacking)
+  static __device__ __forceinline__ void moments(const uint4& r, float& s1, float& s2) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const bf16x2 one = __builtin_bit_cast(bf16x2, 0x3f803f80u);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+    s1 = s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bf16x2 v = __builtin_bit_cast(bf16x2, w[i]);
+      s1 = __builtin_amdgcn_fdot2_f32_bf16(v, one, s1, false);
+      s2 = __builtin_amdgcn_fdot2_f32_bf16(v, v, s2, false);
+    }
+  }
   static __device__ __forceinline__ void unpack(const uint4& r, float* f) {
     const uint32_t w[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
@@ -462,15 +479,17 @@ void tsn_fwd_wave_kernel(const TsnParams p, int tiles) {
   float* sb = s_b[wave];
   int* sv = s_valid[wave];
 
+  // element offset of this lane's vector in pass 0; a pass advances RPW rows
+  const int64_t off0 =
+      (static_cast<int64_t>(b) * p.L + t0 + lane / LPR) * p.D + g * p.Dg + col * VEC;
+  const int64_t pass_stride = static_cast<int64_t>(RPW) * p.D;
+  const int rows_left = p.L - t0 - lane / LPR;  // pass q is in range iff q * RPW < rows_left
+  const typename Elem<DT>::type* xp = static_cast<const typename Elem<DT>::type*>(p.x) + off0;
   uint4 xv[P];
 #pragma unroll
   for (int q = 0; q < P; ++q) {
-    const int t = t0 + q * RPW + lane / LPR;
     xv[q] = make_uint4(0, 0, 0, 0);
-    if (t < p.L && col_ok) {
-      const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
-      xv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.x) + off);
-    }
+    if (q * RPW < rows_left && col_ok) xv[q] = *reinterpret_cast<const uint4*>(xp + q * pass_stride);
   }
   uint4 gmv = make_uint4(0, 0, 0, 0), btv = make_uint4(0, 0, 0, 0);
   if (col_ok) {
@@ -485,18 +504,28 @@ void tsn_fwd_wave_kernel(const TsnParams p, int tiles) {
 #pragma unroll
   for (int q = 0; q < P; ++q) {
     const int r = q * RPW + lane / LPR;
-    float f[VEC];
-    Vec<DT>::unpack(xv[q], f);
-    float s = 0.f;
+    float mu, var;
+    if (DT == MEGA_BF16) {
+      // one pass over the packed words.  E[x^2] - mu^2 in fp32 is exact to
+      // ~1e-7 (1 + mu^2 / var), and bf16 data cannot hold |mu| / sigma > 256
+      float s1, s2;
+      Vec<MEGA_BF16>::moments(xv[q], s1, s2);  // lanes past the group hold zeros
+      mu = row_sum<LPR>(s1) * inv_dg;
+      var = fmaxf(row_sum<LPR>(s2) * inv_dg - mu * mu, 0.f);
+    } else {
+      float f[VEC];
+      Vec<DT>::unpack(xv[q], f);
+      float s = 0.f;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) s += f[e];
-    const float mu = row_sum<LPR>(s) * inv_dg;
-    float s2 = 0.f;
-    if (col_ok) {
+      for (int e = 0; e < VEC; ++e) s += f[e];
+      mu = row_sum<LPR>(s) * inv_dg;
+      float s2 = 0.f;
+      if (col_ok) {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) s2 += (f[e] - mu) * (f[e] - mu);
+        for (int e = 0; e < VEC; ++e) s2 += (f[e] - mu) * (f[e] - mu);
+      }
+      var = row_sum<LPR>(s2) * inv_dg;
     }
-    const float var = row_sum<LPR>(s2) * inv_dg;
     if (col == 0) {
       sa[r] = mu;
       sb[r] = var;
@@ -535,8 +564,10 @@ void tsn_fwd_wave_kernel(const TsnParams p, int tiles) {
   }
   // the row moments were read before the scan (the shuffles above depend on
   // them); a wave runs in program order, so they can be overwritten now
-  sa[lane] = st.u;
-  sb[lane] = rstd;
+  // y = x rstd - mean rstd per row (then gamma, beta per column); masked rows
+  // get the zero map and are cleared after packing
+  sa[lane] = valid ? -st.u * rstd : 0.f;
+  sb[lane] = valid ? rstd : 0.f;
   sv[lane] = valid ? 1 : 0;
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __builtin_amdgcn_wave_barrier();
@@ -544,19 +575,19 @@ void tsn_fwd_wave_kernel(const TsnParams p, int tiles) {
   float gm[VEC], bt[VEC];
   Vec<DT>::unpack(gmv, gm);
   Vec<DT>::unpack(btv, bt);
+  typename Elem<DT>::type* yp = static_cast<typename Elem<DT>::type*>(p.y) + off0;
 #pragma unroll
   for (int q = 0; q < P; ++q) {
     const int r = q * RPW + lane / LPR;
-    const int tr = t0 + r;
-    if (tr < p.L && col_ok) {
+    if (q * RPW < rows_left && col_ok) {
       float f[VEC], o[VEC];
       Vec<DT>::unpack(reload(xv[q]), f);
-      const float u = sa[r], rs = sb[r];
-      const bool ok = sv[r] != 0;
+      const float nur = sa[r], rs = sb[r];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) o[e] = ok ? (f[e] - u) * rs * gm[e] + bt[e] : 0.f;
-      const int64_t off = (static_cast<int64_t>(b) * p.L + tr) * p.D + g * p.Dg + col * VEC;
-      *reinterpret_cast<uint4*>(static_cast<typename Elem<DT>::type*>(p.y) + off) = Vec<DT>::pack(o);
+      for (int e = 0; e < VEC; ++e) o[e] = fmaf(fmaf(f[e], rs, nur), gm[e], bt[e]);
+      uint4 packed = Vec<DT>::pack(o);
+      if (sv[r] == 0) packed = make_uint4(0, 0, 0, 0);
+      *reinterpret_cast<uint4*>(yp + q * pass_stride) = packed;
     }
   }
 }

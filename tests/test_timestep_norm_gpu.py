@@ -69,6 +69,7 @@ def _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed, check_stats_everywhere=Tr
     (2, 130, 64, 2, 2, "holes"),     # Dg = 32
     (2, 77, 1024, 2, 1, "trailing"), # Dg = 512 (64 lanes per row in 16-bit)
     (2, 50, 48, 48, 4, "holes"),     # one feature per group: serial path
+    (2, 150, 256, 2, 0, "holes"),    # masked steps before the first counted one, no prior
     (2, 33, 36, 1, 0, None),         # one group, Dg not a multiple of the vector width
     (1, 1, 128, 1, 0, None),         # single step
 ])
@@ -76,9 +77,24 @@ def test_fwd_bwd_match_oracle(B, L, H, G, prior, mask, dtype):
     _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed=B * 1000 + L)
 
 
-def test_all_steps_masked_keeps_prior():
+@pytest.mark.parametrize("offset", [8.0, 40.0])
+def test_bf16_forward_with_large_channel_offsets(offset):
+    """bfloat16 rows take their moments in one pass (E[x^2] - mean^2 in float32);
+    a mean many standard deviations from zero must stay within the bfloat16 bar."""
+    B, L, H, G = 2, 300, 512, 4
+    x, pc, pm, pv, gamma, beta, m, *_ = _case(B, L, H, G, 7, torch.float32, 0, "holes")
+    x = (x + offset).to(torch.bfloat16)
+    pm, pv, gamma, beta = (t.to(torch.bfloat16) for t in (pm, pv, gamma, beta))
+    y, count, mean, var, cummean, cumrstd = ops.group_timestep_norm_fwd(*_cuda(x, pc, pm, pv, gamma, beta, m), G, 1e-5)
+    wy, wcount, wmean, wvar, wcm, wcr = tn.group_timestep_norm_closed_form_full(x, pc, pm, pv, gamma, beta, m, G, 1e-5)
+    assert rel_err(y, wy) <= 2e-2 and rel_err(var, wvar) <= 2e-2
+    assert rel_err(cummean, wcm) <= 1e-4 and rel_err(cumrstd, wcr) <= 2e-3
+
+
+@pytest.mark.parametrize("prior", [4, 0])
+def test_all_steps_masked_keeps_prior(prior):
     B, L, H, G = 2, 70, 256, 2
-    x, pc, pm, pv, gamma, beta, _, *_ = _case(B, L, H, G, 3, torch.float32, prior=4, mask=None)
+    x, pc, pm, pv, gamma, beta, _, *_ = _case(B, L, H, G, 3, torch.float32, prior=prior, mask=None)
     m = torch.ones(B, L, dtype=torch.bool)
     y, count, mean, var, cm, cr = ops.group_timestep_norm_fwd(*_cuda(x, pc, pm, pv, gamma, beta, m), G, 1e-5)
     assert y.abs().max().item() == 0
