@@ -4,9 +4,12 @@
 A step is one CEMA layer forward+backward at the 7B layer width (BASELINE
 config 1): k = ema_parameters(p, q, gamma) -> y = fftconv(x, k) + x*omega, then
 backward through both ops to dx, d(alpha, delta, theta, gamma, omega), with
-B=1, L=32768, D=4096, ndim=16, x and the upstream gradient in bf16, arithmetic
-in fp32.  Inputs are synthetic, seeded, and resident in HBM before the timed
-region.  Prints one JSON line.
+B=1, L=32768, D=4096, ndim=16, x and the upstream gradient in bf16.  The
+convolution's DFT stages run on the matrix cores (fp16 operands, fp32
+accumulation; twiddles, the spectral product and every sum in fp32); the same
+step through the all-fp32 VALU convolution engine is timed beside it
+("fp32_fft_engine").  Inputs are synthetic, seeded, and resident in HBM before
+the timed region.  Prints one JSON line.
 """
 import argparse
 import json
@@ -22,7 +25,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes one forward convolution launch moves at config 1: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from
 # two rocprofv3 --pmc passes of this script, the factors being what the same counters read for a plain
 # copy of 2^30 bytes (--copy-calibration).  A measured constant: counters cannot be read from in here.
-FFTCONV_TRAFFIC_BYTES = 1.40e9
+FFTCONV_TRAFFIC_BYTES = 1.37e9
 
 
 def cpu_baseline(B, D, N, L, seed, budget_s=25.0):
@@ -225,6 +228,23 @@ def main():
     kernels["ema_weight_fwd_GBps"] = 4 * E / (kernels["ema_weight_fwd_ms"] * 1e-3) / 1e9
     kernels["ema_weight_bwd_GBps"] = 4 * E / (kernels["ema_weight_bwd_ms"] * 1e-3) / 1e9
 
+    # the same step with every FFT butterfly in fp32 on the vector ALUs
+    fp32_engine = None
+    if not args.skip_other_ops:
+        os.environ["MEGA_FFTCONV_VALU"] = "1"
+        try:
+            step()
+            torch.cuda.synchronize()
+            n32 = max(1, min(5, args.steps))
+            t1 = time.perf_counter()
+            for _ in range(n32):
+                step()
+            torch.cuda.synchronize()
+            dt32 = (time.perf_counter() - t1) / n32
+        finally:
+            os.environ.pop("MEGA_FFTCONV_VALU", None)
+        fp32_engine = {"ms_per_step": dt32 * 1e3, "tokens_per_s": B * L / dt32, "steps": n32}
+
     if args.copy_calibration:
         src = torch.ones(1 << 29, dtype=torch.bfloat16, device=dev)
         dst = torch.empty_like(src)
@@ -246,10 +266,11 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f16*f16+f32",
         "data": "synthetic",
         "config": {"workload": "configs[1]: CEMA + causal FFT convolution forward+backward, "
-                               "B=1 L=32768 D=4096 ndim=16, x/dy bf16, fp32 arithmetic",
+                               "B=1 L=32768 D=4096 ndim=16, x/dy bf16, k/dk fp32; DFT stages fp16 operands "
+                               "with fp32 accumulation on the matrix cores, everything else fp32",
                    "global_batch": B, "seq_len": L},
         "roofline": {
             "bound": "hbm", "kernel": "fftconv_mfma_kernel<bf16, MODE=0> (one launch = forward conv of all rows, skip term included)",
@@ -257,6 +278,7 @@ def main():
             "frac": achieved / HBM_PEAK_GBS, "traffic": FFTCONV_TRAFFIC_BYTES,
         },
         "kernels": kernels,
+        "fp32_fft_engine": fp32_engine,
         "other_ops": other,
     }
     if not args.no_cpu_baseline:
