@@ -4,7 +4,7 @@
 //   megalodon/csrc/ops/attention_kernel.cu:40-133 (forward), :135-257 (backward)
 //   megalodon/csrc/softmax.cuh:86-131,198-234 (causal softmax forward / backward):
 //   S = scale * Q K^T rounded to the element type, P = softmax_fp32(S) over the
-//   causal prefix (row r sees columns 0..r), P stored in the element type,
+//   causal prefix (row r sees columns 0..L2-L1+r), P stored in the element type,
 //   Y = P V;  dV = P^T dY, dP = dY V^T, dS = P o (dP - rowsum(P o dP)),
 //   dQ = scale dS K, dK = scale dS^T Q.  Layout BLNH in and out; w = P is
 //   returned (B, N, L1, L2) as the reference does.
@@ -12,13 +12,14 @@
 // Differences in execution: the reference runs full-square cuBLAS GEMMs and a
 // full-row softmax; here every product is one hand-written MFMA GEMM
 // (v_mfma_f32_32x32x16, 256x256 workgroup tile, 128x128 per wavefront,
-// double-buffered LDS staging of 64-wide k slabs) that skips the tiles above
+// double-buffered LDS staging of 32-wide k slabs) that skips the tiles above
 // the causal diagonal and the k-ranges where P / dS are structurally zero, so
 // causal attention costs half the flops and half the P traffic.  Operands whose
 // reduction index is not the contiguous one (V, dY, K, Q, P, dS in the
-// backward products) are transposed first by a tiled copy kernel; the GEMM
-// itself only ever sees k-contiguous rows, which is the form the MFMA operand
-// registers want (8 consecutive k per lane).
+// backward products) are staged k-major in LDS and read with the transposing
+// LDS read, which hands each lane the 8 consecutive k an MFMA operand wants.
+// A key/value prefix (L2 > L1, cached keys in front of the chunk) shifts the
+// diagonal by L2 - L1 columns in every one of these rules.
 #include "common.hpp"
 
 namespace mega {
@@ -77,8 +78,12 @@ struct GemmParams {
   int64_t sa0, sa1, sb0, sb1, sc0, sc1;  // batch z = z0 * nh + z1 -> offset z0*s0 + z1*s1
   int nh;
   float alpha;
-  int tri_out;  // 1: tiles with nt > mt are skipped (left unwritten)
-  int k_mode;   // 0: all k; 1: k < (mt+1)*256; 2: k >= mt*256
+  // Causal structure with rows = queries r, columns = keys c, c <= r + off
+  // (off = L2 - L1 >= 0, the length of a key/value prefix):
+  int tri_out;  // 1: tiles wholly above that diagonal are skipped (left unwritten)
+  int k_mode;   // 0: all k; 1: m = queries, k = keys: k < (mt+1)*256 + off, rounded up to a slab;
+                // 2: m = keys, k = queries: k >= mt*256 - off, rounded down to a slab
+  int off;
   int ta, tb;   // operand is k-major: element (m, k) at [k * ld + m]
 };
 
@@ -143,15 +148,15 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
   const int mt_raw = (id / gridDim.x) % gridDim.y;
   const int mt = (p.tri_out || p.k_mode) ? static_cast<int>(gridDim.y) - 1 - mt_raw : mt_raw;
   const int zz = id / (gridDim.x * gridDim.y);
-  if (p.tri_out && nt > mt) return;
+  if (p.tri_out && nt * kTile > mt * kTile + (kTile - 1) + p.off) return;
   const int z0 = zz / p.nh, z1 = zz % p.nh;
   const uint16_t* A = p.A + z0 * p.sa0 + z1 * p.sa1;
   const uint16_t* B = p.B + z0 * p.sb0 + z1 * p.sb1;
   uint16_t* C = p.C + z0 * p.sc0 + z1 * p.sc1;
   const int m0 = mt * kTile, n0 = nt * kTile;
   int kb = 0, ke = p.K;
-  if (p.k_mode == 1) ke = min(p.K, (mt + 1) * kTile);
-  if (p.k_mode == 2) kb = min(p.K, mt * kTile);
+  if (p.k_mode == 1) ke = min(p.K, ((mt + 1) * kTile + p.off + kSlab - 1) / kSlab * kSlab);
+  if (p.k_mode == 2) kb = min(p.K, max(0, mt * kTile - p.off) / kSlab * kSlab);
   const int nslab = (ke - kb + kSlab - 1) / kSlab;
 
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
@@ -348,19 +353,21 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
 }
 
 // ---- causal softmax over rows (in place), one wavefront per row ---------------
-// row r of matrix z keeps columns [0, n) with n = causal ? r + 1 : L2; the rest
-// of the row up to the end of its 256-column tile is set to 0 (that is all the
-// later products read).  softmax.cuh:86-131.
+// `coff` < 0: every row keeps all L2 columns.  `coff` = L2 - L1 >= 0 (causal,
+// bottom-right aligned, softmax.cuh:99-100): row r keeps columns [0, n) with
+// n = r + 1 + coff.  The rest of the row is set to 0 -- with coff = 0 only up
+// to the end of its 256-column tile, which is all the later products read.
+// softmax.cuh:86-131.
 template <int DT>
 __global__ __launch_bounds__(kThreads) void softmax_fwd_kernel(uint16_t* w, int L1, int L2,
-                                                              int causal) {
+                                                              int coff) {
   // grid.y carries the batch*heads index; grid.x covers the L1 rows
   const int lane = threadIdx.x % kWave;
   const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   if (r >= L1) return;
   uint16_t* x = w + (static_cast<int64_t>(blockIdx.y) * L1 + r) * L2;
-  const int n = causal ? min(r + 1, L2) : L2;
-  const int nz = causal ? min(L2, (r / kTile + 1) * kTile) : L2;
+  const int n = coff >= 0 ? min(r + 1 + coff, L2) : L2;
+  const int nz = coff == 0 ? min(L2, (r / kTile + 1) * kTile) : L2;
   float m = -INFINITY;
   for (int j = lane; j < n; j += kWave) m = fmaxf(m, Elem<DT>::load(x + j));
   m = wave_max(m);
@@ -407,13 +414,13 @@ __device__ __forceinline__ uint4 pack8(const float* v) {
 // aligned base and L2 <= 64 * 8 * NCH; one read and one write of the row.
 template <int DT, int NCH>
 __global__ __launch_bounds__(kThreads) void softmax_fwd_vec_kernel(uint16_t* w, int L1, int L2,
-                                                                  int causal) {
+                                                                  int coff) {
   const int lane = threadIdx.x % kWave;
   const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   if (r >= L1) return;
   uint16_t* x = w + (static_cast<int64_t>(blockIdx.y) * L1 + r) * L2;
-  const int n = causal ? min(r + 1, L2) : L2;
-  const int nz = causal ? min(L2, (r / kTile + 1) * kTile) : L2;
+  const int n = coff >= 0 ? min(r + 1 + coff, L2) : L2;
+  const int nz = coff == 0 ? min(L2, (r / kTile + 1) * kTile) : L2;
   float v[NCH][8];
   float m = -INFINITY;
 #pragma unroll
@@ -456,15 +463,15 @@ __global__ __launch_bounds__(kThreads) void softmax_fwd_vec_kernel(uint16_t* w, 
 // dS = P o (dP - sum_j P_j dP_j), written over dP.  softmax.cuh:198-234.
 template <int DT>
 __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const uint16_t* w, uint16_t* dw,
-                                                              int L1, int L2, int causal) {
+                                                              int L1, int L2, int coff) {
   const int lane = threadIdx.x % kWave;
   const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   if (r >= L1) return;
   const int64_t o = (static_cast<int64_t>(blockIdx.y) * L1 + r) * L2;
   const uint16_t* pw = w + o;
   uint16_t* pd = dw + o;
-  const int n = causal ? min(r + 1, L2) : L2;
-  const int nz = causal ? min(L2, (r / kTile + 1) * kTile) : L2;
+  const int n = coff >= 0 ? min(r + 1 + coff, L2) : L2;
+  const int nz = coff == 0 ? min(L2, (r / kTile + 1) * kTile) : L2;
   float s = 0.f;
   for (int j = lane; j < n; j += kWave) s += Elem<DT>::load(pw + j) * Elem<DT>::load(pd + j);
   s = wave_sum(s);
@@ -476,15 +483,15 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const uint16_t* w
 
 template <int DT, int NCH>
 __global__ __launch_bounds__(kThreads) void softmax_bwd_vec_kernel(const uint16_t* w, uint16_t* dw,
-                                                                  int L1, int L2, int causal) {
+                                                                  int L1, int L2, int coff) {
   const int lane = threadIdx.x % kWave;
   const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   if (r >= L1) return;
   const int64_t o = (static_cast<int64_t>(blockIdx.y) * L1 + r) * L2;
   const uint16_t* pw = w + o;
   uint16_t* pd = dw + o;
-  const int n = causal ? min(r + 1, L2) : L2;
-  const int nz = causal ? min(L2, (r / kTile + 1) * kTile) : L2;
+  const int n = coff >= 0 ? min(r + 1 + coff, L2) : L2;
+  const int nz = coff == 0 ? min(L2, (r / kTile + 1) * kTile) : L2;
   float pv[NCH][8], dv[NCH][8];
   float s = 0.f;
 #pragma unroll
@@ -518,6 +525,7 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_vec_kernel(const uint16_
 template <int DT>
 int launch_softmax(const uint16_t* p, uint16_t* x, int64_t Z, int64_t L1, int64_t L2, int causal,
                    hipStream_t s) {
+  const int coff = causal ? static_cast<int>(L2 - L1) : -1;
   // p == nullptr: forward over x in place; else backward with probabilities p
   if (Z == 0 || L1 == 0 || L2 == 0) return MEGA_OK;
   const dim3 grid((unsigned)((L1 + 3) / 4), (unsigned)Z);
@@ -525,9 +533,9 @@ int launch_softmax(const uint16_t* p, uint16_t* x, int64_t Z, int64_t L1, int64_
                    reinterpret_cast<uintptr_t>(p) % 16 == 0;
 #define MEGA_SOFTMAX(NCH)                                                                   \
   if (p == nullptr)                                                                         \
-    softmax_fwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, causal); \
+    softmax_fwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff); \
   else                                                                                      \
-    softmax_bwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, causal);
+    softmax_bwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, coff);
   if (vec && L2 <= 512) {
     MEGA_SOFTMAX(1)
   } else if (vec && L2 <= 1024) {
@@ -537,9 +545,9 @@ int launch_softmax(const uint16_t* p, uint16_t* x, int64_t Z, int64_t L1, int64_
   } else if (vec && L2 <= 4096) {
     MEGA_SOFTMAX(8)
   } else if (p == nullptr) {
-    softmax_fwd_kernel<DT><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, causal);
+    softmax_fwd_kernel<DT><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff);
   } else {
-    softmax_bwd_kernel<DT><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, causal);
+    softmax_bwd_kernel<DT><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, coff);
   }
 #undef MEGA_SOFTMAX
   MEGA_CHECK_LAUNCH();
@@ -595,9 +603,8 @@ int check_attn(const char* who, int dtype, int64_t B, int64_t L1, int64_t L2, in
   MEGA_CHECK_ARG(B >= 0 && L1 >= 0 && L2 >= 0 && NH >= 1 && H1 >= 1 && H2 >= 1, "%s: bad sizes", who);
   MEGA_CHECK_ARG(B * NH <= 65535, "%s: batch * heads exceeds 65535", who);
   MEGA_CHECK_ARG(L1 <= (1 << 24) && L2 <= (1 << 24), "%s: sequence too long", who);
-  if (causal && L1 != L2)
-    return set_error(MEGA_ERR_UNSUPPORTED,
-                     "%s: causal attention with L1 != L2 (key/value cache prefix) is not implemented", who);
+  MEGA_CHECK_ARG(!causal || L2 >= L1,
+                 "%s: causal attention needs L2 >= L1 (row r sees keys 0 .. L2 - L1 + r)", who);
   return MEGA_OK;
 }
 
@@ -613,7 +620,7 @@ int attn_fwd_impl(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64
   g.lda = NH * H1; g.ldb = NH * H1; g.ldc = L2;
   g.sa0 = L1 * NH * H1; g.sa1 = H1; g.sb0 = L2 * NH * H1; g.sb1 = H1;
   g.sc0 = NH * L1 * L2; g.sc1 = L1 * L2; g.nh = (int)NH; g.alpha = scale;
-  g.tri_out = causal; g.k_mode = 0;
+  g.tri_out = causal; g.k_mode = 0; g.off = causal ? (int)(L2 - L1) : 0;
   int rc = launch_gemm<DT>(g, Z, s);
   if (rc != MEGA_OK) return rc;
   // P = softmax(S) in place
@@ -624,7 +631,7 @@ int attn_fwd_impl(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64
   o.lda = L2; o.ldb = NH * H2; o.ldc = NH * H2; o.tb = 1;
   o.sa0 = NH * L1 * L2; o.sa1 = L1 * L2; o.sb0 = L2 * NH * H2; o.sb1 = H2;
   o.sc0 = L1 * NH * H2; o.sc1 = H2; o.nh = (int)NH; o.alpha = 1.f;
-  o.tri_out = 0; o.k_mode = causal ? 1 : 0;
+  o.tri_out = 0; o.k_mode = causal ? 1 : 0; o.off = causal ? (int)(L2 - L1) : 0;
   return launch_gemm<DT>(o, Z, s);
 }
 
@@ -643,7 +650,7 @@ int attn_bwd_impl(const uint16_t* dy, const uint16_t* q, const uint16_t* k, cons
   g.lda = NH * H2; g.ldb = NH * H2; g.ldc = L2;
   g.sa0 = L1 * NH * H2; g.sa1 = H2; g.sb0 = L2 * NH * H2; g.sb1 = H2;
   g.sc0 = NH * L1 * L2; g.sc1 = L1 * L2; g.nh = (int)NH; g.alpha = 1.f;
-  g.tri_out = causal; g.k_mode = 0;
+  g.tri_out = causal; g.k_mode = 0; g.off = causal ? (int)(L2 - L1) : 0;
   if ((rc = launch_gemm<DT>(g, Z, s)) != MEGA_OK) return rc;
   // dS = P o (dP - rowsum(P o dP)) in place
   if ((rc = launch_softmax<DT>(w, dp, Z, L1, L2, causal, s)) != MEGA_OK) return rc;
@@ -652,21 +659,21 @@ int attn_bwd_impl(const uint16_t* dy, const uint16_t* q, const uint16_t* k, cons
   a.A = dp; a.B = k; a.C = dq; a.M = (int)L1; a.N = (int)H1; a.K = (int)L2;
   a.lda = L2; a.ldb = NH * H1; a.ldc = NH * H1; a.tb = 1;
   a.sa0 = NH * L1 * L2; a.sa1 = L1 * L2; a.sb0 = L2 * NH * H1; a.sb1 = H1;
-  a.sc0 = L1 * NH * H1; a.sc1 = H1; a.nh = (int)NH; a.alpha = scale; a.k_mode = causal ? 1 : 0;
+  a.sc0 = L1 * NH * H1; a.sc1 = H1; a.nh = (int)NH; a.alpha = scale; a.k_mode = causal ? 1 : 0; a.off = causal ? (int)(L2 - L1) : 0;
   if ((rc = launch_gemm<DT>(a, Z, s)) != MEGA_OK) return rc;
   // dK = scale dS^T Q: dS[q][key] and Q[q][h] are both k-major (k = q)
   GemmParams b{};
   b.A = dp; b.B = q; b.C = dk; b.M = (int)L2; b.N = (int)H1; b.K = (int)L1;
   b.lda = L2; b.ldb = NH * H1; b.ldc = NH * H1; b.ta = 1; b.tb = 1;
   b.sa0 = NH * L1 * L2; b.sa1 = L1 * L2; b.sb0 = L1 * NH * H1; b.sb1 = H1;
-  b.sc0 = L2 * NH * H1; b.sc1 = H1; b.nh = (int)NH; b.alpha = scale; b.k_mode = causal ? 2 : 0;
+  b.sc0 = L2 * NH * H1; b.sc1 = H1; b.nh = (int)NH; b.alpha = scale; b.k_mode = causal ? 2 : 0; b.off = causal ? (int)(L2 - L1) : 0;
   if ((rc = launch_gemm<DT>(b, Z, s)) != MEGA_OK) return rc;
   // dV = P^T dY: P[q][key] and dY[q][c] are both k-major (k = q)
   GemmParams c{};
   c.A = w; c.B = dy; c.C = dv; c.M = (int)L2; c.N = (int)H2; c.K = (int)L1;
   c.lda = L2; c.ldb = NH * H2; c.ldc = NH * H2; c.ta = 1; c.tb = 1;
   c.sa0 = NH * L1 * L2; c.sa1 = L1 * L2; c.sb0 = L1 * NH * H2; c.sb1 = H2;
-  c.sc0 = L2 * NH * H2; c.sc1 = H2; c.nh = (int)NH; c.alpha = 1.f; c.k_mode = causal ? 2 : 0;
+  c.sc0 = L2 * NH * H2; c.sc1 = H2; c.nh = (int)NH; c.alpha = 1.f; c.k_mode = causal ? 2 : 0; c.off = causal ? (int)(L2 - L1) : 0;
   return launch_gemm<DT>(c, Z, s);
 }
 

@@ -2,8 +2,10 @@
 (megalodon/modules/moving_average_gated_attention.py:43-142): view the
 sequence as chunks, rotary on q/k, causal attention inside each chunk through
 the fused operator.  The rotary product is plain PyTorch (restating
-megalodon/modules/rotary_positional_embedding.py:53-77); the key/value cache
-branch (:92-101) belongs to cached inference and is not implemented."""
+megalodon/modules/rotary_positional_embedding.py:53-77).  With a key/value
+cache (:92-101) the cached keys and values of the unfinished chunk are put in
+front of the new ones: the fused operator then sees L2 > L1 (row r attends to
+keys 0 .. L2 - L1 + r), and a single new token attends to everything (:132-135)."""
 from typing import Optional, Tuple
 
 import torch
@@ -46,23 +48,35 @@ class _InnerAttention(nn.Module):
 
     def forward(self, xq: Tensor, xk: Tensor, xv: Tensor, mask: Optional[Tensor], freqs_cis: Optional[Tensor],
                 cache: Optional[Tuple[Tensor, Tensor, int]] = None):
-        if cache is not None:
-            raise NotImplementedError("key/value cache (cached inference) is not implemented")
         bs, slen, _ = xq.shape
         xq = xq.view(bs, slen, self.n_heads, self.z_head_dim)
         xk = xk.view(bs, slen, self.n_heads, self.z_head_dim)
         xv = xv.view(bs, slen, self.n_heads, self.v_head_dim)
 
-        # shorter than a chunk: rope before chunking
+        # shorter than a chunk: rope before the cached keys are put in front
         if slen <= self.chunk_size:
             xq, xk = apply_rotary_emb(xq, xk, freqs_cis=freqs_cis, backward=False)
+
+        new_cache = None
+        clen = slen
+        if cache is not None:
+            cache_k, cache_v, count = cache
+            xk = torch.cat([cache_k, xk], dim=1)
+            xv = torch.cat([cache_v, xv], dim=1)
+            clen = count + slen
+            # what is left of the last, unfinished chunk goes to the next call
+            new_count = clen % self.chunk_size
+            new_cache = (xk.detach()[:, clen - new_count:], xv.detach()[:, clen - new_count:], new_count)
 
         if self.chunk_size < slen:
             nc = slen // self.chunk_size
             xq = xq.reshape(bs * nc, self.chunk_size, self.n_heads, self.z_head_dim)
+        if self.chunk_size < clen:
+            nc = clen // self.chunk_size
             xk = xk.reshape(bs * nc, self.chunk_size, self.n_heads, self.z_head_dim)
             xv = xv.reshape(bs * nc, self.chunk_size, self.n_heads, self.v_head_dim)
-            # seq length > chunk: rope after the chunk split
+        # seq length > chunk: rope after the chunk split
+        if slen > self.chunk_size:
             xq, xk = apply_rotary_emb(xq, xk, freqs_cis=freqs_cis, backward=False)
 
         if self.efficient_attn is None:
@@ -74,10 +88,12 @@ class _InnerAttention(nn.Module):
             output = torch.matmul(scores, xv).transpose(1, 2).contiguous()
         else:
             assert mask is None
-            output = self.attn_fn(xq, xk, xv, 1.0, self.dropout, True, self.training)
+            use_causal_mask = not (slen == 1 and cache is not None)
+            output = self.attn_fn(xq.contiguous(), xk.contiguous(), xv.contiguous(), 1.0, self.dropout,
+                                  use_causal_mask, self.training)
 
         output = output.reshape(bs, slen, -1)
-        return output, None
+        return output, new_cache
 
     def extra_repr(self) -> str:
         return 'heads={}, z_head_dim={}, v_head_dim={}, chunk={}'.format(

@@ -3,8 +3,11 @@
 megalodon/model/mega.py:43-88): TimestepNorm -> CEMA -> RMSNorm -> z/q/k, v, r
 projections -> chunk attention -> gate -> wh1 + wh2 -> residual, then the
 normalised feed-forward network.  World size 1: the Column/RowParallelLinear
-layers are `nn.Linear`, the chunk-parallel send/recv and the key/value cache
-branches are not part of this path, dropout is 0."""
+layers are `nn.Linear`, the chunk-parallel send/recv branches are not part of
+this path, dropout is 0.  With `cache` = (attention cache, (count, mean, var)
+of TimestepNorm, EMA state) a sequence can be fed piece by piece (:283-297,
+:306-308, :345-346): every piece continues the running statistics, the EMA
+state and the unfinished attention chunk of the one before."""
 import math
 from typing import Optional
 
@@ -59,15 +62,23 @@ class MovingAverageGatedAttention(nn.Module):
         self.beta = Parameter(torch.zeros(2, self.z_head_dim * self.local_heads))
 
     def forward(self, x: Tensor, freqs_cis: Optional[Tensor] = None, mask: Optional[Tensor] = None, cache=None):
-        if cache is not None:
-            raise NotImplementedError("cached inference is not implemented")
         bsz, seq_len, _ = x.size()
         residual = x
 
+        if cache is not None:
+            cache_attn, cache_norm, hx = cache
+            prev_count, prev_mean, prev_var = cache_norm
+        else:
+            prev_count, prev_mean, prev_var = None, None, None
+            cache_attn, hx = None, None
+
         # B x L x D
-        out_tsn, prev_count, prev_mean, prev_var = self.timenorm(x, None, None, None)
+        out_tsn, prev_count, prev_mean, prev_var = self.timenorm(x, prev_count, prev_mean, prev_var)
         # B x D x L
-        out_cema, _ = self.cema(out_tsn.transpose(1, 2), None, compute_last_state=False)
+        out_cema, hx = self.cema(out_tsn.transpose(1, 2), hx, compute_last_state=cache_attn is not None)
+        if cache is not None:
+            cache_norm = (prev_count.detach(), prev_mean.detach(), prev_var.detach())
+            hx = None if hx is None else hx.detach()
         # B x L x D
         out_cema = out_cema.transpose(1, 2)
         mx = self.rmsnorm(out_cema)
@@ -84,13 +95,15 @@ class MovingAverageGatedAttention(nn.Module):
         v = F.silu(self.wv(out_tsn))
         r = F.silu(self.wr(mx))
 
-        attn, _ = self.inner_attention(q.contiguous(), k.contiguous(), v, mask, freqs_cis, None)
+        attn, cache_attn = self.inner_attention(q.contiguous(), k.contiguous(), v, mask, freqs_cis, cache_attn)
         attn = attn * r
 
         # B x L x E -> B x L x D
         h = self.wh1(mx) + self.wh2(attn)
         out = h + residual
-        return out, None
+        if cache is not None:
+            cache = (cache_attn, cache_norm, hx)
+        return out, cache
 
     def extra_repr(self) -> str:
         return 'edim={}, zdim={}, hdim={}, heads={}, chunk={}, eff_attn={}'.format(

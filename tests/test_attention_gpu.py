@@ -27,7 +27,7 @@ def _run(B, L1, L2, NH, H1, H2, causal, dtype, seed, scale=1.0):
     assert rel_err(y, wy) <= TOL
     if causal:
         # compare the probabilities on and below the diagonal (blocks right of the diagonal block are not written)
-        assert rel_err(torch.tril(w.float()), wp) <= TOL
+        assert rel_err(torch.tril(w.float(), diagonal=L2 - L1), wp) <= TOL
     else:
         assert rel_err(w, wp) <= TOL
     dq, dk, dv = ops.attention_bwd(dy.cuda(), q.cuda(), k.cuda(), v.cuda(), w, scale, causal)
@@ -46,6 +46,28 @@ def _run(B, L1, L2, NH, H1, H2, causal, dtype, seed, scale=1.0):
 ])
 def test_causal_fwd_bwd(B, L, NH, H1, H2, dtype):
     _run(B, L, L, NH, H1, H2, True, dtype, seed=L + H2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L1,L2,NH,H1,H2", [
+    (2, 212, 512, 2, 64, 128),    # cached keys in front: diagonal shifted by 300 columns
+    (1, 256, 768, 1, 256, 256),   # shift by two whole tiles
+    (1, 520, 1000, 2, 32, 64),    # three row tiles, shift not a multiple of the k slab
+    (2, 100, 131, 3, 32, 72),     # ragged, unaligned operand path
+    (1, 1, 40, 1, 16, 16),        # one new query, causal flag kept: sees all keys
+    (1, 1024, 1280, 1, 256, 512), # config-3 head dims, prefix of 256
+])
+def test_causal_with_key_value_prefix(B, L1, L2, NH, H1, H2, dtype):
+    """L2 > L1: row r attends to keys 0 .. L2 - L1 + r (bottom-right aligned
+    mask), forward values, probabilities and all three gradients."""
+    _run(B, L1, L2, NH, H1, H2, True, dtype, seed=L1 + L2)
+
+
+def test_causal_with_fewer_keys_than_queries_fails_loudly():
+    q = torch.zeros(1, 8, 1, 16, dtype=torch.bfloat16, device="cuda")
+    k = torch.zeros(1, 4, 1, 16, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="L2 >= L1"):
+        ops.attention_fwd(q, k, k.clone(), 1.0, 0.0, True)
 
 
 @pytest.mark.parametrize("B,L1,L2,NH,H1,H2", [(2, 1, 77, 2, 32, 64), (1, 130, 260, 1, 64, 64)])
@@ -105,9 +127,6 @@ def test_autograd_function_and_module():
 
 def test_unsupported_cases_fail_loudly():
     q = torch.zeros(1, 8, 1, 8, device="cuda", dtype=torch.bfloat16)
-    k = torch.zeros(1, 16, 1, 8, device="cuda", dtype=torch.bfloat16)
-    with pytest.raises(RuntimeError, match="not implemented"):
-        ops.attention_fwd(q, k, k, 1.0, 0.0, True)   # causal with a key prefix
     with pytest.raises(NotImplementedError):
         ops.attention_fwd(q, q, q, 1.0, 0.1, True)   # DropKey
     with pytest.raises(RuntimeError, match="bfloat16"):
