@@ -85,12 +85,19 @@ int mega_ema_weight_bwd(const float* dw, const float* p, const float* log_q,
  *   x, y (B, D, L) of `dtype` (MEGA_F32 / MEGA_BF16 / MEGA_F16);
  *   k (D, L) float32 in the TIME domain (the reference passes rfft(k); here
  *   the transform of k happens inside the kernel and nothing is saved).
- *   Arithmetic is float32 throughout; y is rounded once on store.
+ *   float32 rows: arithmetic is float32 throughout; y is rounded once on
+ *   store.  bfloat16 / float16 rows with 2048 < L, L % 8 == 0 and 16-byte
+ *   aligned x, k, y: the DFT stages run on the matrix cores (fp16 operands,
+ *   fp32 accumulation, fp16 between stages, rows pre-scaled by a power of
+ *   two), twiddles, the spectral product and all sums in float32; measured
+ *   error against a float64 convolution <= 4e-3 of the largest output
+ *   (the bfloat16 rounding of y alone is 2e-3).  Other 16-bit rows take the
+ *   float32 path.
  *   L <= mega_fftconv_max_length() (32768); longer rows return
  *   MEGA_ERR_UNSUPPORTED.
- *   The first call for a transform size on a device allocates the twiddle
- *   tables and a per-workgroup scratch (kept until process exit) and
- *   synchronises `stream` once.
+ *   The float32 path's first call for a transform size on a device allocates
+ *   the twiddle tables and a per-workgroup scratch (kept until process exit)
+ *   and synchronises `stream` once; the matrix-core path allocates nothing.
  * ---------------------------------------------------------------------- */
 int mega_fftconv_max_length(void);
 int mega_fftconv_fwd(const void* x, int dtype, const float* k, int64_t B,
@@ -175,12 +182,14 @@ int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, const void* 
  *   q (B, L1, NH, H1), k (B, L2, NH, H1), v (B, L2, NH, H2), y (B, L1, NH, H2),
  *   w (B, NH, L1, L2), all of `dtype` (MEGA_BF16 or MEGA_F16), contiguous; B
  *   counts chunks (the module views (batch, L) as (batch*L/chunk, chunk)).
- *   S = scale * q k^T rounded to `dtype`; row r keeps columns 0..r when
- *   `causal` (L1 == L2 required), all columns otherwise; P = softmax in fp32,
- *   stored in `dtype` into w; y = P v.  With `causal`, w is written only up to
- *   the end of the 256-column block holding the diagonal of each row (zeros
- *   above the diagonal inside that block); the blocks to the right are never
- *   read by the backward and are left untouched.  DropKey dropout is not
+ *   S = scale * q k^T rounded to `dtype`; with `causal` row r keeps columns
+ *   0 .. L2 - L1 + r (L2 >= L1 required: cached keys / values in front of the
+ *   chunk, softmax.cuh:99-100), all columns otherwise; P = softmax in fp32,
+ *   stored in `dtype` into w; y = P v.  With `causal` and L1 == L2, w is
+ *   written only up to the end of the 256-column block holding the diagonal of
+ *   each row (zeros above the diagonal inside that block); the blocks to the
+ *   right are never read by the backward and are left untouched.  With
+ *   L2 > L1 every row of w is written to its end.  DropKey dropout is not
  *   implemented (dropout must be 0).
  *   `workspace`: mega_attention_workspace_bytes(B, L1, L2, NH, H1, H2, 0) bytes.
  * ---------------------------------------------------------------------- */
