@@ -22,6 +22,8 @@
 // diagonal by L2 - L1 columns in every one of these rules.
 #include "common.hpp"
 
+#include <algorithm>
+
 namespace mega {
 namespace {
 
@@ -84,6 +86,11 @@ struct GemmParams {
   int k_mode;   // 0: all k; 1: m = queries, k = keys: k < (mt+1)*256 + off, rounded up to a slab;
                 // 2: m = keys, k = queries: k >= mt*256 - off, rounded down to a slab
   int off;
+  // persistent schedule (filled in by the launcher): work items of equal weight,
+  // walked by gridDim.x workgroups
+  int mt_count, nt_count;  // tiles along m and n
+  int per_batch;           // work items per batch index
+  int items;               // per_batch * batch
   int ta, tb;   // operand is k-major: element (m, k) at [k * ld + m]
 };
 
@@ -134,33 +141,69 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
   extern __shared__ __align__(16) uint16_t smem[];
   // main loop: [buf][A|B] operand slabs; epilogue: [wave][128][kEpiPitch]
   constexpr int kOperand = kOperandElems;
-  // Workgroups are handed to the 8 XCDs round-robin by linear index, and each
-  // XCD has its own L2.  Renumber so that one XCD runs a contiguous run of
-  // tiles (n fastest, then m, then batch): neighbours that share an A row
-  // block or the B matrix of a head then hit the same L2.
-  const unsigned total = gridDim.x * gridDim.y * gridDim.z;
-  const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-  const unsigned xcd = lin % kXcds, slot = lin / kXcds;
-  const unsigned id = xcd * (total / kXcds) + min(xcd, total % kXcds) + slot;
-  // with a triangular k range or output the work of a tile grows with mt:
-  // start the heavy rows first so the light ones fill the tail
-  const int nt = id % gridDim.x;
-  const int mt_raw = (id / gridDim.x) % gridDim.y;
-  const int mt = (p.tri_out || p.k_mode) ? static_cast<int>(gridDim.y) - 1 - mt_raw : mt_raw;
-  const int zz = id / (gridDim.x * gridDim.y);
-  if (p.tri_out && nt * kTile > mt * kTile + (kTile - 1) + p.off) return;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // Persistent workgroups (one per CU) walk a list of work items of equal
+  // weight, so nothing is launched for skipped tiles and no CU ends up with
+  // the long tail of a triangular problem:
+  //   tri_out: one item per tile on or below the (shifted) diagonal;
+  //   k_mode:  one item = the tile pair (mt, mt_count - 1 - mt) of a column
+  //            block, whose k ranges add up to the same length for every pair;
+  //   else:    one item per tile.
+  // Items are numbered n fastest, then m, then batch.  Workgroups are handed
+  // to the 8 XCDs round-robin by index and each XCD has its own L2: an XCD
+  // takes a contiguous eighth of the list and its workgroups interleave inside
+  // it, so neighbours that share an A row block or the B matrix of a head hit
+  // the same L2 at the same time.
+  const int G = static_cast<int>(gridDim.x), lin = static_cast<int>(blockIdx.x);
+  int it_lo, it_hi, it_step;
+  if (G % kXcds == 0) {
+    const int xcd = lin % kXcds;
+    it_lo = static_cast<int>(static_cast<int64_t>(p.items) * xcd / kXcds) + lin / kXcds;
+    it_hi = static_cast<int>(static_cast<int64_t>(p.items) * (xcd + 1) / kXcds);
+    it_step = G / kXcds;
+  } else {
+    it_lo = lin;
+    it_hi = p.items;
+    it_step = G;
+  }
+  for (int item = it_lo; item < it_hi; item += it_step) {
+  const int zz = item / p.per_batch;
+  const int rem = item % p.per_batch;
+  int nt, mt_first, mt_second = -1;
+  if (p.tri_out) {
+    // row mt holds the tiles nt <= (mt * 256 + 255 + off) / 256
+    int t = rem, m = 0;
+    while (true) {
+      const int cnt = min(p.nt_count, (m * kTile + (kTile - 1) + p.off) / kTile + 1);
+      if (t < cnt) break;
+      t -= cnt;
+      ++m;
+    }
+    mt_first = m;
+    nt = t;
+  } else if (p.k_mode) {
+    nt = rem % p.nt_count;
+    const int pr = rem / p.nt_count;
+    mt_first = p.mt_count - 1 - pr;
+    if (mt_first != pr) mt_second = pr;
+  } else {
+    nt = rem % p.nt_count;
+    mt_first = rem / p.nt_count;
+  }
   const int z0 = zz / p.nh, z1 = zz % p.nh;
   const uint16_t* A = p.A + z0 * p.sa0 + z1 * p.sa1;
   const uint16_t* B = p.B + z0 * p.sb0 + z1 * p.sb1;
   uint16_t* C = p.C + z0 * p.sc0 + z1 * p.sc1;
+  for (int half = 0; half < 2; ++half) {
+  const int mt = half == 0 ? mt_first : mt_second;
+  if (mt < 0) break;
   const int m0 = mt * kTile, n0 = nt * kTile;
   int kb = 0, ke = p.K;
   if (p.k_mode == 1) ke = min(p.K, ((mt + 1) * kTile + p.off + kSlab - 1) / kSlab * kSlab);
   if (p.k_mode == 2) kb = min(p.K, max(0, mt * kTile - p.off) / kSlab * kSlab);
   const int nslab = (ke - kb + kSlab - 1) / kSlab;
-
-  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const int wm = wave >> 1, wn = wave & 1;
 
   floatx16 acc[4][4];
 #pragma unroll
@@ -350,6 +393,11 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
       }
     }
   }
+  // the staging regions overlap the operand buffers of every wave: all reads
+  // of this tile's epilogue retire before the next tile's first slab lands
+  lds_barrier();
+  }  // tile of the pair
+  }  // work item
 }
 
 // ---- causal softmax over rows (in place), one wavefront per row ---------------
@@ -564,16 +612,40 @@ int launch_gemm_t(const GemmParams& p, int batch, hipStream_t s) {
   const bool fast_b = a16(p.B) && p.ldb % 8 == 0 && p.sb0 % 8 == 0 && p.sb1 % 8 == 0 &&
                       (TB ? (p.N % 8 == 0 && p.N >= 8 && p.K * p.ldb < lim) : p.N * p.ldb < lim);
   const bool fast = fast_a && fast_b && p.K % kSlab == 0 && p.K >= kSlab;
-  const dim3 grid((p.N + kTile - 1) / kTile, (p.M + kTile - 1) / kTile, batch);
+  GemmParams q = p;
+  q.mt_count = (p.M + kTile - 1) / kTile;
+  q.nt_count = (p.N + kTile - 1) / kTile;
+  int64_t per_batch;
+  if (p.tri_out) {
+    per_batch = 0;
+    for (int m = 0; m < q.mt_count; ++m)
+      per_batch += std::min<int64_t>(q.nt_count, (static_cast<int64_t>(m) * kTile + (kTile - 1) + p.off) / kTile + 1);
+  } else if (p.k_mode) {
+    per_batch = static_cast<int64_t>(q.nt_count) * ((q.mt_count + 1) / 2);
+  } else {
+    per_batch = static_cast<int64_t>(q.nt_count) * q.mt_count;
+  }
+  const int64_t items = per_batch * batch;
+  MEGA_CHECK_ARG(items <= 0x7fffffff, "attention: too many tiles");
+  q.per_batch = static_cast<int>(per_batch);
+  q.items = static_cast<int>(items);
+  int dev = 0, cus = 0;
+  MEGA_CHECK_HIP(hipGetDevice(&dev));
+  MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  // one workgroup per CU (its LDS and registers fill one); a multiple of the
+  // XCD count whenever there are that many items
+  int64_t g = std::min<int64_t>(items, cus);
+  if (g >= kXcds) g -= g % kXcds;
+  const dim3 grid(static_cast<unsigned>(g));
   const size_t lds = kGemmLds;
   if (fast) {
     MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, true, TA, TB>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    gemm_kernel<DT, true, TA, TB><<<grid, kThreads, lds, s>>>(p);
+    gemm_kernel<DT, true, TA, TB><<<grid, kThreads, lds, s>>>(q);
   } else {
     MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, false, TA, TB>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    gemm_kernel<DT, false, TA, TB><<<grid, kThreads, lds, s>>>(p);
+    gemm_kernel<DT, false, TA, TB><<<grid, kThreads, lds, s>>>(q);
   }
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
