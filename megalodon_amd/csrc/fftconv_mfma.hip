@@ -673,13 +673,40 @@ __device__ __forceinline__ void write_quad(uint16_t* p, const float* v) {
   *reinterpret_cast<uint2*>(p) = make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
 }
 
-// E = (Z(k) + conj Z(m)) / 2,  O = (Z(k) - conj Z(m)) / (2i)
+// Twice the even / odd spectra of a real signal packed as z = even + i odd:
+// 2E = Z(k) + conj Z(m), 2O = (Z(k) - conj Z(m)) / i, m the mirror bin.  The
+// factors of two of both operands are taken out again by the final scale.
 __device__ __forceinline__ void untangle(float zkr, float zki, float zmr, float zmi, float& er,
                                          float& ei, float& orr, float& oi) {
-  er = 0.5f * (zkr + zmr);
-  ei = 0.5f * (zki - zmi);
-  orr = 0.5f * (zki + zmi);
-  oi = 0.5f * (zmr - zkr);
+  er = zkr + zmr;
+  ei = zki - zmi;
+  orr = zki + zmi;
+  oi = zmr - zkr;
+}
+// The same on a quad of bins (elements 0..3 of the re and im runs) and the
+// reversed quad of mirror bins, in packed fp16: element e pairs with mirror
+// element 3 - e.  Results: index 0 holds elements (0, 1), index 1 elements (2, 3).
+struct Quad2 {
+  half2v er[2], ei[2], orr[2], oi[2];
+};
+__device__ __forceinline__ half2v as_h2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
+__device__ __forceinline__ half2v swap_h2(half2v v) { return __builtin_shufflevector(v, v, 1, 0); }
+__device__ __forceinline__ Quad2 untangle_quads(uint2 kr, uint2 ki, uint2 mr, uint2 mi) {
+  const half2v mr0 = swap_h2(as_h2(mr.y)), mr1 = swap_h2(as_h2(mr.x));  // mirror of elements (0,1), (2,3)
+  const half2v mi0 = swap_h2(as_h2(mi.y)), mi1 = swap_h2(as_h2(mi.x));
+  Quad2 q;
+  q.er[0] = as_h2(kr.x) + mr0;
+  q.er[1] = as_h2(kr.y) + mr1;
+  q.ei[0] = as_h2(ki.x) - mi0;
+  q.ei[1] = as_h2(ki.y) - mi1;
+  q.orr[0] = as_h2(ki.x) + mi0;
+  q.orr[1] = as_h2(ki.y) + mi1;
+  q.oi[0] = mr0 - as_h2(kr.x);
+  q.oi[1] = mr1 - as_h2(kr.y);
+  return q;
+}
+__device__ __forceinline__ uint2 read_quad_raw(const uint16_t* p) {
+  return *reinterpret_cast<const uint2*>(p);
 }
 // Zy(k) = Ey + i Oy and Zy(m) = conj Ey + i conj Oy with
 // Ey = Ea Eb + W_N^k Oa Ob, Oy = Ea Ob + Oa Eb;  W_N^k = wc - i ws
@@ -698,8 +725,10 @@ __device__ __forceinline__ void bin_product(float ar, float ai, float pr, float 
 }
 
 struct Spectrum {
-  uint32_t e[8][4], o[8][4];  // E(k), O(k) of the parked operand per task and element, fp16 (re, im)
-  uint32_t e0, o0;            // row (0, 0), lane = k3 (threads 0..31)
+  // 2E(k), 2O(k) of the parked operand per task, packed fp16:
+  // e = (re of elements 0,1), (re 2,3), (im 0,1), (im 2,3); o likewise
+  uint32_t e[8][4], o[8][4];
+  uint32_t e0, o0;  // row (0, 0), lane = k3 (threads 0..31), fp16 (re, im)
 };
 
 template <int LOGA>
@@ -710,17 +739,14 @@ __device__ __forceinline__ void capture_spectrum(const uint16_t* pre, Spectrum& 
   for (int i = 0; i < 8; ++i) {
     tid = opaque(tid) & (kThreads - 1);
     const RowPair rp = row_pair<LOGA>(tid + kThreads * i);
-    float kr[4], ki[4], mr[4], mi[4];
-    read_quad(pre + rp.ok, kr);
-    read_quad(pim + rp.ok, ki);
-    read_quad(pre + rp.om, mr);
-    read_quad(pim + rp.om, mi);
+    const Quad2 q = untangle_quads(read_quad_raw(pre + rp.ok), read_quad_raw(pim + rp.ok),
+                                   read_quad_raw(pre + rp.om), read_quad_raw(pim + rp.om));
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float er, ei, orr, oi;
-      untangle(kr[e], ki[e], mr[3 - e], mi[3 - e], er, ei, orr, oi);
-      sp.e[i][e] = pack_h2(er, ei);
-      sp.o[i][e] = pack_h2(orr, oi);
+    for (int h = 0; h < 2; ++h) {
+      sp.e[i][h] = __builtin_bit_cast(uint32_t, q.er[h]);
+      sp.e[i][2 + h] = __builtin_bit_cast(uint32_t, q.ei[h]);
+      sp.o[i][h] = __builtin_bit_cast(uint32_t, q.orr[h]);
+      sp.o[i][2 + h] = __builtin_bit_cast(uint32_t, q.oi[h]);
     }
   }
   sp.e0 = sp.o0 = 0u;
@@ -744,11 +770,8 @@ __device__ __forceinline__ void pointwise(uint16_t* pre, const Spectrum& sp, int
   for (int i = 0; i < 8; ++i) {
     tid = opaque(tid) & (kThreads - 1);
     const RowPair rp = row_pair<LOGA>(tid + kThreads * i);
-    float kr[4], ki[4], mr[4], mi[4];
-    read_quad(pre + rp.ok, kr);
-    read_quad(pim + rp.ok, ki);
-    read_quad(pre + rp.om, mr);
-    read_quad(pim + rp.om, mi);
+    const Quad2 qa = untangle_quads(read_quad_raw(pre + rp.ok), read_quad_raw(pim + rp.ok),
+                                    read_quad_raw(pre + rp.om), read_quad_raw(pim + rp.om));
     float w0c, w0s;
     cis(rp.k0, 1.f / NP, w0c, w0s);
     // W_N'^(k0 + 32 A e) = W_N'^k0 W_32^e
@@ -757,10 +780,14 @@ __device__ __forceinline__ void pointwise(uint16_t* pre, const Spectrum& sp, int
     float okr[4], oki[4], omr[4], omi[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      float ar, ai, pr, pi, br, bi, qr, qi, wc, ws;
-      untangle(kr[e], ki[e], mr[3 - e], mi[3 - e], ar, ai, pr, pi);
-      unpack_h2(sp.e[i][e], br, bi);
-      unpack_h2(sp.o[i][e], qr, qi);
+      const int hp = e >> 1, hh = e & 1;  // which packed pair, which half of it
+      const float ar = static_cast<float>(qa.er[hp][hh]), ai = static_cast<float>(qa.ei[hp][hh]);
+      const float pr = static_cast<float>(qa.orr[hp][hh]), pi = static_cast<float>(qa.oi[hp][hh]);
+      const float br = static_cast<float>(as_h2(sp.e[i][hp])[hh]);
+      const float bi = static_cast<float>(as_h2(sp.e[i][2 + hp])[hh]);
+      const float qr = static_cast<float>(as_h2(sp.o[i][hp])[hh]);
+      const float qi = static_cast<float>(as_h2(sp.o[i][2 + hp])[hh]);
+      float wc, ws;
       cmul(w0c, w0s, c32[e], s32[e], wc, ws);
       bin_product(ar, ai, pr, pi, br, bi, qr, qi, wc, ws, okr[e], oki[e], omr[3 - e], omi[3 - e]);
     }
@@ -790,11 +817,12 @@ __device__ __forceinline__ void pointwise(uint16_t* pre, const Spectrum& sp, int
   }
 }
 
-// sqrt(N') / (the two operands' row scales): undoes the three unitary transforms
+// sqrt(N') / 4 / (the two operands' row scales): undoes the three unitary transforms
 template <int LOGA>
 __device__ __forceinline__ void final_scales(const float* sa, const float* sb, float* out) {
-  constexpr float root = LOGA == 5 ? 181.01933598375618f
-                                   : (LOGA == 4 ? 128.f : (LOGA == 3 ? 90.509667991878086f : 64.f));
+  // sqrt(N') / 4: the spectra of both operands are carried at twice their size
+  constexpr float root = 0.25f * (LOGA == 5 ? 181.01933598375618f
+                                            : (LOGA == 4 ? 128.f : (LOGA == 3 ? 90.509667991878086f : 64.f)));
 #pragma unroll
   for (int i = 0; i < Geo<LOGA>::R; ++i) out[i] = root / (sa[i] * sb[i]);
 }
