@@ -211,6 +211,27 @@ int mega_attention_bwd(const void* dy, const void* q, const void* k, const void*
                        int64_t NH, int64_t H1, int64_t H2, double scale, int causal,
                        void* dq, void* dk, void* dv, void* workspace, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Standalone softmax of attention scores, in place.
+ *
+ * Replaces attention_softmax_fwd(x, dropout=0, use_causal_mask) -> y
+ *   reference: megalodon/csrc/ops/attention_softmax_kernel.cu:22-66,96-108,
+ *              megalodon/csrc/softmax.cuh:86-131, binding attention_softmax.cc:6-10,20-22.
+ *   x: Z matrices (L1, L2) of `dtype` (MEGA_BF16 or MEGA_F16), contiguous,
+ *   overwritten by y = softmax over the last axis in float32; with `causal`
+ *   row r keeps columns 0 .. L2 - L1 + r (L2 >= L1) and the rest of the row
+ *   becomes 0.  The caller copies x first if it must survive (the reference
+ *   returns a new tensor).  DropKey dropout is not implemented.
+ * Replaces attention_softmax_bwd(y_grad, y, use_causal_mask) -> x_grad
+ *   reference: attention_softmax_kernel.cu:68-94,110-123, softmax.cuh:198-234,
+ *              binding attention_softmax.cc:12-18.
+ *   dy is overwritten by dx = y o (dy - rowsum(y o dy)) (0 where masked).
+ * ---------------------------------------------------------------------- */
+int mega_attention_softmax_fwd(void* x, int dtype, int64_t Z, int64_t L1, int64_t L2,
+                               int causal, void* stream);
+int mega_attention_softmax_bwd(const void* y, void* dy, int dtype, int64_t Z, int64_t L1,
+                               int64_t L2, int causal, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

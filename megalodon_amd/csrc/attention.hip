@@ -403,19 +403,20 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
 // ---- causal softmax over rows (in place), one wavefront per row ---------------
 // `coff` < 0: every row keeps all L2 columns.  `coff` = L2 - L1 >= 0 (causal,
 // bottom-right aligned, softmax.cuh:99-100): row r keeps columns [0, n) with
-// n = r + 1 + coff.  The rest of the row is set to 0 -- with coff = 0 only up
-// to the end of its 256-column tile, which is all the later products read.
+// n = r + 1 + coff.  The rest of the row is set to 0 -- with coff = 0 and
+// `zfull` = 0 only up to the end of its 256-column tile, which is all the
+// products of the fused attention read.
 // softmax.cuh:86-131.
 template <int DT>
 __global__ __launch_bounds__(kThreads) void softmax_fwd_kernel(uint16_t* w, int L1, int L2,
-                                                              int coff) {
+                                                              int coff, int zfull) {
   // grid.y carries the batch*heads index; grid.x covers the L1 rows
   const int lane = threadIdx.x % kWave;
   const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   if (r >= L1) return;
   uint16_t* x = w + (static_cast<int64_t>(blockIdx.y) * L1 + r) * L2;
   const int n = coff >= 0 ? min(r + 1 + coff, L2) : L2;
-  const int nz = coff == 0 ? min(L2, (r / kTile + 1) * kTile) : L2;
+  const int nz = (coff == 0 && !zfull) ? min(L2, (r / kTile + 1) * kTile) : L2;
   float m = -INFINITY;
   for (int j = lane; j < n; j += kWave) m = fmaxf(m, Elem<DT>::load(x + j));
   m = wave_max(m);
@@ -462,13 +463,13 @@ __device__ __forceinline__ uint4 pack8(const float* v) {
 // aligned base and L2 <= 64 * 8 * NCH; one read and one write of the row.
 template <int DT, int NCH>
 __global__ __launch_bounds__(kThreads) void softmax_fwd_vec_kernel(uint16_t* w, int L1, int L2,
-                                                                  int coff) {
+                                                                  int coff, int zfull) {
   const int lane = threadIdx.x % kWave;
   const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   if (r >= L1) return;
   uint16_t* x = w + (static_cast<int64_t>(blockIdx.y) * L1 + r) * L2;
   const int n = coff >= 0 ? min(r + 1 + coff, L2) : L2;
-  const int nz = coff == 0 ? min(L2, (r / kTile + 1) * kTile) : L2;
+  const int nz = (coff == 0 && !zfull) ? min(L2, (r / kTile + 1) * kTile) : L2;
   float v[NCH][8];
   float m = -INFINITY;
 #pragma unroll
@@ -511,7 +512,7 @@ __global__ __launch_bounds__(kThreads) void softmax_fwd_vec_kernel(uint16_t* w, 
 // dS = P o (dP - sum_j P_j dP_j), written over dP.  softmax.cuh:198-234.
 template <int DT>
 __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const uint16_t* w, uint16_t* dw,
-                                                              int L1, int L2, int coff) {
+                                                              int L1, int L2, int coff, int zfull) {
   const int lane = threadIdx.x % kWave;
   const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   if (r >= L1) return;
@@ -519,7 +520,7 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const uint16_t* w
   const uint16_t* pw = w + o;
   uint16_t* pd = dw + o;
   const int n = coff >= 0 ? min(r + 1 + coff, L2) : L2;
-  const int nz = coff == 0 ? min(L2, (r / kTile + 1) * kTile) : L2;
+  const int nz = (coff == 0 && !zfull) ? min(L2, (r / kTile + 1) * kTile) : L2;
   float s = 0.f;
   for (int j = lane; j < n; j += kWave) s += Elem<DT>::load(pw + j) * Elem<DT>::load(pd + j);
   s = wave_sum(s);
@@ -531,7 +532,7 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const uint16_t* w
 
 template <int DT, int NCH>
 __global__ __launch_bounds__(kThreads) void softmax_bwd_vec_kernel(const uint16_t* w, uint16_t* dw,
-                                                                  int L1, int L2, int coff) {
+                                                                  int L1, int L2, int coff, int zfull) {
   const int lane = threadIdx.x % kWave;
   const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   if (r >= L1) return;
@@ -539,7 +540,7 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_vec_kernel(const uint16_
   const uint16_t* pw = w + o;
   uint16_t* pd = dw + o;
   const int n = coff >= 0 ? min(r + 1 + coff, L2) : L2;
-  const int nz = coff == 0 ? min(L2, (r / kTile + 1) * kTile) : L2;
+  const int nz = (coff == 0 && !zfull) ? min(L2, (r / kTile + 1) * kTile) : L2;
   float pv[NCH][8], dv[NCH][8];
   float s = 0.f;
 #pragma unroll
@@ -572,7 +573,7 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_vec_kernel(const uint16_
 
 template <int DT>
 int launch_softmax(const uint16_t* p, uint16_t* x, int64_t Z, int64_t L1, int64_t L2, int causal,
-                   hipStream_t s) {
+                   hipStream_t s, int zfull = 0) {
   const int coff = causal ? static_cast<int>(L2 - L1) : -1;
   // p == nullptr: forward over x in place; else backward with probabilities p
   if (Z == 0 || L1 == 0 || L2 == 0) return MEGA_OK;
@@ -581,9 +582,9 @@ int launch_softmax(const uint16_t* p, uint16_t* x, int64_t Z, int64_t L1, int64_
                    reinterpret_cast<uintptr_t>(p) % 16 == 0;
 #define MEGA_SOFTMAX(NCH)                                                                   \
   if (p == nullptr)                                                                         \
-    softmax_fwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff); \
+    softmax_fwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff, zfull); \
   else                                                                                      \
-    softmax_bwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, coff);
+    softmax_bwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, coff, zfull);
   if (vec && L2 <= 512) {
     MEGA_SOFTMAX(1)
   } else if (vec && L2 <= 1024) {
@@ -593,9 +594,9 @@ int launch_softmax(const uint16_t* p, uint16_t* x, int64_t Z, int64_t L1, int64_
   } else if (vec && L2 <= 4096) {
     MEGA_SOFTMAX(8)
   } else if (p == nullptr) {
-    softmax_fwd_kernel<DT><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff);
+    softmax_fwd_kernel<DT><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff, zfull);
   } else {
-    softmax_bwd_kernel<DT><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, coff);
+    softmax_bwd_kernel<DT><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, coff, zfull);
   }
 #undef MEGA_SOFTMAX
   MEGA_CHECK_LAUNCH();
@@ -797,4 +798,41 @@ extern "C" int mega_attention_bwd(const void* dy, const void* q, const void* k, 
                                     (float)scale, causal, m(dq), m(dk), m(dv), m(workspace), s);
   return attn_bwd_impl<MEGA_F16>(u(dy), u(q), u(k), u(v), u(w), B, L1, L2, NH, H1, H2,
                                  (float)scale, causal, m(dq), m(dk), m(dv), m(workspace), s);
+}
+
+// ---- standalone causal softmax ---------------------------------------------------
+static int check_softmax(const char* who, int dtype, int64_t Z, int64_t L1, int64_t L2, int causal) {
+  if (dtype != MEGA_BF16 && dtype != MEGA_F16)
+    return set_error(MEGA_ERR_UNSUPPORTED, "%s: only bfloat16 / float16 tensors are supported", who);
+  MEGA_CHECK_ARG(Z >= 0 && L1 >= 0 && L2 >= 0, "%s: bad sizes", who);
+  MEGA_CHECK_ARG(Z <= 65535, "%s: more than 65535 matrices", who);
+  MEGA_CHECK_ARG(L1 <= (1 << 24) && L2 <= (1 << 24), "%s: rows too long", who);
+  MEGA_CHECK_ARG(!causal || L2 >= L1, "%s: causal softmax needs L2 >= L1", who);
+  return MEGA_OK;
+}
+
+extern "C" int mega_attention_softmax_fwd(void* x, int dtype, int64_t Z, int64_t L1, int64_t L2,
+                                          int causal, void* stream) {
+  int rc = check_softmax("mega_attention_softmax_fwd", dtype, Z, L1, L2, causal);
+  if (rc != MEGA_OK) return rc;
+  MEGA_CHECK_ARG(x != nullptr || Z * L1 * L2 == 0, "mega_attention_softmax_fwd: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MEGA_BF16)
+    return launch_softmax<MEGA_BF16>(nullptr, static_cast<uint16_t*>(x), Z, L1, L2, causal, s, 1);
+  return launch_softmax<MEGA_F16>(nullptr, static_cast<uint16_t*>(x), Z, L1, L2, causal, s, 1);
+}
+
+extern "C" int mega_attention_softmax_bwd(const void* y, void* dy, int dtype, int64_t Z, int64_t L1,
+                                          int64_t L2, int causal, void* stream) {
+  int rc = check_softmax("mega_attention_softmax_bwd", dtype, Z, L1, L2, causal);
+  if (rc != MEGA_OK) return rc;
+  MEGA_CHECK_ARG((y != nullptr && dy != nullptr) || Z * L1 * L2 == 0,
+                 "mega_attention_softmax_bwd: null pointer");
+  if (Z * L1 * L2 == 0) return MEGA_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MEGA_BF16)
+    return launch_softmax<MEGA_BF16>(static_cast<const uint16_t*>(y), static_cast<uint16_t*>(dy), Z, L1,
+                                     L2, causal, s, 1);
+  return launch_softmax<MEGA_F16>(static_cast<const uint16_t*>(y), static_cast<uint16_t*>(dy), Z, L1, L2,
+                                  causal, s, 1);
 }

@@ -473,3 +473,66 @@ def attention_bwd(y_grad: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: tor
                   _lib.i64(H1), _lib.i64(H2), _lib.f64(scale), _lib.i32(1 if use_causal_mask else 0),
                   _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(ws), _lib.stream_ptr(dev))
     return dq, dk, dv
+
+
+def _softmax_dims(x: torch.Tensor):
+    if x.dim() < 2:
+        raise RuntimeError("attention_softmax: x needs at least two dimensions")
+    L1, L2 = x.shape[-2], x.shape[-1]
+    Z = x.numel() // max(1, L1 * L2)
+    return Z, L1, L2
+
+
+def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool) -> torch.Tensor:
+    """y = softmax(x) over the last axis (float32 inside), rows masked causally
+    (bottom-right aligned) when asked; x (..., L1, L2) bfloat16 / float16
+    (attention_softmax_kernel.cu:96-108)."""
+    dev = _require_cuda(x)
+    if dropout != 0.0:
+        raise NotImplementedError("DropKey dropout is not implemented (dropout must be 0)")
+    Z, L1, L2 = _softmax_dims(x)
+    y = x.contiguous().clone()
+    with torch.cuda.device(dev):
+        _lib.call("mega_attention_softmax_fwd", _lib.ptr(y), _lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(Z),
+                  _lib.i64(L1), _lib.i64(L2), _lib.i32(1 if use_causal_mask else 0), _lib.stream_ptr(dev))
+    return y
+
+
+def attention_softmax_bwd(y_grad: torch.Tensor, y: torch.Tensor, use_causal_mask: bool) -> torch.Tensor:
+    """x_grad = y o (y_grad - rowsum(y o y_grad)) (attention_softmax_kernel.cu:110-123)."""
+    dev = _require_cuda(y_grad, y)
+    if y_grad.shape != y.shape or y_grad.dtype != y.dtype:
+        raise RuntimeError("attention_softmax_bwd: y_grad and y must have the same shape and dtype")
+    Z, L1, L2 = _softmax_dims(y)
+    yc = y.contiguous()
+    dx = y_grad.contiguous().clone()
+    with torch.cuda.device(dev):
+        _lib.call("mega_attention_softmax_bwd", _lib.ptr(yc), _lib.ptr(dx), _lib.i32(_lib.dtype_code(y.dtype)),
+                  _lib.i64(Z), _lib.i64(L1), _lib.i64(L2), _lib.i32(1 if use_causal_mask else 0),
+                  _lib.stream_ptr(dev))
+    return dx
+
+
+def timestep_norm_fwd(x: torch.Tensor, prev_count: torch.Tensor, prev_mean: torch.Tensor, prev_var: torch.Tensor,
+                      gamma: torch.Tensor, beta: torch.Tensor, padding_mask: Optional[torch.Tensor], eps: float):
+    """The non-group operator (megalodon/csrc/ops/timestep_norm.cc:23-105,
+    binding :700-701): every feature keeps its own running mean / variance,
+    i.e. the group operator with one feature per group.  Returns (y, count,
+    mean, var, cummean, cumrstd) with the saved statistics in x's dtype, as the
+    reference does for this variant (:53-54).  The module path never calls it
+    (modules/timestep_norm.py:123-125 always takes the group operator), so it
+    runs on the general one-wave-per-chain kernel."""
+    H = x.shape[-1]
+    y, count, mean, var, cummean, cumrstd = group_timestep_norm_fwd(
+        x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask, H, eps)
+    return y, count, mean, var, cummean.to(x.dtype), cumrstd.to(x.dtype)
+
+
+def timestep_norm_bwd(y_grad: torch.Tensor, mean_grad: torch.Tensor, var_grad: torch.Tensor, x: torch.Tensor,
+                      prev_mean: torch.Tensor, count: torch.Tensor, cummean: torch.Tensor, cumrstd: torch.Tensor,
+                      gamma: torch.Tensor, padding_mask: Optional[torch.Tensor]):
+    """(dx, dprev_mean, dprev_var, dgamma, dbeta) of the non-group operator
+    (timestep_norm.cc:107-216, binding :702-703)."""
+    H = x.shape[-1]
+    return group_timestep_norm_bwd(y_grad, mean_grad, var_grad, x, prev_mean, count, cummean.float(),
+                                   cumrstd.float(), gamma, padding_mask, H)

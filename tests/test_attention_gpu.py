@@ -131,3 +131,35 @@ def test_unsupported_cases_fail_loudly():
         ops.attention_fwd(q, q, q, 1.0, 0.1, True)   # DropKey
     with pytest.raises(RuntimeError, match="bfloat16"):
         ops.attention_fwd(q.float(), q.float(), q.float(), 1.0, 0.0, True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,causal", [
+    ((2, 3, 300, 300), True), ((1, 2, 100, 260), True), ((4, 64, 512), False), ((1, 1, 1, 40), True),
+    ((2, 1, 50, 4100), False),   # rows longer than the register-resident kernels take
+])
+def test_standalone_softmax(shape, causal, dtype):
+    """attention_softmax_fwd/bwd against float64: y = softmax over the last
+    axis with the bottom-right aligned causal mask, zeros above it;
+    dx = y o (dy - sum(y o dy))."""
+    from megalodon_amd.fused_ops import attention_softmax
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (2.0 * torch.randn(*shape, generator=g)).to(dtype)
+    dy = torch.randn(*shape, generator=g).to(dtype)
+    L1, L2 = shape[-2], shape[-1]
+    xd = x.double().requires_grad_(True)
+    if causal:
+        r = torch.arange(L1).view(L1, 1)
+        c = torch.arange(L2).view(1, L2)
+        want = torch.softmax(xd.masked_fill(c > r + (L2 - L1), float("-inf")), dim=-1)
+    else:
+        want = torch.softmax(xd, dim=-1)
+    want.backward(dy.double())
+    xg = x.cuda().requires_grad_(True)
+    y = attention_softmax(xg, 0.0, causal, True)
+    assert y.dtype == dtype and y.shape == x.shape
+    assert rel_err(y, want.detach()) <= TOL
+    if causal:
+        assert torch.count_nonzero(torch.triu(y.float(), diagonal=L2 - L1 + 1)) == 0
+    y.backward(dy.cuda())
+    assert rel_err(xg.grad, xd.grad) <= TOL

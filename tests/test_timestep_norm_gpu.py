@@ -183,3 +183,21 @@ def test_dtype_mismatch_is_an_error():
         ops.group_timestep_norm_fwd(x.cuda(), pc.cuda(), pm.float().cuda(), pv.cuda(), gamma.cuda(), beta.cuda(), None, 2, 1e-5)
     with pytest.raises(RuntimeError, match="divisible"):
         ops.group_timestep_norm_fwd(x.cuda(), pc.cuda(), pm.cuda(), pv.cuda(), gamma.cuda(), beta.cuda(), None, 3, 1e-5)
+
+
+@pytest.mark.parametrize("mask", [None, "holes"])
+def test_non_group_operator(mask):
+    """timestep_norm_fwd/bwd (one running mean / variance per feature) equals
+    the float64 oracle of the group operator with one feature per group."""
+    B, L, H = 2, 90, 24
+    x, pc, pm, pv, gamma, beta, m, dy, dmean, dvar = _case(B, L, H, H, 21, torch.float32, 2, mask)
+    y, count, mean, var, cm, cr = ops.timestep_norm_fwd(*_cuda(x, pc, pm, pv, gamma, beta, m), 1e-5)
+    wy, wcount, wmean, wvar, wcm, wcr = tn.group_timestep_norm_closed_form_full(x, pc, pm, pv, gamma, beta, m, H, 1e-5)
+    assert torch.equal(count.cpu(), wcount) and cm.dtype == x.dtype and cm.shape == (B, L, H)
+    assert rel_err(y, wy) <= 1e-4 and rel_err(mean, wmean) <= 1e-4 and rel_err(var, wvar) <= 1e-4
+    assert rel_err(cm, wcm) <= 1e-4 and rel_err(cr, wcr) <= 1e-4
+    got = ops.timestep_norm_bwd(*_cuda(dy, dmean, dvar, x, pm), count, cm, cr, gamma.cuda(),
+                                None if m is None else m.cuda())
+    want = tn.group_timestep_norm_bwd_autograd(dy, dmean, dvar, x, pc, pm, pv, gamma, beta, m, H, 1e-5)
+    for name, a, b_ in zip(["dx", "dprev_mean", "dprev_var", "dgamma", "dbeta"], got, want):
+        assert rel_err(a, b_) <= 1e-4, name
