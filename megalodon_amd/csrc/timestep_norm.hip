@@ -714,7 +714,7 @@ __device__ __forceinline__ State2 bwd_lookahead(const TsnParams& p, int64_t chai
 
 template <int DT, int LPR>
 __global__ __launch_bounds__(kThreads)
-__attribute__((amdgpu_waves_per_eu(LPR <= 16 ? 4 : (LPR == 32 ? 2 : 1))))  // 132 -> 128 registers at LPR 16: one more wave per SIMD
+__attribute__((amdgpu_waves_per_eu(LPR <= 16 ? 4 : (LPR == 32 ? 2 : 1))))  // at least this many waves per SIMD
 void tsn_bwd_kernel(const TsnParams p) {
   constexpr int VEC = Vec<DT>::N;
   constexpr int RPW = kWave / LPR;
@@ -786,22 +786,22 @@ void tsn_bwd_kernel(const TsnParams p) {
     float f[VEC], d[VEC];
     Vec<DT>::unpack(xv[q], f);
     Vec<DT>::unpack(dv[q], d);
-    const float u = s_u[r];
-    float sx = 0.f, sds = 0.f, sdb = 0.f;
-    if (col_ok) {
+    // ds = sum dy gamma (x - u) = sum (dy gamma) x - u sum (dy gamma): lanes past
+    // the group hold zeros and add nothing
+    float sx = 0.f, sa = 0.f, sdb = 0.f;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        sx += f[e];
-        sds += d[e] * (f[e] - u) * gm[e];
-        sdb += d[e] * gm[e];
-      }
+    for (int e = 0; e < VEC; ++e) {
+      const float dg = d[e] * gm[e];
+      sx += f[e];
+      sa = fmaf(dg, f[e], sa);
+      sdb += dg;
     }
     sx = row_sum<LPR>(sx);
-    sds = row_sum<LPR>(sds);
+    sa = row_sum<LPR>(sa);
     sdb = row_sum<LPR>(sdb);
     if (col == 0) {
       s_ux[r] = sx * inv_dg;
-      s_ds[r] = sds;
+      s_ds[r] = sa - s_u[r] * sdb;
       s_db[r] = sdb;
     }
   }
@@ -854,8 +854,12 @@ void tsn_bwd_kernel(const TsnParams p) {
     const float dvx = c2 * dvv;
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // LDS reads above retired
     __builtin_amdgcn_wave_barrier();
-    s_ds[lane] = dux;
-    s_db[lane] = dvx;
+    // dx = dy gamma r + c0 + c1 x with c1 = 2 dvx / Dg, c0 = (dux - 2 dvx ux) / Dg;
+    // masked rows get the zero map (their x and dy are cleared before use, so
+    // whatever the padding holds stays out of dx and the parameter sums)
+    s_ds[lane] = valid ? (dux - 2.f * dvx * ux) * inv_dg : 0.f;
+    s_db[lane] = valid ? 2.f * dvx * inv_dg : 0.f;
+    s_r[lane] = valid ? r : 0.f;
   }
   __syncthreads();
 
@@ -868,17 +872,16 @@ void tsn_bwd_kernel(const TsnParams p) {
     const int t = t0 + r;
     if (t < p.L && col_ok) {
       float f[VEC], d[VEC], o[VEC];
-      Vec<DT>::unpack(xv[q], f);
-      Vec<DT>::unpack(dv[q], d);
-      const bool valid = s_valid[r] != 0;
-      const float u = s_u[r], rs = s_r[r], ux = s_ux[r], dux = s_ds[r], dvx = s_db[r];
+      uint4 xq = xv[q], dq = dv[q];
+      if (s_valid[r] == 0) xq = dq = make_uint4(0, 0, 0, 0);
+      Vec<DT>::unpack(xq, f);
+      Vec<DT>::unpack(dq, d);
+      const float u = s_u[r], rs = s_r[r], c0 = s_ds[r], c1 = s_db[r];
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        o[e] = valid ? d[e] * rs * gm[e] + (dux + 2.f * dvx * (f[e] - ux)) * inv_dg : 0.f;
-        if (valid) {
-          pg[e] += d[e] * (f[e] - u) * rs;
-          pb[e] += d[e];
-        }
+        o[e] = fmaf(d[e] * gm[e], rs, fmaf(c1, f[e], c0));
+        pg[e] = fmaf(d[e] * rs, f[e] - u, pg[e]);
+        pb[e] += d[e];
       }
       const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
       *reinterpret_cast<uint4*>(static_cast<typename Elem<DT>::type*>(p.y) + off) = Vec<DT>::pack(o);
