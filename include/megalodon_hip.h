@@ -212,6 +212,30 @@ int mega_attention_bwd(const void* dy, const void* q, const void* k, const void*
                        void* dq, void* dk, void* dv, void* workspace, void* stream);
 
 /* ------------------------------------------------------------------------
+ * Convolution with spectra kept between forward and backward.
+ *
+ * The reference's fused operator returns the spectrum of x for the backward
+ * pass and takes the spectrum of k (fftconv_fwd(x, k_f) -> (y, x_f),
+ * fftconv_bwd(dy, x_f, k_f, k_dtype), megalodon/modules/fused_ops/fftconv.py:
+ * 21-28,62-75, csrc/ops/fftconv_kernel.cu:34-164).  This pair does the same for
+ * the matrix-core path: the forward also writes the spectra of x and of k (an
+ * opaque fp16 layout with the rows' scales, mega_fftconv_spectrum_bytes(...)
+ * bytes each, 16-byte aligned), the backward needs only dy and the two
+ * buffers: dx = corr(dy, k) + omega dy, dk = sum_b corr(dy, x) from three
+ * transforms per row instead of five.  mega_fftconv_spectrum_bytes returns 0
+ * for shapes outside this path (float32 rows, L <= 2048, L % 8 != 0, D not a
+ * multiple of the rows per pass: 32768 / 2^ceil(log2 L) for L > 2048); use
+ * mega_fftconv_residual_fwd / _bwd then.  omega may be null (no skip term).
+ * ---------------------------------------------------------------------- */
+int64_t mega_fftconv_spectrum_bytes(int dtype, int64_t B, int64_t D, int64_t L);
+int mega_fftconv_residual_fwd_saving(const void* x, int dtype, const float* k, const float* omega,
+                                     int64_t B, int64_t D, int64_t L, void* y, void* spec_x,
+                                     void* spec_k, void* stream);
+int mega_fftconv_residual_bwd_saved(const void* dy, int dtype, const void* spec_x,
+                                    const void* spec_k, const float* omega, int64_t B, int64_t D,
+                                    int64_t L, void* dx, float* dk, void* stream);
+
+/* ------------------------------------------------------------------------
  * Standalone softmax of attention scores, in place.
  *
  * Replaces attention_softmax_fwd(x, dropout=0, use_causal_mask) -> y

@@ -540,3 +540,38 @@ extern "C" int mega_fftconv_residual_bwd(const void* dy, const void* x, int dtyp
   return fftconv_bwd_impl("mega_fftconv_residual_bwd", dy, x, dtype, k, omega, B, D, L, dx, dk,
                           stream);
 }
+
+// ---- forward that keeps the spectra of x and k, backward that uses them ----------
+extern "C" int64_t mega_fftconv_spectrum_bytes(int dtype, int64_t B, int64_t D, int64_t L) {
+  if (B <= 0 || D <= 0 || L <= 0 || getenv("MEGA_FFTCONV_VALU") != nullptr) return 0;
+  return fftm::spectrum_bytes(dtype, B, D, L);
+}
+
+extern "C" int mega_fftconv_residual_fwd_saving(const void* x, int dtype, const float* k,
+                                                const float* omega, int64_t B, int64_t D,
+                                                int64_t L, void* y, void* spec_x, void* spec_k,
+                                                void* stream) {
+  const char* who = "mega_fftconv_residual_fwd_saving";
+  MEGA_CHECK_ARG(x && k && y && spec_x && spec_k, "%s: null pointer", who);
+  MEGA_CHECK_ARG(fftm::spectrum_bytes(dtype, B, D, L) > 0 && fftm::applicable(dtype, L, x, k, y) &&
+                     reinterpret_cast<uintptr_t>(spec_x) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(spec_k) % 16 == 0,
+                 "%s: shape, dtype or alignment outside the saved-spectrum path "
+                 "(mega_fftconv_spectrum_bytes returns 0 for it)", who);
+  return fftm::launch_forward_saving(dtype, x, k, y, B, D, L, omega, spec_x, spec_k,
+                                     static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mega_fftconv_residual_bwd_saved(const void* dy, int dtype, const void* spec_x,
+                                               const void* spec_k, const float* omega, int64_t B,
+                                               int64_t D, int64_t L, void* dx, float* dk,
+                                               void* stream) {
+  const char* who = "mega_fftconv_residual_bwd_saved";
+  MEGA_CHECK_ARG(dy && spec_x && spec_k && dx && dk, "%s: null pointer", who);
+  MEGA_CHECK_ARG(fftm::spectrum_bytes(dtype, B, D, L) > 0 && fftm::applicable(dtype, L, dy, dx, dk) &&
+                     reinterpret_cast<uintptr_t>(spec_x) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(spec_k) % 16 == 0,
+                 "%s: shape, dtype or alignment outside the saved-spectrum path", who);
+  return fftm::launch_backward_saved(dtype, dy, spec_x, spec_k, dx, dk, B, D, L, omega,
+                                     static_cast<hipStream_t>(stream));
+}

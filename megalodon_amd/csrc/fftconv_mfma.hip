@@ -731,6 +731,25 @@ struct Spectrum {
   uint32_t e0, o0;  // row (0, 0), lane = k3 (threads 0..31), fp16 (re, im)
 };
 
+// A spectrum kept in memory between the forward and the backward launch: the
+// registers of `Spectrum` as they are, per pass
+//   [task 0..7][thread 0..511][8 words]  then  [thread][e0, o0]  then  8 row scales (float).
+constexpr int kSpecRowWords = 8 * kThreads * 8;              // offset of the (e0, o0) pairs
+constexpr int kSpecScaleWords = kSpecRowWords + kThreads * 2;  // offset of the scales
+constexpr int kSpecWords = kSpecScaleWords + 8;              // words per pass (a multiple of 4)
+
+__device__ __forceinline__ void store_spec_task(uint32_t* spec, int i, int tid, const uint32_t* e,
+                                                const uint32_t* o) {
+  u32x4* q = reinterpret_cast<u32x4*>(spec + (static_cast<size_t>(i) * kThreads + tid) * 8);
+  q[0] = u32x4{e[0], e[1], e[2], e[3]};
+  q[1] = u32x4{o[0], o[1], o[2], o[3]};
+}
+__device__ __forceinline__ void store_spectrum(uint32_t* spec, const Spectrum& sp, int tid) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) store_spec_task(spec, i, tid, sp.e[i], sp.o[i]);
+  *reinterpret_cast<uint2*>(spec + kSpecRowWords + 2 * tid) = make_uint2(sp.e0, sp.o0);
+}
+
 template <int LOGA>
 __device__ __forceinline__ void capture_spectrum(const uint16_t* pre, Spectrum& sp, int tid) {
   constexpr int A = Geo<LOGA>::A, R = Geo<LOGA>::R;
@@ -762,8 +781,11 @@ __device__ __forceinline__ void capture_spectrum(const uint16_t* pre, Spectrum& 
 }
 
 // the product of the two real signals' spectra, written over Za
+// `save` != nullptr: the untangled spectrum of the operand in LDS is also
+// written out in the saved-spectrum layout.
 template <int LOGA>
-__device__ __forceinline__ void pointwise(uint16_t* pre, const Spectrum& sp, int tid) {
+__device__ __forceinline__ void pointwise(uint16_t* pre, const Spectrum& sp, int tid,
+                                          uint32_t* save = nullptr) {
   constexpr int A = Geo<LOGA>::A, R = Geo<LOGA>::R, NP = Geo<LOGA>::NP;
   uint16_t* pim = pre + kIm;
 #pragma unroll
@@ -772,6 +794,13 @@ __device__ __forceinline__ void pointwise(uint16_t* pre, const Spectrum& sp, int
     const RowPair rp = row_pair<LOGA>(tid + kThreads * i);
     const Quad2 qa = untangle_quads(read_quad_raw(pre + rp.ok), read_quad_raw(pim + rp.ok),
                                     read_quad_raw(pre + rp.om), read_quad_raw(pim + rp.om));
+    if (save != nullptr) {
+      const uint32_t se[4] = {__builtin_bit_cast(uint32_t, qa.er[0]), __builtin_bit_cast(uint32_t, qa.er[1]),
+                              __builtin_bit_cast(uint32_t, qa.ei[0]), __builtin_bit_cast(uint32_t, qa.ei[1])};
+      const uint32_t so[4] = {__builtin_bit_cast(uint32_t, qa.orr[0]), __builtin_bit_cast(uint32_t, qa.orr[1]),
+                              __builtin_bit_cast(uint32_t, qa.oi[0]), __builtin_bit_cast(uint32_t, qa.oi[1])};
+      store_spec_task(save, i, tid, se, so);
+    }
     float w0c, w0s;
     cis(rp.k0, 1.f / NP, w0c, w0s);
     // W_N'^(k0 + 32 A e) = W_N'^k0 W_32^e
@@ -804,8 +833,80 @@ __device__ __forceinline__ void pointwise(uint16_t* pre, const Spectrum& sp, int
     const int ok = pos(a0, 0, k3), om = pos(a0, 0, m3);
     float ar, ai, pr, pi, br, bi, qr, qi, wc, ws, zkr, zki, zmr, zmi;
     untangle(h2f(pre[ok]), h2f(pim[ok]), h2f(pre[om]), h2f(pim[om]), ar, ai, pr, pi);
+    if (save != nullptr)
+      *reinterpret_cast<uint2*>(save + kSpecRowWords + 2 * tid) = make_uint2(pack_h2(ar, ai), pack_h2(pr, pi));
     unpack_h2(sp.e0, br, bi);
     unpack_h2(sp.o0, qr, qi);
+    cis(k3, 1.f / 32.f, wc, ws);
+    bin_product(ar, ai, pr, pi, br, bi, qr, qi, wc, ws, zkr, zki, zmr, zmi);
+    if (k3 <= m3) {
+      pre[ok] = f2h(zkr);
+      pim[ok] = f2h(zki);
+      pre[om] = f2h(zmr);
+      pim[om] = f2h(zmi);
+    }
+  } else if (save != nullptr) {
+    *reinterpret_cast<uint2*>(save + kSpecRowWords + 2 * tid) = make_uint2(0u, 0u);
+  }
+}
+
+// The same product with both spectra untangled already: `sa` in registers, the
+// other read from a saved spectrum; the result goes to the LDS planes.
+template <int LOGA>
+__device__ __forceinline__ void pointwise_saved(uint16_t* pre, const Spectrum& sa,
+                                                const uint32_t* __restrict__ spec, int tid) {
+  constexpr int A = Geo<LOGA>::A, R = Geo<LOGA>::R, NP = Geo<LOGA>::NP;
+  uint16_t* pim = pre + kIm;
+  // the saved spectrum is read two tasks ahead of its use
+  const u32x4* q = reinterpret_cast<const u32x4*>(spec) + static_cast<size_t>(tid) * 2;
+  const uint2 b0 = *reinterpret_cast<const uint2*>(spec + kSpecRowWords + 2 * tid);
+  u32x4 be_n = q[0], bo_n = q[1];
+  u32x4 be_nn = q[2 * kThreads], bo_nn = q[2 * kThreads + 1];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    tid = opaque(tid) & (kThreads - 1);
+    const RowPair rp = row_pair<LOGA>(tid + kThreads * i);
+    const u32x4 be = be_n, bo = bo_n;
+    be_n = be_nn;
+    bo_n = bo_nn;
+    if (i + 2 < 8) {
+      be_nn = q[static_cast<size_t>(i + 2) * 2 * kThreads];
+      bo_nn = q[static_cast<size_t>(i + 2) * 2 * kThreads + 1];
+    }
+    float w0c, w0s;
+    cis(rp.k0, 1.f / NP, w0c, w0s);
+    const float c32[4] = {1.f, 0.98078528040323043f, 0.92387953251128674f, 0.83146961230254524f};
+    const float s32[4] = {0.f, 0.19509032201612825f, 0.38268343236508978f, 0.55557023301960218f};
+    float okr[4], oki[4], omr[4], omi[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int hp = e >> 1, hh = e & 1;
+      const float ar = static_cast<float>(as_h2(sa.e[i][hp])[hh]);
+      const float ai = static_cast<float>(as_h2(sa.e[i][2 + hp])[hh]);
+      const float pr = static_cast<float>(as_h2(sa.o[i][hp])[hh]);
+      const float pi = static_cast<float>(as_h2(sa.o[i][2 + hp])[hh]);
+      const float br = static_cast<float>(as_h2(be[hp])[hh]), bi = static_cast<float>(as_h2(be[2 + hp])[hh]);
+      const float qr = static_cast<float>(as_h2(bo[hp])[hh]), qi = static_cast<float>(as_h2(bo[2 + hp])[hh]);
+      float wc, ws;
+      cmul(w0c, w0s, c32[e], s32[e], wc, ws);
+      bin_product(ar, ai, pr, pi, br, bi, qr, qi, wc, ws, okr[e], oki[e], omr[3 - e], omi[3 - e]);
+    }
+    if (rp.writes) {
+      write_quad(pre + rp.ok, okr);
+      write_quad(pim + rp.ok, oki);
+      write_quad(pre + rp.om, omr);
+      write_quad(pim + rp.om, omi);
+    }
+  }
+  tid = opaque(tid) & (kThreads - 1);
+  if (tid < 32 * R) {
+    const int a0 = (tid >> 5) * A, k3 = tid & 31, m3 = (32 - k3) & 31;
+    const int ok = pos(a0, 0, k3), om = pos(a0, 0, m3);
+    float ar, ai, pr, pi, br, bi, qr, qi, wc, ws, zkr, zki, zmr, zmi;
+    unpack_h2(sa.e0, ar, ai);
+    unpack_h2(sa.o0, pr, pi);
+    unpack_h2(b0.x, br, bi);
+    unpack_h2(b0.y, qr, qi);
     cis(k3, 1.f / 32.f, wc, ws);
     bin_product(ar, ai, pr, pi, br, bi, qr, qi, wc, ws, zkr, zki, zmr, zmi);
     if (k3 <= m3) {
@@ -835,7 +936,8 @@ __device__ __forceinline__ void final_scales(const float* sa, const float* sb, f
 template <int DT, int MODE, int LOGA>
 __global__ __launch_bounds__(kThreads) void fftconv_mfma_kernel(
     const void* __restrict__ a, const void* __restrict__ b, void* __restrict__ out, int rows,
-    int D, int L, int flip, const float* __restrict__ omega) {
+    int D, int L, int flip, const float* __restrict__ omega, uint32_t* __restrict__ spec_a,
+    uint32_t* __restrict__ spec_b) {
   constexpr int R = Geo<LOGA>::R;
   extern __shared__ __align__(16) uint16_t lds[];
   uint16_t* pre = lds;
@@ -844,6 +946,8 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_kernel(
   const Dft w = make_dft(lane);
   const int64_t esz = 2;
   const int passes = (rows + R - 1) / R;
+  // spec_a / spec_b (both or neither): the untangled spectra of the two
+  // operands of every pass and their row scales are kept for the backward launch
 
   // Software pipeline over the passes of this workgroup: the first-operand rows
   // are fetched while the second operand is transformed, and the next pass's
@@ -884,10 +988,24 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_kernel(
     transform<LOGA, false>(pre, w, wave, lane);
     Spectrum sp;
     capture_spectrum<LOGA>(pre, sp, tid);
+    uint32_t* const save_a = spec_a == nullptr ? nullptr : spec_a + static_cast<size_t>(pass) * kSpecWords;
     lds_barrier();
     place_rows<LOGA>(pre, red, ra, flip_a, tid, sa);
     transform<LOGA, false>(pre, w, wave, lane);
-    pointwise<LOGA>(pre, sp, tid);
+    if (spec_b != nullptr) {
+      // Stores go here, after the wait for the first operand's rows and with
+      // no wait on memory before the next pass: issued right after the capture
+      // they would be waited for in front of place_rows (loads and stores
+      // share one in-order counter).
+      uint32_t* const save_b = spec_b + static_cast<size_t>(pass) * kSpecWords;
+      store_spectrum(save_b, sp, tid);
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        if (tid == i) reinterpret_cast<float*>(save_b + kSpecScaleWords)[i] = sb[i];
+        if (tid == i) reinterpret_cast<float*>(save_a + kSpecScaleWords)[i] = sa[i];
+      }
+    }
+    pointwise<LOGA>(pre, sp, tid, save_a);
     lds_barrier();
     if (pass + static_cast<int>(gridDim.x) < passes)
       fetch_rows<LOGA>(rb, brows_of(pass + gridDim.x), L, false, tid);
@@ -982,6 +1100,79 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_bwd_kernel(
   }
 }
 
+// Backward from the spectra the forward launch kept (those of x and k, one pass
+// = R consecutive channels of one batch index, D % R == 0): dy is transformed
+// once, multiplied with either spectrum and transformed back -- three
+// transforms per pass instead of five, and neither x nor k is read.
+//   dx[b,d,:] = reverse(conv(reverse(dy[b,d,:]), k[d,:])) (+ omega[d] dy[b,d,:])
+//   dk[d,:]   = sum_b reverse(conv(reverse(dy[b,d,:]), x[b,d,:]))
+// As in the kernel above a workgroup owns channel groups and walks the batch.
+template <int DT, int LOGA>
+__global__ __launch_bounds__(kThreads) void fftconv_mfma_bwd_saved_kernel(
+    const void* __restrict__ dy, const uint32_t* __restrict__ spec_x,
+    const uint32_t* __restrict__ spec_k, void* __restrict__ dx, float* __restrict__ dk, int B,
+    int D, int L, const float* __restrict__ omega) {
+  constexpr int R = Geo<LOGA>::R;
+  extern __shared__ __align__(16) uint16_t lds[];
+  uint16_t* pre = lds;
+  float* red = reinterpret_cast<float*>(lds + 2 * kPlane);
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const Dft w = make_dft(lane);
+  const int64_t groups = D / R;
+  const int64_t total = (groups - blockIdx.x + gridDim.x - 1) / gridDim.x * B;
+  auto rows_of = [&](int64_t it, const void* base, int64_t esz, bool batched) {
+    const int64_t d0 = (blockIdx.x + (it / B) * gridDim.x) * R, bb = it % B;
+    RowPtrs<LOGA> p;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      p.p[i] = static_cast<const char*>(base) + ((batched ? bb * D : 0) + d0 + i) * L * esz;
+    return p;
+  };
+  RowRegs<DT> rdy;
+  if (total > 0) fetch_rows<LOGA>(rdy, rows_of(0, dy, 2, true), L, true, tid);
+  for (int64_t it = 0; it < total; ++it) {
+    const int64_t d0 = (blockIdx.x + (it / B) * gridDim.x) * R, bb = it % B;
+    const bool first = bb == 0;
+    // the forward's pass of rows (bb, d0 .. d0 + R - 1)
+    const size_t pass = static_cast<size_t>((bb * D + d0) / R);
+    const uint32_t* sx = spec_x + pass * kSpecWords;
+    const uint32_t* sk = spec_k + pass * kSpecWords;
+    const RowPtrs<LOGA> dyrows = rows_of(it, dy, 2, true);
+    float wres[R], sdy[R], s2[R], scale[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) wres[i] = omega != nullptr ? omega[d0 + i] : 0.f;
+    place_rows<LOGA>(pre, red, rdy, true, tid, sdy);
+    transform<LOGA, false>(pre, w, wave, lane);
+    Spectrum sp;
+    capture_spectrum<LOGA>(pre, sp, tid);
+    lds_barrier();
+    // dx
+    pointwise_saved<LOGA>(pre, sp, sk, tid);
+    lds_barrier();
+    transform<LOGA, true>(pre, w, wave, lane);
+#pragma unroll
+    for (int i = 0; i < R; ++i) s2[i] = reinterpret_cast<const float*>(sk + kSpecScaleWords)[i];
+    final_scales<LOGA>(sdy, s2, scale);
+    store_rows<LOGA, DT, false>(pre, rows_of(it, dx, 2, true), L, true, scale,
+                                omega != nullptr ? &dyrows : nullptr, wres, tid);
+    lds_barrier();
+    // dk
+    pointwise_saved<LOGA>(pre, sp, sx, tid);
+    lds_barrier();
+    if (it + 1 < total) fetch_rows<LOGA>(rdy, rows_of(it + 1, dy, 2, true), L, true, tid);
+    transform<LOGA, true>(pre, w, wave, lane);
+#pragma unroll
+    for (int i = 0; i < R; ++i) s2[i] = reinterpret_cast<const float*>(sx + kSpecScaleWords)[i];
+    final_scales<LOGA>(sdy, s2, scale);
+    const RowPtrs<LOGA> krows = rows_of(it, dk, 4, false);
+    if (first)
+      store_rows<LOGA, MEGA_F32, false>(pre, krows, L, true, scale, nullptr, wres, tid);
+    else
+      store_rows<LOGA, MEGA_F32, true>(pre, krows, L, true, scale, nullptr, wres, tid);
+    lds_barrier();
+  }
+}
+
 // digits a per row for a row of L samples: the smallest of 4, 8, 16, 32 with L <= 1024 A
 inline int loga_of(int64_t L) { return L > 16384 ? 5 : (L > 8192 ? 4 : (L > 4096 ? 3 : 2)); }
 
@@ -1003,9 +1194,29 @@ int launch_bwd(const void* dy, const void* x, const float* k, void* dx, float* d
   return MEGA_OK;
 }
 
+template <int DT, int LOGA>
+int launch_bwd_saved(const void* dy, const uint32_t* spec_x, const uint32_t* spec_k, void* dx,
+                     float* dk, int64_t B, int64_t D, int64_t L, const float* omega,
+                     hipStream_t stream) {
+  int dev = 0, cus = 0;
+  MEGA_CHECK_HIP(hipGetDevice(&dev));
+  MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  MEGA_CHECK_HIP(hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&fftconv_mfma_bwd_saved_kernel<DT, LOGA>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBytes)));
+  MEGA_CHECK_ARG(B * D <= 0x7fffffff, "fftconv: too many rows");
+  const int64_t groups = D / Geo<LOGA>::R;
+  const unsigned grid = static_cast<unsigned>(groups < cus ? groups : cus);
+  fftconv_mfma_bwd_saved_kernel<DT, LOGA><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
+      dy, spec_x, spec_k, dx, dk, static_cast<int>(B), static_cast<int>(D), static_cast<int>(L), omega);
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
+}
+
 template <int DT, int MODE, int LOGA>
 int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_t L, int flip,
-           const float* omega, hipStream_t stream) {
+           const float* omega, hipStream_t stream, uint32_t* spec_a = nullptr,
+           uint32_t* spec_b = nullptr) {
   int dev = 0, cus = 0;
   MEGA_CHECK_HIP(hipGetDevice(&dev));
   MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
@@ -1019,7 +1230,8 @@ int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_
     const int64_t passes = (rows + R - 1) / R;
     const unsigned grid = static_cast<unsigned>(passes < cus ? passes : cus);
     fftconv_mfma_kernel<DT, MODE, LOGA><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
-        a, b, out, static_cast<int>(rows), static_cast<int>(D), static_cast<int>(L), flip, omega);
+        a, b, out, static_cast<int>(rows), static_cast<int>(D), static_cast<int>(L), flip, omega,
+        spec_a, spec_b);
     MEGA_CHECK_LAUNCH();
   } else {
     const int64_t passes = (D + R - 1) / R;
@@ -1029,7 +1241,7 @@ int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_
       const char* xb = static_cast<const char*>(b) + bb * D * L * 2;
       fftconv_mfma_kernel<DT, MODE, LOGA><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
           ab, xb, out, static_cast<int>(D), static_cast<int>(D), static_cast<int>(L),
-          bb > 0 ? 1 : 0, nullptr);
+          bb > 0 ? 1 : 0, nullptr, nullptr, nullptr);
       MEGA_CHECK_LAUNCH();
     }
   }
@@ -1038,12 +1250,24 @@ int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_
 
 template <int DT, int MODE>
 int launch_len(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_t L, int flip,
-               const float* omega, hipStream_t stream) {
+               const float* omega, hipStream_t stream, uint32_t* spec_a = nullptr,
+               uint32_t* spec_b = nullptr) {
   switch (loga_of(L)) {
-    case 5: return launch<DT, MODE, 5>(a, b, out, B, D, L, flip, omega, stream);
-    case 4: return launch<DT, MODE, 4>(a, b, out, B, D, L, flip, omega, stream);
-    case 3: return launch<DT, MODE, 3>(a, b, out, B, D, L, flip, omega, stream);
-    default: return launch<DT, MODE, 2>(a, b, out, B, D, L, flip, omega, stream);
+    case 5: return launch<DT, MODE, 5>(a, b, out, B, D, L, flip, omega, stream, spec_a, spec_b);
+    case 4: return launch<DT, MODE, 4>(a, b, out, B, D, L, flip, omega, stream, spec_a, spec_b);
+    case 3: return launch<DT, MODE, 3>(a, b, out, B, D, L, flip, omega, stream, spec_a, spec_b);
+    default: return launch<DT, MODE, 2>(a, b, out, B, D, L, flip, omega, stream, spec_a, spec_b);
+  }
+}
+template <int DT>
+int launch_bwd_saved_len(const void* dy, const uint32_t* spec_x, const uint32_t* spec_k, void* dx,
+                         float* dk, int64_t B, int64_t D, int64_t L, const float* omega,
+                         hipStream_t stream) {
+  switch (loga_of(L)) {
+    case 5: return launch_bwd_saved<DT, 5>(dy, spec_x, spec_k, dx, dk, B, D, L, omega, stream);
+    case 4: return launch_bwd_saved<DT, 4>(dy, spec_x, spec_k, dx, dk, B, D, L, omega, stream);
+    case 3: return launch_bwd_saved<DT, 3>(dy, spec_x, spec_k, dx, dk, B, D, L, omega, stream);
+    default: return launch_bwd_saved<DT, 2>(dy, spec_x, spec_k, dx, dk, B, D, L, omega, stream);
   }
 }
 template <int DT>
@@ -1072,6 +1296,32 @@ int launch_conv(int dtype, int mode, const void* a, const void* b, void* out, in
                      : launch_len<MEGA_BF16, 1>(a, b, out, B, D, L, flip, omega, stream);
   return mode == 0 ? launch_len<MEGA_F16, 0>(a, b, out, B, D, L, flip, omega, stream)
                    : launch_len<MEGA_F16, 1>(a, b, out, B, D, L, flip, omega, stream);
+}
+
+int64_t spectrum_bytes(int dtype, int64_t B, int64_t D, int64_t L) {
+  if ((dtype != MEGA_BF16 && dtype != MEGA_F16) || L <= 2048 || L > 32768 || L % 8 != 0) return 0;
+  const int64_t R = 32 >> loga_of(L);
+  if (D % R != 0) return 0;
+  return B * D / R * kSpecWords * 4;
+}
+
+int launch_forward_saving(int dtype, const void* x, const float* k, void* y, int64_t B, int64_t D,
+                          int64_t L, const float* omega, void* spec_x, void* spec_k,
+                          hipStream_t stream) {
+  uint32_t* sx = static_cast<uint32_t*>(spec_x);
+  uint32_t* sk = static_cast<uint32_t*>(spec_k);
+  if (dtype == MEGA_BF16) return launch_len<MEGA_BF16, 0>(x, k, y, B, D, L, 0, omega, stream, sx, sk);
+  return launch_len<MEGA_F16, 0>(x, k, y, B, D, L, 0, omega, stream, sx, sk);
+}
+
+int launch_backward_saved(int dtype, const void* dy, const void* spec_x, const void* spec_k, void* dx,
+                          float* dk, int64_t B, int64_t D, int64_t L, const float* omega,
+                          hipStream_t stream) {
+  const uint32_t* sx = static_cast<const uint32_t*>(spec_x);
+  const uint32_t* sk = static_cast<const uint32_t*>(spec_k);
+  if (dtype == MEGA_BF16)
+    return launch_bwd_saved_len<MEGA_BF16>(dy, sx, sk, dx, dk, B, D, L, omega, stream);
+  return launch_bwd_saved_len<MEGA_F16>(dy, sx, sk, dx, dk, B, D, L, omega, stream);
 }
 
 int launch_backward(int dtype, const void* dy, const void* x, const float* k, void* dx, float* dk,

@@ -314,6 +314,57 @@ def fftconv_residual_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
     return dx, dk, dk[:, 0].clone()
 
 
+def fftconv_spectrum_bytes(dtype: torch.dtype, B: int, D: int, L: int) -> int:
+    """Bytes of one saved-spectrum buffer for this shape, 0 when the shape does
+    not take the saved-spectrum path."""
+    if dtype not in (torch.bfloat16, torch.float16):
+        return 0
+    fn = _lib.load().mega_fftconv_spectrum_bytes
+    fn.restype = _lib.ctypes.c_int64
+    return int(fn(_lib.i32(_lib.dtype_code(dtype)), _lib.i64(B), _lib.i64(D), _lib.i64(L)))
+
+
+def fftconv_residual_fwd_saving(x: torch.Tensor, k: torch.Tensor, omega: torch.Tensor):
+    """(y, spec_x, spec_k): ``fftconv_residual_fwd`` that also keeps the spectra
+    of x and k for ``fftconv_residual_bwd_saved`` (the reference keeps x_f and
+    k_f the same way, fused_ops/fftconv.py:21-28).  Only for shapes with
+    ``fftconv_spectrum_bytes(...) > 0``."""
+    dev = _require_cuda(x, k, omega)
+    B, D, L = x.shape
+    nbytes = fftconv_spectrum_bytes(x.dtype, B, D, L)
+    if nbytes == 0:
+        raise RuntimeError("fftconv: this shape / dtype has no saved-spectrum path")
+    xc = x.contiguous()
+    kc = k.contiguous().float()
+    wc = omega.reshape(-1).contiguous().float()
+    y = torch.empty_like(xc)
+    spec_x = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    spec_k = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_fftconv_residual_fwd_saving", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
+                  _lib.ptr(kc), _lib.ptr(wc), _lib.i64(B), _lib.i64(D), _lib.i64(L), _lib.ptr(y),
+                  _lib.ptr(spec_x), _lib.ptr(spec_k), _lib.stream_ptr(dev))
+    return y, spec_x, spec_k
+
+
+def fftconv_residual_bwd_saved(y_grad: torch.Tensor, spec_x: torch.Tensor, spec_k: torch.Tensor,
+                               omega: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dx, dk, domega) from y_grad (B, D, L) and the two saved spectra."""
+    dev = _require_cuda(y_grad, spec_x, spec_k, omega)
+    B, D, L = y_grad.shape
+    if spec_x.numel() != fftconv_spectrum_bytes(y_grad.dtype, B, D, L) or spec_k.numel() != spec_x.numel():
+        raise RuntimeError("fftconv_bwd: the saved spectra do not belong to this shape")
+    dy = y_grad.contiguous()
+    wc = omega.reshape(-1).contiguous().float()
+    dx = torch.empty_like(dy)
+    dk = torch.empty((D, L), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_fftconv_residual_bwd_saved", _lib.ptr(dy), _lib.i32(_lib.dtype_code(dy.dtype)),
+                  _lib.ptr(spec_x), _lib.ptr(spec_k), _lib.ptr(wc), _lib.i64(B), _lib.i64(D), _lib.i64(L),
+                  _lib.ptr(dx), _lib.ptr(dk), _lib.stream_ptr(dev))
+    return dx, dk, dk[:, 0].clone()
+
+
 # --------------------------------------------------------------------------
 # group_timestep_norm (reference: csrc/ops/timestep_norm.cc:621-705)
 # --------------------------------------------------------------------------

@@ -1,13 +1,16 @@
 """`fftconv` autograd op (mirror of megalodon/modules/fused_ops/fftconv.py:9-27).
 
-The reference saves the spectra ``(x_f, k_f)`` for backward; this op saves
-``(x, k)`` and the backward kernel recomputes the transforms on chip."""
+The reference saves the spectra ``(x_f, k_f)`` for backward; `fftconv` saves
+``(x, k)`` and the backward kernel recomputes the transforms on chip, while
+`fftconv_residual` (the op the CEMA layer uses) keeps the two spectra whenever
+the shape runs on the matrix-core path."""
 from typing import Tuple
 
 import torch
 from torch.autograd.function import FunctionCtx
 
-from ..extension import fftconv_bwd, fftconv_fwd, fftconv_residual_bwd, fftconv_residual_fwd
+from ..extension import (fftconv_bwd, fftconv_fwd, fftconv_residual_bwd, fftconv_residual_bwd_saved,
+                         fftconv_residual_fwd, fftconv_residual_fwd_saving, fftconv_spectrum_bytes)
 
 
 class FFTConvFunc(torch.autograd.Function):
@@ -36,15 +39,28 @@ class FFTConvResidualFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx: FunctionCtx, x: torch.Tensor, k: torch.Tensor, omega: torch.Tensor) -> torch.Tensor:
-        y = fftconv_residual_fwd(x, k, omega)
-        ctx.save_for_backward(x, k, omega)
+        # 16-bit rows on the matrix-core path keep the spectra of x and k for
+        # the backward pass, as the reference keeps x_f and k_f
+        # (fused_ops/fftconv.py:21-28); other shapes keep x and k themselves
+        ctx.k_dtype = k.dtype
+        ctx.spectra = x.is_cuda and fftconv_spectrum_bytes(x.dtype, *x.shape) > 0
+        if ctx.spectra:
+            y, spec_x, spec_k = fftconv_residual_fwd_saving(x, k, omega)
+            ctx.save_for_backward(spec_x, spec_k, omega)
+        else:
+            y = fftconv_residual_fwd(x, k, omega)
+            ctx.save_for_backward(x, k, omega)
         return y
 
     @staticmethod
     def backward(ctx: FunctionCtx, y_grad: torch.Tensor):
-        x, k, omega = ctx.saved_tensors
-        dx, dk, dw = fftconv_residual_bwd(y_grad, x, k, omega)
-        return dx, dk.to(k.dtype), dw.to(omega.dtype).view_as(omega)
+        if ctx.spectra:
+            spec_x, spec_k, omega = ctx.saved_tensors
+            dx, dk, dw = fftconv_residual_bwd_saved(y_grad, spec_x, spec_k, omega)
+        else:
+            x, k, omega = ctx.saved_tensors
+            dx, dk, dw = fftconv_residual_bwd(y_grad, x, k, omega)
+        return dx, dk.to(ctx.k_dtype), dw.to(omega.dtype).view_as(omega)
 
 
 fftconv_residual = FFTConvResidualFunc.apply

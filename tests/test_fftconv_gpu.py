@@ -75,6 +75,48 @@ def test_residual_variant_matches_oracle(B, D, L, dtype):
     assert dw.shape == (D,) and rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("B,D,L", [(1, 3, 32768), (2, 2, 20000), (2, 4, 16384), (1, 8, 8192), (3, 16, 4096),
+                                   (2, 8, 2056), (1, 4, 12344)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_saved_spectrum_pair_matches_oracle(B, D, L, dtype):
+    """Forward that keeps the spectra of x and k, backward from dy and the two
+    buffers alone: same values and gradients as the float64 oracle."""
+    x, k, dy = _data(B, D, L, dtype, 13 * L + B)
+    omega = torch.randn(D, 1, generator=torch.Generator().manual_seed(L)) * 0.5
+    assert ops.fftconv_spectrum_bytes(dtype, B, D, L) > 0
+    y, sx, sk = ops.fftconv_residual_fwd_saving(x.cuda(), k.cuda(), omega.cuda())
+    w64 = omega.double().view(1, D, 1)
+    assert rel_err(y, fftconv.fftconv_fwd(x, k).double() + w64 * x.double()) <= TOL[dtype]
+    dx, dk, dw = ops.fftconv_residual_bwd_saved(dy.cuda(), sx, sk, omega.cuda())
+    wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
+    assert rel_err(dx, wdx.double() + w64 * dy.double()) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= TOL[dtype]
+    assert rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= TOL[dtype]
+    # the recomputing pair gives the same forward bits
+    assert torch.equal(y, ops.fftconv_residual_fwd(x.cuda(), k.cuda(), omega.cuda()))
+
+
+def test_saved_spectrum_path_is_refused_outside_its_shapes():
+    assert ops.fftconv_spectrum_bytes(torch.float32, 1, 8, 4096) == 0
+    assert ops.fftconv_spectrum_bytes(torch.bfloat16, 1, 8, 2048) == 0
+    assert ops.fftconv_spectrum_bytes(torch.bfloat16, 1, 3, 4096) == 0   # 8 rows per pass, D = 3
+    assert ops.fftconv_spectrum_bytes(torch.bfloat16, 1, 8, 4097) == 0
+    x = torch.zeros(1, 3, 4096, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="saved-spectrum"):
+        ops.fftconv_residual_fwd_saving(x, torch.zeros(3, 4096, device="cuda"), torch.zeros(3, device="cuda"))
+
+
+def test_residual_autograd_function_16bit_uses_saved_spectra():
+    x, k, dy = _data(2, 8, 6000, torch.bfloat16, 3)
+    omega = torch.randn(8, 1)
+    xg, kg, wg = (t.cuda().requires_grad_() for t in (x, k, omega))
+    fftconv_residual(xg, kg, wg).backward(dy.cuda())
+    wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
+    assert rel_err(xg.grad, wdx.double() + omega.double().view(1, 8, 1) * dy.double()) <= 2e-2
+    assert rel_err(kg.grad, wdk) <= 2e-2
+    assert rel_err(wg.grad.view(-1), (dy.double() * x.double()).sum(dim=(0, 2))) <= 2e-2
+
+
 def test_residual_autograd_function():
     x, k, dy = _data(2, 3, 3000, torch.float32, 3)
     omega = torch.randn(3, 1)
