@@ -22,10 +22,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
-# HBM bytes one forward convolution launch moves at config 1: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from
+# HBM bytes one forward convolution launch moves at config 1 (1.11e9 of them the spectra kept for the backward): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from
 # two rocprofv3 --pmc passes of this script, the factors being what the same counters read for a plain
 # copy of 2^30 bytes (--copy-calibration).  A measured constant: counters cannot be read from in here.
-FFTCONV_TRAFFIC_BYTES = 1.37e9
+FFTCONV_TRAFFIC_BYTES = 2.49e9
 
 
 def cpu_baseline(B, D, N, L, seed, budget_s=25.0):
