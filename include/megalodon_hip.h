@@ -74,6 +74,30 @@ int mega_ema_weight_bwd(const float* dw, const float* p, const float* log_q,
                         float* dp, float* dq, float* dgamma, void* stream);
 
 /* ------------------------------------------------------------------------
+ * CEMA coefficients from the raw parameters, and their gradients.
+ *
+ * Replaces MultiHeadComplexEMA._calc_coeffs and its autograd graph
+ *   reference: megalodon/modules/complex_exponential_moving_average.py:100-117
+ *   (about thirty elementwise PyTorch kernels per training step there).
+ *   alpha, delta (D, N), theta (D), gamma (D, N, 2) float32 ->
+ *   p = sigmoid(alpha) (D, N) float32;
+ *   log_q = (ln(1 - sigmoid(alpha) sigmoid(delta)), n sigmoid(theta) 2 pi / N),
+ *   n = 1 .. N, (D, N) complex64 -- the logarithm of the reference's q, which is
+ *   what mega_ema_weight_fwd takes;
+ *   gamma_hat = (gamma_0 + i gamma_1) sqrt(1 / N) (D, N) complex64.  N <= 64.
+ * Backward: dp (D, N) float32, dq and dgamma_hat (D, N) complex64 as
+ *   mega_ema_weight_bwd returns them (gradient w.r.t. q, PyTorch's complex
+ *   convention) -> dalpha, ddelta (D, N), dtheta (D), dgamma (D, N, 2).
+ * ---------------------------------------------------------------------- */
+int mega_cema_coeffs_fwd(const float* alpha, const float* delta, const float* theta,
+                         const float* gamma, int64_t D, int64_t N, float* p, float* log_q,
+                         float* gamma_hat, void* stream);
+int mega_cema_coeffs_bwd(const float* dp, const float* dq, const float* dgamma_hat,
+                         const float* alpha, const float* delta, const float* theta, int64_t D,
+                         int64_t N, float* dalpha, float* ddelta, float* dtheta, float* dgamma,
+                         void* stream);
+
+/* ------------------------------------------------------------------------
  * Causal FFT convolution.
  *
  * Replaces fftconv_fwd(x, k_f) -> (y, x_f) and the torch.fft branch used for

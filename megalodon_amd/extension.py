@@ -167,6 +167,52 @@ def ema_parameters_bwd(
 
 
 # --------------------------------------------------------------------------
+# CEMA coefficients (reference: modules/complex_exponential_moving_average.py:100-117)
+# --------------------------------------------------------------------------
+def _coeff_shapes(alpha, delta, theta, gamma):
+    D, N = alpha.shape[0], alpha.shape[1]
+    if alpha.numel() != D * N or delta.shape != alpha.shape or theta.numel() != D or gamma.numel() != 2 * D * N:
+        raise RuntimeError("cema_coeffs: expected alpha, delta (D, N, 1), theta (D, 1, 1), gamma (D, N, 2)")
+    for name, t in (("alpha", alpha), ("delta", delta), ("theta", theta), ("gamma", gamma)):
+        if t.dtype != torch.float32:
+            raise RuntimeError(f"cema_coeffs: {name} must be float32 (got {t.dtype})")
+    return D, N
+
+
+def cema_coeffs_fwd(alpha: torch.Tensor, delta: torch.Tensor, theta: torch.Tensor, gamma: torch.Tensor):
+    """(p (D, N, 1) float32, log_q (D, N, 1) complex64, gamma_hat (D, N) complex64) in
+    one launch: ``_calc_coeffs`` followed by ``q.log()``."""
+    dev = _require_cuda(alpha, delta, theta, gamma)
+    D, N = _coeff_shapes(alpha, delta, theta, gamma)
+    a, d, t, g = alpha.contiguous(), delta.contiguous(), theta.contiguous(), gamma.contiguous()
+    p = torch.empty((D, N, 1), dtype=torch.float32, device=dev)
+    log_q = torch.empty((D, N, 1), dtype=torch.complex64, device=dev)
+    gamma_hat = torch.empty((D, N), dtype=torch.complex64, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_cema_coeffs_fwd", _lib.ptr(a), _lib.ptr(d), _lib.ptr(t), _lib.ptr(g), _lib.i64(D),
+                  _lib.i64(N), _lib.ptr(p), _lib.ptr(log_q), _lib.ptr(gamma_hat), _lib.stream_ptr(dev))
+    return p, log_q, gamma_hat
+
+
+def cema_coeffs_bwd(dp: torch.Tensor, dq: torch.Tensor, dgamma_hat: torch.Tensor, alpha: torch.Tensor,
+                    delta: torch.Tensor, theta: torch.Tensor):
+    """(dalpha, ddelta, dtheta, dgamma) from the gradients ``ema_parameters_bwd``
+    returns (dp real, dq / dgamma_hat complex, PyTorch's convention)."""
+    dev = _require_cuda(dp, dq, dgamma_hat, alpha, delta, theta)
+    D, N = alpha.shape[0], alpha.shape[1]
+    a, d, t = alpha.contiguous(), delta.contiguous(), theta.contiguous()
+    dpc = dp.contiguous().float()
+    dqc, dgc = _as_c64(dq, "dq"), _as_c64(dgamma_hat, "dgamma_hat")
+    dalpha, ddelta, dtheta = torch.empty_like(a), torch.empty_like(d), torch.empty_like(t)
+    dgamma = torch.empty((D, N, 2), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_cema_coeffs_bwd", _lib.ptr(dpc), _lib.ptr(dqc), _lib.ptr(dgc), _lib.ptr(a), _lib.ptr(d),
+                  _lib.ptr(t), _lib.i64(D), _lib.i64(N), _lib.ptr(dalpha), _lib.ptr(ddelta), _lib.ptr(dtheta),
+                  _lib.ptr(dgamma), _lib.stream_ptr(dev))
+    return dalpha, ddelta, dtheta, dgamma
+
+
+# --------------------------------------------------------------------------
 # ema_hidden (reference: csrc/ops/ema_hidden.cc:16-159, fused_ops/ema_hidden.py)
 # --------------------------------------------------------------------------
 def ema_hidden_fwd(

@@ -1,9 +1,10 @@
 """Fused ops with the reference's names (megalodon/modules/fused_ops/__init__.py:1-14)."""
 from .attention import (attention_softmax, swift_efficient_attention, swift_efficient_attention_bwd,
                         swift_efficient_attention_fwd)
+from .cema_kernel import cema_kernel
 from .ema_hidden import ema_hidden
 from .ema_parameters import ema_parameters
 from .fftconv import fftconv, fftconv_residual
 
-__all__ = ["attention_softmax", "ema_hidden", "ema_parameters", "fftconv", "fftconv_residual", "swift_efficient_attention", "swift_efficient_attention_fwd",
+__all__ = ["attention_softmax", "cema_kernel", "ema_hidden", "ema_parameters", "fftconv", "fftconv_residual", "swift_efficient_attention", "swift_efficient_attention_fwd",
            "swift_efficient_attention_bwd"]

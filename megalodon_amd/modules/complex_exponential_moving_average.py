@@ -9,7 +9,7 @@ import math
 import torch
 from torch import nn
 
-from ..fused_ops import ema_hidden, ema_parameters, fftconv_residual
+from ..fused_ops import cema_kernel, ema_hidden, ema_parameters, fftconv_residual
 
 _r2c = torch.view_as_complex
 
@@ -85,8 +85,15 @@ class MultiHeadComplexEMA(nn.Module):
     ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
         # B x D x L
         bsz, _, seq_len = x.size()
-        p, q, gamma = self.coeffs()
-        k, b = ema_parameters(p, q, gamma, hx, seq_len)
+        if hx is None and not compute_last_state and self.alpha.is_cuda:
+            # no carried state: coefficients and kernel as one autograd node
+            # (two launches per direction instead of the coefficient graph)
+            k, b = cema_kernel(self.alpha.float(), self.delta.float(), self.theta.float(), self.gamma.float(),
+                               seq_len), None
+            p = q = None
+        else:
+            p, q, gamma = self.coeffs()
+            k, b = ema_parameters(p, q, gamma, hx, seq_len)
         # fftconv(x, k) + x * omega, the skip term folded into the convolution's
         # output pass (the reference adds `residual = x * self.omega` afterwards)
         output = fftconv_residual(x, k, self.omega)

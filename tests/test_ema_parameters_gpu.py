@@ -107,3 +107,33 @@ def test_errors_are_loud():
     g40 = torch.randn(2, 40, dtype=torch.complex64).cuda()
     with pytest.raises(RuntimeError, match="outside"):
         ops.ema_parameters_fwd(p40, q40.log(), g40, None, 8)
+
+
+@pytest.mark.parametrize("D,N", [(5, 16), (64, 16), (7, 3), (33, 1), (4, 64)])
+def test_fused_coefficients_match_oracle(D, N):
+    """mega_cema_coeffs_fwd/bwd against the float64 restatement of
+    _calc_coeffs and autograd over it (log q instead of q on the forward side,
+    gradients w.r.t. q on the backward side, as the weight operator uses them)."""
+    g = torch.Generator().manual_seed(D * 100 + N)
+    alpha = torch.randn(D, N, 1, generator=g)
+    delta = torch.randn(D, N, 1, generator=g)
+    theta = torch.randn(D, 1, 1, generator=g)
+    gamma = torch.randn(D, N, 2, generator=g)
+    p, log_q, gh = ops.cema_coeffs_fwd(alpha.cuda(), delta.cuda(), theta.cuda(), gamma.cuda())
+    a64, d64, t64, g64 = (t.double().requires_grad_(True) for t in (alpha, delta, theta, gamma))
+    wp, wq, wg = cema.calc_coeffs(a64, d64, t64, g64, N)
+    assert p.shape == (D, N, 1) and log_q.shape == (D, N, 1) and gh.shape == (D, N)
+    assert rel_err(p, wp) <= 1e-6
+    assert rel_err(torch.exp(log_q), wq) <= 1e-5
+    assert rel_err(log_q.real, wq.abs().log()) <= 1e-5   # the phase is n theta_hat in (0, 2 pi), not the wrapped one
+    assert float(log_q.imag.min()) > 0.0 and float(log_q.imag.max()) < 2 * math.pi
+    assert rel_err(torch.view_as_real(gh), torch.view_as_real(wg)) <= 1e-6
+    dp = torch.randn(D, N, 1, generator=g)
+    dq = torch.view_as_complex(torch.randn(D, N, 1, 2, generator=g))
+    dg = torch.view_as_complex(torch.randn(D, N, 2, generator=g))
+    # PyTorch convention: backward with grad_output g gives dL/dRe + i dL/dIm for L = Re(sum conj(g) z)
+    torch.autograd.backward([wp, wq, wg], [dp.double(), dq.to(torch.complex128), dg.to(torch.complex128)])
+    got = ops.cema_coeffs_bwd(dp.cuda(), dq.cuda(), dg.cuda(), alpha.cuda(), delta.cuda(), theta.cuda())
+    for name, a, b in zip(["dalpha", "ddelta", "dtheta", "dgamma"], got, (a64.grad, d64.grad, t64.grad, g64.grad)):
+        assert a.shape == b.shape, name
+        assert rel_err(a, b) <= 1e-5, name
