@@ -259,6 +259,84 @@ __device__ __forceinline__ void split8(const float* v, u32x4& hi, u32x4& lo) {
   }
 }
 
+// ---- forward on the matrix cores (N <= 16) ------------------------------------
+// With j = 1024 h + lo the kernel row of a channel is a small GEMM,
+//   w[1024 h + lo] = sum_c T[h][c] Q[lo][c],  c = 2 n + part,
+//   T[h] = (Re, Im)(c_n q_n^(1024 h)),  Q[lo] = (Re, -Im)(q_n^lo),
+// 32 rows h x 1024 columns lo x 32 values c per workgroup: the VALU version
+// spends 2 FMA per (element, mode) and is bound by them, this one by its
+// stores.  Same split-bf16 products as the backward kernel.
+__global__ __launch_bounds__(kThreads) void ema_weight_fwd_mfma_kernel(
+    const float* __restrict__ p, const cf* __restrict__ log_q, const cf* __restrict__ gamma, int N,
+    int64_t L, float* __restrict__ w) {
+  __shared__ LowTables<16, 4> low;  // q^b (b < 64), q^(64 a) (a < 16)
+  __shared__ cf hi[32][16];         // c_n q_n^(1024 h) for the 32 rows of this workgroup
+  const int64_t d = blockIdx.x;
+  const int64_t h0 = static_cast<int64_t>(blockIdx.y) * 32;
+  const cf* lq = log_q + d * N;
+  fill_low_tables<16, 4>(low, lq, N);
+  for (int i = threadIdx.x; i < 32 * 16; i += kThreads) {
+    const int h = i >> 4, n = i & 15;
+    cf v{0.f, 0.f};
+    if (n < N && (h0 + h) * 1024 < L) {
+      const cf g = gamma[d * N + n];
+      const float pp = p[d * N + n];
+      v = cmul(cf{pp * g.x, pp * g.y}, qpow(lq[n].x, lq[n].y, (h0 + h) * 1024));
+    }
+    hi[h][n] = v;
+  }
+  __syncthreads();
+
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int g = lane >> 5, col = lane & 31;
+  // A operand: lane <-> row h = col, k = c = 16 s + 8 g + e  ->  modes 8 s + 4 g + e / 2
+  u32x4 ahi[2], alo[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    float v[8];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const cf t = hi[col][8 * s + 4 * g + m];
+      v[2 * m] = t.x;
+      v[2 * m + 1] = t.y;
+    }
+    split8(v, ahi[s], alo[s]);
+  }
+  float* wrow = w + d * L + h0 * 1024;
+  const int64_t left = L - h0 * 1024;  // samples of this workgroup's rows
+  for (int lt = wave; lt < 32; lt += kThreads / kWave) {
+    const int lo = 32 * lt + col;
+    u32x4 bhi[2], blo[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      float v[8];
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int n = 8 * s + 4 * g + m;
+        const cf q = cmul(low.p2[n][lo >> 6], low.p1[n][lo & 63]);
+        v[2 * m] = q.x;
+        v[2 * m + 1] = -q.y;
+      }
+      split8(v, bhi[s], blo[s]);
+    }
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      acc = mfma_bf16(ahi[s], bhi[s], acc);
+      acc = mfma_bf16(ahi[s], blo[s], acc);
+      acc = mfma_bf16(alo[s], bhi[s], acc);
+    }
+    // result: lane <-> column lo, register r <-> row h = 8 (r / 4) + 4 g + r % 4
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int64_t j = static_cast<int64_t>(8 * (r >> 2) + 4 * g + (r & 3)) * 1024 + lo;
+      if (j < left) wrow[j] = acc[r];
+    }
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void ema_weight_bwd_mfma_kernel(
     const float* __restrict__ dw, const float* __restrict__ p, const cf* __restrict__ log_q,
     const cf* __restrict__ gamma, int N, int64_t L, float* __restrict__ dp, cf* __restrict__ dq,
@@ -399,7 +477,11 @@ extern "C" int mega_ema_weight_fwd(const float* p, const float* log_q,
   const cf* lq = reinterpret_cast<const cf*>(log_q);
   const cf* gm = reinterpret_cast<const cf*>(gamma);
   const bool vec = (L % 4 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0);
-  if (N <= 16) {
+  if (N <= 16 && (L + 1023) / 1024 <= 32 * 65535 && getenv("MEGA_EMA_FWD_VALU") == nullptr) {
+    const int64_t hrows = (L + 1023) / 1024;
+    dim3 grid(static_cast<unsigned>(D), static_cast<unsigned>((hrows + 31) / 32));
+    ema_weight_fwd_mfma_kernel<<<grid, kThreads, 0, s>>>(p, lq, gm, (int)N, L, w);
+  } else if (N <= 16) {
     constexpr int kTile = kThreads * 4;
     const int64_t tiles = (L + kTile - 1) / kTile;
     dim3 grid(static_cast<unsigned>(D), static_cast<unsigned>((tiles + kSlab - 1) / kSlab));
