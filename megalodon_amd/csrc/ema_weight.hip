@@ -342,6 +342,8 @@ __global__ __launch_bounds__(kThreads) void ema_weight_bwd_mfma_kernel(
     const cf* __restrict__ gamma, int N, int64_t L, float* __restrict__ dp, cf* __restrict__ dq,
     cf* __restrict__ dgamma) {
   __shared__ float red[kThreads][4];
+  __shared__ u32x4 qop[4][4][kWave];  // [k-step][re hi, re lo, im hi, im lo][lane]
+  static_assert(kThreads / kWave == 4, "one wave per k-step of the B operand");
   const int64_t d = blockIdx.x;
   const cf* lq = log_q + d * N;
   const float* drow = dw + d * L;
@@ -352,11 +354,12 @@ __global__ __launch_bounds__(kThreads) void ema_weight_bwd_mfma_kernel(
   const float la = live ? lq[n].x : 0.f, lphi = live ? lq[n].y : 0.f;
 
   // B operand: lane <-> column (kind, n), k = h = 16 s + 8 g + e; real and
-  // imaginary parts are the two 32-column tiles
-  u32x4 qre_hi[4], qre_lo[4], qim_hi[4], qim_lo[4];
-  const cf q1 = qpow(la, lphi, 1);
-#pragma unroll
-  for (int s = 0; s < 4; ++s) {
+  // imaginary parts are the two 32-column tiles.  It is the same for the four
+  // waves: wave s builds k-step s and the operand lives in LDS (64 registers
+  // less per lane, one more workgroup per CU).
+  {
+    const int s = wave;
+    const cf q1 = qpow(la, lphi, 1);
     float vr[8], vi[8];
     cf v = qpow(la, lphi, 16 * s + 8 * g);
 #pragma unroll
@@ -366,9 +369,15 @@ __global__ __launch_bounds__(kThreads) void ema_weight_bwd_mfma_kernel(
       vi[e] = v.y * sc;
       v = cmul(v, q1);
     }
-    split8(vr, qre_hi[s], qre_lo[s]);
-    split8(vi, qim_hi[s], qim_lo[s]);
+    u32x4 rh, rl, ih, il;
+    split8(vr, rh, rl);
+    split8(vi, ih, il);
+    qop[s][0][lane] = rh;
+    qop[s][1][lane] = rl;
+    qop[s][2][lane] = ih;
+    qop[s][3][lane] = il;
   }
+  __syncthreads();
   // q^(64 lo) for the rows a lane meets: lo = 32 mt + 8 qd + 4 g + e
   const cf st1 = qpow(la, lphi, 64), st2 = cmul(st1, st1), st3 = cmul(st2, st1);
   const cf st8 = qpow(la, lphi, 512);
@@ -404,14 +413,20 @@ __global__ __launch_bounds__(kThreads) void ema_weight_bwd_mfma_kernel(
     floatx16 cr, ci;
 #pragma unroll
     for (int r = 0; r < 16; ++r) cr[r] = ci[r] = 0.f;
+    // re-read per tile: left to itself the compiler hoists these 64 registers
+    // out of the loop again
+    int ql = lane;
+    asm volatile("" : "+v"(ql));
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      cr = mfma_bf16(ahi[s], qre_hi[s], cr);
-      ci = mfma_bf16(ahi[s], qim_hi[s], ci);
-      cr = mfma_bf16(ahi[s], qre_lo[s], cr);
-      ci = mfma_bf16(ahi[s], qim_lo[s], ci);
-      cr = mfma_bf16(alo[s], qre_hi[s], cr);
-      ci = mfma_bf16(alo[s], qim_hi[s], ci);
+      const u32x4 qre_hi = qop[s][0][ql], qre_lo = qop[s][1][ql];
+      const u32x4 qim_hi = qop[s][2][ql], qim_lo = qop[s][3][ql];
+      cr = mfma_bf16(ahi[s], qre_hi, cr);
+      ci = mfma_bf16(ahi[s], qim_hi, ci);
+      cr = mfma_bf16(ahi[s], qre_lo, cr);
+      ci = mfma_bf16(ahi[s], qim_lo, ci);
+      cr = mfma_bf16(alo[s], qre_hi, cr);
+      ci = mfma_bf16(alo[s], qim_hi, ci);
     }
     // result: lane <-> column, register r <-> row lo = 32 mt + 8 (r / 4) + 4 g + r % 4
     const int64_t lo0 = 32 * mt + 4 * g;
