@@ -43,8 +43,9 @@ class FFTConvResidualFunc(torch.autograd.Function):
         # the backward pass, as the reference keeps x_f and k_f
         # (fused_ops/fftconv.py:21-28); other shapes keep x and k themselves
         ctx.k_dtype = k.dtype
+        x = x.contiguous()  # the CEMA layer hands in a transposed view
         ctx.spectra = (x.is_cuda and x.dim() == 3 and fftconv_spectrum_bytes(x.dtype, *x.shape) > 0
-                       and x.is_contiguous() and x.data_ptr() % 16 == 0)
+                       and x.data_ptr() % 16 == 0)
         if ctx.spectra:
             y, spec_x, spec_k = fftconv_residual_fwd_saving(x, k, omega)
             ctx.save_for_backward(spec_x, spec_k, omega)
