@@ -96,6 +96,23 @@ def test_saved_spectrum_pair_matches_oracle(B, D, L, dtype):
     assert torch.equal(y, ops.fftconv_residual_fwd(x.cuda(), k.cuda(), omega.cuda()))
 
 
+def test_saved_spectrum_pair_at_full_row_count_agrees_with_recomputing_pair():
+    """Config-1 rows (L = 32768, bf16) over 512 channels and two batch entries:
+    the backward from kept spectra and the backward that re-transforms x and k
+    see the same fp16 spectra, so they agree far inside the bfloat16 bar."""
+    B, D, L = 2, 512, 32768
+    g = torch.Generator().manual_seed(91)
+    x = torch.randn(B, D, L, generator=g).bfloat16().cuda()
+    dy = torch.randn(B, D, L, generator=g).bfloat16().cuda()
+    k = (torch.randn(D, L, generator=g) * (0.9995 ** torch.arange(L, dtype=torch.float32))).cuda()
+    omega = torch.randn(D, generator=g).cuda()
+    y, sx, sk = ops.fftconv_residual_fwd_saving(x, k, omega)
+    assert torch.equal(y, ops.fftconv_residual_fwd(x, k, omega))
+    dx, dk, dw = ops.fftconv_residual_bwd_saved(dy, sx, sk, omega)
+    rdx, rdk, rdw = ops.fftconv_residual_bwd(dy, x, k, omega)
+    assert rel_err(dx, rdx) <= 4e-3 and rel_err(dk, rdk) <= 1e-3 and rel_err(dw, rdw) <= 1e-3
+
+
 def test_saved_spectrum_path_is_refused_outside_its_shapes():
     assert ops.fftconv_spectrum_bytes(torch.float32, 1, 8, 4096) == 0
     assert ops.fftconv_spectrum_bytes(torch.bfloat16, 1, 8, 2048) == 0
