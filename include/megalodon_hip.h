@@ -213,8 +213,9 @@ int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, const void* 
  *   written only up to the end of the 256-column block holding the diagonal of
  *   each row (zeros above the diagonal inside that block); the blocks to the
  *   right are never read by the backward and are left untouched.  With
- *   L2 > L1 every row of w is written to its end.  DropKey dropout is not
- *   implemented (dropout must be 0).
+ *   L2 > L1 every row of w is written to its end.  Without dropout use
+ *   mega_attention_fwd; with DropKey dropout (softmax.cuh:135-196,
+ *   attention_kernel.cu:99-116) mega_attention_dropkey_fwd, below.
  *   `workspace`: mega_attention_workspace_bytes(B, L1, L2, NH, H1, H2, 0) bytes.
  * ---------------------------------------------------------------------- */
 int64_t mega_attention_workspace_bytes(int64_t B, int64_t L1, int64_t L2, int64_t NH,
@@ -223,6 +224,24 @@ int mega_attention_fwd(const void* q, const void* k, const void* v, int dtype,
                        int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1,
                        int64_t H2, double scale, int causal, void* y, void* w,
                        void* workspace, void* stream);
+
+/* attention_fwd with dropout > 0 (attention_kernel.cu:99-116, softmax.cuh:135-196):
+ *   before the softmax every kept key of every row is taken out (score -> -inf)
+ *   with probability `dropout`; the survivors are not rescaled; a row that
+ *   loses all its keys becomes 0.  The backward is mega_attention_bwd unchanged
+ *   (a dropped key has probability 0 in w).  The draw for (row i, column j),
+ *   i = (b * NH + head) * L1 + r, is word j % 4 of Philox4x32-10 with counter
+ *   (j / 4, i, offset & 0xffffffff, offset >> 32) and key (seed & 0xffffffff,
+ *   seed >> 32): dropped iff (word >> 8) * 2^-24 < (float)dropout.  The reference
+ *   takes (seed, offset) from PyTorch's CUDA generator and walks curand's
+ *   per-thread streams, so the two masks differ for the same seed while their
+ *   distribution is the same; a caller that wants fresh masks advances `offset`
+ *   by any amount between calls.  dropout == 0 is mega_attention_fwd. */
+int mega_attention_dropkey_fwd(const void* q, const void* k, const void* v, int dtype,
+                               int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1,
+                               int64_t H2, double scale, int causal, double dropout,
+                               uint64_t seed, uint64_t offset, void* y, void* w,
+                               void* workspace, void* stream);
 
 /* Replaces attention_bwd(dy, q, k, v, w, scale, use_causal_mask) -> (dq, dk, dv)
  *   reference: attention_kernel.cu:135-257,283-303, softmax.cuh:198-234,
@@ -269,7 +288,9 @@ int mega_fftconv_residual_bwd_saved(const void* dy, int dtype, const void* spec_
  *   overwritten by y = softmax over the last axis in float32; with `causal`
  *   row r keeps columns 0 .. L2 - L1 + r (L2 >= L1) and the rest of the row
  *   becomes 0.  The caller copies x first if it must survive (the reference
- *   returns a new tensor).  DropKey dropout is not implemented.
+ *   returns a new tensor).  mega_attention_softmax_dropkey_fwd is the same with
+ *   DropKey dropout (attention_softmax_kernel.cu:50-65); rows are numbered
+ *   i = matrix * L1 + r and drawn as described at mega_attention_dropkey_fwd.
  * Replaces attention_softmax_bwd(y_grad, y, use_causal_mask) -> x_grad
  *   reference: attention_softmax_kernel.cu:68-94,110-123, softmax.cuh:198-234,
  *              binding attention_softmax.cc:12-18.
@@ -277,8 +298,28 @@ int mega_fftconv_residual_bwd_saved(const void* dy, int dtype, const void* spec_
  * ---------------------------------------------------------------------- */
 int mega_attention_softmax_fwd(void* x, int dtype, int64_t Z, int64_t L1, int64_t L2,
                                int causal, void* stream);
+int mega_attention_softmax_dropkey_fwd(void* x, int dtype, int64_t Z, int64_t L1, int64_t L2,
+                                       int causal, double dropout, uint64_t seed,
+                                       uint64_t offset, void* stream);
 int mega_attention_softmax_bwd(const void* y, void* dy, int dtype, int64_t Z, int64_t L1,
                                int64_t L2, int causal, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Dropout that keeps no mask and no generator state.
+ *
+ * Replaces memory_efficient_dropout_fwd / _bwd
+ *   reference: megalodon/modules/fused_ops/memory_efficient_dropout.py:39-96
+ *   (bernoulli(1 - p) / (1 - p) noise, rebuilt in the backward by replaying the
+ *   CUDA generator from its saved state).
+ *   out[e] = in[e] / (1 - p) if element e is kept, else 0; e is kept iff word
+ *   e % 4 of Philox4x32-10 with counter (e / 4 as two 32-bit words, offset as
+ *   two 32-bit words) and key seed gives (word >> 8) * 2^-24 >= (float)p.  The
+ *   backward is the same call on the gradient with the same (p, seed, offset).
+ *   `in` and `out` (n elements of `dtype`: float32, bfloat16 or float16) may be
+ *   the same buffer.  p == 1 gives zeros (the reference's 0 / 0 gives NaN).
+ * ---------------------------------------------------------------------- */
+int mega_dropout(const void* in, int dtype, int64_t n, double p, uint64_t seed, uint64_t offset,
+                 void* out, void* stream);
 
 #ifdef __cplusplus
 }

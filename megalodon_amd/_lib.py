@@ -59,6 +59,10 @@ def i64(v: int) -> ctypes.c_int64:
     return _c_i64(int(v))
 
 
+def u64(v: int) -> ctypes.c_uint64:
+    return ctypes.c_uint64(int(v))
+
+
 def f64(v: float) -> ctypes.c_double:
     return ctypes.c_double(float(v))
 

@@ -400,6 +400,29 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
   }  // work item
 }
 
+// ---- DropKey (softmax.cuh:135-196) ----------------------------------------------
+// With probability `p` a key is taken out of a row (its score becomes -inf)
+// before the softmax; the survivors are not rescaled, and the backward needs no
+// mask because a dropped key has probability 0.  The reference draws from
+// curand's Philox stream of the thread that holds the element; here the draw of
+// element (row i, column j) is a pure function of its position, so it does not
+// depend on the kernel flavour or the element type: Philox4x32-10 with counter
+// (j / 4, i, offset_lo, offset_hi) and key (seed_lo, seed_hi) gives four words,
+// element j takes word j % 4, u = (word >> 8) * 2^-24, dropped iff u < p.
+// i counts rows over all matrices (i = matrix * L1 + r < 2^32).
+struct DropKey {
+  float p;
+  uint32_t seed_lo, seed_hi, off_lo, off_hi;
+};
+
+// drops[e] for the four columns 4 * quad .. 4 * quad + 3 of row i
+__device__ __forceinline__ void dropkey_quad(const DropKey& dk, uint32_t i, uint32_t quad, bool* drops) {
+  uint32_t w[4];
+  philox4x32_10(quad, i, dk.off_lo, dk.off_hi, dk.seed_lo, dk.seed_hi, w);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) drops[e] = static_cast<float>(w[e] >> 8) * 0x1p-24f < dk.p;
+}
+
 // ---- causal softmax over rows (in place), one wavefront per row ---------------
 // `coff` < 0: every row keeps all L2 columns.  `coff` = L2 - L1 >= 0 (causal,
 // bottom-right aligned, softmax.cuh:99-100): row r keeps columns [0, n) with
@@ -407,25 +430,36 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
 // `zfull` = 0 only up to the end of its 256-column tile, which is all the
 // products of the fused attention read.
 // softmax.cuh:86-131.
-template <int DT>
+template <int DT, bool DROP>
 __global__ __launch_bounds__(kThreads) void softmax_fwd_kernel(uint16_t* w, int L1, int L2,
-                                                              int coff, int zfull) {
+                                                              int coff, int zfull, DropKey dk) {
   // grid.y carries the batch*heads index; grid.x covers the L1 rows
   const int lane = threadIdx.x % kWave;
   const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   if (r >= L1) return;
+  const uint32_t row = blockIdx.y * static_cast<uint32_t>(L1) + r;
   uint16_t* x = w + (static_cast<int64_t>(blockIdx.y) * L1 + r) * L2;
   const int n = coff >= 0 ? min(r + 1 + coff, L2) : L2;
   const int nz = (coff == 0 && !zfull) ? min(L2, (r / kTile + 1) * kTile) : L2;
+  const auto score = [&](int j) {
+    float v = Elem<DT>::load(x + j);
+    if (DROP) {
+      bool drops[4];
+      dropkey_quad(dk, row, static_cast<uint32_t>(j) >> 2, drops);
+      if (drops[j & 3]) v = -INFINITY;
+    }
+    return v;
+  };
   float m = -INFINITY;
-  for (int j = lane; j < n; j += kWave) m = fmaxf(m, Elem<DT>::load(x + j));
+  for (int j = lane; j < n; j += kWave) m = fmaxf(m, score(j));
   m = wave_max(m);
+  if (m == -INFINITY) m = 0.f;  // nothing kept: the row becomes 0 (softmax.cuh:113-116)
   float d = 0.f;
-  for (int j = lane; j < n; j += kWave) d += __expf(Elem<DT>::load(x + j) - m);
+  for (int j = lane; j < n; j += kWave) d += __expf(score(j) - m);
   d = wave_sum(d);
   const float c = d == 0.f ? 0.f : 1.f / d;
   for (int j = lane; j < nz; j += kWave) {
-    const float v = j < n ? __expf(Elem<DT>::load(x + j) - m) * c : 0.f;
+    const float v = j < n ? __expf(score(j) - m) * c : 0.f;
     Elem<DT>::store(x + j, v);
   }
 }
@@ -461,12 +495,13 @@ __device__ __forceinline__ uint4 pack8(const float* v) {
 
 // Same contract with the row held in registers: needs L2 % 8 == 0, a 16-byte
 // aligned base and L2 <= 64 * 8 * NCH; one read and one write of the row.
-template <int DT, int NCH>
+template <int DT, int NCH, bool DROP>
 __global__ __launch_bounds__(kThreads) void softmax_fwd_vec_kernel(uint16_t* w, int L1, int L2,
-                                                                  int coff, int zfull) {
+                                                                  int coff, int zfull, DropKey dk) {
   const int lane = threadIdx.x % kWave;
   const int r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   if (r >= L1) return;
+  const uint32_t row = blockIdx.y * static_cast<uint32_t>(L1) + r;
   uint16_t* x = w + (static_cast<int64_t>(blockIdx.y) * L1 + r) * L2;
   const int n = coff >= 0 ? min(r + 1 + coff, L2) : L2;
   const int nz = (coff == 0 && !zfull) ? min(L2, (r / kTile + 1) * kTile) : L2;
@@ -477,6 +512,14 @@ __global__ __launch_bounds__(kThreads) void softmax_fwd_vec_kernel(uint16_t* w, 
     const int c8 = (lane + kWave * i) * 8;
     if (c8 < n) {
       unpack8<DT>(*reinterpret_cast<const uint4*>(x + c8), v[i]);
+      if (DROP) {
+        bool drops[8];
+        dropkey_quad(dk, row, static_cast<uint32_t>(c8) >> 2, drops);
+        dropkey_quad(dk, row, (static_cast<uint32_t>(c8) >> 2) + 1, drops + 4);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (drops[e]) v[i][e] = -INFINITY;
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         if (c8 + e >= n) v[i][e] = -INFINITY;
@@ -488,6 +531,7 @@ __global__ __launch_bounds__(kThreads) void softmax_fwd_vec_kernel(uint16_t* w, 
     }
   }
   m = wave_max(m);
+  if (m == -INFINITY) m = 0.f;  // nothing kept: the row becomes 0 (softmax.cuh:113-116)
   float d = 0.f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i)
@@ -573,18 +617,21 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_vec_kernel(const uint16_
 
 template <int DT>
 int launch_softmax(const uint16_t* p, uint16_t* x, int64_t Z, int64_t L1, int64_t L2, int causal,
-                   hipStream_t s, int zfull = 0) {
+                   hipStream_t s, int zfull = 0, const DropKey* drop = nullptr) {
   const int coff = causal ? static_cast<int>(L2 - L1) : -1;
   // p == nullptr: forward over x in place; else backward with probabilities p
   if (Z == 0 || L1 == 0 || L2 == 0) return MEGA_OK;
   const dim3 grid((unsigned)((L1 + 3) / 4), (unsigned)Z);
   const bool vec = L2 % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(p) % 16 == 0;
-#define MEGA_SOFTMAX(NCH)                                                                   \
-  if (p == nullptr)                                                                         \
-    softmax_fwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff, zfull); \
-  else                                                                                      \
-    softmax_bwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, coff, zfull);
+  const DropKey dk = drop ? *drop : DropKey{};
+#define MEGA_SOFTMAX(NCH)                                                                        \
+  if (p != nullptr)                                                                              \
+    softmax_bwd_vec_kernel<DT, NCH><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, coff, zfull); \
+  else if (drop)                                                                                 \
+    softmax_fwd_vec_kernel<DT, NCH, true><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff, zfull, dk); \
+  else                                                                                           \
+    softmax_fwd_vec_kernel<DT, NCH, false><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff, zfull, dk);
   if (vec && L2 <= 512) {
     MEGA_SOFTMAX(1)
   } else if (vec && L2 <= 1024) {
@@ -593,10 +640,12 @@ int launch_softmax(const uint16_t* p, uint16_t* x, int64_t Z, int64_t L1, int64_
     MEGA_SOFTMAX(4)
   } else if (vec && L2 <= 4096) {
     MEGA_SOFTMAX(8)
-  } else if (p == nullptr) {
-    softmax_fwd_kernel<DT><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff, zfull);
-  } else {
+  } else if (p != nullptr) {
     softmax_bwd_kernel<DT><<<grid, kThreads, 0, s>>>(p, x, (int)L1, (int)L2, coff, zfull);
+  } else if (drop) {
+    softmax_fwd_kernel<DT, true><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff, zfull, dk);
+  } else {
+    softmax_fwd_kernel<DT, false><<<grid, kThreads, 0, s>>>(x, (int)L1, (int)L2, coff, zfull, dk);
   }
 #undef MEGA_SOFTMAX
   MEGA_CHECK_LAUNCH();
@@ -684,7 +733,7 @@ int check_attn(const char* who, int dtype, int64_t B, int64_t L1, int64_t L2, in
 template <int DT>
 int attn_fwd_impl(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64_t B, int64_t L1,
                   int64_t L2, int64_t NH, int64_t H1, int64_t H2, float scale, int causal,
-                  uint16_t* y, uint16_t* w, uint16_t* ws, hipStream_t s) {
+                  uint16_t* y, uint16_t* w, uint16_t* ws, hipStream_t s, const DropKey* drop) {
   (void)ws;
   const int Z = static_cast<int>(B * NH);
   // S = scale Q K^T  -> w
@@ -697,7 +746,7 @@ int attn_fwd_impl(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64
   int rc = launch_gemm<DT>(g, Z, s);
   if (rc != MEGA_OK) return rc;
   // P = softmax(S) in place
-  if ((rc = launch_softmax<DT>(nullptr, w, Z, L1, L2, causal, s)) != MEGA_OK) return rc;
+  if ((rc = launch_softmax<DT>(nullptr, w, Z, L1, L2, causal, s, 0, drop)) != MEGA_OK) return rc;
   // Y = P V: V[key][c] is the k-major B operand
   GemmParams o{};
   o.A = w; o.B = v; o.C = y; o.M = (int)L1; o.N = (int)H2; o.K = (int)L2;
@@ -761,23 +810,57 @@ extern "C" int64_t mega_attention_workspace_bytes(int64_t B, int64_t L1, int64_t
   return attn_ws(B, L1, L2, NH, H1, H2, backward != 0).total;
 }
 
-extern "C" int mega_attention_fwd(const void* q, const void* k, const void* v, int dtype, int64_t B,
-                                  int64_t L1, int64_t L2, int64_t NH, int64_t H1, int64_t H2,
-                                  double scale, int causal, void* y, void* w, void* workspace,
-                                  void* stream) {
-  int rc = check_attn("mega_attention_fwd", dtype, B, L1, L2, NH, H1, H2, causal);
+// p in [0, 1]; p == 0 means no DropKey
+static int make_dropkey(const char* who, double dropout, uint64_t seed, uint64_t offset, int64_t rows,
+                        DropKey* dk) {
+  MEGA_CHECK_ARG(dropout >= 0.0 && dropout <= 1.0, "%s: dropout must lie in [0, 1]", who);
+  MEGA_CHECK_ARG(rows < (1ll << 32), "%s: more than 2^32 rows", who);
+  dk->p = static_cast<float>(dropout);
+  dk->seed_lo = static_cast<uint32_t>(seed);
+  dk->seed_hi = static_cast<uint32_t>(seed >> 32);
+  dk->off_lo = static_cast<uint32_t>(offset);
+  dk->off_hi = static_cast<uint32_t>(offset >> 32);
+  return MEGA_OK;
+}
+
+static int attention_fwd_entry(const char* who, const void* q, const void* k, const void* v, int dtype,
+                               int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1, int64_t H2,
+                               double scale, int causal, const DropKey* drop, void* y, void* w,
+                               void* workspace, void* stream) {
+  int rc = check_attn(who, dtype, B, L1, L2, NH, H1, H2, causal);
   if (rc != MEGA_OK) return rc;
   if (B == 0 || L1 == 0) return MEGA_OK;
-  MEGA_CHECK_ARG(q && k && v && y && w && workspace, "mega_attention_fwd: null pointer");
-  MEGA_CHECK_ARG(L2 >= 1, "mega_attention_fwd: no keys");
+  MEGA_CHECK_ARG(q && k && v && y && w && workspace, "%s: null pointer", who);
+  MEGA_CHECK_ARG(L2 >= 1, "%s: no keys", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
   auto u = [](const void* p) { return static_cast<const uint16_t*>(p); };
   auto m = [](void* p) { return static_cast<uint16_t*>(p); };
   if (dtype == MEGA_BF16)
     return attn_fwd_impl<MEGA_BF16>(u(q), u(k), u(v), B, L1, L2, NH, H1, H2, (float)scale, causal,
-                                    m(y), m(w), m(workspace), s);
+                                    m(y), m(w), m(workspace), s, drop);
   return attn_fwd_impl<MEGA_F16>(u(q), u(k), u(v), B, L1, L2, NH, H1, H2, (float)scale, causal,
-                                 m(y), m(w), m(workspace), s);
+                                 m(y), m(w), m(workspace), s, drop);
+}
+
+extern "C" int mega_attention_fwd(const void* q, const void* k, const void* v, int dtype, int64_t B,
+                                  int64_t L1, int64_t L2, int64_t NH, int64_t H1, int64_t H2,
+                                  double scale, int causal, void* y, void* w, void* workspace,
+                                  void* stream) {
+  return attention_fwd_entry("mega_attention_fwd", q, k, v, dtype, B, L1, L2, NH, H1, H2, scale,
+                             causal, nullptr, y, w, workspace, stream);
+}
+
+extern "C" int mega_attention_dropkey_fwd(const void* q, const void* k, const void* v, int dtype,
+                                          int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1,
+                                          int64_t H2, double scale, int causal, double dropout,
+                                          uint64_t seed, uint64_t offset, void* y, void* w,
+                                          void* workspace, void* stream) {
+  DropKey dk;
+  int rc = make_dropkey("mega_attention_dropkey_fwd", dropout, seed, offset,
+                        B >= 0 && NH >= 0 && L1 >= 0 ? B * NH * L1 : 0, &dk);
+  if (rc != MEGA_OK) return rc;
+  return attention_fwd_entry("mega_attention_dropkey_fwd", q, k, v, dtype, B, L1, L2, NH, H1, H2,
+                             scale, causal, dropout > 0.0 ? &dk : nullptr, y, w, workspace, stream);
 }
 
 extern "C" int mega_attention_bwd(const void* dy, const void* q, const void* k, const void* v,
@@ -811,15 +894,31 @@ static int check_softmax(const char* who, int dtype, int64_t Z, int64_t L1, int6
   return MEGA_OK;
 }
 
-extern "C" int mega_attention_softmax_fwd(void* x, int dtype, int64_t Z, int64_t L1, int64_t L2,
-                                          int causal, void* stream) {
-  int rc = check_softmax("mega_attention_softmax_fwd", dtype, Z, L1, L2, causal);
+static int softmax_fwd_entry(const char* who, void* x, int dtype, int64_t Z, int64_t L1, int64_t L2,
+                             int causal, const DropKey* drop, void* stream) {
+  int rc = check_softmax(who, dtype, Z, L1, L2, causal);
   if (rc != MEGA_OK) return rc;
-  MEGA_CHECK_ARG(x != nullptr || Z * L1 * L2 == 0, "mega_attention_softmax_fwd: null pointer");
+  MEGA_CHECK_ARG(x != nullptr || Z * L1 * L2 == 0, "%s: null pointer", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == MEGA_BF16)
-    return launch_softmax<MEGA_BF16>(nullptr, static_cast<uint16_t*>(x), Z, L1, L2, causal, s, 1);
-  return launch_softmax<MEGA_F16>(nullptr, static_cast<uint16_t*>(x), Z, L1, L2, causal, s, 1);
+    return launch_softmax<MEGA_BF16>(nullptr, static_cast<uint16_t*>(x), Z, L1, L2, causal, s, 1, drop);
+  return launch_softmax<MEGA_F16>(nullptr, static_cast<uint16_t*>(x), Z, L1, L2, causal, s, 1, drop);
+}
+
+extern "C" int mega_attention_softmax_fwd(void* x, int dtype, int64_t Z, int64_t L1, int64_t L2,
+                                          int causal, void* stream) {
+  return softmax_fwd_entry("mega_attention_softmax_fwd", x, dtype, Z, L1, L2, causal, nullptr, stream);
+}
+
+extern "C" int mega_attention_softmax_dropkey_fwd(void* x, int dtype, int64_t Z, int64_t L1,
+                                                  int64_t L2, int causal, double dropout,
+                                                  uint64_t seed, uint64_t offset, void* stream) {
+  DropKey dk;
+  int rc = make_dropkey("mega_attention_softmax_dropkey_fwd", dropout, seed, offset,
+                        Z >= 0 && L1 >= 0 ? Z * L1 : 0, &dk);
+  if (rc != MEGA_OK) return rc;
+  return softmax_fwd_entry("mega_attention_softmax_dropkey_fwd", x, dtype, Z, L1, L2, causal,
+                           dropout > 0.0 ? &dk : nullptr, stream);
 }
 
 extern "C" int mega_attention_softmax_bwd(const void* y, void* dy, int dtype, int64_t Z, int64_t L1,

@@ -535,13 +535,42 @@ def _attn_dims(q, k, v):
     return B, L1, L2, NH, H1, H2
 
 
+def dropkey_philox_state(dev: torch.device, columns: int) -> Tuple[int, int]:
+    """(seed, offset) for one DropKey launch, taken from PyTorch's generator of
+    the device the way the reference does (attention_kernel.cu:100-109:
+    `philox_cuda_state(capacity)`): the offset is read and then advanced, so
+    successive launches draw different masks and `torch.manual_seed` /
+    `torch.cuda.set_rng_state` reproduce them."""
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    gen = torch.cuda.default_generators[index]
+    seed, offset = gen.initial_seed(), gen.get_offset()
+    gen.set_offset(offset + 4 * max(1, (columns + 3) // 4))
+    return seed & 0xFFFFFFFFFFFFFFFF, offset
+
+
 def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, dropout: float,
                   use_causal_mask: bool) -> Tuple[torch.Tensor, torch.Tensor]:
-    """(y, w): y (B, L1, N, H2), w = softmax probabilities (B, N, L1, L2)."""
+    """(y, w): y (B, L1, N, H2), w = softmax probabilities (B, N, L1, L2).
+    `dropout` > 0 is DropKey (softmax.cuh:135-196): keys leave a row with that
+    probability before the softmax, drawn from the device generator's
+    (seed, offset)."""
     dev = _require_cuda(q, k, v)
-    if dropout != 0.0:
-        raise NotImplementedError("DropKey dropout is not implemented (dropout must be 0)")
+    if not 0.0 <= dropout <= 1.0:
+        raise RuntimeError("attention_fwd: dropout must lie in [0, 1]")
     B, L1, L2, NH, H1, H2 = _attn_dims(q, k, v)
+    if dropout > 0.0:
+        qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
+        y = torch.empty((B, L1, NH, H2), dtype=v.dtype, device=dev)
+        w = torch.empty((B, NH, L1, L2), dtype=v.dtype, device=dev)
+        ws = _attn_workspace(B, L1, L2, NH, H1, H2, False, dev)
+        seed, offset = dropkey_philox_state(dev, L2)
+        with torch.cuda.device(dev):
+            _lib.call("mega_attention_dropkey_fwd", _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc),
+                      _lib.i32(_lib.dtype_code(q.dtype)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2),
+                      _lib.i64(NH), _lib.i64(H1), _lib.i64(H2), _lib.f64(scale),
+                      _lib.i32(1 if use_causal_mask else 0), _lib.f64(dropout), _lib.u64(seed),
+                      _lib.u64(offset), _lib.ptr(y), _lib.ptr(w), _lib.ptr(ws), _lib.stream_ptr(dev))
+        return y, w
     qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
     y = torch.empty((B, L1, NH, H2), dtype=v.dtype, device=dev)
     w = torch.empty((B, NH, L1, L2), dtype=v.dtype, device=dev)
@@ -585,10 +614,17 @@ def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool
     (bottom-right aligned) when asked; x (..., L1, L2) bfloat16 / float16
     (attention_softmax_kernel.cu:96-108)."""
     dev = _require_cuda(x)
-    if dropout != 0.0:
-        raise NotImplementedError("DropKey dropout is not implemented (dropout must be 0)")
+    if not 0.0 <= dropout <= 1.0:
+        raise RuntimeError("attention_softmax_fwd: dropout must lie in [0, 1]")
     Z, L1, L2 = _softmax_dims(x)
     y = x.contiguous().clone()
+    if dropout > 0.0:
+        seed, offset = dropkey_philox_state(dev, L2)
+        with torch.cuda.device(dev):
+            _lib.call("mega_attention_softmax_dropkey_fwd", _lib.ptr(y), _lib.i32(_lib.dtype_code(x.dtype)),
+                      _lib.i64(Z), _lib.i64(L1), _lib.i64(L2), _lib.i32(1 if use_causal_mask else 0),
+                      _lib.f64(dropout), _lib.u64(seed), _lib.u64(offset), _lib.stream_ptr(dev))
+        return y
     with torch.cuda.device(dev):
         _lib.call("mega_attention_softmax_fwd", _lib.ptr(y), _lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(Z),
                   _lib.i64(L1), _lib.i64(L2), _lib.i32(1 if use_causal_mask else 0), _lib.stream_ptr(dev))
@@ -608,6 +644,20 @@ def attention_softmax_bwd(y_grad: torch.Tensor, y: torch.Tensor, use_causal_mask
                   _lib.i64(Z), _lib.i64(L1), _lib.i64(L2), _lib.i32(1 if use_causal_mask else 0),
                   _lib.stream_ptr(dev))
     return dx
+
+
+def dropout(x: torch.Tensor, p: float, seed: int, offset: int) -> torch.Tensor:
+    """x / (1 - p) where element e is kept, 0 elsewhere; the mask is a pure
+    function of (seed, offset, e), so the same call on a gradient is the
+    backward (replaces the generator replay of
+    megalodon/modules/fused_ops/memory_efficient_dropout.py:60-96)."""
+    dev = _require_cuda(x)
+    xc = x.contiguous()
+    y = torch.empty_like(xc)
+    with torch.cuda.device(dev):
+        _lib.call("mega_dropout", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(xc.numel()),
+                  _lib.f64(p), _lib.u64(seed), _lib.u64(offset), _lib.ptr(y), _lib.stream_ptr(dev))
+    return y
 
 
 def timestep_norm_fwd(x: torch.Tensor, prev_count: torch.Tensor, prev_mean: torch.Tensor, prev_var: torch.Tensor,

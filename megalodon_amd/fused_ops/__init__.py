@@ -5,6 +5,8 @@ from .cema_kernel import cema_kernel
 from .ema_hidden import ema_hidden
 from .ema_parameters import ema_parameters
 from .fftconv import fftconv, fftconv_residual
+from .memory_efficient_dropout import memory_efficient_dropout
 
-__all__ = ["attention_softmax", "cema_kernel", "ema_hidden", "ema_parameters", "fftconv", "fftconv_residual", "swift_efficient_attention", "swift_efficient_attention_fwd",
+__all__ = ["attention_softmax", "cema_kernel", "ema_hidden", "ema_parameters", "fftconv", "fftconv_residual", "memory_efficient_dropout",
+           "swift_efficient_attention", "swift_efficient_attention_fwd",
            "swift_efficient_attention_bwd"]

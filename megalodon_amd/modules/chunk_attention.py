@@ -12,7 +12,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from ..fused_ops import swift_efficient_attention
+from ..fused_ops import memory_efficient_dropout, swift_efficient_attention
 
 
 def apply_rotary_emb(xq: Tensor, xk: Tensor, freqs_cis: Optional[Tensor], backward: bool = False):
@@ -85,6 +85,7 @@ class _InnerAttention(nn.Module):
             assert mask is not None
             scores = torch.matmul(xq, xk.transpose(2, 3)) + mask
             scores = F.softmax(scores, dim=-1, dtype=torch.float32).to(xq)
+            scores = memory_efficient_dropout(scores, self.dropout, self.training)
             output = torch.matmul(scores, xv).transpose(1, 2).contiguous()
         else:
             assert mask is None

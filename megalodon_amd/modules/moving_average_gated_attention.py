@@ -4,7 +4,8 @@ megalodon/model/mega.py:43-88): TimestepNorm -> CEMA -> RMSNorm -> z/q/k, v, r
 projections -> chunk attention -> gate -> wh1 + wh2 -> residual, then the
 normalised feed-forward network.  World size 1: the Column/RowParallelLinear
 layers are `nn.Linear`, the chunk-parallel send/recv branches are not part of
-this path, dropout is 0.  With `cache` = (attention cache, (count, mean, var)
+this path.  The three dropouts sit where the reference has them (:316, :336,
+:340; DropKey inside the attention operator).  With `cache` = (attention cache, (count, mean, var)
 of TimestepNorm, EMA state) a sequence can be fed piece by piece (:283-297,
 :306-308, :345-346): every piece continues the running statistics, the EMA
 state and the unfinished attention chunk of the one before."""
@@ -16,6 +17,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 from torch.nn import Parameter
 
+from ..fused_ops import memory_efficient_dropout
 from .chunk_attention import _InnerAttention
 from .complex_exponential_moving_average import MultiHeadComplexEMA
 from .layer_norm import FusedRMSNorm
@@ -31,8 +33,9 @@ class MovingAverageGatedAttention(nn.Module):
                  efficient_attn: Optional[str] = "fused", norm_num_groups: Optional[int] = None,
                  norm_affine: bool = True, norm_eps: float = 1e-5, init_std: float = 0.02):
         super().__init__()
-        assert dropout == 0.0 and attention_dropout == 0.0 and hidden_dropout == 0.0, \
-            "dropout is outside the path built here"
+        self.dropout = dropout
+        self.attention_dropout = attention_dropout
+        self.hidden_dropout = hidden_dropout
         self.mdim, self.hdim, self.zdim, self.ndim = mdim, hdim, zdim, ndim
         self.num_heads = num_heads
         assert zdim % num_heads == 0 and hdim % num_heads == 0
@@ -82,6 +85,7 @@ class MovingAverageGatedAttention(nn.Module):
         # B x L x D
         out_cema = out_cema.transpose(1, 2)
         mx = self.rmsnorm(out_cema)
+        mx = memory_efficient_dropout(mx, self.hidden_dropout, self.training)
 
         # B x L x S -> B x L x H x S/H -> B x L x S
         z = self.wz(mx).view(bsz, seq_len, self.local_heads, self.z_head_dim)
@@ -96,10 +100,11 @@ class MovingAverageGatedAttention(nn.Module):
         r = F.silu(self.wr(mx))
 
         attn, cache_attn = self.inner_attention(q.contiguous(), k.contiguous(), v, mask, freqs_cis, cache_attn)
-        attn = attn * r
+        attn = memory_efficient_dropout(attn * r, self.hidden_dropout, self.training)
 
         # B x L x E -> B x L x D
         h = self.wh1(mx) + self.wh2(attn)
+        h = memory_efficient_dropout(h, self.dropout, self.training)
         out = h + residual
         if cache is not None:
             cache = (cache_attn, cache_norm, hx)
@@ -116,16 +121,19 @@ class MegaBlock(nn.Module):
     def __init__(self, model_dim: int, z_dim: int, value_dim: int, num_heads: int, cema_ndim: int,
                  chunk_size: int, ffn_hidden_dim: int, norm_num_groups: int, swiglu: bool = True,
                  efficient_attn: Optional[str] = "fused", norm_affine: bool = True, norm_eps: float = 1e-5,
-                 rescale_nffn: bool = False, layer_id: int = 0, init_std: float = 0.02):
+                 rescale_nffn: bool = False, layer_id: int = 0, init_std: float = 0.02, dropout: float = 0.0,
+                 attention_dropout: float = 0.0, hidden_dropout: float = 0.0):
         super().__init__()
         self.layer_id = layer_id
         self.mega = MovingAverageGatedAttention(
             mdim=model_dim, zdim=z_dim, hdim=value_dim, num_heads=num_heads, ndim=cema_ndim,
+            dropout=dropout, attention_dropout=attention_dropout, hidden_dropout=hidden_dropout,
             chunk_size=chunk_size, efficient_attn=efficient_attn, norm_num_groups=norm_num_groups,
             norm_affine=norm_affine, norm_eps=norm_eps, init_std=init_std)
         rescale = 0.1 * (0.5 ** layer_id) if rescale_nffn else None
         self.nffn = NormalizedFeedForwardNetwork(
-            model_dim=model_dim, ffn_hidden_dim=ffn_hidden_dim, swiglu=swiglu, norm_affine=norm_affine,
+            model_dim=model_dim, ffn_hidden_dim=ffn_hidden_dim, dropout=dropout, hidden_dropout=hidden_dropout,
+            swiglu=swiglu, norm_affine=norm_affine,
             norm_eps=norm_eps, rescale=rescale, init_std=init_std)
 
     def forward(self, x: Tensor, freqs_cis: Optional[Tensor] = None, mask: Optional[Tensor] = None, cache=None):

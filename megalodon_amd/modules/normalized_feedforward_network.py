@@ -1,10 +1,12 @@
 """`NormalizedFeedForwardNetwork` (megalodon/modules/normalized_feedforward_network.py:15-98)
 for model-parallel world size 1: Column/RowParallelLinear are plain `nn.Linear`
-(megalodon/modules/model_parallel/layers.py:222-235,321-341), dropout 0."""
+(megalodon/modules/model_parallel/layers.py:222-235,321-341); the two dropouts
+sit where the reference has them (:83-90)."""
 import torch
 import torch.nn.functional as F
 from torch import nn
 
+from ..fused_ops import memory_efficient_dropout
 from .layer_norm import FusedLayerNorm
 
 
@@ -12,7 +14,8 @@ class NormalizedFeedForwardNetwork(nn.Module):
     def __init__(self, model_dim, ffn_hidden_dim, dropout=0.0, hidden_dropout=0.0, swiglu=False,
                  norm_affine=True, norm_eps=1e-5, rescale=None, init_std=0.02):
         super().__init__()
-        assert dropout == 0.0 and hidden_dropout == 0.0, "dropout is outside the path built here"
+        self.dropout = dropout
+        self.hidden_dropout = hidden_dropout
         self.model_dim = model_dim
         self.hidden_dim = ffn_hidden_dim
         self.swiglu = swiglu
@@ -39,7 +42,9 @@ class NormalizedFeedForwardNetwork(nn.Module):
             hidden = F.silu(self.fc1(x)) * self.fc3(x)
         else:
             hidden = F.silu(self.fc1(x))
+        hidden = memory_efficient_dropout(hidden, self.hidden_dropout, self.training)
         x = self.fc2(hidden)
+        x = memory_efficient_dropout(x, self.dropout, self.training)
         return self.rescale(x) + residual
 
     def extra_repr(self) -> str:

@@ -26,6 +26,11 @@ Pinning status (what independently fixes each function; see tests/test_oracle_*.
 * ``attention.chunk_attention_fwd/bwd``: pinned by row-0 / permutation /
   softmax-normalisation properties and autograd over the textbook formula
   (which is the reference's own unfused branch).
+* ``philox.philox4x32_10`` and the masks built on it (DropKey, dropout):
+  pinned by the known-answer vectors Random123 ships for Philox4x32-10 and by
+  element-by-element evaluation.  The reference's masks come from curand's
+  per-thread streams and are NOT reproduced: parity unpinned for the mask
+  stream itself; what is checked is the operator under an identical mask.
 
 The reference ships no tests, golden vectors or fixtures for any of these
 functions, so none of them can be checked against reference-held vectors.

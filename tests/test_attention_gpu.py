@@ -127,8 +127,8 @@ def test_autograd_function_and_module():
 
 def test_unsupported_cases_fail_loudly():
     q = torch.zeros(1, 8, 1, 8, device="cuda", dtype=torch.bfloat16)
-    with pytest.raises(NotImplementedError):
-        ops.attention_fwd(q, q, q, 1.0, 0.1, True)   # DropKey
+    with pytest.raises(RuntimeError, match=r"\[0, 1\]"):
+        ops.attention_fwd(q, q, q, 1.0, 1.5, True)   # not a probability
     with pytest.raises(RuntimeError, match="bfloat16"):
         ops.attention_fwd(q.float(), q.float(), q.float(), 1.0, 0.0, True)
 
