@@ -321,6 +321,55 @@ int mega_attention_softmax_bwd(const void* y, void* dy, int dtype, int64_t Z, in
 int mega_dropout(const void* in, int dtype, int64_t n, double p, uint64_t seed, uint64_t offset,
                  void* out, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Block glue: the transposes around the EMA convolution and the SiLU gates.
+ *
+ * mega_transpose: in (Z, R, C) -> out (Z, C, R), contiguous, `in` != `out`.
+ *   Replaces the strided copies behind `out_tsn.transpose(1, 2)` and
+ *   `out_cema.transpose(1, 2)` (megalodon/modules/moving_average_gated_attention.py:
+ *   299-300,314, and their gradients).  16-bit elements with R % 8 == 0,
+ *   C % 8 == 0 and 16-byte aligned buffers move in 128 x 128 tiles with 16-byte
+ *   accesses on both sides; everything else takes a 32 x 32 element-wise path.
+ * mega_silu_mul_fwd: out = silu(a) * b, n elements of `dtype`, float32 inside
+ *   with one rounding (PyTorch's `F.silu(a) * b` rounds twice).
+ *   Replaces `F.silu(self.fc1(x)) * self.fc3(x)`
+ *   (normalized_feedforward_network.py:82) and `attn * F.silu(self.wr(mx))`
+ *   (moving_average_gated_attention.py:333-336).
+ * mega_silu_mul_bwd: da = dout * b * s * (1 + a (1 - s)), db = dout * a * s,
+ *   s = sigmoid(a); the forward's result is not needed.
+ * ---------------------------------------------------------------------- */
+int mega_transpose(const void* in, int dtype, int64_t Z, int64_t R, int64_t C, void* out,
+                   void* stream);
+int mega_silu_mul_fwd(const void* a, const void* b, int dtype, int64_t n, void* out, void* stream);
+int mega_silu_mul_bwd(const void* dout, const void* a, const void* b, int dtype, int64_t n,
+                      void* da, void* db, void* stream);
+
+/* ------------------------------------------------------------------------
+ * LayerNorm / RMSNorm over the last axis, stored weight = gamma - 1.
+ *
+ * Replaces FusedLayerNorm / FusedRMSNorm (megalodon/modules/layer_norm.py:14-66:
+ *   `weight + 1` handed to apex's fused_layer_norm_cuda, which is not in the
+ *   reference tree; apex's definition is the usual one restated here).
+ *   x, y (rows, D) of `dtype`; weight, bias (D) of the same dtype or null
+ *   (no affine parameters); mean, rstd (rows) float32 are saved for the
+ *   backward.  rms == 0: mean = E[x], var = E[(x - mean)^2],
+ *   y = (x - mean) rstd (weight + 1) + bias.  rms != 0: rstd = 1/sqrt(E[x^2] + eps),
+ *   y = x rstd (weight + 1); `bias` and `mean` are ignored.  float32 inside.
+ *   16-bit rows of 128, 256, 512, 1024, 2048 or 4096 elements stay in
+ *   registers (x read once); other shapes re-read the row from cache.
+ * Backward: dx, and (when `dweight` is not null) dweight, dbias (null for rms
+ *   or no bias) in `dtype`, summed over rows in a fixed order.
+ *   `workspace`: mega_layer_norm_workspace_bytes(rows, D) bytes, needed when
+ *   dweight is not null.
+ * ---------------------------------------------------------------------- */
+int64_t mega_layer_norm_workspace_bytes(int64_t rows, int64_t D);
+int mega_layer_norm_fwd(const void* x, const void* weight, const void* bias, int dtype,
+                        int64_t rows, int64_t D, double eps, int rms, void* y, float* mean,
+                        float* rstd, void* stream);
+int mega_layer_norm_bwd(const void* dy, const void* x, const void* weight, const float* mean,
+                        const float* rstd, int dtype, int64_t rows, int64_t D, int rms, void* dx,
+                        void* dweight, void* dbias, void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

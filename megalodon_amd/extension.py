@@ -660,6 +660,101 @@ def dropout(x: torch.Tensor, p: float, seed: int, offset: int) -> torch.Tensor:
     return y
 
 
+def transpose_last2(x: torch.Tensor) -> torch.Tensor:
+    """(..., R, C) -> contiguous (..., C, R): what `x.transpose(-2, -1).contiguous()`
+    returns, in one tiled pass (the BLD <-> BDL moves around the EMA convolution,
+    megalodon/modules/moving_average_gated_attention.py:299-300,314)."""
+    dev = _require_cuda(x)
+    if x.dim() < 2:
+        raise RuntimeError("transpose_last2: x needs at least two dimensions")
+    xc = x.contiguous()
+    R, C = xc.shape[-2], xc.shape[-1]
+    out = torch.empty(xc.shape[:-2] + (C, R), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_transpose", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
+                  _lib.i64(xc.numel() // max(1, R * C)), _lib.i64(R), _lib.i64(C), _lib.ptr(out),
+                  _lib.stream_ptr(dev))
+    return out
+
+
+def silu_mul_fwd(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """silu(a) * b (normalized_feedforward_network.py:82,
+    moving_average_gated_attention.py:333-336), float32 inside."""
+    dev = _require_cuda(a, b)
+    if a.shape != b.shape or a.dtype != b.dtype:
+        raise RuntimeError("silu_mul: a and b must have the same shape and dtype")
+    ac, bc = a.contiguous(), b.contiguous()
+    out = torch.empty_like(ac)
+    with torch.cuda.device(dev):
+        _lib.call("mega_silu_mul_fwd", _lib.ptr(ac), _lib.ptr(bc), _lib.i32(_lib.dtype_code(a.dtype)),
+                  _lib.i64(ac.numel()), _lib.ptr(out), _lib.stream_ptr(dev))
+    return out
+
+
+def silu_mul_bwd(out_grad: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(a_grad, b_grad) of silu(a) * b."""
+    dev = _require_cuda(out_grad, a, b)
+    if not (out_grad.shape == a.shape == b.shape) or not (out_grad.dtype == a.dtype == b.dtype):
+        raise RuntimeError("silu_mul_bwd: out_grad, a and b must have the same shape and dtype")
+    gc, ac, bc = out_grad.contiguous(), a.contiguous(), b.contiguous()
+    da, db = torch.empty_like(ac), torch.empty_like(bc)
+    with torch.cuda.device(dev):
+        _lib.call("mega_silu_mul_bwd", _lib.ptr(gc), _lib.ptr(ac), _lib.ptr(bc), _lib.i32(_lib.dtype_code(a.dtype)),
+                  _lib.i64(ac.numel()), _lib.ptr(da), _lib.ptr(db), _lib.stream_ptr(dev))
+    return da, db
+
+
+def layer_norm_fwd(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float,
+                   rms: bool) -> Tuple[torch.Tensor, Optional[torch.Tensor], torch.Tensor]:
+    """(y, mean, rstd) of LayerNorm / RMSNorm over the last axis with the stored
+    weight = gamma - 1 (megalodon/modules/layer_norm.py:30-33,62-65)."""
+    dev = _require_cuda(x)
+    D = x.shape[-1]
+    for t, name in ((weight, "weight"), (bias, "bias")):
+        if t is not None and (t.shape != (D,) or t.dtype != x.dtype or t.device != x.device):
+            raise RuntimeError(f"layer_norm: {name} must be ({D},) of x's dtype on x's device")
+    xc = x.contiguous()
+    rows = xc.numel() // D
+    y = torch.empty_like(xc)
+    mean = None if rms else torch.empty(rows, dtype=torch.float32, device=dev)
+    rstd = torch.empty(rows, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_layer_norm_fwd", _lib.ptr(xc), _lib.ptr(None if weight is None else weight.contiguous()),
+                  _lib.ptr(None if bias is None or rms else bias.contiguous()), _lib.i32(_lib.dtype_code(x.dtype)),
+                  _lib.i64(rows), _lib.i64(D), _lib.f64(eps), _lib.i32(1 if rms else 0), _lib.ptr(y),
+                  _lib.ptr(mean), _lib.ptr(rstd), _lib.stream_ptr(dev))
+    return y, mean, rstd
+
+
+def layer_norm_bwd(y_grad: torch.Tensor, x: torch.Tensor, weight: Optional[torch.Tensor],
+                   mean: Optional[torch.Tensor], rstd: torch.Tensor, rms: bool, has_bias: bool
+                   ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """(x_grad, weight_grad, bias_grad)."""
+    dev = _require_cuda(y_grad, x)
+    if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
+        raise RuntimeError("layer_norm_bwd: y_grad and x must have the same shape and dtype")
+    D = x.shape[-1]
+    xc, gc = x.contiguous(), y_grad.contiguous()
+    rows = xc.numel() // D
+    dx = torch.empty_like(xc)
+    if rows == 0:
+        return (dx, None if weight is None else torch.zeros_like(weight),
+                torch.zeros(D, dtype=x.dtype, device=dev) if has_bias and not rms else None)
+    dw = None if weight is None else torch.empty_like(weight)
+    db = torch.empty(D, dtype=x.dtype, device=dev) if (has_bias and not rms and weight is not None) else None
+    ws = None
+    if dw is not None:
+        fn = _lib.load().mega_layer_norm_workspace_bytes
+        fn.restype = _lib.ctypes.c_int64
+        ws = torch.empty(int(fn(_lib.i64(rows), _lib.i64(D))), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_layer_norm_bwd", _lib.ptr(gc), _lib.ptr(xc),
+                  _lib.ptr(None if weight is None else weight.contiguous()), _lib.ptr(mean), _lib.ptr(rstd),
+                  _lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(rows), _lib.i64(D), _lib.i32(1 if rms else 0),
+                  _lib.ptr(dx), _lib.ptr(dw), _lib.ptr(db), _lib.ptr(ws), _lib.stream_ptr(dev))
+    return dx, dw, db
+
+
 def timestep_norm_fwd(x: torch.Tensor, prev_count: torch.Tensor, prev_mean: torch.Tensor, prev_var: torch.Tensor,
                       gamma: torch.Tensor, beta: torch.Tensor, padding_mask: Optional[torch.Tensor], eps: float):
     """The non-group operator (megalodon/csrc/ops/timestep_norm.cc:23-105,

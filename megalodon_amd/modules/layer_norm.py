@@ -1,12 +1,20 @@
 """`FusedLayerNorm` / `FusedRMSNorm` with the reference's parameterisation
-(megalodon/modules/layer_norm.py:14-66: stored weight is `gamma - 1`), computed
-with PyTorch's own layer_norm / rms_norm (the reference calls apex's
-fused_layer_norm_cuda, which is not part of the hot path built here)."""
+(megalodon/modules/layer_norm.py:14-66: stored weight is `gamma - 1`; the
+reference adds 1 and calls apex's fused_layer_norm_cuda).  On the GPU the
+normalisation over the last axis runs as one streaming kernel that takes the
+stored weight as it is; CPU tensors and multi-axis shapes use PyTorch's
+layer_norm / rms_norm."""
 import numbers
 
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
+
+from ..fused_ops import layer_norm_plus_one
+
+
+def _param_dtype(weight, input_):
+    return input_.dtype if weight is None else weight.dtype
 
 
 class FusedLayerNorm(nn.Module):
@@ -25,6 +33,8 @@ class FusedLayerNorm(nn.Module):
             self.register_parameter("bias", None)
 
     def forward(self, input_):
+        if input_.is_cuda and len(self.normalized_shape) == 1 and input_.dtype == _param_dtype(self.weight, input_):
+            return layer_norm_plus_one(input_, self.weight, self.bias, self.eps, False)
         weight = None if self.weight is None else self.weight + 1.0
         return F.layer_norm(input_, self.normalized_shape, weight, self.bias, self.eps)
 
@@ -46,6 +56,8 @@ class FusedRMSNorm(nn.Module):
             self.register_parameter("weight", None)
 
     def forward(self, input_):
+        if input_.is_cuda and len(self.normalized_shape) == 1 and input_.dtype == _param_dtype(self.weight, input_):
+            return layer_norm_plus_one(input_, self.weight, None, self.eps, True)
         weight = None if self.weight is None else self.weight + 1.0
         return F.rms_norm(input_, self.normalized_shape, weight, self.eps)
 

@@ -17,7 +17,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 from torch.nn import Parameter
 
-from ..fused_ops import memory_efficient_dropout
+from ..fused_ops import memory_efficient_dropout, silu_mul, transpose_last2
 from .chunk_attention import _InnerAttention
 from .complex_exponential_moving_average import MultiHeadComplexEMA
 from .layer_norm import FusedRMSNorm
@@ -78,12 +78,12 @@ class MovingAverageGatedAttention(nn.Module):
         # B x L x D
         out_tsn, prev_count, prev_mean, prev_var = self.timenorm(x, prev_count, prev_mean, prev_var)
         # B x D x L
-        out_cema, hx = self.cema(out_tsn.transpose(1, 2), hx, compute_last_state=cache_attn is not None)
+        out_cema, hx = self.cema(transpose_last2(out_tsn), hx, compute_last_state=cache_attn is not None)
         if cache is not None:
             cache_norm = (prev_count.detach(), prev_mean.detach(), prev_var.detach())
             hx = None if hx is None else hx.detach()
         # B x L x D
-        out_cema = out_cema.transpose(1, 2)
+        out_cema = transpose_last2(out_cema)
         mx = self.rmsnorm(out_cema)
         mx = memory_efficient_dropout(mx, self.hidden_dropout, self.training)
 
@@ -97,10 +97,11 @@ class MovingAverageGatedAttention(nn.Module):
 
         # B x L x E
         v = F.silu(self.wv(out_tsn))
-        r = F.silu(self.wr(mx))
+        r = self.wr(mx)
 
         attn, cache_attn = self.inner_attention(q.contiguous(), k.contiguous(), v, mask, freqs_cis, cache_attn)
-        attn = memory_efficient_dropout(attn * r, self.hidden_dropout, self.training)
+        # attn * silu(r) in one pass
+        attn = memory_efficient_dropout(silu_mul(r, attn), self.hidden_dropout, self.training)
 
         # B x L x E -> B x L x D
         h = self.wh1(mx) + self.wh2(attn)

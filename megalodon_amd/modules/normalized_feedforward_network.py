@@ -6,7 +6,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
-from ..fused_ops import memory_efficient_dropout
+from ..fused_ops import memory_efficient_dropout, silu_mul
 from .layer_norm import FusedLayerNorm
 
 
@@ -39,7 +39,7 @@ class NormalizedFeedForwardNetwork(nn.Module):
     def forward(self, x, residual):
         x = self.norm(x)
         if self.swiglu:
-            hidden = F.silu(self.fc1(x)) * self.fc3(x)
+            hidden = silu_mul(self.fc1(x), self.fc3(x))
         else:
             hidden = F.silu(self.fc1(x))
         hidden = memory_efficient_dropout(hidden, self.hidden_dropout, self.training)

@@ -1,0 +1,97 @@
+"""The block's glue kernels: tiled transpose (bit-exact, a byte move) and the
+SiLU gates against float64 (`silu(a) * b` and its autograd gradient):
+rel err <= 1e-4 float32, <= 2e-2 bfloat16 / float16."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from conftest import rel_err
+from megalodon_amd import extension as ops
+from megalodon_amd.fused_ops import silu_mul, transpose_last2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [
+    (2, 256, 384),      # whole 128 x 128 tiles
+    (1, 1000, 72),      # partial tiles on both sides, still 16-byte rows
+    (3, 50, 77),        # ragged: element-wise path
+    (2, 3, 8, 4096),    # leading dimensions fold into the batch; R far below a tile
+    (1, 1, 1),
+])
+def test_transpose_is_a_bit_exact_move(shape, dtype):
+    g = torch.Generator().manual_seed(sum(shape))
+    x = torch.randn(*shape, generator=g).to(dtype).cuda()
+    y = ops.transpose_last2(x)
+    assert y.is_contiguous() and y.shape == x.transpose(-2, -1).shape
+    assert torch.equal(y, x.transpose(-2, -1).contiguous())
+    assert torch.equal(ops.transpose_last2(y), x)
+
+
+def test_transpose_of_views_and_unaligned_buffers():
+    base = torch.randn(2 * 64 * 128 + 1, device="cuda").bfloat16()
+    x = base[1:].view(2, 64, 128)                 # 2-byte aligned only
+    assert torch.equal(ops.transpose_last2(x), x.transpose(1, 2).contiguous())
+    v = torch.randn(4, 128, 256, device="cuda").half()[:, :, ::2]   # strided input
+    assert torch.equal(ops.transpose_last2(v), v.transpose(1, 2).contiguous())
+    e = torch.empty(0, 8, 16, device="cuda", dtype=torch.bfloat16)
+    assert ops.transpose_last2(e).shape == (0, 16, 8)
+
+
+def test_transpose_autograd_and_full_size():
+    x = torch.randn(2, 96, 160, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    w = torch.randn(2, 160, 96, device="cuda", dtype=torch.bfloat16)
+    (transpose_last2(x) * w).sum().backward()
+    assert torch.equal(x.grad, w.transpose(1, 2))
+    # config-4 activation: (1, 32768, 4096) both ways
+    big = torch.randn(1, 32768, 4096, device="cuda").bfloat16()
+    t = ops.transpose_last2(big)
+    assert torch.equal(t, big.transpose(1, 2).contiguous()) and torch.equal(ops.transpose_last2(t), big)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2), (torch.float16, 2e-2)])
+@pytest.mark.parametrize("shape", [(4, 300, 64), (1003,), (2, 7, 9), (8,)])
+def test_silu_gate_matches_float64(shape, dtype, tol):
+    g = torch.Generator().manual_seed(len(shape) + shape[0])
+    a = (torch.randn(*shape, generator=g) * 3).to(dtype)
+    b = torch.randn(*shape, generator=g).to(dtype)
+    dy = torch.randn(*shape, generator=g).to(dtype)
+    ag, bg = a.cuda().requires_grad_(True), b.cuda().requires_grad_(True)
+    y = silu_mul(ag, bg)
+    y.backward(dy.cuda())
+    a64, b64 = a.double().requires_grad_(True), b.double().requires_grad_(True)
+    want = F.silu(a64) * b64
+    want.backward(dy.double())
+    assert y.dtype == dtype and rel_err(y, want) <= tol
+    assert rel_err(ag.grad, a64.grad) <= tol and rel_err(bg.grad, b64.grad) <= tol
+
+
+def test_silu_gate_edge_values_and_unaligned():
+    a = torch.tensor([0.0, -100.0, 100.0, -20.0, 20.0, 1e-3, -1e-3, 88.0, -88.0], device="cuda")
+    b = torch.full_like(a, 2.0)
+    y = ops.silu_mul_fwd(a, b)
+    want = (F.silu(a.double()) * 2.0)
+    assert torch.isfinite(y).all() and rel_err(y, want) <= 1e-5
+    da, db = ops.silu_mul_bwd(torch.ones_like(a), a, b)
+    assert torch.isfinite(da).all() and torch.isfinite(db).all()
+    base = torch.randn(4097, device="cuda").bfloat16()
+    u, v = base[1:], base[:-1].clone()
+    assert rel_err(ops.silu_mul_fwd(u, v), F.silu(u.double()) * v.double()) <= 2e-2
+    with pytest.raises(RuntimeError, match="same shape"):
+        ops.silu_mul_fwd(u, v[:-1])
+
+
+def test_silu_gate_at_the_feed_forward_size():
+    # (32768, 11008) bfloat16 as in config 4: compare a strided sample with float64
+    n = 32768 * 11008
+    a = torch.randn(n, device="cuda", dtype=torch.bfloat16)
+    b = torch.randn(n, device="cuda", dtype=torch.bfloat16)
+    y = ops.silu_mul_fwd(a, b)
+    idx = torch.arange(0, n, 4099, device="cuda")
+    assert rel_err(y[idx], F.silu(a[idx].double()) * b[idx].double()) <= 2e-2
+    assert rel_err(y[-70000:], F.silu(a[-70000:].double()) * b[-70000:].double()) <= 2e-2
+    da, db = ops.silu_mul_bwd(y, a, b)
+    s = torch.sigmoid(a[idx].double())
+    assert rel_err(db[idx], y[idx].double() * a[idx].double() * s) <= 2e-2
+    assert rel_err(da[idx], y[idx].double() * b[idx].double() * s * (1 + a[idx].double() * (1 - s))) <= 2e-2
