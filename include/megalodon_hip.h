@@ -370,6 +370,35 @@ int mega_layer_norm_bwd(const void* dy, const void* x, const void* weight, const
                         const float* rstd, int dtype, int64_t rows, int64_t D, int rms, void* dx,
                         void* dweight, void* dbias, void* workspace, void* stream);
 
+/* ------------------------------------------------------------------------
+ * z -> (q, k): per-head RMSNorm, the two affine maps and the rotary product.
+ *
+ * Replaces, in one pass over z, megalodon/modules/moving_average_gated_attention.py:
+ *   319-330 (`self.znorm(z.view(B, L, heads, Dh))`, `z.unsqueeze(2) * (gamma + 1)
+ *   / sqrt(Dh) + beta`, `torch.unbind`) and the rotary product of
+ *   megalodon/modules/rotary_positional_embedding.py:53-77 that
+ *   _InnerAttention applies to q and k (moving_average_gated_attention.py:
+ *   88-90,113-114).
+ *   z, q, k (rows, S) of `dtype` (bfloat16 / float16), rows = batch * L; gamma,
+ *   beta (2, S) of `dtype` as the module stores them; heads of Dh elements,
+ *   Dh in {64, 128, 256, 512}, S in {512, 1024, 2048, 4096}.  `freqs`: (P, Dh/2)
+ *   complex numbers as float32 pairs (cos, sin), or null for no rotary; row r
+ *   uses position (r % L) % P (P = chunk length, or L for a shorter piece).
+ *   rstd (rows, S / Dh) float32 is saved for the backward.  All buffers 16-byte
+ *   aligned.  Other shapes return MEGA_ERR_UNSUPPORTED (the module then keeps
+ *   the PyTorch expressions).
+ * Backward: dz, dgamma (2, S), dbeta (2, S) in `dtype`;
+ *   `workspace`: mega_qk_norm_rotary_workspace_bytes(S) bytes.
+ * ---------------------------------------------------------------------- */
+int64_t mega_qk_norm_rotary_workspace_bytes(int64_t S);
+int mega_qk_norm_rotary_fwd(const void* z, const void* gamma, const void* beta, const float* freqs,
+                            int dtype, int64_t rows, int64_t L, int64_t P, int64_t S, int64_t Dh,
+                            double eps, void* q, void* k, float* rstd, void* stream);
+int mega_qk_norm_rotary_bwd(const void* dq, const void* dk, const void* z, const void* gamma,
+                            const float* rstd, const float* freqs, int dtype, int64_t rows,
+                            int64_t L, int64_t P, int64_t S, int64_t Dh, void* dz, void* dgamma,
+                            void* dbeta, void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -330,16 +330,17 @@ __global__ __launch_bounds__(kThreads) void norm_bwd_any_kernel(NormParams p, in
   }
 }
 
-// out[c] = sum over `groups` rows of part[., c]: 64 columns x 16 row slices per workgroup
+// out[c] = sum over `groups` rows (`stride` floats apart) of part[., c], c < D:
+// 64 columns x 16 row slices per workgroup
 template <int DT>
 __global__ __launch_bounds__(1024) void norm_param_grad_kernel(const float* part, int groups, int D,
-                                                              typename Elem<DT>::type* out) {
+                                                              int stride, typename Elem<DT>::type* out) {
   __shared__ float red[16][65];
   const int cx = threadIdx.x % 64, sy = threadIdx.x / 64;
   const int c = blockIdx.x * 64 + cx;
   float s = 0.f;
   if (c < D)
-    for (int gidx = sy; gidx < groups; gidx += 16) s += part[static_cast<int64_t>(gidx) * D + c];
+    for (int gidx = sy; gidx < groups; gidx += 16) s += part[static_cast<int64_t>(gidx) * stride + c];
   red[sy][cx] = s;
   __syncthreads();
   if (sy == 0 && c < D) {
@@ -348,6 +349,196 @@ __global__ __launch_bounds__(1024) void norm_param_grad_kernel(const float* part
     for (int v = 0; v < 16; ++v) t += red[v][cx];
     Elem<DT>::store(out + c, t);
   }
+}
+
+
+// ---- z -> (q, k): per-head RMSNorm, the two affine maps, rotary ----------------
+// megalodon/modules/moving_average_gated_attention.py:319-330 (znorm over each
+// head of z, `z.unsqueeze(2) * (gamma + 1) / sqrt(Dh) + beta`, unbind into q, k)
+// followed by the rotary product of
+// megalodon/modules/rotary_positional_embedding.py:53-77 on both: neighbouring
+// elements (2i, 2i+1) of a head are one complex number that is multiplied by
+// freqs[p][i], p = (row % L) % P the position inside the chunk.  One wavefront
+// holds a row of S = 512 * NCH elements, G = Dh / 8 lanes per head; z is read
+// once and q, k are written once.  The backward undoes the rotation with the
+// conjugate factor, forms the gradients of the affine parameters as column
+// sums (per-workgroup partials, reduced in a fixed order afterwards) and the
+// RMSNorm gradient per head.
+struct QkParams {
+  const uint16_t* z;
+  const uint16_t* gamma;  // (2, S) as stored: the factor is (gamma + 1) / sqrt(Dh)
+  const uint16_t* beta;   // (2, S)
+  const float* freqs;     // (P, Dh / 2, 2) cos, sin; null = no rotary
+  const uint16_t* dq;
+  const uint16_t* dk;
+  uint16_t* q;  // forward: q, backward: dz
+  uint16_t* k;
+  float* rstd;  // (rows, S / Dh)
+  float* part;  // backward: (groups, 4 S): dgamma_q | dgamma_k | dbeta_q | dbeta_k
+  int64_t rows;
+  int L, P, S, Dh;
+  float eps, inv_sqrt_dh;
+};
+
+__device__ __forceinline__ void rotate8(float* u, const float4& f0, const float4& f1, bool conj) {
+  const float c[4] = {f0.x, f0.z, f1.x, f1.z};
+  const float sn[4] = {f0.y, f0.w, f1.y, f1.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float s = conj ? -sn[i] : sn[i];
+    const float a = u[2 * i], b = u[2 * i + 1];
+    u[2 * i] = a * c[i] - b * s;
+    u[2 * i + 1] = a * s + b * c[i];
+  }
+}
+
+template <int DT, int G, int NCH>
+__global__ __launch_bounds__(kThreads) void qk_fwd_kernel(QkParams p) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int heads = p.S / p.Dh;
+  const float inv_dh = 1.f / static_cast<float>(p.Dh);
+  uint4 gq[NCH], gk[NCH], bq[NCH], bk[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = (lane + kWave * i) * 8;
+    gq[i] = *reinterpret_cast<const uint4*>(p.gamma + c);
+    gk[i] = *reinterpret_cast<const uint4*>(p.gamma + p.S + c);
+    bq[i] = *reinterpret_cast<const uint4*>(p.beta + c);
+    bk[i] = *reinterpret_cast<const uint4*>(p.beta + p.S + c);
+  }
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * kWaves + wave; row < p.rows;
+       row += static_cast<int64_t>(gridDim.x) * kWaves) {
+    const int pos = static_cast<int>(row % p.L) % p.P;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = (lane + kWave * i) * 8;
+      float v[8], uq[8], uk[8], g[8], b[8];
+      unpack8<DT>(*reinterpret_cast<const uint4*>(p.z + row * p.S + c), v);
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
+      const float r = rsqrtf(group_sum<G>(ss) * inv_dh + p.eps);
+      if (lane % G == 0) p.rstd[row * heads + c / p.Dh] = r;
+      opaque(gq[i]); opaque(bq[i]); opaque(gk[i]); opaque(bk[i]);
+      unpack8<DT>(gq[i], g);
+      unpack8<DT>(bq[i], b);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) uq[e] = v[e] * r * ((g[e] + 1.f) * p.inv_sqrt_dh) + b[e];
+      unpack8<DT>(gk[i], g);
+      unpack8<DT>(bk[i], b);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) uk[e] = v[e] * r * ((g[e] + 1.f) * p.inv_sqrt_dh) + b[e];
+      if (p.freqs) {
+        const float4* f = reinterpret_cast<const float4*>(p.freqs + (static_cast<int64_t>(pos) * p.Dh + c % p.Dh));
+        const float4 f0 = f[0], f1 = f[1];
+        rotate8(uq, f0, f1, false);
+        rotate8(uk, f0, f1, false);
+      }
+      *reinterpret_cast<uint4*>(p.q + row * p.S + c) = pack8<DT>(uq);
+      *reinterpret_cast<uint4*>(p.k + row * p.S + c) = pack8<DT>(uk);
+    }
+  }
+}
+
+template <int DT, int G, int NCH>
+__global__ __launch_bounds__(kThreads) void qk_bwd_kernel(QkParams p) {
+  extern __shared__ float acc[];  // 4 S floats
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int heads = p.S / p.Dh;
+  const float inv_dh = 1.f / static_cast<float>(p.Dh);
+  uint4 gq[NCH], gk[NCH];
+  float a_gq[NCH][8], a_gk[NCH][8], a_bq[NCH][8], a_bk[NCH][8];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = (lane + kWave * i) * 8;
+    gq[i] = *reinterpret_cast<const uint4*>(p.gamma + c);
+    gk[i] = *reinterpret_cast<const uint4*>(p.gamma + p.S + c);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a_gq[i][e] = 0.f, a_gk[i][e] = 0.f, a_bq[i][e] = 0.f, a_bk[i][e] = 0.f;
+  }
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * kWaves + wave; row < p.rows;
+       row += static_cast<int64_t>(gridDim.x) * kWaves) {
+    const int pos = static_cast<int>(row % p.L) % p.P;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = (lane + kWave * i) * 8;
+      float zn[8], dq[8], dk[8], g[8], dzn[8];
+      unpack8<DT>(*reinterpret_cast<const uint4*>(p.z + row * p.S + c), zn);
+      unpack8<DT>(*reinterpret_cast<const uint4*>(p.dq + row * p.S + c), dq);
+      unpack8<DT>(*reinterpret_cast<const uint4*>(p.dk + row * p.S + c), dk);
+      const float r = p.rstd[row * heads + c / p.Dh];
+      if (p.freqs) {
+        const float4* f = reinterpret_cast<const float4*>(p.freqs + (static_cast<int64_t>(pos) * p.Dh + c % p.Dh));
+        const float4 f0 = f[0], f1 = f[1];
+        rotate8(dq, f0, f1, true);
+        rotate8(dk, f0, f1, true);
+      }
+      opaque(gq[i]); opaque(gk[i]);
+      unpack8<DT>(gq[i], g);
+      float s = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        zn[e] *= r;
+        a_gq[i][e] += dq[e] * zn[e];
+        a_bq[i][e] += dq[e];
+        dzn[e] = dq[e] * ((g[e] + 1.f) * p.inv_sqrt_dh);
+      }
+      unpack8<DT>(gk[i], g);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        a_gk[i][e] += dk[e] * zn[e];
+        a_bk[i][e] += dk[e];
+        dzn[e] += dk[e] * ((g[e] + 1.f) * p.inv_sqrt_dh);
+        s += dzn[e] * zn[e];
+      }
+      s = group_sum<G>(s) * inv_dh;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dzn[e] = r * (dzn[e] - zn[e] * s);
+      *reinterpret_cast<uint4*>(p.q + row * p.S + c) = pack8<DT>(dzn);
+    }
+  }
+  // column sums of this workgroup, wave by wave in a fixed order
+  for (int w = 0; w < kWaves; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int c = (lane + kWave * i) * 8 + e;
+          const float vg0 = a_gq[i][e] * p.inv_sqrt_dh, vg1 = a_gk[i][e] * p.inv_sqrt_dh;
+          if (w == 0) {
+            acc[c] = vg0; acc[p.S + c] = vg1; acc[2 * p.S + c] = a_bq[i][e]; acc[3 * p.S + c] = a_bk[i][e];
+          } else {
+            acc[c] += vg0; acc[p.S + c] += vg1; acc[2 * p.S + c] += a_bq[i][e]; acc[3 * p.S + c] += a_bk[i][e];
+          }
+        }
+    }
+    __syncthreads();
+  }
+  for (int c = threadIdx.x; c < 4 * p.S; c += kThreads)
+    p.part[static_cast<int64_t>(blockIdx.x) * 4 * p.S + c] = acc[c];
+}
+
+template <int DT, bool BWD>
+int launch_qk(const QkParams& p, int groups, hipStream_t s) {
+  const int G = p.Dh / 8, nch = p.S / 512;
+  const size_t lds = BWD ? static_cast<size_t>(4) * p.S * sizeof(float) : 0;
+  bool hit = false;
+#define MEGA_QK(GG, NN)                                                      \
+  if (G == GG && nch == NN) {                                                \
+    hit = true;                                                              \
+    if (BWD)                                                                 \
+      qk_bwd_kernel<DT, GG, NN><<<groups, kThreads, lds, s>>>(p);            \
+    else                                                                     \
+      qk_fwd_kernel<DT, GG, NN><<<groups, kThreads, 0, s>>>(p);              \
+  }
+#define MEGA_QK_G(GG) MEGA_QK(GG, 1) MEGA_QK(GG, 2) MEGA_QK(GG, 4) MEGA_QK(GG, 8)
+  MEGA_QK_G(8) MEGA_QK_G(16) MEGA_QK_G(32) MEGA_QK_G(64)
+#undef MEGA_QK_G
+#undef MEGA_QK
+  if (!hit) return set_error(MEGA_ERR_UNSUPPORTED, "qk_norm_rotary: unsupported head size / width");
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
 }
 
 struct Shape {
@@ -476,10 +667,10 @@ static int run_bwd(NormParams p, int dtype, void* dweight, void* dbias, float* w
   }
   if (affine) {
     const int blocks = (p.D + 63) / 64;
-    norm_param_grad_kernel<DT><<<blocks, 1024, 0, s>>>(p.part_w, groups, p.D, static_cast<T*>(dweight));
+    norm_param_grad_kernel<DT><<<blocks, 1024, 0, s>>>(p.part_w, groups, p.D, p.D, static_cast<T*>(dweight));
     MEGA_CHECK_LAUNCH();
     if (p.part_b) {
-      norm_param_grad_kernel<DT><<<blocks, 1024, 0, s>>>(p.part_b, groups, p.D, static_cast<T*>(dbias));
+      norm_param_grad_kernel<DT><<<blocks, 1024, 0, s>>>(p.part_b, groups, p.D, p.D, static_cast<T*>(dbias));
       MEGA_CHECK_LAUNCH();
     }
   }
@@ -508,4 +699,79 @@ extern "C" int mega_layer_norm_bwd(const void* dy, const void* x, const void* we
   if (dtype == MEGA_BF16) { MEGA_DISPATCH(MEGA_BF16) }
   MEGA_DISPATCH(MEGA_F16)
 #undef MEGA_DISPATCH
+}
+
+// ---- z -> (q, k) -------------------------------------------------------------------
+static int check_qk(const char* who, int dtype, int64_t rows, int64_t L, int64_t P, int64_t S, int64_t Dh,
+                    const void* freqs) {
+  if (dtype != MEGA_BF16 && dtype != MEGA_F16)
+    return set_error(MEGA_ERR_UNSUPPORTED, "%s: only bfloat16 / float16 tensors are supported", who);
+  MEGA_CHECK_ARG(rows >= 0 && L >= 1 && S >= 1 && Dh >= 1, "%s: bad sizes", who);
+  MEGA_CHECK_ARG(!freqs || P >= 1, "%s: rotary factors without positions", who);
+  if (!(Dh == 64 || Dh == 128 || Dh == 256 || Dh == 512) || S % Dh != 0 ||
+      !(S == 512 || S == 1024 || S == 2048 || S == 4096))
+    return set_error(MEGA_ERR_UNSUPPORTED,
+                     "%s: needs a head size of 64, 128, 256 or 512 and a width of 512, 1024, 2048 or 4096 "
+                     "(got %lld, %lld)", who, (long long)Dh, (long long)S);
+  return MEGA_OK;
+}
+
+extern "C" int64_t mega_qk_norm_rotary_workspace_bytes(int64_t S) {
+  return S < 1 ? 16 : static_cast<int64_t>(kMaxGroups) * 4 * S * static_cast<int64_t>(sizeof(float));
+}
+
+extern "C" int mega_qk_norm_rotary_fwd(const void* z, const void* gamma, const void* beta,
+                                       const float* freqs, int dtype, int64_t rows, int64_t L, int64_t P,
+                                       int64_t S, int64_t Dh, double eps, void* q, void* k, float* rstd,
+                                       void* stream) {
+  int rc = check_qk("mega_qk_norm_rotary_fwd", dtype, rows, L, P, S, Dh, freqs);
+  if (rc != MEGA_OK) return rc;
+  if (rows == 0) return MEGA_OK;
+  MEGA_CHECK_ARG(z && gamma && beta && q && k && rstd, "mega_qk_norm_rotary_fwd: null pointer");
+  for (const void* ptr : {z, gamma, beta, static_cast<const void*>(freqs), static_cast<const void*>(q),
+                          static_cast<const void*>(k)})
+    MEGA_CHECK_ARG(reinterpret_cast<uintptr_t>(ptr) % 16 == 0, "mega_qk_norm_rotary_fwd: buffers must be 16-byte aligned");
+  QkParams p{};
+  p.z = static_cast<const uint16_t*>(z); p.gamma = static_cast<const uint16_t*>(gamma);
+  p.beta = static_cast<const uint16_t*>(beta); p.freqs = freqs;
+  p.q = static_cast<uint16_t*>(q); p.k = static_cast<uint16_t*>(k); p.rstd = rstd;
+  p.rows = rows; p.L = (int)L; p.P = freqs ? (int)P : 1; p.S = (int)S; p.Dh = (int)Dh;
+  p.eps = static_cast<float>(eps); p.inv_sqrt_dh = static_cast<float>(1.0 / sqrt(static_cast<double>(Dh)));
+  const int64_t g = (rows + kWaves - 1) / kWaves;
+  const int groups = static_cast<int>(g > 16384 ? 16384 : g);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return dtype == MEGA_BF16 ? launch_qk<MEGA_BF16, false>(p, groups, s) : launch_qk<MEGA_F16, false>(p, groups, s);
+}
+
+extern "C" int mega_qk_norm_rotary_bwd(const void* dq, const void* dk, const void* z, const void* gamma,
+                                       const float* rstd, const float* freqs, int dtype, int64_t rows,
+                                       int64_t L, int64_t P, int64_t S, int64_t Dh, void* dz, void* dgamma,
+                                       void* dbeta, void* workspace, void* stream) {
+  int rc = check_qk("mega_qk_norm_rotary_bwd", dtype, rows, L, P, S, Dh, freqs);
+  if (rc != MEGA_OK) return rc;
+  MEGA_CHECK_ARG(rows >= 1, "mega_qk_norm_rotary_bwd: no rows");
+  MEGA_CHECK_ARG(dq && dk && z && gamma && rstd && dz && dgamma && dbeta && workspace,
+                 "mega_qk_norm_rotary_bwd: null pointer");
+  for (const void* ptr : {dq, dk, z, gamma, static_cast<const void*>(freqs), static_cast<const void*>(dz)})
+    MEGA_CHECK_ARG(reinterpret_cast<uintptr_t>(ptr) % 16 == 0, "mega_qk_norm_rotary_bwd: buffers must be 16-byte aligned");
+  QkParams p{};
+  p.z = static_cast<const uint16_t*>(z); p.gamma = static_cast<const uint16_t*>(gamma); p.freqs = freqs;
+  p.dq = static_cast<const uint16_t*>(dq); p.dk = static_cast<const uint16_t*>(dk);
+  p.q = static_cast<uint16_t*>(dz); p.rstd = const_cast<float*>(rstd); p.part = static_cast<float*>(workspace);
+  p.rows = rows; p.L = (int)L; p.P = freqs ? (int)P : 1; p.S = (int)S; p.Dh = (int)Dh;
+  p.inv_sqrt_dh = static_cast<float>(1.0 / sqrt(static_cast<double>(Dh)));
+  const int groups = groups_for(rows, kWaves);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  rc = dtype == MEGA_BF16 ? launch_qk<MEGA_BF16, true>(p, groups, s) : launch_qk<MEGA_F16, true>(p, groups, s);
+  if (rc != MEGA_OK) return rc;
+  const int cols = 2 * static_cast<int>(S), blocks = (cols + 63) / 64;
+  if (dtype == MEGA_BF16) {
+    norm_param_grad_kernel<MEGA_BF16><<<blocks, 1024, 0, s>>>(p.part, groups, cols, 2 * cols, static_cast<uint16_t*>(dgamma));
+    norm_param_grad_kernel<MEGA_BF16><<<blocks, 1024, 0, s>>>(p.part + cols, groups, cols, 2 * cols, static_cast<uint16_t*>(dbeta));
+  } else {
+    norm_param_grad_kernel<MEGA_F16><<<blocks, 1024, 0, s>>>(p.part, groups, cols, 2 * cols, static_cast<uint16_t*>(dgamma));
+    norm_param_grad_kernel<MEGA_F16><<<blocks, 1024, 0, s>>>(p.part + cols, groups, cols, 2 * cols, static_cast<uint16_t*>(dbeta));
+  }
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
 }

@@ -755,6 +755,63 @@ def layer_norm_bwd(y_grad: torch.Tensor, x: torch.Tensor, weight: Optional[torch
     return dx, dw, db
 
 
+def qk_norm_rotary_supported(z: torch.Tensor, gamma: torch.Tensor, head_dim: int) -> bool:
+    """Shapes the fused z -> (q, k) kernel takes (include/megalodon_hip.h)."""
+    return (z.is_cuda and z.dtype in (torch.bfloat16, torch.float16) and gamma.dtype == z.dtype
+            and head_dim in (64, 128, 256, 512) and z.shape[-1] in (512, 1024, 2048, 4096)
+            and z.shape[-1] % head_dim == 0 and z.dim() == 3)
+
+
+def _freqs_real(freqs_cis: Optional[torch.Tensor], head_dim: int, dev) -> Tuple[Optional[torch.Tensor], int]:
+    if freqs_cis is None:
+        return None, 1
+    if freqs_cis.dim() != 2 or freqs_cis.shape[1] != head_dim // 2 or not freqs_cis.is_complex():
+        raise RuntimeError("qk_norm_rotary: freqs_cis must be complex (positions, head_dim / 2)")
+    fr = torch.view_as_real(freqs_cis.to(device=dev, dtype=torch.complex64)).contiguous()
+    return fr, freqs_cis.shape[0]
+
+
+def qk_norm_rotary_fwd(z: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor,
+                       freqs_cis: Optional[torch.Tensor], head_dim: int, eps: float
+                       ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(q, k, rstd) from z (B, L, S): RMSNorm per head, `* (gamma + 1) / sqrt(head_dim) + beta`
+    for q and for k, rotary by position inside the chunk
+    (moving_average_gated_attention.py:319-330, rotary_positional_embedding.py:53-77)."""
+    dev = _require_cuda(z, gamma, beta)
+    if z.dim() != 3 or gamma.shape != (2, z.shape[-1]) or beta.shape != gamma.shape:
+        raise RuntimeError("qk_norm_rotary: z must be (B, L, S), gamma and beta (2, S)")
+    B, L, S = z.shape
+    zc, gc, bc = z.contiguous(), gamma.contiguous(), beta.contiguous()
+    fr, P = _freqs_real(freqs_cis, head_dim, dev)
+    q, k = torch.empty_like(zc), torch.empty_like(zc)
+    rstd = torch.empty(B * L, S // head_dim, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_qk_norm_rotary_fwd", _lib.ptr(zc), _lib.ptr(gc), _lib.ptr(bc), _lib.ptr(fr),
+                  _lib.i32(_lib.dtype_code(z.dtype)), _lib.i64(B * L), _lib.i64(L), _lib.i64(P), _lib.i64(S),
+                  _lib.i64(head_dim), _lib.f64(eps), _lib.ptr(q), _lib.ptr(k), _lib.ptr(rstd), _lib.stream_ptr(dev))
+    return q, k, rstd
+
+
+def qk_norm_rotary_bwd(q_grad: torch.Tensor, k_grad: torch.Tensor, z: torch.Tensor, gamma: torch.Tensor,
+                       rstd: torch.Tensor, freqs_cis: Optional[torch.Tensor], head_dim: int
+                       ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(z_grad, gamma_grad, beta_grad)."""
+    dev = _require_cuda(q_grad, k_grad, z, gamma)
+    B, L, S = z.shape
+    zc, gc, dq, dk = z.contiguous(), gamma.contiguous(), q_grad.contiguous(), k_grad.contiguous()
+    fr, P = _freqs_real(freqs_cis, head_dim, dev)
+    dz, dgamma, dbeta = torch.empty_like(zc), torch.empty_like(gc), torch.empty_like(gc)
+    fn = _lib.load().mega_qk_norm_rotary_workspace_bytes
+    fn.restype = _lib.ctypes.c_int64
+    ws = torch.empty(int(fn(_lib.i64(S))), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_qk_norm_rotary_bwd", _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(zc), _lib.ptr(gc), _lib.ptr(rstd),
+                  _lib.ptr(fr), _lib.i32(_lib.dtype_code(z.dtype)), _lib.i64(B * L), _lib.i64(L), _lib.i64(P),
+                  _lib.i64(S), _lib.i64(head_dim), _lib.ptr(dz), _lib.ptr(dgamma), _lib.ptr(dbeta), _lib.ptr(ws),
+                  _lib.stream_ptr(dev))
+    return dz, dgamma, dbeta
+
+
 def timestep_norm_fwd(x: torch.Tensor, prev_count: torch.Tensor, prev_mean: torch.Tensor, prev_var: torch.Tensor,
                       gamma: torch.Tensor, beta: torch.Tensor, padding_mask: Optional[torch.Tensor], eps: float):
     """The non-group operator (megalodon/csrc/ops/timestep_norm.cc:23-105,

@@ -1,7 +1,7 @@
 """Fused ops with the reference's names (megalodon/modules/fused_ops/__init__.py:1-14)."""
 from .attention import (attention_softmax, swift_efficient_attention, swift_efficient_attention_bwd,
                         swift_efficient_attention_fwd)
-from .block_glue import layer_norm_plus_one, silu_mul, transpose_last2
+from .block_glue import layer_norm_plus_one, qk_norm_rotary, silu_mul, transpose_last2
 from .cema_kernel import cema_kernel
 from .ema_hidden import ema_hidden
 from .ema_parameters import ema_parameters
@@ -10,4 +10,4 @@ from .memory_efficient_dropout import memory_efficient_dropout
 
 __all__ = ["attention_softmax", "cema_kernel", "ema_hidden", "ema_parameters", "fftconv", "fftconv_residual", "memory_efficient_dropout",
            "swift_efficient_attention", "swift_efficient_attention_fwd",
-           "swift_efficient_attention_bwd", "silu_mul", "transpose_last2", "layer_norm_plus_one"]
+           "swift_efficient_attention_bwd", "silu_mul", "transpose_last2", "layer_norm_plus_one", "qk_norm_rotary"]

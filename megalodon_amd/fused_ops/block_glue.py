@@ -58,6 +58,30 @@ class LayerNormPlusOneFunc(torch.autograd.Function):
         return dx, dw, db, None, None
 
 
+class QkNormRotaryFunc(torch.autograd.Function):
+    """z -> (q, k) in one pass (moving_average_gated_attention.py:319-330 plus the
+    rotary product of rotary_positional_embedding.py:53-77)."""
+
+    @staticmethod
+    def forward(ctx: FunctionCtx, z: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor,
+                freqs_cis: Optional[torch.Tensor], head_dim: int, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+        q, k, rstd = megalodon_ops.qk_norm_rotary_fwd(z, gamma, beta, freqs_cis, head_dim, eps)
+        ctx.save_for_backward(z, gamma, rstd)
+        ctx.freqs_cis = freqs_cis
+        ctx.head_dim = head_dim
+        return q, k
+
+    @staticmethod
+    def backward(ctx: FunctionCtx, q_grad: torch.Tensor, k_grad: torch.Tensor):
+        z, gamma, rstd = ctx.saved_tensors
+        dz, dgamma, dbeta = megalodon_ops.qk_norm_rotary_bwd(q_grad, k_grad, z, gamma, rstd, ctx.freqs_cis,
+                                                             ctx.head_dim)
+        return dz, dgamma, dbeta, None, None, None
+
+
+qk_norm_rotary = QkNormRotaryFunc.apply
+
+
 def layer_norm_plus_one(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],
                         eps: float = 1e-5, rms: bool = False) -> torch.Tensor:
     return LayerNormPlusOneFunc.apply(x, weight, bias, eps, rms)

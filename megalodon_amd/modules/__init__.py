@@ -4,8 +4,9 @@ from .complex_exponential_moving_average import MultiHeadComplexEMA
 from .layer_norm import FusedLayerNorm, FusedRMSNorm
 from .moving_average_gated_attention import MegaBlock, MovingAverageGatedAttention
 from .normalized_feedforward_network import NormalizedFeedForwardNetwork
+from .rotary_positional_embedding import RotaryEmbedding
 from .timestep_norm import TimestepNorm, TimestepNormFunc, timestep_norm
 
 __all__ = ["MegaBlock", "MovingAverageGatedAttention", "NormalizedFeedForwardNetwork", "FusedLayerNorm",
            "FusedRMSNorm", "MultiHeadComplexEMA", "TimestepNorm", "TimestepNormFunc", "timestep_norm", "_InnerAttention",
-           "apply_rotary_emb"]
+           "apply_rotary_emb", "RotaryEmbedding"]

@@ -17,7 +17,8 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 from torch.nn import Parameter
 
-from ..fused_ops import memory_efficient_dropout, silu_mul, transpose_last2
+from .. import extension as megalodon_ops
+from ..fused_ops import memory_efficient_dropout, qk_norm_rotary, silu_mul, transpose_last2
 from .chunk_attention import _InnerAttention
 from .complex_exponential_moving_average import MultiHeadComplexEMA
 from .layer_norm import FusedRMSNorm
@@ -87,13 +88,22 @@ class MovingAverageGatedAttention(nn.Module):
         mx = self.rmsnorm(out_cema)
         mx = memory_efficient_dropout(mx, self.hidden_dropout, self.training)
 
-        # B x L x S -> B x L x H x S/H -> B x L x S
-        z = self.wz(mx).view(bsz, seq_len, self.local_heads, self.z_head_dim)
-        z = self.znorm(z).view(bsz, seq_len, -1)
-        # B x L x 1 x S -> B x L x 2 x S
-        gamma = (self.gamma + 1.0) / math.sqrt(self.z_head_dim)
-        z = z.unsqueeze(2) * gamma + self.beta
-        q, k = torch.unbind(z, dim=2)
+        z = self.wz(mx)
+        if (not self.znorm.elementwise_affine
+                and megalodon_ops.qk_norm_rotary_supported(z, self.gamma, self.z_head_dim)
+                and (freqs_cis is None or freqs_cis.shape[0] == min(seq_len, self.chunk_size))):
+            # per-head norm, both affine maps and the rotary product in one pass over z:
+            # position = index inside the chunk, which is what _InnerAttention applies
+            # before (short piece) or after (long sequence) its chunk split
+            q, k = qk_norm_rotary(z, self.gamma, self.beta, freqs_cis, self.z_head_dim, self.znorm.eps)
+            freqs_cis = None
+        else:
+            # B x L x S -> B x L x H x S/H -> B x L x S
+            z = self.znorm(z.view(bsz, seq_len, self.local_heads, self.z_head_dim)).view(bsz, seq_len, -1)
+            # B x L x 1 x S -> B x L x 2 x S
+            gamma = (self.gamma + 1.0) / math.sqrt(self.z_head_dim)
+            z = z.unsqueeze(2) * gamma + self.beta
+            q, k = torch.unbind(z, dim=2)
 
         # B x L x E
         v = F.silu(self.wv(out_tsn))

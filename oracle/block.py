@@ -24,7 +24,16 @@ def _rms(x, weight, eps):
     return y if weight is None else y * (weight + 1.0)
 
 
-def mega_block_forward(p, x, *, num_heads, ndim, chunk_size, groups, eps=1e-5, swiglu=True):
+def rotary(x, freqs_cis):
+    """x (B', C, heads, Dh), freqs_cis (C, Dh / 2) complex: neighbouring elements
+    (2i, 2i+1) form a complex number that is multiplied by freqs_cis[position, i]
+    (megalodon/modules/rotary_positional_embedding.py:53-77)."""
+    xc = torch.view_as_complex(x.double().reshape(*x.shape[:-1], -1, 2))
+    out = xc * freqs_cis.to(torch.complex128).unsqueeze(1)
+    return torch.view_as_real(out).flatten(3)
+
+
+def mega_block_forward(p, x, *, num_heads, ndim, chunk_size, groups, eps=1e-5, swiglu=True, freqs_cis=None):
     B, L, D = x.shape
     x = x.double()
     # TimestepNorm (prior count 0: buffers, not parameters)
@@ -53,8 +62,11 @@ def mega_block_forward(p, x, *, num_heads, ndim, chunk_size, groups, eps=1e-5, s
     vh = hdim // num_heads
     nc = max(1, L // chunk_size)
     C = L // nc
-    y, _ = oattn.chunk_attention_fwd(qq.reshape(B * nc, C, num_heads, zh), kk.reshape(B * nc, C, num_heads, zh),
-                                     v.reshape(B * nc, C, num_heads, vh), 1.0, True)
+    qq, kk = qq.reshape(B * nc, C, num_heads, zh), kk.reshape(B * nc, C, num_heads, zh)
+    if freqs_cis is not None:
+        # position = index inside the chunk (moving_average_gated_attention.py:88-90,113-114)
+        qq, kk = rotary(qq, freqs_cis), rotary(kk, freqs_cis)
+    y, _ = oattn.chunk_attention_fwd(qq, kk, v.reshape(B * nc, C, num_heads, vh), 1.0, True)
     attn = y.reshape(B, L, hdim) * r
     h = F.linear(mx, p["mega.wh1.weight"], p["mega.wh1.bias"]) + F.linear(attn, p["mega.wh2.weight"])
     y1 = h + x
