@@ -262,9 +262,10 @@ int mega_attention_bwd(const void* dy, const void* q, const void* k, const void*
  * fftconv_bwd(dy, x_f, k_f, k_dtype), megalodon/modules/fused_ops/fftconv.py:
  * 21-28,62-75, csrc/ops/fftconv_kernel.cu:34-164).  This pair does the same for
  * the matrix-core path: the forward also writes the spectra of x and of k (an
- * opaque fp16 layout with the rows' scales, mega_fftconv_spectrum_bytes(...)
- * bytes each, 16-byte aligned), the backward needs only dy and the two
- * buffers: dx = corr(dy, k) + omega dy, dk = sum_b corr(dy, x) from three
+ * opaque fp16 layout with the rows' scales, 16-byte aligned: spec_x takes
+ * mega_fftconv_spectrum_bytes(dtype, B, D, L) bytes, spec_k, which depends on
+ * the channel only, mega_fftconv_spectrum_bytes(dtype, 1, D, L)), the backward
+ * needs only dy and the two buffers: dx = corr(dy, k) + omega dy, dk = sum_b corr(dy, x) from three
  * transforms per row instead of five.  mega_fftconv_spectrum_bytes returns 0
  * for shapes outside this path (float32 rows, L <= 2048, L % 8 != 0, D not a
  * multiple of the rows per pass: 32768 / 2^ceil(log2 L) for L > 2048); use

@@ -997,13 +997,18 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_kernel(
       // no wait on memory before the next pass: issued right after the capture
       // they would be waited for in front of place_rows (loads and stores
       // share one in-order counter).
-      uint32_t* const save_b = spec_b + static_cast<size_t>(pass) * kSpecWords;
-      store_spectrum(save_b, sp, tid);
+      // The second operand depends on the channel only: its spectrum is kept
+      // once per channel group, by the pass of batch index 0.
+      if (static_cast<int64_t>(pass) * R < D) {
+        uint32_t* const save_b = spec_b + static_cast<size_t>(pass) * kSpecWords;
+        store_spectrum(save_b, sp, tid);
 #pragma unroll
-      for (int i = 0; i < R; ++i) {
-        if (tid == i) reinterpret_cast<float*>(save_b + kSpecScaleWords)[i] = sb[i];
-        if (tid == i) reinterpret_cast<float*>(save_a + kSpecScaleWords)[i] = sa[i];
+        for (int i = 0; i < R; ++i)
+          if (tid == i) reinterpret_cast<float*>(save_b + kSpecScaleWords)[i] = sb[i];
       }
+#pragma unroll
+      for (int i = 0; i < R; ++i)
+        if (tid == i) reinterpret_cast<float*>(save_a + kSpecScaleWords)[i] = sa[i];
     }
     pointwise<LOGA>(pre, sp, tid, save_a);
     lds_barrier();
@@ -1136,7 +1141,7 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_bwd_saved_kernel(
     // the forward's pass of rows (bb, d0 .. d0 + R - 1)
     const size_t pass = static_cast<size_t>((bb * D + d0) / R);
     const uint32_t* sx = spec_x + pass * kSpecWords;
-    const uint32_t* sk = spec_k + pass * kSpecWords;
+    const uint32_t* sk = spec_k + static_cast<size_t>(d0 / R) * kSpecWords;  // one per channel group
     const RowPtrs<LOGA> dyrows = rows_of(it, dy, 2, true);
     float wres[R], sdy[R], s2[R], scale[R];
 #pragma unroll
@@ -1169,6 +1174,79 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_bwd_saved_kernel(
       store_rows<LOGA, MEGA_F32, false>(pre, krows, L, true, scale, nullptr, wres, tid);
     else
       store_rows<LOGA, MEGA_F32, true>(pre, krows, L, true, scale, nullptr, wres, tid);
+    lds_barrier();
+  }
+}
+
+// Forward for B > 1: the kernel row k[d, :] is the same for every batch index,
+// so a workgroup owns channel groups (as the backward kernels do) and walks
+// the batch itself: k is transformed once per channel group and its spectrum
+// stays parked while the B rows of x are transformed, multiplied and
+// transformed back -- 2 transforms per row instead of 3.  spec_x / spec_k as
+// in fftconv_mfma_kernel (both or neither).
+template <int DT, int LOGA>
+__global__ __launch_bounds__(kThreads) void fftconv_mfma_fwd_batch_kernel(
+    const void* __restrict__ x, const float* __restrict__ k, void* __restrict__ y, int B, int D, int L,
+    const float* __restrict__ omega, uint32_t* __restrict__ spec_x, uint32_t* __restrict__ spec_k) {
+  constexpr int R = Geo<LOGA>::R;
+  extern __shared__ __align__(16) uint16_t lds[];
+  uint16_t* pre = lds;
+  float* red = reinterpret_cast<float*>(lds + 2 * kPlane);
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const Dft w = make_dft(lane);
+  const int64_t groups = (static_cast<int64_t>(D) + R - 1) / R;
+  const int64_t total = (groups - blockIdx.x + gridDim.x - 1) / gridDim.x * B;
+  auto rows_of = [&](int64_t it, const void* base, int64_t esz, bool batched) {
+    const int64_t d0 = (blockIdx.x + (it / B) * gridDim.x) * R, bb = it % B;
+    RowPtrs<LOGA> p;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      p.p[i] = d0 + i < D ? static_cast<const char*>(base) + ((batched ? bb * D : 0) + d0 + i) * L * esz
+                          : nullptr;
+    return p;
+  };
+  RowRegs<DT> rx;
+  if (total > 0) fetch_rows<LOGA>(rx, rows_of(0, x, 2, true), L, false, tid);
+  Spectrum spk;
+  float sk[R];
+  for (int64_t it = 0; it < total; ++it) {
+    const int64_t d0 = (blockIdx.x + (it / B) * gridDim.x) * R, bb = it % B;
+    if (bb == 0) {
+      // a new channel group: its kernel rows, transformed once
+      RowRegs<MEGA_F32> rk;
+      fetch_rows<LOGA>(rk, rows_of(it, k, 4, false), L, false, tid);
+      place_rows<LOGA>(pre, red, rk, false, tid, sk);
+      transform<LOGA, false>(pre, w, wave, lane);
+      capture_spectrum<LOGA>(pre, spk, tid);
+      if (spec_k != nullptr) {
+        uint32_t* const save_k = spec_k + static_cast<size_t>(d0 / R) * kSpecWords;
+        store_spectrum(save_k, spk, tid);
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+          if (tid == i) reinterpret_cast<float*>(save_k + kSpecScaleWords)[i] = sk[i];
+      }
+      lds_barrier();
+    }
+    const RowPtrs<LOGA> xrows = rows_of(it, x, 2, true);
+    float wres[R], sx[R], scale[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) wres[i] = (omega != nullptr && d0 + i < D) ? omega[d0 + i] : 0.f;
+    place_rows<LOGA>(pre, red, rx, false, tid, sx);
+    transform<LOGA, false>(pre, w, wave, lane);
+    uint32_t* save_x = nullptr;
+    if (spec_x != nullptr) {
+      save_x = spec_x + static_cast<size_t>((bb * D + d0) / R) * kSpecWords;
+#pragma unroll
+      for (int i = 0; i < R; ++i)
+        if (tid == i) reinterpret_cast<float*>(save_x + kSpecScaleWords)[i] = sx[i];
+    }
+    pointwise<LOGA>(pre, spk, tid, save_x);
+    lds_barrier();
+    if (it + 1 < total) fetch_rows<LOGA>(rx, rows_of(it + 1, x, 2, true), L, false, tid);
+    transform<LOGA, true>(pre, w, wave, lane);
+    final_scales<LOGA>(sx, sk, scale);
+    store_rows<LOGA, DT, false>(pre, rows_of(it, y, 2, true), L, false, scale,
+                                omega != nullptr ? &xrows : nullptr, wres, tid);
     lds_barrier();
   }
 }
@@ -1224,6 +1302,20 @@ int launch(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_
       reinterpret_cast<const void*>(&fftconv_mfma_kernel<DT, MODE, LOGA>),
       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBytes)));
   constexpr int R = Geo<LOGA>::R;
+  if (MODE == 0 && B >= 2 && flip == 0 && 2 * ((D + R - 1) / R) >= cus) {
+    // enough channel groups to fill the chip: one transform of k per group instead of one per row
+    MEGA_CHECK_HIP(hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&fftconv_mfma_fwd_batch_kernel<DT, LOGA>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBytes)));
+    MEGA_CHECK_ARG(B * D <= 0x7fffffff, "fftconv: too many rows");
+    const int64_t groups = (D + R - 1) / R;
+    const unsigned grid = static_cast<unsigned>(groups < cus ? groups : cus);
+    fftconv_mfma_fwd_batch_kernel<DT, LOGA><<<dim3(grid), kThreads, kLdsBytes, stream>>>(
+        a, static_cast<const float*>(b), out, static_cast<int>(B), static_cast<int>(D),
+        static_cast<int>(L), omega, spec_a, spec_b);
+    MEGA_CHECK_LAUNCH();
+    return MEGA_OK;
+  }
   if (MODE == 0) {
     const int64_t rows = B * D;
     MEGA_CHECK_ARG(rows <= 0x7fffffff, "fftconv: too many rows");

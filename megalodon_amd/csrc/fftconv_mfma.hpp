@@ -20,8 +20,8 @@ int launch_conv(int dtype, int mode, const void* a, const void* b, void* out, in
 int launch_backward(int dtype, const void* dy, const void* x, const float* k, void* dx, float* dk,
                     int64_t B, int64_t D, int64_t L, const float* omega, hipStream_t stream);
 
-// Saved spectra.  spectrum_bytes: size of one spectrum buffer (that of x or of k)
-// for the shape, 0 when the shape cannot take this path (16-bit rows, 2048 < L
+// Saved spectra.  spectrum_bytes: size of the spectrum buffer of x for the shape
+// (that of k, kept once per channel, has the size for B = 1), 0 when the shape cannot take this path (16-bit rows, 2048 < L
 // <= 32768, L % 8 == 0, D a multiple of the rows per pass).  launch_forward_saving
 // is launch_conv mode 0 that also fills both buffers; launch_backward_saved
 // computes dx (+ omega dy) and dk from dy and the two buffers alone.

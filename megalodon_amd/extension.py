@@ -385,7 +385,8 @@ def fftconv_residual_fwd_saving(x: torch.Tensor, k: torch.Tensor, omega: torch.T
     wc = omega.reshape(-1).contiguous().float()
     y = torch.empty_like(xc)
     spec_x = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    spec_k = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    # the spectrum of k is kept once per channel, whatever the batch size
+    spec_k = torch.empty(fftconv_spectrum_bytes(x.dtype, 1, D, L), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         _lib.call("mega_fftconv_residual_fwd_saving", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
                   _lib.ptr(kc), _lib.ptr(wc), _lib.i64(B), _lib.i64(D), _lib.i64(L), _lib.ptr(y),
@@ -398,7 +399,8 @@ def fftconv_residual_bwd_saved(y_grad: torch.Tensor, spec_x: torch.Tensor, spec_
     """(dx, dk, domega) from y_grad (B, D, L) and the two saved spectra."""
     dev = _require_cuda(y_grad, spec_x, spec_k, omega)
     B, D, L = y_grad.shape
-    if spec_x.numel() != fftconv_spectrum_bytes(y_grad.dtype, B, D, L) or spec_k.numel() != spec_x.numel():
+    if (spec_x.numel() != fftconv_spectrum_bytes(y_grad.dtype, B, D, L)
+            or spec_k.numel() != fftconv_spectrum_bytes(y_grad.dtype, 1, D, L)):
         raise RuntimeError("fftconv_bwd: the saved spectra do not belong to this shape")
     dy = y_grad.contiguous()
     wc = omega.reshape(-1).contiguous().float()

@@ -96,6 +96,36 @@ def test_saved_spectrum_pair_matches_oracle(B, D, L, dtype):
     assert torch.equal(y, ops.fftconv_residual_fwd(x.cuda(), k.cuda(), omega.cuda()))
 
 
+@pytest.mark.parametrize("B,D,L", [(3, 256, 20000), (2, 1024, 4096), (2, 130, 32768), (4, 520, 9000)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_batch_walking_forward_matches_oracle(B, D, L, dtype):
+    """B > 1 with at least half as many channel groups as compute units: the
+    forward that transforms k once per channel group and walks the batch, with
+    and without kept spectra, and the backward from those spectra (the
+    spectrum of k is kept once per channel)."""
+    x, k, dy = _data(B, D, L, dtype, 17 * L + B)
+    omega = torch.randn(D, 1, generator=torch.Generator().manual_seed(L)) * 0.5
+    w64 = omega.double().view(1, D, 1)
+    want = fftconv.fftconv_fwd(x, k).double()
+    y0 = ops.fftconv_fwd(x.cuda(), k.cuda())
+    assert rel_err(y0, want) <= TOL[dtype]
+    y1 = ops.fftconv_residual_fwd(x.cuda(), k.cuda(), omega.cuda())
+    assert rel_err(y1, want + w64 * x.double()) <= TOL[dtype]
+    if ops.fftconv_spectrum_bytes(dtype, B, D, L) == 0:
+        return
+    y, sx, sk = ops.fftconv_residual_fwd_saving(x.cuda(), k.cuda(), omega.cuda())
+    assert torch.equal(y, y1)
+    assert sk.numel() == ops.fftconv_spectrum_bytes(dtype, 1, D, L) and sx.numel() == B * sk.numel()
+    dx, dk, dw = ops.fftconv_residual_bwd_saved(dy.cuda(), sx, sk, omega.cuda())
+    wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
+    assert rel_err(dx, wdx.double() + w64 * dy.double()) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= TOL[dtype]
+    assert rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= TOL[dtype]
+    # every batch entry on its own (B = 1: the kernel that transforms k per row) gives the same rows
+    for b in range(B):
+        assert torch.equal(ops.fftconv_residual_fwd(x[b:b + 1].cuda(), k.cuda(), omega.cuda())[0], y1[b])
+
+
 def test_saved_spectrum_pair_at_full_row_count_agrees_with_recomputing_pair():
     """Config-1 rows (L = 32768, bf16) over 512 channels and two batch entries:
     the backward from kept spectra and the backward that re-transforms x and k
