@@ -21,6 +21,7 @@ from .. import extension as megalodon_ops
 from ..fused_ops import memory_efficient_dropout, qk_norm_rotary, silu_mul, transpose_last2
 from .chunk_attention import _InnerAttention
 from .complex_exponential_moving_average import MultiHeadComplexEMA
+from .linear import Linear
 from .layer_norm import FusedRMSNorm
 from .normalized_feedforward_network import NormalizedFeedForwardNetwork
 from .timestep_norm import TimestepNorm
@@ -51,11 +52,11 @@ class MovingAverageGatedAttention(nn.Module):
         self.rmsnorm = FusedRMSNorm(mdim, elementwise_affine=norm_affine, eps=norm_eps)
         self.znorm = FusedRMSNorm(self.z_head_dim, elementwise_affine=False, eps=norm_eps)
 
-        self.wv = nn.Linear(mdim, hdim, bias=True)
-        self.wz = nn.Linear(mdim, zdim, bias=True)
-        self.wr = nn.Linear(mdim, hdim, bias=True)
-        self.wh1 = nn.Linear(mdim, mdim, bias=True)
-        self.wh2 = nn.Linear(hdim, mdim, bias=False)
+        self.wv = Linear(mdim, hdim, bias=True)
+        self.wz = Linear(mdim, zdim, bias=True)
+        self.wr = Linear(mdim, hdim, bias=True)
+        self.wh1 = Linear(mdim, mdim, bias=True)
+        self.wh2 = Linear(hdim, mdim, bias=False)
         for lin in (self.wv, self.wz, self.wr, self.wh1, self.wh2):
             nn.init.normal_(lin.weight, mean=0.0, std=init_std)
             if lin.bias is not None:

@@ -7,6 +7,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from ..fused_ops import memory_efficient_dropout, silu_mul
+from .linear import Linear
 from .layer_norm import FusedLayerNorm
 
 
@@ -21,9 +22,9 @@ class NormalizedFeedForwardNetwork(nn.Module):
         self.swiglu = swiglu
         self.rescale_init = rescale
         self.norm = FusedLayerNorm(model_dim, elementwise_affine=norm_affine, eps=norm_eps)
-        self.fc1 = nn.Linear(model_dim, ffn_hidden_dim, bias=False)
-        self.fc2 = nn.Linear(ffn_hidden_dim, model_dim, bias=False)
-        self.fc3 = nn.Linear(model_dim, ffn_hidden_dim, bias=False) if swiglu else None
+        self.fc1 = Linear(model_dim, ffn_hidden_dim, bias=False)
+        self.fc2 = Linear(ffn_hidden_dim, model_dim, bias=False)
+        self.fc3 = Linear(model_dim, ffn_hidden_dim, bias=False) if swiglu else None
         for lin in (self.fc1, self.fc2, self.fc3):
             if lin is not None:
                 nn.init.normal_(lin.weight, mean=0.0, std=init_std)

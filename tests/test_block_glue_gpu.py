@@ -95,3 +95,29 @@ def test_silu_gate_at_the_feed_forward_size():
     s = torch.sigmoid(a[idx].double())
     assert rel_err(db[idx], y[idx].double() * a[idx].double() * s) <= 2e-2
     assert rel_err(da[idx], y[idx].double() * b[idx].double() * s * (1 + a[idx].double() * (1 - s))) <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,out,bias", [((2, 300, 256), 512, True), ((640, 1024), 264, False), ((3, 5, 7, 64), 72, True)])
+def test_linear_with_transposed_weight_backward_matches_float64(shape, out, bias, dtype):
+    from megalodon_amd.modules.linear import Linear
+    torch.manual_seed(out)
+    lin = Linear(shape[-1], out, bias=bias).cuda().to(dtype)
+    x = torch.randn(*shape, device="cuda").to(dtype).requires_grad_(True)
+    dy = torch.randn(*shape[:-1], out, device="cuda").to(dtype)
+    y = lin(x)
+    y.backward(dy)
+    x64 = x.detach().double().requires_grad_(True)
+    w64 = lin.weight.detach().double().requires_grad_(True)
+    b64 = lin.bias.detach().double().requires_grad_(True) if bias else None
+    want = F.linear(x64, w64, b64)
+    want.backward(dy.double())
+    assert rel_err(y, want) <= 2e-2 and rel_err(x.grad, x64.grad) <= 2e-2
+    assert rel_err(lin.weight.grad, w64.grad) <= 2e-2
+    if bias:
+        assert rel_err(lin.bias.grad, b64.grad) <= 2e-2
+    # state dicts are those of nn.Linear; without gradients the module is F.linear itself
+    ref = torch.nn.Linear(shape[-1], out, bias=bias).cuda().to(dtype)
+    ref.load_state_dict(lin.state_dict())
+    with torch.no_grad():
+        assert torch.equal(lin(x), ref(x))
