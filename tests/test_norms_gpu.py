@@ -116,3 +116,32 @@ def test_full_size_rows_are_independent():
         assert rel_err(dw, (dy.double() * xh).sum(0)) <= 2e-2
         if not rms:
             assert rel_err(db, dy.double().sum(0)) <= 2e-2
+
+
+@pytest.mark.parametrize("D,rms", [(4096, False), (8192, False), (8192, True), (10000, True)])
+def test_float32_rows_wider_than_one_stripe_per_wave(D, rms):
+    """float32 rows take the element-wise kernels, whose parameter-gradient
+    stripes share 64 KB of LDS: 4, 2 or 1 working waves per workgroup."""
+    g = torch.Generator().manual_seed(D)
+    x = torch.randn(3, 11, D, generator=g)
+    dy = torch.randn(3, 11, D, generator=g)
+    w = torch.randn(D, generator=g) * 0.2
+    b = None if rms else torch.randn(D, generator=g) * 0.2
+    xg, wg = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    bg = None if b is None else b.cuda().requires_grad_(True)
+    y = layer_norm_plus_one(xg, wg, bg, 1e-5, rms)
+    y.backward(dy.cuda())
+    wy, wdx, wdw, wdb = _reference(x, w, b, 1e-5, rms, dy)
+    assert rel_err(y, wy) <= 1e-4 and rel_err(xg.grad, wdx) <= 1e-4 and rel_err(wg.grad, wdw) <= 1e-4
+    if not rms:
+        assert rel_err(bg.grad, wdb) <= 1e-4
+
+
+def test_parameter_gradients_that_do_not_fit_are_refused():
+    x = torch.randn(4, 10000, device="cuda")
+    w = torch.zeros(10000, device="cuda")
+    y, mean, rstd = ops.layer_norm_fwd(x, w, w, 1e-5, False)
+    with pytest.raises(RuntimeError, match="do not fit"):
+        ops.layer_norm_bwd(torch.ones_like(x), x, w, mean, rstd, False, True)
+    dx, dw, db = ops.layer_norm_bwd(torch.ones_like(x), x, None, mean, rstd, False, False)   # no parameters: fine
+    assert dw is None and db is None and torch.isfinite(dx).all()
