@@ -302,26 +302,56 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
   };
 
   // One step per slab, one barrier per step, placed between the two k-steps:
-  //   write slab cur+1 to the other LDS buffer, request slab cur+3,
-  //   read the second fragment set of slab cur, first 16 MFMAs,
+  //   first half:  read the second fragment set of slab cur, write slab cur+1
+  //                to the other LDS buffer, 16 MFMAs on the first set,
   //   barrier,
-  //   read the first fragment set of slab cur+1, last 16 MFMAs.
-  // Each wait (LDS writes, barrier skew, fragment reads) then has 16 MFMAs
-  // already issued behind it.  Loads and LDS stores are unconditional, so every
-  // path has the same number of loads in flight and the waits can count.
+  //   second half: read the first fragment set of slab cur+1, request slab
+  //                cur+3, 16 MFMAs on the second set.
+  // Loads and LDS stores are unconditional, so every path has the same number
+  // of loads in flight and the waits can count.
+  // Inside each half the 16 MFMAs and the half's memory instructions are one
+  // scheduling region, interleaved by sched_group_barrier: one MFMA, then one
+  // LDS write or global load, then one LDS read.  An MFMA occupies the matrix
+  // pipe for 8 passes while the wave may issue other instructions, and a wave
+  // issues in order -- memory instructions bunched in front of the MFMAs leave
+  // the matrix pipe idle while they issue (one wave per SIMD: nobody else
+  // feeds it).
+#define MEGA_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+  // What the barrier waits for goes first: the fragment reads of this slab
+  // (their buffer is overwritten after the barrier) under the first four
+  // MFMAs, the LDS writes of the next slab under the next eight; the global
+  // loads (nobody waits for them here) go under the MFMAs of the second half,
+  // behind the fragment reads for the next slab.
+  constexpr int kFragReads = (TA ? 2 : 1) + (TB ? 2 : 1);  // LDS reads per MFMA of the first four
 #define MEGA_GEMM_STEP(R, CA, CB, NA, NB)                                  \
   {                                                                        \
     const int cur = it + (R);                                              \
-    sstore(NA, NB, cur + 1);                                               \
-    gload(CA, CB, cur + kRing);                                            \
     fread(fa1, fb1, 1, cur & 1);                                           \
-    __builtin_amdgcn_sched_barrier(0);                                     \
+    sstore(NA, NB, cur + 1);                                               \
     mma(fa0, fb0);                                                         \
+    _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
+      MEGA_SGB(0x008, 1);                                                  \
+      MEGA_SGB(0x100, kFragReads);                                         \
+    }                                                                      \
+    _Pragma("unroll") for (int sg = 0; sg < 8; ++sg) {                     \
+      MEGA_SGB(0x008, 1);                                                  \
+      MEGA_SGB(0x200, 1);                                                  \
+    }                                                                      \
+    MEGA_SGB(0x008, 4);                                                    \
     __builtin_amdgcn_sched_barrier(0);                                     \
     lds_barrier();                                                         \
     fread(fa0, fb0, 0, (cur + 1) & 1);                                     \
-    __builtin_amdgcn_sched_barrier(0);                                     \
+    gload(CA, CB, cur + kRing);                                            \
     mma(fa1, fb1);                                                         \
+    _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
+      MEGA_SGB(0x008, 1);                                                  \
+      MEGA_SGB(0x100, kFragReads);                                         \
+    }                                                                      \
+    _Pragma("unroll") for (int sg = 0; sg < 8; ++sg) {                     \
+      MEGA_SGB(0x008, 1);                                                  \
+      MEGA_SGB(0x020, 1);                                                  \
+    }                                                                      \
+    MEGA_SGB(0x008, 4);                                                    \
     __builtin_amdgcn_sched_barrier(0);                                     \
   }
   if (nslab > 0) {
@@ -344,6 +374,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
     lds_barrier();  // every wave is done with the slab buffers before they are reused
   }
 #undef MEGA_GEMM_STEP
+#undef MEGA_SGB
 
   // epilogue: stage the wave's 128x128 tile in LDS ([row][col], element type),
   // then write it with 16-byte row segments.  The products are issued as
