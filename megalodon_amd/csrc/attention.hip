@@ -11,7 +11,7 @@
 //
 // Differences in execution: the reference runs full-square cuBLAS GEMMs and a
 // full-row softmax; here every product is one hand-written MFMA GEMM
-// (v_mfma_f32_32x32x16, 256x256 workgroup tile, 128x128 per wavefront,
+// (v_mfma_f32_32x32x16, 256x256 workgroup tile, eight wavefronts of 128x64,
 // double-buffered LDS staging of 32-wide k slabs) that skips the tiles above
 // the causal diagonal and the k-ranges where P / dS are structurally zero, so
 // causal attention costs half the flops and half the P traffic.  Operands whose
@@ -23,6 +23,7 @@
 #include "common.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace mega {
 namespace {
@@ -136,13 +137,18 @@ __device__ __forceinline__ uint2 lds_read_tr(const uint16_t* q) {
 
 // C[m][n] = alpha * sum_k A(m, k) B(n, k).  An operand is either k-contiguous
 // (rows m, `ld` between rows) or, with TA / TB, k-major (rows k, m contiguous).
-template <int DT, bool FAST, bool TA, bool TB>
-__global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
+template <int DT, bool FAST, bool TA, bool TB, bool W8>
+__global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(const GemmParams p) {
   extern __shared__ __align__(16) uint16_t smem[];
-  // main loop: [buf][A|B] operand slabs; epilogue: [wave][128][kEpiPitch]
+  // main loop: [buf][A|B] operand slabs; epilogue: [wave][128][pitch]
   constexpr int kOperand = kOperandElems;
+  // W8: eight waves (two per SIMD) of 128 x 64 each instead of four of 128 x 128
+  constexpr int T = W8 ? 2 * kThreads : kThreads;  // threads
+  constexpr int JN = W8 ? 2 : 4;                   // 32-column blocks per wave
+  constexpr int NL = W8 ? 2 : 4;                   // 16-byte chunks per thread, operand and slab
+  constexpr int EP = W8 ? 64 + 8 : kEpiPitch;      // staging pitch
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = W8 ? wave >> 2 : wave >> 1, wn = W8 ? wave & 3 : wave & 1;
 
   // Persistent workgroups (one per CU) walk a list of work items of equal
   // weight, so nothing is launched for skipped tiles and no CU ends up with
@@ -205,32 +211,33 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
   if (p.k_mode == 2) kb = min(p.K, max(0, mt * kTile - p.off) / kSlab * kSlab);
   const int nslab = (ke - kb + kSlab - 1) / kSlab;
 
-  floatx16 acc[4][4];
+  floatx16 acc[4][JN];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < JN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // register ring: slab s lives in ring slot s % 3 from its issue (three steps
   // before use) until it is written to LDS
-  u32x4 ra0[4], ra1[4], ra2[4], rb0[4], rb1[4], rb2[4];
+  constexpr int RING = W8 ? 4 : kRing;  // slabs in flight from memory
+  u32x4 ra0[NL], ra1[NL], ra2[NL], ra3[W8 ? NL : 1], rb0[NL], rb1[NL], rb2[NL], rb3[W8 ? NL : 1];
 
   // Global -> register chunk i of a thread (16 bytes):
-  //   k-contiguous operand: row (tid >> 2) + 64 i, k chunk tid & 3
-  //   k-major operand:      k row (tid >> 5) + 8 i, m chunk tid & 31
+  //   k-contiguous operand: row (tid >> 2) + T / 4 i, k chunk tid & 3
+  //   k-major operand:      k row (tid >> 5) + T / 32 i, m chunk tid & 31
   // FAST (16-byte aligned rows, K % 32 == 0, extents % 8 == 0 and below 1 GiB):
   // branch-free loads from a uniform base plus 32-bit byte offsets with rows,
   // columns and slab index clamped into the matrix, so nothing forces a wait
   // on the loads in flight.  Otherwise: bounds-checked element loads.
-  uint32_t offa[4], offb[4];
+  uint32_t offa[NL], offb[NL];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if (TA) offa[i] = static_cast<uint32_t>(((kb + (tid >> 5) + 8 * i) * p.lda + min(m0 + (tid & 31) * 8, p.M - 8)) * 2);
-    else offa[i] = static_cast<uint32_t>((static_cast<int64_t>(min(m0 + (tid >> 2) + 64 * i, p.M - 1)) * p.lda + kb + (tid & 3) * 8) * 2);
-    if (TB) offb[i] = static_cast<uint32_t>(((kb + (tid >> 5) + 8 * i) * p.ldb + min(n0 + (tid & 31) * 8, p.N - 8)) * 2);
-    else offb[i] = static_cast<uint32_t>((static_cast<int64_t>(min(n0 + (tid >> 2) + 64 * i, p.N - 1)) * p.ldb + kb + (tid & 3) * 8) * 2);
+  for (int i = 0; i < NL; ++i) {
+    if (TA) offa[i] = static_cast<uint32_t>(((kb + (tid >> 5) + (T / 32) * i) * p.lda + min(m0 + (tid & 31) * 8, p.M - 8)) * 2);
+    else offa[i] = static_cast<uint32_t>((static_cast<int64_t>(min(m0 + (tid >> 2) + (T / 4) * i, p.M - 1)) * p.lda + kb + (tid & 3) * 8) * 2);
+    if (TB) offb[i] = static_cast<uint32_t>(((kb + (tid >> 5) + (T / 32) * i) * p.ldb + min(n0 + (tid & 31) * 8, p.N - 8)) * 2);
+    else offb[i] = static_cast<uint32_t>((static_cast<int64_t>(min(n0 + (tid >> 2) + (T / 4) * i, p.N - 1)) * p.ldb + kb + (tid & 3) * 8) * 2);
   }
   const uint32_t stepa = static_cast<uint32_t>((TA ? p.lda : 1) * kSlab * 2);
   const uint32_t stepb = static_cast<uint32_t>((TB ? p.ldb : 1) * kSlab * 2);
@@ -238,18 +245,18 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
     if (FAST) {
       const uint32_t sc = static_cast<uint32_t>(min(s, nslab - 1));
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < NL; ++i) {
         qa[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(A) + (offa[i] + sc * stepa));
         qb[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(B) + (offb[i] + sc * stepb));
       }
     } else {
       const int k0 = kb + s * kSlab;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (TA) qa[i] = load_chunk<false>(A, p.lda, k0 + (tid >> 5) + 8 * i, ke, m0 + (tid & 31) * 8, p.M);
-        else qa[i] = load_chunk<false>(A, p.lda, m0 + (tid >> 2) + 64 * i, p.M, k0 + (tid & 3) * 8, ke);
-        if (TB) qb[i] = load_chunk<false>(B, p.ldb, k0 + (tid >> 5) + 8 * i, ke, n0 + (tid & 31) * 8, p.N);
-        else qb[i] = load_chunk<false>(B, p.ldb, n0 + (tid >> 2) + 64 * i, p.N, k0 + (tid & 3) * 8, ke);
+      for (int i = 0; i < NL; ++i) {
+        if (TA) qa[i] = load_chunk<false>(A, p.lda, k0 + (tid >> 5) + (T / 32) * i, ke, m0 + (tid & 31) * 8, p.M);
+        else qa[i] = load_chunk<false>(A, p.lda, m0 + (tid >> 2) + (T / 4) * i, p.M, k0 + (tid & 3) * 8, ke);
+        if (TB) qb[i] = load_chunk<false>(B, p.ldb, k0 + (tid >> 5) + (T / 32) * i, ke, n0 + (tid & 31) * 8, p.N);
+        else qb[i] = load_chunk<false>(B, p.ldb, n0 + (tid >> 2) + (T / 4) * i, p.N, k0 + (tid & 3) * 8, ke);
       }
     }
   };
@@ -261,19 +268,19 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
     uint16_t* sa = smem + (s & 1) * 2 * kOperand + st_a;
     uint16_t* sb = smem + (s & 1) * 2 * kOperand + kOperand + st_b;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<u32x4*>(sa + i * (TA ? 8 * kPitchT : 64 * 8)) = qa[i];
-      *reinterpret_cast<u32x4*>(sb + i * (TB ? 8 * kPitchT : 64 * 8)) = qb[i];
+    for (int i = 0; i < NL; ++i) {
+      *reinterpret_cast<u32x4*>(sa + i * (TA ? (T / 32) * kPitchT : (T / 4) * 8)) = qa[i];
+      *reinterpret_cast<u32x4*>(sb + i * (TB ? (T / 32) * kPitchT : (T / 4) * 8)) = qb[i];
     }
   };
 
   // MFMA fragments: set ks holds the k-step ks (16 k values) of a slab; lane l
   // owns row l % 32 of a 32-row tile and k values 8 (l / 32) .. + 7
   static_assert(kSlab == 32, "the pipeline below is written for two k-steps per slab");
-  u32x4 fa0[4], fb0[4], fa1[4], fb1[4];
+  u32x4 fa0[4], fb0[JN], fa1[4], fb1[JN];
   const int tr_lane = (8 * (lane >> 5) + ((lane & 15) >> 2)) * kPitchT + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
   const int frag_a = TA ? tr_lane + wm * 128 : ((lane >> 5) * kChunkPitch + wm * 128 + (lane & 31)) * 8;
-  const int frag_b = kOperand + (TB ? tr_lane + wn * 128 : ((lane >> 5) * kChunkPitch + wn * 128 + (lane & 31)) * 8);
+  const int frag_b = kOperand + (TB ? tr_lane + wn * (32 * JN) : ((lane >> 5) * kChunkPitch + wn * (32 * JN) + (lane & 31)) * 8);
   auto fread = [&](u32x4* fa, u32x4* fb, int set, int buf) {
     const uint16_t* base = smem + buf * 2 * kOperand;
     const uint16_t* qa = base + frag_a + set * (TA ? 16 * kPitchT : 2 * kChunkPitch * 8);
@@ -286,11 +293,13 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
       } else {
         fa[i] = *reinterpret_cast<const u32x4*>(qa + i * 32 * 8);
       }
-      if (TB) {
-        const uint2 lo = lds_read_tr(qb + i * 32), hi = lds_read_tr(qb + i * 32 + 4 * kPitchT);
-        fb[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
-      } else {
-        fb[i] = *reinterpret_cast<const u32x4*>(qb + i * 32 * 8);
+      if (i < JN) {
+        if (TB) {
+          const uint2 lo = lds_read_tr(qb + i * 32), hi = lds_read_tr(qb + i * 32 + 4 * kPitchT);
+          fb[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        } else {
+          fb[i] = *reinterpret_cast<const u32x4*>(qb + i * 32 * 8);
+        }
       }
     }
   };
@@ -298,7 +307,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = Mma<DT>::run(fb[j], fa[i], acc[i][j]);
+      for (int j = 0; j < JN; ++j) acc[i][j] = Mma<DT>::run(fb[j], fa[i], acc[i][j]);
   };
 
   // One step per slab, one barrier per step, placed between the two k-steps:
@@ -322,7 +331,8 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
   // MFMAs, the LDS writes of the next slab under the next eight; the global
   // loads (nobody waits for them here) go under the MFMAs of the second half,
   // behind the fragment reads for the next slab.
-  constexpr int kFragReads = (TA ? 2 : 1) + (TB ? 2 : 1);  // LDS reads per MFMA of the first four
+  constexpr int kFragReads = (TA ? 2 : 1) + (TB ? JN / 2 : (JN + 3) / 4);  // LDS reads per MFMA of the first four
+  constexpr int kRest = 4 * JN - 4 - 2 * NL;  // MFMAs of a half with nothing to carry
 #define MEGA_GEMM_STEP(R, CA, CB, NA, NB)                                  \
   {                                                                        \
     const int cur = it + (R);                                              \
@@ -333,44 +343,57 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
       MEGA_SGB(0x008, 1);                                                  \
       MEGA_SGB(0x100, kFragReads);                                         \
     }                                                                      \
-    _Pragma("unroll") for (int sg = 0; sg < 8; ++sg) {                     \
+    _Pragma("unroll") for (int sg = 0; sg < 2 * NL; ++sg) {                \
       MEGA_SGB(0x008, 1);                                                  \
       MEGA_SGB(0x200, 1);                                                  \
     }                                                                      \
-    MEGA_SGB(0x008, 4);                                                    \
+    if (kRest > 0) MEGA_SGB(0x008, kRest);                                 \
     __builtin_amdgcn_sched_barrier(0);                                     \
     lds_barrier();                                                         \
     fread(fa0, fb0, 0, (cur + 1) & 1);                                     \
-    gload(CA, CB, cur + kRing);                                            \
+    gload(CA, CB, cur + RING);                                             \
     mma(fa1, fb1);                                                         \
     _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
       MEGA_SGB(0x008, 1);                                                  \
       MEGA_SGB(0x100, kFragReads);                                         \
     }                                                                      \
-    _Pragma("unroll") for (int sg = 0; sg < 8; ++sg) {                     \
+    _Pragma("unroll") for (int sg = 0; sg < 2 * NL; ++sg) {                \
       MEGA_SGB(0x008, 1);                                                  \
       MEGA_SGB(0x020, 1);                                                  \
     }                                                                      \
-    MEGA_SGB(0x008, 4);                                                    \
+    if (kRest > 0) MEGA_SGB(0x008, kRest);                                 \
     __builtin_amdgcn_sched_barrier(0);                                     \
   }
   if (nslab > 0) {
     gload(ra0, rb0, 0);
     gload(ra1, rb1, 1);
     gload(ra2, rb2, 2);
+    if constexpr (RING == 4) gload(ra3, rb3, 3);
     sstore(ra0, rb0, 0);
     lds_barrier();
     fread(fa0, fb0, 0, 0);
     // ring slot R held slab cur, already written to LDS, so it is free for
     // slab cur + kRing
     int it = 0;
-    for (; it + kRing <= nslab; it += kRing) {
-      MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
-      MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
-      MEGA_GEMM_STEP(2, ra2, rb2, ra0, rb0)
+    if constexpr (RING == 4) {
+      for (; it + 4 <= nslab; it += 4) {
+        MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
+        MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
+        MEGA_GEMM_STEP(2, ra2, rb2, ra3, rb3)
+        MEGA_GEMM_STEP(3, ra3, rb3, ra0, rb0)
+      }
+      if (it < nslab) MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
+      if (it + 1 < nslab) MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
+      if (it + 2 < nslab) MEGA_GEMM_STEP(2, ra2, rb2, ra3, rb3)
+    } else {
+      for (; it + kRing <= nslab; it += kRing) {
+        MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
+        MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
+        MEGA_GEMM_STEP(2, ra2, rb2, ra0, rb0)
+      }
+      if (it < nslab) MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
+      if (it + 1 < nslab) MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
     }
-    if (it < nslab) MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
-    if (it + 1 < nslab) MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
     lds_barrier();  // every wave is done with the slab buffers before they are reused
   }
 #undef MEGA_GEMM_STEP
@@ -381,11 +404,11 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
   // B-fragment x A-fragment, so a 32x32 MFMA tile holds C transposed: lane l has
   // row m = l % 32 and register r the column n = 8 (r / 4) + 4 (l / 32) + r % 4,
   // i.e. four consecutive columns per register quad -> one 8-byte LDS write.
-  uint16_t* stage = smem + wave * 128 * kEpiPitch;
+  uint16_t* stage = smem + wave * 128 * EP;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < JN; ++j) {
       const int row = i * 32 + (lane & 31);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -401,19 +424,19 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
           w.x = static_cast<uint32_t>(float_to_f16_bits(v[0])) | (static_cast<uint32_t>(float_to_f16_bits(v[1])) << 16);
           w.y = static_cast<uint32_t>(float_to_f16_bits(v[2])) | (static_cast<uint32_t>(float_to_f16_bits(v[3])) << 16);
         }
-        *reinterpret_cast<uint2*>(stage + row * kEpiPitch + col) = w;
+        *reinterpret_cast<uint2*>(stage + row * EP + col) = w;
       }
     }
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave reads back only its own region
   const bool vec_ok = (p.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
 #pragma unroll 4
-  for (int i = 0; i < 32; ++i) {
+  for (int i = 0; i < 8 * JN; ++i) {
     const int c = lane + kWave * i;
-    const int row = c >> 4, kc = (c & 15) * 8;
-    const int grow = m0 + wm * 128 + row, gcol = n0 + wn * 128 + kc;
+    const int row = c / (4 * JN), kc = (c % (4 * JN)) * 8;
+    const int grow = m0 + wm * 128 + row, gcol = n0 + wn * (32 * JN) + kc;
     if (grow < p.M && gcol < p.N) {
-      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * kEpiPitch + kc);
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * EP + kc);
       uint16_t* dst = C + static_cast<int64_t>(grow) * p.ldc + gcol;
       if (vec_ok && gcol + 8 <= p.N) {
         *reinterpret_cast<u32x4*>(dst) = v;
@@ -719,14 +742,24 @@ int launch_gemm_t(const GemmParams& p, int batch, hipStream_t s) {
   if (g >= kXcds) g -= g % kXcds;
   const dim3 grid(static_cast<unsigned>(g));
   const size_t lds = kGemmLds;
-  if (fast) {
-    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, true, TA, TB>),
+  // Eight waves of 128 x 64 (two per SIMD, accumulators in the unified register
+  // file, a ring of four slabs) hide more latency than four of 128 x 128 with
+  // one per SIMD; MEGA_GEMM_W4=1 in the environment selects the latter for
+  // comparison.
+  const char* w4 = getenv("MEGA_GEMM_W4");
+  if (fast && !(w4 != nullptr && w4[0] == '1')) {
+    const size_t lds8 = sizeof(uint16_t) * 8 * 128 * (64 + 8) > lds ? sizeof(uint16_t) * 8 * 128 * (64 + 8) : lds;
+    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, true, TA, TB, true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds8));
+    gemm_kernel<DT, true, TA, TB, true><<<grid, 2 * kThreads, lds8, s>>>(q);
+  } else if (fast) {
+    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, true, TA, TB, false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    gemm_kernel<DT, true, TA, TB><<<grid, kThreads, lds, s>>>(q);
+    gemm_kernel<DT, true, TA, TB, false><<<grid, kThreads, lds, s>>>(q);
   } else {
-    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, false, TA, TB>),
+    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, false, TA, TB, false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    gemm_kernel<DT, false, TA, TB><<<grid, kThreads, lds, s>>>(q);
+    gemm_kernel<DT, false, TA, TB, false><<<grid, kThreads, lds, s>>>(q);
   }
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
