@@ -32,9 +32,11 @@ constexpr int kTile = 256;     // workgroup tile (M and N)
 constexpr int kSlab = 32;      // k elements staged per iteration
 // LDS slab layout: 16-byte chunks (8 k values of one row), chunk (c, row) at
 // index c * kChunkPitch + row.  A fragment read then has consecutive lanes on
-// consecutive chunks, and the 4 (c) x 4 (row) chunks a group of 16 lanes writes
-// land on 16 different bank groups (260 = 4 mod 16).
-constexpr int kChunkPitch = kTile + 4;
+// consecutive chunks.  16-byte LDS accesses go eight lanes at a time over 32
+// banks (measured: a pitch of 260 chunks left a third of the LDS cycles as bank
+// conflicts, 264 was worse, 258 leaves 3 %): the 4 (c) x 2 (row) chunks that
+// eight neighbouring lanes write must differ mod 8, so the pitch is 2 mod 8.
+constexpr int kChunkPitch = kTile + 2;
 // k-major operands keep their rows of k: 256 + 32 elements per row, so that the
 // four rows a transposing read touches start 16 banks apart.
 constexpr int kPitchT = kTile + 32;
@@ -278,13 +280,16 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
   // owns row l % 32 of a 32-row tile and k values 8 (l / 32) .. + 7
   static_assert(kSlab == 32, "the pipeline below is written for two k-steps per slab");
   u32x4 fa0[4], fb0[JN], fa1[4], fb1[JN];
-  const int tr_lane = (8 * (lane >> 5) + ((lane & 15) >> 2)) * kPitchT + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-  const int frag_a = TA ? tr_lane + wm * 128 : ((lane >> 5) * kChunkPitch + wm * 128 + (lane & 31)) * 8;
-  const int frag_b = kOperand + (TB ? tr_lane + wn * (32 * JN) : ((lane >> 5) * kChunkPitch + wn * (32 * JN) + (lane & 31)) * 8);
+  // Which k a fragment slot holds only has to agree between A and B: k-step
+  // `set` of a slab takes k = 16 g + 8 set + e for lane half g = lane / 32, i.e.
+  // chunk planes set and set + 2.
+  const int tr_lane = (16 * (lane >> 5) + ((lane & 15) >> 2)) * kPitchT + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const int frag_a = TA ? tr_lane + wm * 128 : ((lane >> 5) * 2 * kChunkPitch + wm * 128 + (lane & 31)) * 8;
+  const int frag_b = kOperand + (TB ? tr_lane + wn * (32 * JN) : ((lane >> 5) * 2 * kChunkPitch + wn * (32 * JN) + (lane & 31)) * 8);
   auto fread = [&](u32x4* fa, u32x4* fb, int set, int buf) {
     const uint16_t* base = smem + buf * 2 * kOperand;
-    const uint16_t* qa = base + frag_a + set * (TA ? 16 * kPitchT : 2 * kChunkPitch * 8);
-    const uint16_t* qb = base + frag_b + set * (TB ? 16 * kPitchT : 2 * kChunkPitch * 8);
+    const uint16_t* qa = base + frag_a + set * (TA ? 8 * kPitchT : kChunkPitch * 8);
+    const uint16_t* qb = base + frag_b + set * (TB ? 8 * kPitchT : kChunkPitch * 8);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (TA) {
