@@ -290,7 +290,7 @@ __device__ __forceinline__ Dft make_dft_a(int lane) {
 // F1 (a -> k1): then twiddle W_(32 A)^(b k1), one factor per lane.  With A = 32
 // only a < 16 holds data (zero padding) -> one k-step; shorter rows have their
 // padding written as zeros and take both.  I3 (k1 -> a): no twiddle.
-template <int LOGA, bool INV>
+template <int LOGA, bool INV, bool PF>
 __device__ __forceinline__ void stage_a(uint16_t* pre, const Dft& w32, int wave, int lane) {
   constexpr int A = Geo<LOGA>::A;
   constexpr int KS = (INV || LOGA < 5) ? 2 : 1;
@@ -303,10 +303,21 @@ __device__ __forceinline__ void stage_a(uint16_t* pre, const Dft& w32, int wave,
   const int rd1 = (rsrc + 4) * kRS + (csrc ^ (((2 * g + 1) & 3) << 3));
   const int wr = f * kRS + 4 * g, fx = (f >> 2) & 3;
   const int wv = __builtin_amdgcn_readfirstlane(wave);
+  // PF: the operands of the wave's next tile are read before this tile's
+  // twiddles and write-back (tiles are disjoint, but the compiler cannot move
+  // LDS reads over LDS writes by itself); the loop is then fully unrolled.
+  u32x4 xr[2], xi[2], nr[2], ni[2];
+  if (PF) read_tile_tr<KS, 16 * kRS>(pre, (rd0 ^ (((wv >> 2) & 3) << 3)) + 32 * wv,
+                                     (rd1 ^ (((wv >> 2) & 3) << 3)) + 32 * wv, xr, xi);
+#pragma unroll(PF ? 4 : 1)
   for (int b = wv; b < 32; b += kWaves) {
     const int bx = ((b >> 2) & 3) << 3;
-    u32x4 xr[2], xi[2];
-    read_tile_tr<KS, 16 * kRS>(pre, (rd0 ^ bx) + 32 * b, (rd1 ^ bx) + 32 * b, xr, xi);
+    if (!PF) {
+      read_tile_tr<KS, 16 * kRS>(pre, (rd0 ^ bx) + 32 * b, (rd1 ^ bx) + 32 * b, xr, xi);
+    } else if (b + kWaves < 32) {
+      const int b2 = b + kWaves, bx2 = ((b2 >> 2) & 3) << 3;
+      read_tile_tr<KS, 16 * kRS>(pre, (rd0 ^ bx2) + 32 * b2, (rd1 ^ bx2) + 32 * b2, nr, ni);
+    }
     floatx16 dr, di;
     dft_xa<INV, KS>(xr, xi, w, dr, di);
     if (!INV) {
@@ -320,13 +331,17 @@ __device__ __forceinline__ void stage_a(uint16_t* pre, const Dft& w32, int wave,
       }
     }
     write_tile_x(pre, dr, di, wr + 32 * b, fx ^ (bx >> 3));
+    if (PF) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) xr[s] = nr[s], xi[s] = ni[s];
+    }
   }
 }
 
 // ---- stages over b (F2 / I2): tile = fixed a, rows b, bystander c -------------
 // With k1 = a % A: F2 (b -> k2): then twiddle W_N'^(c (k1 + A k2)).  I2 (k2 ->
 // n2): undoes F1's twiddle, conj W_(32 A)^(n2 k1), one factor per lane.
-template <int LOGA, bool INV>
+template <int LOGA, bool INV, bool PF>
 __device__ __forceinline__ void stage_b(uint16_t* pre, const Dft& w, int wave, int lane) {
   constexpr int A = Geo<LOGA>::A;
   lane = opaque(lane) & 63;
@@ -336,10 +351,18 @@ __device__ __forceinline__ void stage_b(uint16_t* pre, const Dft& w, int wave, i
   const int rd1 = 32 * (rsrc + 4) + (csrc ^ (((2 * g + 1) & 3) << 3));
   const int wr = 32 * f + 4 * g, fx = (f >> 2) & 3;
   const int wv = __builtin_amdgcn_readfirstlane(wave);
+  u32x4 xr[2], xi[2], nr[2], ni[2];
+  if (PF) read_tile_tr<2, 512>(pre, (rd0 ^ (((wv >> 2) & 3) << 3)) + wv * kRS,
+                               (rd1 ^ (((wv >> 2) & 3) << 3)) + wv * kRS, xr, xi);
+#pragma unroll(PF ? 4 : 1)
   for (int a = wv; a < 32; a += kWaves) {
     const int ax = ((a >> 2) & 3) << 3, k1 = a & (A - 1);
-    u32x4 xr[2], xi[2];
-    read_tile_tr<2, 512>(pre, (rd0 ^ ax) + a * kRS, (rd1 ^ ax) + a * kRS, xr, xi);
+    if (!PF) {
+      read_tile_tr<2, 512>(pre, (rd0 ^ ax) + a * kRS, (rd1 ^ ax) + a * kRS, xr, xi);
+    } else if (a + kWaves < 32) {
+      const int a2 = a + kWaves, ax2 = ((a2 >> 2) & 3) << 3;
+      read_tile_tr<2, 512>(pre, (rd0 ^ ax2) + a2 * kRS, (rd1 ^ ax2) + a2 * kRS, nr, ni);
+    }
     floatx16 dr, di;
     dft_xa<INV, 2>(xr, xi, w, dr, di);
     if (!INV) {
@@ -356,29 +379,43 @@ __device__ __forceinline__ void stage_b(uint16_t* pre, const Dft& w, int wave, i
       }
     }
     write_tile_x(pre, dr, di, wr + a * kRS, fx ^ (ax >> 3));
+    if (PF) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) xr[s] = nr[s], xi[s] = ni[s];
+    }
   }
 }
 
 // ---- stages over c (F3 / I1): tile = fixed a, lanes b, rows c (contiguous) ----
 // F3 (c -> k3): no twiddle.  I1 (k3 -> n3): then undoes F2's twiddle,
 // conj W_N'^(n3 (k1 + A b)).
-template <int LOGA, bool INV>
+template <int LOGA, bool INV, bool PF>
 __device__ __forceinline__ void stage_c(uint16_t* pre, const Dft& w, int wave, int lane) {
   constexpr int A = Geo<LOGA>::A;
   lane = opaque(lane) & 63;
   const int g = lane >> 5, b = lane & 31;
   const int bx = (b >> 2) & 3, row = 32 * b;
   const int wv = __builtin_amdgcn_readfirstlane(wave);
-  for (int a = wv; a < 32; a += kWaves) {
+  // pos(a, b, 16 s + 8 g) = row part + 8 ((2 s + g) ^ x), x = bx ^ bits 2-3 of a
+  auto read_tile = [&](int a, u32x4* r, u32x4* i) {
     const int x = bx ^ ((a >> 2) & 3);
-    // pos(a, b, 16 s + 8 g) = row part + 8 ((2 s + g) ^ x)
-    const int base = a * kRS + row;
-    u32x4 xr[2], xi[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const uint16_t* q = pre + base + (((2 * s + g) ^ x) << 3);
-      xr[s] = *reinterpret_cast<const u32x4*>(q);
-      xi[s] = *reinterpret_cast<const u32x4*>(q + kIm);
+      const uint16_t* q = pre + a * kRS + row + (((2 * s + g) ^ x) << 3);
+      r[s] = *reinterpret_cast<const u32x4*>(q);
+      i[s] = *reinterpret_cast<const u32x4*>(q + kIm);
+    }
+  };
+  u32x4 xr[2], xi[2], nr[2], ni[2];
+  if (PF) read_tile(wv, xr, xi);
+#pragma unroll(PF ? 4 : 1)
+  for (int a = wv; a < 32; a += kWaves) {
+    const int x = bx ^ ((a >> 2) & 3);
+    const int base = a * kRS + row;
+    if (!PF) {
+      read_tile(a, xr, xi);
+    } else if (a + kWaves < 32) {
+      read_tile(a + kWaves, nr, ni);
     }
     floatx16 dr, di;
     dft_xb<INV>(xr, xi, w, dr, di);
@@ -387,24 +424,32 @@ __device__ __forceinline__ void stage_c(uint16_t* pre, const Dft& w, int wave, i
       apply_tw<true>(dr, di, t);
     }
     write_tile_x(pre, dr, di, base + 4 * g, x);
+    if (PF) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) xr[s] = nr[s], xi[s] = ni[s];
+    }
   }
 }
 
-template <int LOGA, bool INV>
+// PF: every stage reads the operands of a wave's next tile before it twiddles
+// and writes back the current one: 16 more live registers, worth ~5 % where they
+// are free.  The kernels that hold a parked spectrum plus prefetched rows sit at
+// the 256-register limit already and leave it off.
+template <int LOGA, bool INV, bool PF = false>
 __device__ __forceinline__ void transform(uint16_t* pre, const Dft& w, int wave, int lane) {
   if (!INV) {
-    stage_a<LOGA, false>(pre, w, wave, lane);
+    stage_a<LOGA, false, PF>(pre, w, wave, lane);
     lds_barrier();
-    stage_b<LOGA, false>(pre, w, wave, lane);
+    stage_b<LOGA, false, PF>(pre, w, wave, lane);
     lds_barrier();
-    stage_c<LOGA, false>(pre, w, wave, lane);
+    stage_c<LOGA, false, PF>(pre, w, wave, lane);
     lds_barrier();
   } else {
-    stage_c<LOGA, true>(pre, w, wave, lane);
+    stage_c<LOGA, true, PF>(pre, w, wave, lane);
     lds_barrier();
-    stage_b<LOGA, true>(pre, w, wave, lane);
+    stage_b<LOGA, true, PF>(pre, w, wave, lane);
     lds_barrier();
-    stage_a<LOGA, true>(pre, w, wave, lane);
+    stage_a<LOGA, true, PF>(pre, w, wave, lane);
     lds_barrier();
   }
 }
@@ -1216,7 +1261,7 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_fwd_batch_kernel(
       RowRegs<MEGA_F32> rk;
       fetch_rows<LOGA>(rk, rows_of(it, k, 4, false), L, false, tid);
       place_rows<LOGA>(pre, red, rk, false, tid, sk);
-      transform<LOGA, false>(pre, w, wave, lane);
+      transform<LOGA, false, LOGA == 5>(pre, w, wave, lane);
       capture_spectrum<LOGA>(pre, spk, tid);
       if (spec_k != nullptr) {
         uint32_t* const save_k = spec_k + static_cast<size_t>(d0 / R) * kSpecWords;
@@ -1232,7 +1277,7 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_fwd_batch_kernel(
 #pragma unroll
     for (int i = 0; i < R; ++i) wres[i] = (omega != nullptr && d0 + i < D) ? omega[d0 + i] : 0.f;
     place_rows<LOGA>(pre, red, rx, false, tid, sx);
-    transform<LOGA, false>(pre, w, wave, lane);
+    transform<LOGA, false, LOGA == 5>(pre, w, wave, lane);
     uint32_t* save_x = nullptr;
     if (spec_x != nullptr) {
       save_x = spec_x + static_cast<size_t>((bb * D + d0) / R) * kSpecWords;
@@ -1243,7 +1288,7 @@ __global__ __launch_bounds__(kThreads) void fftconv_mfma_fwd_batch_kernel(
     pointwise<LOGA>(pre, spk, tid, save_x);
     lds_barrier();
     if (it + 1 < total) fetch_rows<LOGA>(rx, rows_of(it + 1, x, 2, true), L, false, tid);
-    transform<LOGA, true>(pre, w, wave, lane);
+    transform<LOGA, true, LOGA == 5>(pre, w, wave, lane);
     final_scales<LOGA>(sx, sk, scale);
     store_rows<LOGA, DT, false>(pre, rows_of(it, y, 2, true), L, false, scale,
                                 omega != nullptr ? &xrows : nullptr, wres, tid);
