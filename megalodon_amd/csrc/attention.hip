@@ -523,34 +523,6 @@ __global__ __launch_bounds__(kThreads) void softmax_fwd_kernel(uint16_t* w, int 
   }
 }
 
-template <int DT>
-__device__ __forceinline__ void unpack8(const uint4& q, float* v) {
-  const uint32_t u[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    if (DT == MEGA_BF16) {
-      v[2 * e] = __uint_as_float(u[e] << 16);
-      v[2 * e + 1] = __uint_as_float(u[e] & 0xffff0000u);
-    } else {
-      v[2 * e] = f16_bits_to_float(static_cast<uint16_t>(u[e] & 0xffffu));
-      v[2 * e + 1] = f16_bits_to_float(static_cast<uint16_t>(u[e] >> 16));
-    }
-  }
-}
-template <int DT>
-__device__ __forceinline__ uint4 pack8(const float* v) {
-  uint32_t u[4];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    if (DT == MEGA_BF16) {
-      u[e] = pack_bf16x2(v[2 * e], v[2 * e + 1]);
-    } else {
-      u[e] = static_cast<uint32_t>(float_to_f16_bits(v[2 * e])) |
-             (static_cast<uint32_t>(float_to_f16_bits(v[2 * e + 1])) << 16);
-    }
-  }
-  return make_uint4(u[0], u[1], u[2], u[3]);
-}
 
 // Same contract with the row held in registers: needs L2 % 8 == 0, a 16-byte
 // aligned base and L2 <= 64 * 8 * NCH; one read and one write of the row.

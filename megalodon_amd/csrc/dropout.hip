@@ -42,43 +42,19 @@ __global__ __launch_bounds__(kThreads) void dropout_vec_kernel(const typename El
     if (DT == MEGA_F32) {
       const float4* src = reinterpret_cast<const float4*>(in) + g * 2;
       float4* dst = reinterpret_cast<float4*>(out) + g * 2;
-      float4 a = src[0], b = src[1];
-      a.x *= sc[0]; a.y *= sc[1]; a.z *= sc[2]; a.w *= sc[3];
-      b.x *= sc[4]; b.y *= sc[5]; b.z *= sc[6]; b.w *= sc[7];
+      const float4 a = src[0], b = src[1];
+      float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
       // a dropped element is 0 whatever it held (0 * inf would be NaN)
-      if (sc[0] == 0.f) a.x = 0.f;
-      if (sc[1] == 0.f) a.y = 0.f;
-      if (sc[2] == 0.f) a.z = 0.f;
-      if (sc[3] == 0.f) a.w = 0.f;
-      if (sc[4] == 0.f) b.x = 0.f;
-      if (sc[5] == 0.f) b.y = 0.f;
-      if (sc[6] == 0.f) b.z = 0.f;
-      if (sc[7] == 0.f) b.w = 0.f;
-      dst[0] = a;
-      dst[1] = b;
-    } else {
-      const uint4 q = reinterpret_cast<const uint4*>(in)[g];
-      const uint32_t u[4] = {q.x, q.y, q.z, q.w};
-      uint32_t r[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float lo, hi;
-        if (DT == MEGA_BF16) {
-          lo = __uint_as_float(u[e] << 16);
-          hi = __uint_as_float(u[e] & 0xffff0000u);
-        } else {
-          lo = f16_bits_to_float(static_cast<uint16_t>(u[e] & 0xffffu));
-          hi = f16_bits_to_float(static_cast<uint16_t>(u[e] >> 16));
-        }
-        lo = sc[2 * e] == 0.f ? 0.f : lo * sc[2 * e];
-        hi = sc[2 * e + 1] == 0.f ? 0.f : hi * sc[2 * e + 1];
-        if (DT == MEGA_BF16)
-          r[e] = pack_bf16x2(lo, hi);
-        else
-          r[e] = static_cast<uint32_t>(float_to_f16_bits(lo)) |
-                 (static_cast<uint32_t>(float_to_f16_bits(hi)) << 16);
-      }
-      reinterpret_cast<uint4*>(out)[g] = make_uint4(r[0], r[1], r[2], r[3]);
+      for (int e = 0; e < 8; ++e) v[e] = sc[e] == 0.f ? 0.f : v[e] * sc[e];
+      dst[0] = make_float4(v[0], v[1], v[2], v[3]);
+      dst[1] = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+      float v[8];
+      unpack8<DT>(reinterpret_cast<const uint4*>(in)[g], v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = sc[e] == 0.f ? 0.f : v[e] * sc[e];
+      reinterpret_cast<uint4*>(out)[g] = pack8<DT>(v);
     }
   }
 }

@@ -17,33 +17,6 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 constexpr int kMaxGroups = 1024;  // workgroups of the backward = partial-sum rows
 
-template <int DT>
-__device__ __forceinline__ void unpack8(const uint4& q, float* v) {
-  const uint32_t u[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    if (DT == MEGA_BF16) {
-      v[2 * e] = __uint_as_float(u[e] << 16);
-      v[2 * e + 1] = __uint_as_float(u[e] & 0xffff0000u);
-    } else {
-      v[2 * e] = f16_bits_to_float(static_cast<uint16_t>(u[e] & 0xffffu));
-      v[2 * e + 1] = f16_bits_to_float(static_cast<uint16_t>(u[e] >> 16));
-    }
-  }
-}
-template <int DT>
-__device__ __forceinline__ uint4 pack8(const float* v) {
-  uint32_t u[4];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    if (DT == MEGA_BF16)
-      u[e] = pack_bf16x2(v[2 * e], v[2 * e + 1]);
-    else
-      u[e] = static_cast<uint32_t>(float_to_f16_bits(v[2 * e])) |
-             (static_cast<uint32_t>(float_to_f16_bits(v[2 * e + 1])) << 16);
-  }
-  return make_uint4(u[0], u[1], u[2], u[3]);
-}
 
 // hides a register from common-subexpression elimination: values derived from it
 // afterwards are recomputed instead of being kept alive across the row reduction
@@ -541,16 +514,19 @@ int launch_qk(const QkParams& p, int groups, hipStream_t s) {
   return MEGA_OK;
 }
 
+// How a row is split over a wavefront: `lpr` lanes per row, `nch` 16-byte chunks
+// per lane (D = lpr * 8 * nch); lpr == 0: no register-resident variant.
 struct Shape {
-  int lpr, nch;  // 0: no register-resident variant
+  int lpr, nch;
 };
 Shape vec_shape(int dtype, int64_t D, const NormParams& p) {
   if (dtype == MEGA_F32) return {0, 0};
   for (const void* q : {p.x, p.dy, p.weight, p.bias, static_cast<const void*>(p.y)})
     if (reinterpret_cast<uintptr_t>(q) % 16 != 0) return {0, 0};
-  for (int lpr : {64, 32, 16})
-    for (int nch : {1, 2, 4, 8})
-      if (D == static_cast<int64_t>(lpr) * 8 * nch) return {lpr, nch};
+  for (int nch : {1, 2, 4, 8})
+    if (D == 512 * nch) return {64, nch};  // one row per wavefront
+  if (D == 256) return {32, 1};            // two rows per wavefront
+  if (D == 128) return {16, 1};            // four
   return {0, 0};
 }
 
@@ -576,19 +552,9 @@ int launch_vec(const NormParams& p, Shape sh, int groups, hipStream_t s) {
   return MEGA_OK;
 }
 
-// D = lpr * 8 * nch has several factorisations; keep the widest row split that exists
-Shape canonical(Shape sh) {
-  if (sh.lpr == 0) return sh;
-  const int d = sh.lpr * 8 * sh.nch;
-  if (d % 512 == 0 && d / 512 <= 8 && ((d / 512) & (d / 512 - 1)) == 0) return {64, d / 512};
-  if (d == 256) return {32, 1};
-  if (d == 128) return {16, 1};
-  return {0, 0};
-}
-
 template <int DT, bool RMS>
 int run_fwd(const NormParams& p, int dtype, hipStream_t s) {
-  const Shape sh = canonical(vec_shape(dtype, p.D, p));
+  const Shape sh = vec_shape(dtype, p.D, p);
   if constexpr (DT != MEGA_F32) {
     if (sh.lpr) {
       const int rpg = kWaves * (kWave / sh.lpr);
@@ -642,7 +608,7 @@ template <int DT, bool RMS>
 static int run_bwd(NormParams p, int dtype, void* dweight, void* dbias, float* ws, hipStream_t s) {
   using T = typename Elem<DT>::type;
   const bool affine = dweight != nullptr;
-  const Shape sh = canonical(vec_shape(dtype, p.D, p));
+  const Shape sh = vec_shape(dtype, p.D, p);
   const int rpg = sh.lpr ? kWaves * (kWave / sh.lpr) : kWaves;
   const int groups = groups_for(p.rows, rpg);
   p.part_w = affine ? ws : nullptr;
