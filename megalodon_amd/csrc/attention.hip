@@ -45,7 +45,7 @@ static_assert((kSlab / 8) * kChunkPitch * 8 <= kOperandElems, "chunk layout must
 constexpr int kThreads = 256;
 constexpr int kXcds = 8;       // accelerator dies, each with a private L2
 constexpr int kRing = 3;       // slabs in flight in registers (prefetch distance)
-constexpr int kEpiPitch = 128 + 8;  // epilogue staging pitch (elements) of a wave's 128x128 tile
+constexpr int kEpiPitch = 128 + 8;  // epilogue staging pitch (elements) of a wave's 128x128 tile (4-wave form)
 constexpr size_t kGemmLds =
     sizeof(uint16_t) * (4 * 128 * kEpiPitch > 2 * 2 * kOperandElems ? 4 * 128 * kEpiPitch
                                                                      : 2 * 2 * kOperandElems);
@@ -328,7 +328,7 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
   // LDS write or global load, then one LDS read.  An MFMA occupies the matrix
   // pipe for 8 passes while the wave may issue other instructions, and a wave
   // issues in order -- memory instructions bunched in front of the MFMAs leave
-  // the matrix pipe idle while they issue (one wave per SIMD: nobody else
+  // the matrix pipe idle while they issue (one or two waves per SIMD: hardly anybody else
   // feeds it).
 #define MEGA_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
   // What the barrier waits for goes first: the fragment reads of this slab
@@ -404,7 +404,7 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
 #undef MEGA_GEMM_STEP
 #undef MEGA_SGB
 
-  // epilogue: stage the wave's 128x128 tile in LDS ([row][col], element type),
+  // epilogue: stage the wave's 128 x 32 JN tile in LDS ([row][col], element type),
   // then write it with 16-byte row segments.  The products are issued as
   // B-fragment x A-fragment, so a 32x32 MFMA tile holds C transposed: lane l has
   // row m = l % 32 and register r the column n = 8 (r / 4) + 4 (l / 32) + r % 4,
