@@ -121,3 +121,30 @@ def test_linear_with_transposed_weight_backward_matches_float64(shape, out, bias
     ref.load_state_dict(lin.state_dict())
     with torch.no_grad():
         assert torch.equal(lin(x), ref(x))
+
+
+def test_random_shapes_sweep():
+    """Forty seeded random shapes per kernel: transpose against PyTorch's own
+    (bit-exact), the SiLU gate and the norms against float64 (2e-2, bfloat16)."""
+    import random
+    from megalodon_amd.fused_ops import layer_norm_plus_one
+    rnd = random.Random(20240)
+    for _ in range(40):
+        Z, R, C = rnd.randint(1, 3), rnd.choice([8, 40, 129, 256, 264, 1000]), rnd.choice([8, 24, 130, 256, 520])
+        x = torch.randn(Z, R, C, device="cuda").bfloat16()
+        assert torch.equal(ops.transpose_last2(x), x.transpose(1, 2).contiguous()), (Z, R, C)
+        n = rnd.randint(1, 5000)
+        a, b = torch.randn(n, device="cuda").bfloat16(), torch.randn(n, device="cuda").bfloat16()
+        assert rel_err(ops.silu_mul_fwd(a, b), F.silu(a.double()) * b.double()) <= 2e-2, n
+        rows, D = rnd.randint(1, 70), rnd.choice([128, 256, 512, 1024, 2048, 4096, 96, 300, 1000])
+        rms = rnd.random() < 0.5
+        xx = (torch.randn(rows, D, device="cuda") + 0.3).bfloat16()
+        w = (torch.randn(D, device="cuda") * 0.2).bfloat16()
+        bb = None if rms else (torch.randn(D, device="cuda") * 0.2).bfloat16()
+        y = layer_norm_plus_one(xx, w, bb, 1e-5, rms)
+        x64 = xx.double()
+        if rms:
+            want = x64 * torch.rsqrt(x64.pow(2).mean(-1, keepdim=True) + 1e-5) * (w.double() + 1)
+        else:
+            want = F.layer_norm(x64, (D,), w.double() + 1, bb.double(), 1e-5)
+        assert rel_err(y, want) <= 2e-2, (rows, D, rms)
