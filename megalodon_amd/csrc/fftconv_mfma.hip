@@ -50,6 +50,7 @@ struct Geo {
 // every access folds into the instruction's immediate offset.
 constexpr int kIm = 1024 + 16;        // elements from a re value to its im value
 constexpr int kRS = 2 * kIm;          // elements between consecutive a
+static_assert(kRS % 32 == 0, "the stages XOR swizzle bits 3-4 into offsets that include a * kRS");
 constexpr int kPlane = 16 * kRS;      // half of the LDS elements (two "planes" of 32 half rows)
 constexpr int kThreads = 512;         // 8 waves, two per SIMD
 constexpr int kWaves = kThreads / kWave;
