@@ -225,13 +225,6 @@ __device__ __forceinline__ void apply_tw(floatx16& dr, floatx16& di, const Tw16&
   }
 }
 
-// Per-lane pieces of the LDS offsets (elements), computed once per stage call.
-// A tile adds its own digit (wave-uniform, scalar) and XORs its swizzle bits.
-struct LaneGeo {
-  int g, f;         // lane / 32, lane % 32
-  int rd[2];        // transposing read, h = 0, 1: row part + swizzled source column
-  int wr;           // tile write: lane part
-};
 // quad slot q of a tile write lands at 8 (q ^ x): x = swizzle bits of (tile digit, lane digit)
 __device__ __forceinline__ void write_tile_x(uint16_t* pre, const floatx16& dr, const floatx16& di,
                                              int base, int x) {
@@ -709,11 +702,6 @@ __device__ __forceinline__ RowPair row_pair(int task) {
   rp.k0 = k1 + A * k2 + 128 * A * u;
   rp.writes = q != 16 * A - 1 || u < 4;
   return rp;
-}
-__device__ __forceinline__ void read_quad(const uint16_t* p, float* v) {
-  const uint2 u = *reinterpret_cast<const uint2*>(p);
-  unpack_h2(u.x, v[0], v[1]);
-  unpack_h2(u.y, v[2], v[3]);
 }
 __device__ __forceinline__ void write_quad(uint16_t* p, const float* v) {
   *reinterpret_cast<uint2*>(p) = make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
