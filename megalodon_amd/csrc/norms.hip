@@ -672,7 +672,7 @@ static int check_qk(const char* who, int dtype, int64_t rows, int64_t L, int64_t
                     const void* freqs) {
   if (dtype != MEGA_BF16 && dtype != MEGA_F16)
     return set_error(MEGA_ERR_UNSUPPORTED, "%s: only bfloat16 / float16 tensors are supported", who);
-  MEGA_CHECK_ARG(rows >= 0 && L >= 1 && S >= 1 && Dh >= 1, "%s: bad sizes", who);
+  MEGA_CHECK_ARG(rows >= 0 && (rows == 0 || L >= 1) && S >= 1 && Dh >= 1, "%s: bad sizes", who);
   MEGA_CHECK_ARG(!freqs || P >= 1, "%s: rotary factors without positions", who);
   if (!(Dh == 64 || Dh == 128 || Dh == 256 || Dh == 512) || S % Dh != 0 ||
       !(S == 512 || S == 1024 || S == 2048 || S == 4096))

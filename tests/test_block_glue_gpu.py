@@ -148,3 +148,16 @@ def test_random_shapes_sweep():
         else:
             want = F.layer_norm(x64, (D,), w.double() + 1, bb.double(), 1e-5)
         assert rel_err(y, want) <= 2e-2, (rows, D, rms)
+
+
+def test_empty_inputs_are_accepted():
+    from megalodon_amd.fused_ops import qk_norm_rotary
+    e = torch.empty(0, device="cuda", dtype=torch.bfloat16)
+    assert ops.silu_mul_fwd(e, e).numel() == 0
+    da, db = ops.silu_mul_bwd(e, e, e)
+    assert da.numel() == 0 and db.numel() == 0
+    assert ops.dropout(e, 0.5, 1, 0).numel() == 0
+    z = torch.empty(2, 0, 512, device="cuda", dtype=torch.bfloat16)
+    g = torch.zeros(2, 512, device="cuda", dtype=torch.bfloat16)
+    q, k = qk_norm_rotary(z, g, g, None, 64, 1e-5)
+    assert q.shape == (2, 0, 512) and k.shape == (2, 0, 512)
