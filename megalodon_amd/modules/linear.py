@@ -19,12 +19,21 @@ from .. import extension as megalodon_ops
 
 
 class LinearFunc(torch.autograd.Function):
+    """y = x W^T (+ bias) (+ residual).  A residual goes into the GEMM as its
+    accumulator input (`addmm`, one pass fewer over the activation than a
+    separate add); it needs a layer without bias."""
 
     @staticmethod
-    def forward(ctx: FunctionCtx, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    def forward(ctx: FunctionCtx, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                residual: Optional[torch.Tensor]) -> torch.Tensor:
         ctx.save_for_backward(x, weight)
         ctx.has_bias = bias is not None
-        return F.linear(x, weight, bias)
+        ctx.has_residual = residual is not None
+        if residual is None:
+            return F.linear(x, weight, bias)
+        out_shape = x.shape[:-1] + (weight.shape[0],)
+        y = torch.addmm(residual.reshape(-1, weight.shape[0]), x.reshape(-1, x.shape[-1]), weight.t())
+        return y.view(out_shape)
 
     @staticmethod
     def backward(ctx: FunctionCtx, y_grad: torch.Tensor) -> Tuple[Optional[torch.Tensor], ...]:
@@ -38,14 +47,21 @@ class LinearFunc(torch.autograd.Function):
             dw = g2.t() @ x.reshape(-1, x.shape[-1])
         if ctx.has_bias and ctx.needs_input_grad[2]:
             db = g2.sum(0)
-        return dx, dw, db
+        return dx, dw, db, (y_grad if ctx.has_residual and ctx.needs_input_grad[3] else None)
 
 
 class Linear(nn.Linear):
-    """Drop-in for `nn.Linear` (same parameters, same values)."""
+    """Drop-in for `nn.Linear` (same parameters, same values); `residual`, for
+    layers without bias, is added inside the GEMM."""
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and self.weight.dtype == x.dtype
-                and torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad)):
-            return LinearFunc.apply(x, self.weight, self.bias)
+    def forward(self, x: torch.Tensor, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        fused = (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and self.weight.dtype == x.dtype)
+        if residual is not None and (self.bias is not None or not fused or residual.dtype != x.dtype):
+            return F.linear(x, self.weight, self.bias) + residual
+        if fused and torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad
+                                                  or (residual is not None and residual.requires_grad)):
+            return LinearFunc.apply(x, self.weight, self.bias, residual)
+        if residual is not None:
+            return torch.addmm(residual.reshape(-1, self.weight.shape[0]), x.reshape(-1, x.shape[-1]),
+                               self.weight.t()).view(x.shape[:-1] + (self.weight.shape[0],))
         return F.linear(x, self.weight, self.bias)

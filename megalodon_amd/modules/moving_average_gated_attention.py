@@ -115,7 +115,7 @@ class MovingAverageGatedAttention(nn.Module):
         attn = memory_efficient_dropout(silu_mul(r, attn), self.hidden_dropout, self.training)
 
         # B x L x E -> B x L x D
-        h = self.wh1(mx) + self.wh2(attn)
+        h = self.wh2(attn, residual=self.wh1(mx))   # wh1(mx) + wh2(attn), the sum formed inside the GEMM
         h = memory_efficient_dropout(h, self.dropout, self.training)
         out = h + residual
         if cache is not None:

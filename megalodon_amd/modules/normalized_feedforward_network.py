@@ -44,6 +44,8 @@ class NormalizedFeedForwardNetwork(nn.Module):
         else:
             hidden = F.silu(self.fc1(x))
         hidden = memory_efficient_dropout(hidden, self.hidden_dropout, self.training)
+        if self.alpha is None and (self.dropout == 0.0 or not self.training):
+            return self.fc2(hidden, residual=residual)   # fc2(hidden) + residual, the sum formed inside the GEMM
         x = self.fc2(hidden)
         x = memory_efficient_dropout(x, self.dropout, self.training)
         return self.rescale(x) + residual

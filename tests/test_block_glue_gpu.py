@@ -161,3 +161,25 @@ def test_empty_inputs_are_accepted():
     g = torch.zeros(2, 512, device="cuda", dtype=torch.bfloat16)
     q, k = qk_norm_rotary(z, g, g, None, 64, 1e-5)
     assert q.shape == (2, 0, 512) and k.shape == (2, 0, 512)
+
+
+def test_linear_with_residual_inside_the_gemm():
+    from megalodon_amd.modules.linear import Linear
+    torch.manual_seed(4)
+    lin = Linear(256, 384, bias=False).cuda().bfloat16()
+    x = torch.randn(3, 70, 256, device="cuda").bfloat16().requires_grad_(True)
+    r = torch.randn(3, 70, 384, device="cuda").bfloat16().requires_grad_(True)
+    dy = torch.randn(3, 70, 384, device="cuda").bfloat16()
+    y = lin(x, residual=r)
+    y.backward(dy)
+    x64, r64 = x.detach().double().requires_grad_(True), r.detach().double().requires_grad_(True)
+    w64 = lin.weight.detach().double().requires_grad_(True)
+    want = F.linear(x64, w64) + r64
+    want.backward(dy.double())
+    assert rel_err(y, want) <= 2e-2 and rel_err(x.grad, x64.grad) <= 2e-2
+    assert rel_err(lin.weight.grad, w64.grad) <= 2e-2 and torch.equal(r.grad, dy)
+    with torch.no_grad():
+        assert rel_err(lin(x, residual=r), want) <= 2e-2
+    # a layer with bias keeps the separate add
+    lb = Linear(256, 384, bias=True).cuda().bfloat16()
+    assert rel_err(lb(x, residual=r), F.linear(x64, lb.weight.double(), lb.bias.double()) + r64) <= 2e-2
