@@ -400,6 +400,21 @@ int mega_qk_norm_rotary_bwd(const void* dq, const void* dk, const void* z, const
                             int64_t L, int64_t P, int64_t S, int64_t Dh, void* dz, void* dgamma,
                             void* dbeta, void* workspace, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Real FFT of zero-padded rows.
+ *
+ * Replaces rfft(x, flip) -> y (megalodon/csrc/ops/fftconv.cc:6-8,22,
+ *   fftconv_kernel.cu:23-32,170-215; called for a 16-bit convolution kernel in
+ *   fused_ops/fftconv.py:88-91).
+ *   x (rows, L) of `dtype`, L <= 16384; y (rows, M + 1) complex64 as float32
+ *   pairs, M = max(2^ceil(log2 L), 32) = mega_rfft_bins(L) - 1:
+ *   y = rfft(x, n = 2 M), with x reversed in time first when `flip` is set.
+ *   The convolution entry points above take k in the time domain and do not
+ *   need this operator.
+ * ---------------------------------------------------------------------- */
+int64_t mega_rfft_bins(int64_t L);
+int mega_rfft(const void* x, int dtype, int64_t rows, int64_t L, int flip, void* y, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -814,6 +814,24 @@ def qk_norm_rotary_bwd(q_grad: torch.Tensor, k_grad: torch.Tensor, z: torch.Tens
     return dz, dgamma, dbeta
 
 
+def rfft(x: torch.Tensor, flip: bool = False) -> torch.Tensor:
+    """`torch.fft.rfft(x, n=2 M)` over the last axis, M = max(2^ceil(log2 L), 32),
+    on the (optionally time-reversed) rows; complex64 (..., M + 1)
+    (megalodon/csrc/ops/fftconv.cc:6-8, fftconv_kernel.cu:170-215)."""
+    dev = _require_cuda(x)
+    L = x.shape[-1]
+    xc = x.contiguous()
+    rows = xc.numel() // max(1, L)
+    fn = _lib.load().mega_rfft_bins
+    fn.restype = _lib.ctypes.c_int64
+    bins = int(fn(_lib.i64(L)))
+    y = torch.empty(x.shape[:-1] + (bins,), dtype=torch.complex64, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_rfft", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(rows), _lib.i64(L),
+                  _lib.i32(1 if flip else 0), _lib.ptr(y), _lib.stream_ptr(dev))
+    return y
+
+
 def timestep_norm_fwd(x: torch.Tensor, prev_count: torch.Tensor, prev_mean: torch.Tensor, prev_var: torch.Tensor,
                       gamma: torch.Tensor, beta: torch.Tensor, padding_mask: Optional[torch.Tensor], eps: float):
     """The non-group operator (megalodon/csrc/ops/timestep_norm.cc:23-105,
