@@ -415,6 +415,38 @@ int mega_qk_norm_rotary_bwd(const void* dq, const void* dk, const void* z, const
 int64_t mega_rfft_bins(int64_t L);
 int mega_rfft(const void* x, int dtype, int64_t rows, int64_t L, int flip, void* y, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Whole-sequence (non-causal) group normalisation.
+ *
+ * Replaces group_sequence_norm_fwd(X, gamma, beta, padding_mask, num_groups,
+ *   eps, length_last) -> (Y, count, mean, rstd) and group_sequence_norm_bwd(
+ *   Y_grad, X, count, mean, rstd, gamma, padding_mask, num_groups,
+ *   length_last) -> (X_grad, gamma_grad, beta_grad)
+ *   (megalodon/csrc/ops/sequence_norm.cc:531-842,953-1063, binding :1068-1071),
+ *   and with num_groups = H the per-feature pair sequence_norm_fwd/bwd
+ *   (:258-529,844-951, binding :1066-1067).
+ *   x, y, dy, dx: (B, L, H) when length_last = 0, (B, H, L) when 1, of
+ *   `dtype`; gamma, beta, dgamma, dbeta (H) of `dtype`; padding_mask (B, L)
+ *   bytes, nonzero = step left out (may be null); count (B) int64 = unmasked
+ *   steps; mean, rstd (B, num_groups) float32 over the unmasked steps and the
+ *   H / num_groups features of a group (biased variance);
+ *   y = (x - mean) rstd gamma + beta, 0 at masked steps.
+ *   workspace: mega_group_sequence_norm_workspace_bytes(...) bytes, contents
+ *   not kept between calls.
+ * ---------------------------------------------------------------------- */
+int64_t mega_group_sequence_norm_workspace_bytes(int64_t B, int64_t L, int64_t H, int64_t num_groups,
+                                                 int length_last);
+int mega_group_sequence_norm_fwd(const void* x, const void* gamma, const void* beta,
+                                 const uint8_t* padding_mask, int dtype, int64_t B, int64_t L,
+                                 int64_t H, int64_t num_groups, double eps, int length_last, void* y,
+                                 int64_t* count, float* mean, float* rstd, void* workspace,
+                                 void* stream);
+int mega_group_sequence_norm_bwd(const void* dy, const void* x, const int64_t* count,
+                                 const float* mean, const float* rstd, const void* gamma,
+                                 const uint8_t* padding_mask, int dtype, int64_t B, int64_t L,
+                                 int64_t H, int64_t num_groups, int length_last, void* dx,
+                                 void* dgamma, void* dbeta, void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -855,3 +855,93 @@ def timestep_norm_bwd(y_grad: torch.Tensor, mean_grad: torch.Tensor, var_grad: t
     H = x.shape[-1]
     return group_timestep_norm_bwd(y_grad, mean_grad, var_grad, x, prev_mean, count, cummean.float(),
                                    cumrstd.float(), gamma, padding_mask, H)
+
+
+def _sequence_norm_geometry(x: torch.Tensor, gamma: torch.Tensor, padding_mask, num_groups: int, length_last: bool):
+    if x.dim() != 3:
+        raise RuntimeError("sequence_norm: x must be (B, L, H) or, with length_last, (B, H, L)")
+    B = x.shape[0]
+    L, H = (x.shape[2], x.shape[1]) if length_last else (x.shape[1], x.shape[2])
+    if gamma.shape != (H,) or gamma.dtype != x.dtype:
+        raise RuntimeError(f"sequence_norm: gamma and beta must be ({H},) of x's dtype")
+    if num_groups < 1 or H % num_groups != 0:
+        raise RuntimeError(f"sequence_norm: num_groups {num_groups} does not divide H={H}")
+    if padding_mask is not None and padding_mask.shape != (B, L):
+        raise RuntimeError(f"sequence_norm: padding_mask must be ({B}, {L})")
+    return B, L, H
+
+
+def _sequence_norm_workspace(dev, B, L, H, num_groups, length_last):
+    fn = _lib.load().mega_group_sequence_norm_workspace_bytes
+    fn.restype = _lib.ctypes.c_int64
+    size = int(fn(_lib.i64(B), _lib.i64(L), _lib.i64(H), _lib.i64(num_groups), _lib.i32(1 if length_last else 0)))
+    return torch.empty(max(size, 256), dtype=torch.uint8, device=dev)
+
+
+def group_sequence_norm_fwd(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor,
+                            padding_mask: Optional[torch.Tensor], num_groups: int, eps: float,
+                            length_last: bool = False):
+    """(y, count, mean, rstd): normalisation of every (sequence, feature group)
+    over its unmasked steps and the group's features
+    (megalodon/csrc/ops/sequence_norm.cc:953-1010, binding :1068-1069)."""
+    dev = _require_cuda(x, gamma, beta, padding_mask)
+    B, L, H = _sequence_norm_geometry(x, gamma, padding_mask, num_groups, length_last)
+    if beta.shape != gamma.shape or beta.dtype != x.dtype:
+        raise RuntimeError(f"sequence_norm: gamma and beta must be ({H},) of x's dtype")
+    xc = x.contiguous()
+    y = torch.empty_like(xc)
+    count = torch.empty(B, dtype=torch.int64, device=dev)
+    mean = torch.empty(B, num_groups, dtype=torch.float32, device=dev)
+    rstd = torch.empty(B, num_groups, dtype=torch.float32, device=dev)
+    mask = _mask_bytes(padding_mask)
+    ws = _sequence_norm_workspace(dev, B, L, H, num_groups, length_last)
+    with torch.cuda.device(dev):
+        _lib.call("mega_group_sequence_norm_fwd", _lib.ptr(xc), _lib.ptr(gamma.contiguous()),
+                  _lib.ptr(beta.contiguous()), _lib.ptr(mask), _lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(B),
+                  _lib.i64(L), _lib.i64(H), _lib.i64(num_groups), _lib.f64(eps), _lib.i32(1 if length_last else 0),
+                  _lib.ptr(y), _lib.ptr(count), _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(ws), _lib.stream_ptr(dev))
+    return y, count, mean, rstd
+
+
+def group_sequence_norm_bwd(y_grad: torch.Tensor, x: torch.Tensor, count: torch.Tensor, mean: torch.Tensor,
+                            rstd: torch.Tensor, gamma: torch.Tensor, padding_mask: Optional[torch.Tensor],
+                            num_groups: int, length_last: bool = False):
+    """(x_grad, gamma_grad, beta_grad)
+    (megalodon/csrc/ops/sequence_norm.cc:1012-1063, binding :1070-1071)."""
+    dev = _require_cuda(y_grad, x, count, mean, rstd, gamma, padding_mask)
+    B, L, H = _sequence_norm_geometry(x, gamma, padding_mask, num_groups, length_last)
+    if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
+        raise RuntimeError("sequence_norm_bwd: y_grad and x must have the same shape and dtype")
+    if (count.shape != (B,) or count.dtype != torch.int64 or mean.shape != (B, num_groups)
+            or rstd.shape != (B, num_groups) or mean.dtype != torch.float32 or rstd.dtype != torch.float32):
+        raise RuntimeError("sequence_norm_bwd: count must be int64 (B,), mean and rstd float32 (B, num_groups)")
+    xc, gc = x.contiguous(), y_grad.contiguous()
+    dx = torch.empty_like(xc)
+    dgamma = torch.empty_like(gamma, memory_format=torch.contiguous_format)
+    dbeta = torch.empty_like(dgamma)
+    mask = _mask_bytes(padding_mask)
+    ws = _sequence_norm_workspace(dev, B, L, H, num_groups, length_last)
+    with torch.cuda.device(dev):
+        _lib.call("mega_group_sequence_norm_bwd", _lib.ptr(gc), _lib.ptr(xc), _lib.ptr(count.contiguous()),
+                  _lib.ptr(mean.contiguous()), _lib.ptr(rstd.contiguous()), _lib.ptr(gamma.contiguous()),
+                  _lib.ptr(mask), _lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(B), _lib.i64(L), _lib.i64(H),
+                  _lib.i64(num_groups), _lib.i32(1 if length_last else 0), _lib.ptr(dx), _lib.ptr(dgamma),
+                  _lib.ptr(dbeta), _lib.ptr(ws), _lib.stream_ptr(dev))
+    return dx, dgamma, dbeta
+
+
+def sequence_norm_fwd(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor,
+                      padding_mask: Optional[torch.Tensor], eps: float, length_last: bool = False):
+    """The per-feature operator: one group per feature, statistics (B, H)
+    (megalodon/csrc/ops/sequence_norm.cc:844-900, binding :1066)."""
+    H = x.shape[1] if length_last else x.shape[-1]
+    return group_sequence_norm_fwd(x, gamma, beta, padding_mask, H, eps, length_last)
+
+
+def sequence_norm_bwd(y_grad: torch.Tensor, x: torch.Tensor, count: torch.Tensor, mean: torch.Tensor,
+                      rstd: torch.Tensor, gamma: torch.Tensor, padding_mask: Optional[torch.Tensor],
+                      length_last: bool = False):
+    """(x_grad, gamma_grad, beta_grad) of the per-feature operator
+    (megalodon/csrc/ops/sequence_norm.cc:902-951, binding :1067)."""
+    H = x.shape[1] if length_last else x.shape[-1]
+    return group_sequence_norm_bwd(y_grad, x, count, mean, rstd, gamma, padding_mask, H, length_last)

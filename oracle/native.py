@@ -169,3 +169,35 @@ def ema_hidden_bwd(lib, dy, x, p, log_q, h):
                            _p(_c64_as_f32(log_q.reshape(D, N))), _p(None if h is None else _c64_as_f32(h)),
                            _i(B), _i(D), _i(N), _i(L), _p(dx), _p(dp), _p(dq), _p(dh))
     return dx, dp, torch.view_as_complex(dq), (None if h is None else torch.view_as_complex(dh))
+
+
+# ---- whole-sequence group normalisation (reference build only) --------------------
+def group_sequence_norm_fwd(lib, x, gamma, beta, mask, G, eps, length_last=False):
+    B = x.shape[0]
+    L, H = (x.shape[2], x.shape[1]) if length_last else (x.shape[1], x.shape[2])
+    xf = x.float().contiguous()
+    gm, bt = gamma.float().contiguous(), beta.float().contiguous()
+    mk = None if mask is None else mask.to(torch.uint8).contiguous()
+    y = torch.empty_like(xf)
+    count = torch.empty(B, dtype=torch.int64)
+    mean = torch.empty(B, G)
+    rstd = torch.empty(B, G)
+    lib.ref_group_sequence_norm_fwd(_p(xf), _p(gm), _p(bt), _p(mk), _i(B), _i(L), _i(H), _i(G), ctypes.c_double(eps),
+                                    ctypes.c_int(1 if length_last else 0), _p(y), _p(count), _p(mean), _p(rstd))
+    return y, count, mean, rstd
+
+
+def group_sequence_norm_bwd(lib, dy, x, count, mean, rstd, gamma, mask, G, length_last=False):
+    B = x.shape[0]
+    L, H = (x.shape[2], x.shape[1]) if length_last else (x.shape[1], x.shape[2])
+    dyf, xf = dy.float().contiguous(), x.float().contiguous()
+    cnt = count.to(torch.int64).contiguous()
+    mn, rs = mean.float().contiguous(), rstd.float().contiguous()
+    gm = gamma.float().contiguous()
+    mk = None if mask is None else mask.to(torch.uint8).contiguous()
+    dx = torch.empty_like(xf)
+    dg = torch.empty(H)
+    db = torch.empty(H)
+    lib.ref_group_sequence_norm_bwd(_p(dyf), _p(xf), _p(cnt), _p(mn), _p(rs), _p(gm), _p(mk), _i(B), _i(L), _i(H),
+                                    _i(G), ctypes.c_int(1 if length_last else 0), _p(dx), _p(dg), _p(db))
+    return dx, dg, db

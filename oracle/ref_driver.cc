@@ -3,11 +3,13 @@
 // TEST INFRASTRUCTURE ONLY: used to validate the oracle restatements and,
 // optionally, as the timed CPU baseline.  Only the reference's *CPU* entry
 // points are called (EMAParametersCPUFwd/Bwd, EMAHiddenCPUFwd/Bwd, GroupTimestepNormCPUFwd/Bwd,
-// declared in megalodon/csrc/ops/ema_parameters.h:19-49 and timestep_norm.h).
+// GroupSequenceNormCPUFwd/Bwd, declared in megalodon/csrc/ops/ema_parameters.h:19-49,
+// timestep_norm.h and sequence_norm.h:57-83).
 #include <torch/torch.h>
 
 #include "ops/ema_hidden.h"
 #include "ops/ema_parameters.h"
+#include "ops/sequence_norm.h"
 #include "ops/timestep_norm.h"
 
 namespace mo = megalodon::ops;
@@ -130,5 +132,38 @@ extern "C" __attribute__((visibility("default"))) int ref_ema_hidden_bwd(
   std::memcpy(dp, std::get<1>(out).data_ptr<float>(), sizeof(float) * D * N);
   std::memcpy(dq, std::get<2>(out).data_ptr(), sizeof(float) * 2 * D * N);
   if (h) std::memcpy(dh, std::get<3>(out)->data_ptr(), sizeof(float) * 2 * B * D * N);
+  return 0;
+}
+
+// ---- whole-sequence group normalisation (float32) ---------------------------------
+// x, y, dy, dx: (B, L, H), or (B, H, L) when length_last; mean, rstd (B, G).
+extern "C" __attribute__((visibility("default"))) int ref_group_sequence_norm_fwd(
+    const float* x, const float* gamma, const float* beta, const uint8_t* mask, int64_t B, int64_t L, int64_t H,
+    int64_t G, double eps, int length_last, float* y, int64_t* count, float* mean, float* rstd) {
+  c10::optional<torch::Tensor> m = c10::nullopt;
+  if (mask) m = torch::from_blob(const_cast<uint8_t*>(mask), {B, L}, torch::kBool);
+  const std::vector<int64_t> shape = length_last ? std::vector<int64_t>{B, H, L} : std::vector<int64_t>{B, L, H};
+  auto out = mo::GroupSequenceNormCPUFwd(f32(x, shape), f32(gamma, {H}), f32(beta, {H}), m, G, eps,
+                                         length_last != 0);
+  std::memcpy(y, std::get<0>(out).data_ptr<float>(), sizeof(float) * B * L * H);
+  std::memcpy(count, std::get<1>(out).data_ptr<int64_t>(), sizeof(int64_t) * B);
+  std::memcpy(mean, std::get<2>(out).data_ptr<float>(), sizeof(float) * B * G);
+  std::memcpy(rstd, std::get<3>(out).data_ptr<float>(), sizeof(float) * B * G);
+  return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int ref_group_sequence_norm_bwd(
+    const float* dy, const float* x, const int64_t* count, const float* mean, const float* rstd, const float* gamma,
+    const uint8_t* mask, int64_t B, int64_t L, int64_t H, int64_t G, int length_last, float* dx, float* dgamma,
+    float* dbeta) {
+  c10::optional<torch::Tensor> m = c10::nullopt;
+  if (mask) m = torch::from_blob(const_cast<uint8_t*>(mask), {B, L}, torch::kBool);
+  const std::vector<int64_t> shape = length_last ? std::vector<int64_t>{B, H, L} : std::vector<int64_t>{B, L, H};
+  auto cnt = torch::from_blob(const_cast<int64_t*>(count), {B}, torch::kInt64);
+  auto out = mo::GroupSequenceNormCPUBwd(f32(dy, shape), f32(x, shape), cnt, f32(mean, {B, G}), f32(rstd, {B, G}),
+                                         f32(gamma, {H}), m, G, length_last != 0);
+  std::memcpy(dx, std::get<0>(out).data_ptr<float>(), sizeof(float) * B * L * H);
+  std::memcpy(dgamma, std::get<1>(out).data_ptr<float>(), sizeof(float) * H);
+  std::memcpy(dbeta, std::get<2>(out).data_ptr<float>(), sizeof(float) * H);
   return 0;
 }
