@@ -71,61 +71,94 @@ __device__ __forceinline__ void block_sum2(float& a, float& b, float* lds) {
   for (int w = 0; w < kThreads / kWave; ++w) a += lds[2 * w], b += lds[2 * w + 1];
 }
 
-// Features last.  A thread owns one feature and walks the tile's time steps;
-// the padding mask is per step, so the branch is uniform.
+// One 16-byte access of `dtype` elements as floats.
+template <int DT> struct Vec {
+  static constexpr int N = DT == MEGA_F32 ? 4 : 8;  // elements of one 16-byte access
+  static __device__ __forceinline__ void load(const typename Elem<DT>::type* p, float* v) {
+    const uint4 q = *reinterpret_cast<const uint4*>(p);
+    if constexpr (DT == MEGA_F32) {
+      v[0] = __uint_as_float(q.x), v[1] = __uint_as_float(q.y), v[2] = __uint_as_float(q.z),
+      v[3] = __uint_as_float(q.w);
+    } else {
+      unpack8<DT>(q, v);
+    }
+  }
+  static __device__ __forceinline__ void store(typename Elem<DT>::type* p, const float* v) {
+    if constexpr (DT == MEGA_F32) {
+      *reinterpret_cast<uint4*>(p) =
+          make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3]));
+    } else {
+      *reinterpret_cast<uint4*>(p) = pack8<DT>(v);
+    }
+  }
+};
+
+// Features last.  A thread owns V consecutive features (one 16-byte load per
+// step when V > 1) and walks the tile's time steps; the padding mask is per
+// step, so the branch is uniform.
 //   BWD == false: part = (mean, M2) of the unmasked steps, cnt = their number
 //   BWD == true : part = (sum dy (x - mean_g), sum dy)
-template <int DT, bool BWD>
+template <int DT, bool BWD, int V>
 __global__ __launch_bounds__(kThreads) void moments_feat_last_kernel(
     const typename Elem<DT>::type* __restrict__ x, const typename Elem<DT>::type* __restrict__ dy,
     const uint8_t* __restrict__ mask, const float* __restrict__ mean, int64_t L, int64_t H, int G, int D, int tiles,
     float2* __restrict__ part, int* __restrict__ cnt) {
-  const int64_t h = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t h = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) * V;
   const int tile = blockIdx.y;
   const int64_t b = blockIdx.z;
   const int64_t l0 = static_cast<int64_t>(tile) * kTileFeatLast;
   const int64_t l1 = l0 + kTileFeatLast < L ? l0 + kTileFeatLast : L;
-  const bool live = h < H;
+  const bool live = h < H;  // V > 1 is only used when H % V == 0
   const uint8_t* mrow = mask ? mask + b * L : nullptr;
-  const float u = (BWD && live) ? mean[b * G + h / D] : 0.f;
+  float u[V], x0[V], s1[V], s2[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    u[e] = (BWD && live) ? mean[b * G + (h + e) / D] : 0.f;
+    x0[e] = s1[e] = s2[e] = 0.f;
+  }
   int n = 0;
-  float x0 = 0.f, s1 = 0.f, s2 = 0.f;
   for (int64_t l = l0; l < l1; ++l) {
     if (mrow && mrow[l]) continue;
     if (live) {
       const int64_t at = (b * L + l) * H + h;
-      const float v = Elem<DT>::load(x + at);
-      if (BWD) {
-        const float g = Elem<DT>::load(dy + at);
-        s1 += g * (v - u);
-        s2 += g;
+      float v[V], g[V];
+      if constexpr (V == 1) {
+        v[0] = Elem<DT>::load(x + at);
+        if (BWD) g[0] = Elem<DT>::load(dy + at);
       } else {
-        if (n == 0) x0 = v;
-        const float d = v - x0;
-        s1 += d;
-        s2 += d * d;
+        Vec<DT>::load(x + at, v);
+        if (BWD) Vec<DT>::load(dy + at, g);
+      }
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        if (BWD) {
+          s1[e] += g[e] * (v[e] - u[e]);
+          s2[e] += g[e];
+        } else {
+          if (n == 0) x0[e] = v[e];
+          const float d = v[e] - x0[e];
+          s1[e] += d;
+          s2[e] += d * d;
+        }
       }
     }
     ++n;
   }
   if (live) {
-    float2 out;
-    if (BWD) {
-      out = make_float2(s1, s2);
-    } else if (n > 0) {
-      const float inv = 1.f / static_cast<float>(n);
-      out = make_float2(x0 + s1 * inv, fmaxf(s2 - s1 * s1 * inv, 0.f));
-    } else {
-      out = make_float2(0.f, 0.f);
+    const float inv = n > 0 ? 1.f / static_cast<float>(n) : 0.f;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float2 out = BWD ? make_float2(s1[e], s2[e])
+                             : make_float2(x0[e] + s1[e] * inv, fmaxf(s2[e] - s1[e] * s1[e] * inv, 0.f));
+      part[(b * tiles + tile) * H + h + e] = out;
     }
-    part[(b * tiles + tile) * H + h] = out;
   }
   if (!BWD && blockIdx.x == 0 && threadIdx.x == 0) cnt[b * tiles + tile] = n;
 }
 
 // Length last.  A workgroup owns one tile of one (b, feature) row; lanes run
-// along the time axis.
-template <int DT, bool BWD>
+// along the time axis, V consecutive steps per load (V > 1 needs L % V == 0).
+template <int DT, bool BWD, int V>
 __global__ __launch_bounds__(kThreads) void moments_len_last_kernel(
     const typename Elem<DT>::type* __restrict__ x, const typename Elem<DT>::type* __restrict__ dy,
     const uint8_t* __restrict__ mask, const float* __restrict__ mean, int64_t L, int64_t H, int G, int D, int tiles,
@@ -140,19 +173,28 @@ __global__ __launch_bounds__(kThreads) void moments_len_last_kernel(
   const uint8_t* mrow = mask ? mask + b * L : nullptr;
   const float u = BWD ? mean[b * G + h / D] : 0.f;
   float n = 0.f, x0 = 0.f, s1 = 0.f, s2 = 0.f;
-  for (int64_t l = l0 + threadIdx.x; l < l1; l += kThreads) {
-    if (mrow && mrow[l]) continue;
-    const float v = Elem<DT>::load(x + row + l);
-    if (BWD) {
-      const float g = Elem<DT>::load(dy + row + l);
-      s1 += g * (v - u);
-      s2 += g;
+  for (int64_t l = l0 + static_cast<int64_t>(threadIdx.x) * V; l < l1; l += kThreads * V) {
+    float v[V], g[V];
+    if constexpr (V == 1) {
+      v[0] = Elem<DT>::load(x + row + l);
+      if (BWD) g[0] = Elem<DT>::load(dy + row + l);
     } else {
-      if (n == 0.f) x0 = v;
-      const float d = v - x0;
-      s1 += d;
-      s2 += d * d;
-      n += 1.f;
+      Vec<DT>::load(x + row + l, v);
+      if (BWD) Vec<DT>::load(dy + row + l, g);
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      if (mrow && mrow[l + e]) continue;
+      if (BWD) {
+        s1 += g[e] * (v[e] - u);
+        s2 += g[e];
+      } else {
+        if (n == 0.f) x0 = v[e];
+        const float d = v[e] - x0;
+        s1 += d;
+        s2 += d * d;
+        n += 1.f;
+      }
     }
   }
   if (BWD) {
@@ -237,6 +279,51 @@ __global__ __launch_bounds__(kThreads) void finalize_bwd_kernel(
   }
 }
 
+// The per-feature operator (D == 1): one thread per (b, feature) walks the
+// tiles, neighbouring threads read neighbouring features.
+__global__ __launch_bounds__(kThreads) void finalize_fwd_cols_kernel(const float2* __restrict__ part,
+                                                                     const int* __restrict__ cnt, int64_t H, int tiles,
+                                                                     float eps, int64_t* __restrict__ count,
+                                                                     float* __restrict__ mean,
+                                                                     float* __restrict__ rstd) {
+  const int64_t h = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t b = blockIdx.y;
+  if (h >= H) return;
+  float n = 0.f, m = 0.f, s = 0.f;
+  int64_t c = 0;
+  for (int t = 0; t < tiles; ++t) {
+    const float2 p = part[(b * tiles + t) * H + h];
+    const int ct = cnt[b * tiles + t];
+    c += ct;
+    merge(n, m, s, static_cast<float>(ct), p.x, p.y);
+  }
+  mean[b * H + h] = m;
+  rstd[b * H + h] = 1.f / sqrtf((n > 0.f ? s / n : 0.f) + eps);
+  if (h == 0) count[b] = c;
+}
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void finalize_bwd_cols_kernel(
+    const float2* __restrict__ part, const int64_t* __restrict__ count, const float* __restrict__ rstd,
+    const typename Elem<DT>::type* __restrict__ gamma, int64_t H, int tiles, float2* __restrict__ col,
+    float2* __restrict__ coef) {
+  const int64_t h = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t b = blockIdx.y;
+  if (h >= H) return;
+  float a = 0.f, c = 0.f;
+  for (int t = 0; t < tiles; ++t) {
+    const float2 p = part[(b * tiles + t) * H + h];
+    a += p.x;
+    c += p.y;
+  }
+  const float r = rstd[b * H + h];
+  const float w = Elem<DT>::load(gamma + h);
+  const int64_t cn = count[b];
+  const float k = cn > 0 ? 1.f / static_cast<float>(cn) : 0.f;
+  col[b * H + h] = make_float2(r * a, c);
+  coef[b * H + h] = make_float2(k * r * r * r * w * a, k * r * w * c);
+}
+
 template <int DT>
 __global__ __launch_bounds__(kThreads) void param_grad_kernel(const float2* __restrict__ col, int64_t B, int64_t H,
                                                               typename Elem<DT>::type* __restrict__ dgamma,
@@ -254,30 +341,9 @@ __global__ __launch_bounds__(kThreads) void param_grad_kernel(const float2* __re
 }
 
 // ---- elementwise passes -------------------------------------------------------
-template <int DT> struct Vec {
-  static constexpr int N = DT == MEGA_F32 ? 4 : 8;  // elements of one 16-byte access
-  static __device__ __forceinline__ void load(const typename Elem<DT>::type* p, float* v) {
-    const uint4 q = *reinterpret_cast<const uint4*>(p);
-    if constexpr (DT == MEGA_F32) {
-      v[0] = __uint_as_float(q.x), v[1] = __uint_as_float(q.y), v[2] = __uint_as_float(q.z),
-      v[3] = __uint_as_float(q.w);
-    } else {
-      unpack8<DT>(q, v);
-    }
-  }
-  static __device__ __forceinline__ void store(typename Elem<DT>::type* p, const float* v) {
-    if constexpr (DT == MEGA_F32) {
-      *reinterpret_cast<uint4*>(p) =
-          make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3]));
-    } else {
-      *reinterpret_cast<uint4*>(p) = pack8<DT>(v);
-    }
-  }
-};
-
 // y (BWD == false) or dx (BWD == true) for V consecutive elements per thread.
-// V = Vec<DT>::N needs the V elements to share a group (features last:
-// D % V == 0) or a row (length last: L % V == 0) and 16-byte aligned
+// V = Vec<DT>::N needs the V elements to lie in one step (features last:
+// H % V == 0) or one row (length last: L % V == 0) and 16-byte aligned
 // pointers; V = 1 is the general path.
 template <int DT, bool LAST, bool BWD, int V>
 __global__ __launch_bounds__(kThreads) void apply_kernel(
@@ -300,12 +366,23 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(
     l = bl % L;
     b = bl / L;
   }
-  const int64_t sg = b * G + h / D;
-  const float u = mean[sg], r = rstd[sg];
-  float c1 = 0.f, c2 = 0.f;
-  if (BWD) {
-    const float2 c = coef[sg];
-    c1 = c.x, c2 = c.y;
+  // statistics of each element's group: shared by the V elements when they
+  // lie in one row (length last) or one group (D % V == 0)
+  float uv[V], rv[V], c1v[V], c2v[V];
+  const bool shared = LAST || V == 1 || D % V == 0;
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    if (e > 0 && shared) {
+      uv[e] = uv[0], rv[e] = rv[0], c1v[e] = c1v[0], c2v[e] = c2v[0];
+      continue;
+    }
+    const int64_t sg = b * G + (h + (LAST ? 0 : e)) / D;
+    uv[e] = mean[sg], rv[e] = rstd[sg];
+    c1v[e] = c2v[e] = 0.f;
+    if (BWD) {
+      const float2 c = coef[sg];
+      c1v[e] = c.x, c2v[e] = c.y;
+    }
   }
   float xv[V], gv[V], wv[V], bv[V], ov[V];
   if constexpr (V == 1) {
@@ -329,7 +406,8 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(
 #pragma unroll
   for (int e = 0; e < V; ++e) {
     const bool masked = mask && mask[b * L + (LAST ? l + e : l)];
-    const float v = BWD ? r * wv[e] * gv[e] - (xv[e] - u) * c1 - c2 : (xv[e] - u) * r * wv[e] + bv[e];
+    const float v = BWD ? rv[e] * wv[e] * gv[e] - (xv[e] - uv[e]) * c1v[e] - c2v[e]
+                        : (xv[e] - uv[e]) * rv[e] * wv[e] + bv[e];
     ov[e] = masked ? 0.f : v;
   }
   if constexpr (V == 1) {
@@ -379,18 +457,22 @@ template <int DT, bool BWD>
 int launch_moments(const Shape& s, const void* x, const void* dy, const uint8_t* mask, const float* mean,
                    const Workspace& w, hipStream_t st) {
   using T = typename Elem<DT>::type;
+  constexpr int V = Vec<DT>::N;
   if (s.tiles == 0) return MEGA_OK;  // empty sequences: nothing to sum
+  const T* xp = static_cast<const T*>(x);
+  const T* gp = static_cast<const T*>(dy);
+  const bool vec = aligned16(x) && (!BWD || aligned16(dy)) && (s.last ? s.L : s.H) % V == 0;
+#define MEGA_MOMENTS(KERNEL_, V_, GRID_) \
+  KERNEL_<DT, BWD, V_><<<GRID_, kThreads, 0, st>>>(xp, gp, mask, mean, s.L, s.H, s.G, s.D, s.tiles, w.part, w.cnt)
   if (s.last) {
     const dim3 grid(s.tiles, static_cast<unsigned>(s.H), static_cast<unsigned>(s.B));
-    moments_len_last_kernel<DT, BWD><<<grid, kThreads, 0, st>>>(static_cast<const T*>(x), static_cast<const T*>(dy),
-                                                                 mask, mean, s.L, s.H, s.G, s.D, s.tiles, w.part,
-                                                                 w.cnt);
+    if (vec) MEGA_MOMENTS(moments_len_last_kernel, V, grid); else MEGA_MOMENTS(moments_len_last_kernel, 1, grid);
   } else {
-    const dim3 grid(static_cast<unsigned>((s.H + kThreads - 1) / kThreads), s.tiles, static_cast<unsigned>(s.B));
-    moments_feat_last_kernel<DT, BWD><<<grid, kThreads, 0, st>>>(static_cast<const T*>(x), static_cast<const T*>(dy),
-                                                                  mask, mean, s.L, s.H, s.G, s.D, s.tiles, w.part,
-                                                                  w.cnt);
+    const int64_t per = static_cast<int64_t>(kThreads) * (vec ? V : 1);
+    const dim3 grid(static_cast<unsigned>((s.H + per - 1) / per), s.tiles, static_cast<unsigned>(s.B));
+    if (vec) MEGA_MOMENTS(moments_feat_last_kernel, V, grid); else MEGA_MOMENTS(moments_feat_last_kernel, 1, grid);
   }
+#undef MEGA_MOMENTS
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
 }
@@ -407,7 +489,7 @@ int launch_apply(const Shape& s, const void* x, const void* dy, const void* gamm
   if (s.last)
     vec = vec && s.L % V == 0;
   else
-    vec = vec && s.D % V == 0 && aligned16(gamma) && (BWD || aligned16(beta));
+    vec = vec && s.H % V == 0 && aligned16(gamma) && (BWD || aligned16(beta));
   const int64_t threads = vec ? total / V : total;
   const int64_t blocks = (threads + kThreads - 1) / kThreads;
   MEGA_CHECK_ARG(blocks < (1ll << 31), "mega_group_sequence_norm: tensor too large");
@@ -435,8 +517,13 @@ int run_fwd(const Shape& s, const void* x, const void* gamma, const void* beta, 
             void* y, int64_t* count, float* mean, float* rstd, void* workspace, hipStream_t st) {
   const Workspace w = carve(workspace, s.B, s.H, s.G, s.tiles);
   if (int rc = launch_moments<DT, false>(s, x, nullptr, mask, nullptr, w, st)) return rc;
-  finalize_fwd_kernel<<<dim3(s.G, static_cast<unsigned>(s.B)), kThreads, 0, st>>>(w.part, w.cnt, s.H, s.G, s.D,
-                                                                                   s.tiles, eps, count, mean, rstd);
+  if (s.D == 1)
+    finalize_fwd_cols_kernel<<<dim3(static_cast<unsigned>((s.H + kThreads - 1) / kThreads),
+                                    static_cast<unsigned>(s.B)), kThreads, 0, st>>>(w.part, w.cnt, s.H, s.tiles, eps,
+                                                                                     count, mean, rstd);
+  else
+    finalize_fwd_kernel<<<dim3(s.G, static_cast<unsigned>(s.B)), kThreads, 0, st>>>(w.part, w.cnt, s.H, s.G, s.D,
+                                                                                     s.tiles, eps, count, mean, rstd);
   MEGA_CHECK_LAUNCH();
   return launch_apply<DT, false>(s, x, nullptr, gamma, beta, mask, mean, rstd, nullptr, y, st);
 }
@@ -454,8 +541,13 @@ int run_bwd(const Shape& s, const void* dy, const void* x, const int64_t* count,
     return MEGA_OK;
   }
   if (int rc = launch_moments<DT, true>(s, x, dy, mask, mean, w, st)) return rc;
-  finalize_bwd_kernel<DT><<<dim3(s.G, static_cast<unsigned>(s.B)), kThreads, 0, st>>>(
-      w.part, count, rstd, static_cast<const T*>(gamma), s.H, s.G, s.D, s.tiles, w.col, w.coef);
+  if (s.D == 1)
+    finalize_bwd_cols_kernel<DT><<<dim3(static_cast<unsigned>((s.H + kThreads - 1) / kThreads),
+                                        static_cast<unsigned>(s.B)), kThreads, 0, st>>>(
+        w.part, count, rstd, static_cast<const T*>(gamma), s.H, s.tiles, w.col, w.coef);
+  else
+    finalize_bwd_kernel<DT><<<dim3(s.G, static_cast<unsigned>(s.B)), kThreads, 0, st>>>(
+        w.part, count, rstd, static_cast<const T*>(gamma), s.H, s.G, s.D, s.tiles, w.col, w.coef);
   MEGA_CHECK_LAUNCH();
   param_grad_kernel<DT><<<static_cast<unsigned>((s.H + kThreads - 1) / kThreads), kThreads, 0, st>>>(
       w.col, s.B, s.H, static_cast<T*>(dgamma), static_cast<T*>(dbeta));

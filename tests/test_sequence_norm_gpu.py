@@ -61,6 +61,8 @@ def _check(B, L, H, G, dtype, seed, mask, length_last):
     (1, 4104, 16, 2),    # three tiles of the length-last layout, L % 8 == 0
     (2, 2049, 6, 1),     # one group over everything, odd length
     (1, 1, 8, 2),        # single step
+    (2, 200, 48, 16),    # 16-byte loads that straddle groups of D = 3
+    (2, 260, 32, 32),    # per-feature operator on the 16-byte path
 ])
 def test_matches_oracle(shape, length_last, dtype):
     B, L, H, G = shape
