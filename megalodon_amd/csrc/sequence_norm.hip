@@ -111,38 +111,52 @@ __global__ __launch_bounds__(kThreads) void moments_feat_last_kernel(
   const bool live = h < H;  // V > 1 is only used when H % V == 0
   const uint8_t* mrow = mask ? mask + b * L : nullptr;
   float u[V], x0[V], s1[V], s2[V];
+  int64_t sg = b * G + h / D;
+  int rem = static_cast<int>(h % D);
 #pragma unroll
   for (int e = 0; e < V; ++e) {
-    u[e] = (BWD && live) ? mean[b * G + (h + e) / D] : 0.f;
+    if (e > 0 && ++rem == D) rem = 0, ++sg;
+    u[e] = (BWD && live) ? mean[sg] : 0.f;
     x0[e] = s1[e] = s2[e] = 0.f;
   }
   int n = 0;
-  for (int64_t l = l0; l < l1; ++l) {
-    if (mrow && mrow[l]) continue;
-    if (live) {
-      const int64_t at = (b * L + l) * H + h;
-      float v[V], g[V];
-      if constexpr (V == 1) {
-        v[0] = Elem<DT>::load(x + at);
-        if (BWD) g[0] = Elem<DT>::load(dy + at);
-      } else {
-        Vec<DT>::load(x + at, v);
-        if (BWD) Vec<DT>::load(dy + at, g);
-      }
+  // U steps per round: their loads are issued together, then summed in order
+  constexpr int U = BWD ? 4 : 8;
+  for (int64_t l = l0; l < l1; l += U) {
+    float v[U][V], g[U][V];
+    bool ok[U];
 #pragma unroll
-      for (int e = 0; e < V; ++e) {
-        if (BWD) {
-          s1[e] += g[e] * (v[e] - u[e]);
-          s2[e] += g[e];
-        } else {
-          if (n == 0) x0[e] = v[e];
-          const float d = v[e] - x0[e];
-          s1[e] += d;
-          s2[e] += d * d;
-        }
+    for (int i = 0; i < U; ++i) {
+      ok[i] = l + i < l1 && !(mrow && mrow[l + i]);
+      if (!(ok[i] && live)) continue;
+      const int64_t at = (b * L + l + i) * H + h;
+      if constexpr (V == 1) {
+        v[i][0] = Elem<DT>::load(x + at);
+        if (BWD) g[i][0] = Elem<DT>::load(dy + at);
+      } else {
+        Vec<DT>::load(x + at, v[i]);
+        if (BWD) Vec<DT>::load(dy + at, g[i]);
       }
     }
-    ++n;
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      if (!ok[i]) continue;
+      if (live) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          if (BWD) {
+            s1[e] += g[i][e] * (v[i][e] - u[e]);
+            s2[e] += g[i][e];
+          } else {
+            if (n == 0) x0[e] = v[i][e];
+            const float d = v[i][e] - x0[e];
+            s1[e] += d;
+            s2[e] += d * d;
+          }
+        }
+      }
+      ++n;
+    }
   }
   if (live) {
     const float inv = n > 0 ? 1.f / static_cast<float>(n) : 0.f;
@@ -215,6 +229,11 @@ __global__ __launch_bounds__(kThreads) void moments_len_last_kernel(
   }
 }
 
+// Shape of the combination passes: lanes along features, waves along tiles.
+constexpr int kColFeat = kWave;               // features per workgroup
+constexpr int kColSlices = kThreads / kWave;  // tile slices per workgroup
+constexpr int kColAhead = 8;                  // loads issued before their merges
+
 // One workgroup per (b, g): combine the (tile, feature) partial moments.
 __global__ __launch_bounds__(kThreads) void finalize_fwd_kernel(const float2* __restrict__ part,
                                                                 const int* __restrict__ cnt, int64_t H, int G, int D,
@@ -223,13 +242,24 @@ __global__ __launch_bounds__(kThreads) void finalize_fwd_kernel(const float2* __
   __shared__ float lds[3 * kThreads / kWave];
   const int g = blockIdx.x;
   const int64_t b = blockIdx.y;
-  const int64_t items = static_cast<int64_t>(D) * tiles;
+  const int lane = threadIdx.x % kWave, slice = threadIdx.x / kWave;
   float n = 0.f, m = 0.f, s = 0.f;
-  for (int64_t it = threadIdx.x; it < items; it += kThreads) {
-    const int k = static_cast<int>(it % D);
-    const int64_t t = it / D;
-    const float2 p = part[(b * tiles + t) * H + static_cast<int64_t>(g) * D + k];
-    merge(n, m, s, static_cast<float>(cnt[b * tiles + t]), p.x, p.y);
+  for (int k0 = 0; k0 < D; k0 += kColFeat) {
+    const bool live = k0 + lane < D;
+    const int64_t h = static_cast<int64_t>(g) * D + k0 + lane;
+    for (int t0 = slice; t0 < tiles; t0 += kColSlices * kColAhead) {
+      float2 p[kColAhead];
+      int ct[kColAhead];
+#pragma unroll
+      for (int i = 0; i < kColAhead; ++i) {
+        const int t = t0 + i * kColSlices;
+        const bool ok = live && t < tiles;
+        p[i] = ok ? part[(b * tiles + t) * H + h] : make_float2(0.f, 0.f);
+        ct[i] = ok ? cnt[b * tiles + t] : 0;
+      }
+#pragma unroll
+      for (int i = 0; i < kColAhead; ++i) merge(n, m, s, static_cast<float>(ct[i]), p[i].x, p[i].y);
+    }
   }
   block_merge(n, m, s, lds);
   if (threadIdx.x == 0) {
@@ -254,22 +284,36 @@ __global__ __launch_bounds__(kThreads) void finalize_bwd_kernel(
     const typename Elem<DT>::type* __restrict__ gamma, int64_t H, int G, int D, int tiles, float2* __restrict__ col,
     float2* __restrict__ coef) {
   __shared__ float lds[2 * kThreads / kWave];
+  __shared__ float cols[kColSlices][2][kColFeat];
   const int g = blockIdx.x;
   const int64_t b = blockIdx.y;
   const float r = rstd[b * G + g];
+  const int lane = threadIdx.x % kWave, slice = threadIdx.x / kWave;
   float A = 0.f, Bs = 0.f;
-  for (int k = threadIdx.x; k < D; k += kThreads) {
-    const int64_t h = static_cast<int64_t>(g) * D + k;
+  for (int k0 = 0; k0 < D; k0 += kColFeat) {
+    const bool live = k0 + lane < D;
+    const int64_t h = static_cast<int64_t>(g) * D + k0 + lane;
     float a = 0.f, c = 0.f;
-    for (int t = 0; t < tiles; ++t) {
-      const float2 p = part[(b * tiles + t) * H + h];
-      a += p.x;
-      c += p.y;
+    for (int t0 = slice; t0 < tiles; t0 += kColSlices * kColAhead) {
+      float2 p[kColAhead];
+#pragma unroll
+      for (int i = 0; i < kColAhead; ++i) {
+        const int t = t0 + i * kColSlices;
+        p[i] = (live && t < tiles) ? part[(b * tiles + t) * H + h] : make_float2(0.f, 0.f);
+      }
+#pragma unroll
+      for (int i = 0; i < kColAhead; ++i) a += p[i].x, c += p[i].y;
     }
-    col[b * H + h] = make_float2(r * a, c);
-    const float w = Elem<DT>::load(gamma + h);
-    A += w * a;
-    Bs += w * c;
+    cols[slice][0][lane] = a, cols[slice][1][lane] = c;
+    __syncthreads();
+    if (slice == 0 && live) {
+      for (int w = 1; w < kColSlices; ++w) a += cols[w][0][lane], c += cols[w][1][lane];
+      col[b * H + h] = make_float2(r * a, c);
+      const float w = Elem<DT>::load(gamma + h);
+      A += w * a;
+      Bs += w * c;
+    }
+    __syncthreads();
   }
   block_sum2(A, Bs, lds);
   if (threadIdx.x == 0) {
@@ -279,27 +323,45 @@ __global__ __launch_bounds__(kThreads) void finalize_bwd_kernel(
   }
 }
 
-// The per-feature operator (D == 1): one thread per (b, feature) walks the
-// tiles, neighbouring threads read neighbouring features.
+// The per-feature operator (D == 1): a workgroup owns 64 neighbouring features
+// of one batch entry; wave w walks tiles w, w + 4, ... (eight loads in flight
+// per lane), the four partial results are combined in wave order through LDS.
+
 __global__ __launch_bounds__(kThreads) void finalize_fwd_cols_kernel(const float2* __restrict__ part,
                                                                      const int* __restrict__ cnt, int64_t H, int tiles,
                                                                      float eps, int64_t* __restrict__ count,
                                                                      float* __restrict__ mean,
                                                                      float* __restrict__ rstd) {
-  const int64_t h = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  __shared__ float lds[kColSlices][3][kColFeat];
+  const int lane = threadIdx.x % kWave, slice = threadIdx.x / kWave;
+  const int64_t h = static_cast<int64_t>(blockIdx.x) * kColFeat + lane;
   const int64_t b = blockIdx.y;
-  if (h >= H) return;
+  const bool live = h < H;
   float n = 0.f, m = 0.f, s = 0.f;
-  int64_t c = 0;
-  for (int t = 0; t < tiles; ++t) {
-    const float2 p = part[(b * tiles + t) * H + h];
-    const int ct = cnt[b * tiles + t];
-    c += ct;
-    merge(n, m, s, static_cast<float>(ct), p.x, p.y);
+  for (int t0 = slice; t0 < tiles; t0 += kColSlices * kColAhead) {
+    float2 p[kColAhead];
+    int ct[kColAhead];
+#pragma unroll
+    for (int i = 0; i < kColAhead; ++i) {
+      const int t = t0 + i * kColSlices;
+      const bool ok = live && t < tiles;
+      p[i] = ok ? part[(b * tiles + t) * H + h] : make_float2(0.f, 0.f);
+      ct[i] = ok ? cnt[b * tiles + t] : 0;
+    }
+#pragma unroll
+    for (int i = 0; i < kColAhead; ++i) merge(n, m, s, static_cast<float>(ct[i]), p[i].x, p[i].y);
   }
+  lds[slice][0][lane] = n, lds[slice][1][lane] = m, lds[slice][2][lane] = s;
+  __syncthreads();
+  if (slice != 0 || !live) return;
+  for (int w = 1; w < kColSlices; ++w) merge(n, m, s, lds[w][0][lane], lds[w][1][lane], lds[w][2][lane]);
   mean[b * H + h] = m;
   rstd[b * H + h] = 1.f / sqrtf((n > 0.f ? s / n : 0.f) + eps);
-  if (h == 0) count[b] = c;
+  if (h == 0) {
+    int64_t c = 0;
+    for (int t = 0; t < tiles; ++t) c += cnt[b * tiles + t];
+    count[b] = c;
+  }
 }
 
 template <int DT>
@@ -307,15 +369,26 @@ __global__ __launch_bounds__(kThreads) void finalize_bwd_cols_kernel(
     const float2* __restrict__ part, const int64_t* __restrict__ count, const float* __restrict__ rstd,
     const typename Elem<DT>::type* __restrict__ gamma, int64_t H, int tiles, float2* __restrict__ col,
     float2* __restrict__ coef) {
-  const int64_t h = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  __shared__ float lds[kColSlices][2][kColFeat];
+  const int lane = threadIdx.x % kWave, slice = threadIdx.x / kWave;
+  const int64_t h = static_cast<int64_t>(blockIdx.x) * kColFeat + lane;
   const int64_t b = blockIdx.y;
-  if (h >= H) return;
+  const bool live = h < H;
   float a = 0.f, c = 0.f;
-  for (int t = 0; t < tiles; ++t) {
-    const float2 p = part[(b * tiles + t) * H + h];
-    a += p.x;
-    c += p.y;
+  for (int t0 = slice; t0 < tiles; t0 += kColSlices * kColAhead) {
+    float2 p[kColAhead];
+#pragma unroll
+    for (int i = 0; i < kColAhead; ++i) {
+      const int t = t0 + i * kColSlices;
+      p[i] = (live && t < tiles) ? part[(b * tiles + t) * H + h] : make_float2(0.f, 0.f);
+    }
+#pragma unroll
+    for (int i = 0; i < kColAhead; ++i) a += p[i].x, c += p[i].y;
   }
+  lds[slice][0][lane] = a, lds[slice][1][lane] = c;
+  __syncthreads();
+  if (slice != 0 || !live) return;
+  for (int w = 1; w < kColSlices; ++w) a += lds[w][0][lane], c += lds[w][1][lane];
   const float r = rstd[b * H + h];
   const float w = Elem<DT>::load(gamma + h);
   const int64_t cn = count[b];
@@ -370,13 +443,35 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(
   // lie in one row (length last) or one group (D % V == 0)
   float uv[V], rv[V], c1v[V], c2v[V];
   const bool shared = LAST || V == 1 || D % V == 0;
+  // group of element e: one division, then a running remainder
+  int64_t sg = b * G + h / D;
+  int rem = static_cast<int>(h % D);
+  // one feature per group: the V statistics are V neighbouring floats
+  const bool rowwise = !LAST && V > 1 && D == 1 &&
+                       ((reinterpret_cast<uintptr_t>(mean) | reinterpret_cast<uintptr_t>(rstd)) & 15) == 0;
+  if (rowwise) {
+#pragma unroll
+    for (int e = 0; e < V; e += 4) {
+      const float4 u4 = *reinterpret_cast<const float4*>(mean + sg + e);
+      const float4 r4 = *reinterpret_cast<const float4*>(rstd + sg + e);
+      uv[e] = u4.x, uv[e + 1 < V ? e + 1 : e] = u4.y, uv[e + 2 < V ? e + 2 : e] = u4.z, uv[e + 3 < V ? e + 3 : e] = u4.w;
+      rv[e] = r4.x, rv[e + 1 < V ? e + 1 : e] = r4.y, rv[e + 2 < V ? e + 2 : e] = r4.z, rv[e + 3 < V ? e + 3 : e] = r4.w;
+    }
+#pragma unroll
+    for (int e = 0; e < V; e += 2) {
+      float4 c4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (BWD) c4 = *reinterpret_cast<const float4*>(coef + sg + e);
+      c1v[e] = c4.x, c2v[e] = c4.y, c1v[e + 1 < V ? e + 1 : e] = c4.z, c2v[e + 1 < V ? e + 1 : e] = c4.w;
+    }
+  }
 #pragma unroll
   for (int e = 0; e < V; ++e) {
+    if (rowwise) break;
     if (e > 0 && shared) {
       uv[e] = uv[0], rv[e] = rv[0], c1v[e] = c1v[0], c2v[e] = c2v[0];
       continue;
     }
-    const int64_t sg = b * G + (h + (LAST ? 0 : e)) / D;
+    if (e > 0 && ++rem == D) rem = 0, ++sg;
     uv[e] = mean[sg], rv[e] = rstd[sg];
     c1v[e] = c2v[e] = 0.f;
     if (BWD) {
@@ -518,7 +613,7 @@ int run_fwd(const Shape& s, const void* x, const void* gamma, const void* beta, 
   const Workspace w = carve(workspace, s.B, s.H, s.G, s.tiles);
   if (int rc = launch_moments<DT, false>(s, x, nullptr, mask, nullptr, w, st)) return rc;
   if (s.D == 1)
-    finalize_fwd_cols_kernel<<<dim3(static_cast<unsigned>((s.H + kThreads - 1) / kThreads),
+    finalize_fwd_cols_kernel<<<dim3(static_cast<unsigned>((s.H + kColFeat - 1) / kColFeat),
                                     static_cast<unsigned>(s.B)), kThreads, 0, st>>>(w.part, w.cnt, s.H, s.tiles, eps,
                                                                                      count, mean, rstd);
   else
@@ -542,7 +637,7 @@ int run_bwd(const Shape& s, const void* dy, const void* x, const int64_t* count,
   }
   if (int rc = launch_moments<DT, true>(s, x, dy, mask, mean, w, st)) return rc;
   if (s.D == 1)
-    finalize_bwd_cols_kernel<DT><<<dim3(static_cast<unsigned>((s.H + kThreads - 1) / kThreads),
+    finalize_bwd_cols_kernel<DT><<<dim3(static_cast<unsigned>((s.H + kColFeat - 1) / kColFeat),
                                         static_cast<unsigned>(s.B)), kThreads, 0, st>>>(
         w.part, count, rstd, static_cast<const T*>(gamma), s.H, s.tiles, w.col, w.coef);
   else
