@@ -280,6 +280,82 @@ def fftconv_max_length() -> int:
     return int(_lib.load().mega_fftconv_max_length())
 
 
+# Rows longer than one kernel launch takes are cut into nb blocks of S samples
+# (zero padded at the end).  With head(a, c) = the first S outputs of the
+# linear convolution of two blocks (what one launch computes) and tail(a, c) =
+# its outputs S .. 2S-1,
+#   y_b = sum_{i+j=b} head(x_i, k_j) + sum_{i+j=b-1} tail(x_i, k_j),
+# and the tail is a head of the reversed blocks:
+#   tail(a, c)[t] = head(flip a, flip c)[S-2-t]  (t <= S-2),  tail[S-1] = 0.
+# All blocks x_i that meet one kernel block k_j go through one launch, stacked
+# along the batch axis; the backward pass sends the gradient of every term
+# through the backward launch of the same pair (which also sums dk over the
+# stack).  Sums over terms are float32.  The reference takes rows of any
+# length through torch.fft (fused_ops/fftconv.py:84,103).
+def _long_blocks(L: int) -> Tuple[int, int]:
+    nb = -(-L // fftconv_max_length())
+    S = -(-L // nb)
+    return nb, (S + 7) // 8 * 8
+
+
+def _cut(t: torch.Tensor, nb: int, S: int) -> torch.Tensor:
+    """(..., L) -> (nb, ..., S), zero padded."""
+    L = t.shape[-1]
+    if nb * S != L:
+        t = torch.nn.functional.pad(t, (0, nb * S - L))
+    return t.reshape(*t.shape[:-1], nb, S).movedim(-2, 0).contiguous()
+
+
+def _head_to_tail(h: torch.Tensor) -> torch.Tensor:
+    """h[..., m] -> t[..., S-2-m] for m <= S-2, last entry 0 (its own inverse)."""
+    t = torch.zeros_like(h)
+    t[..., :-1] = h[..., :-1].flip(-1)
+    return t
+
+
+def _fftconv_long_fwd(x: torch.Tensor, k: torch.Tensor, blocks=None, head=None) -> torch.Tensor:
+    """`blocks` = (nb, S) and `head` = the one-launch operator; the defaults are
+    the library's limits and `fftconv_fwd` (tests pass others)."""
+    B, D, L = x.shape
+    nb, S = blocks or _long_blocks(L)
+    head = head or fftconv_fwd
+    xb, kb = _cut(x, nb, S), _cut(k.float(), nb, S)
+    xr, kr = xb.flip(-1), kb.flip(-1)
+    y = torch.zeros((nb, B, D, S), dtype=torch.float32, device=x.device)
+    for j in range(nb):
+        n = nb - j
+        y[j:] += head(xb[:n].reshape(n * B, D, S), kb[j]).view(n, B, D, S)
+        n = nb - 1 - j
+        if n > 0:
+            h = head(xr[:n].reshape(n * B, D, S), kr[j]).view(n, B, D, S)
+            y[j + 1:] += _head_to_tail(h.float())
+    return y.movedim(0, -2).reshape(B, D, nb * S)[..., :L].to(x.dtype)
+
+
+def _fftconv_long_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor, blocks=None,
+                      head_bwd=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    B, D, L = x.shape
+    nb, S = blocks or _long_blocks(L)
+    head_bwd = head_bwd or (lambda g, a, c: fftconv_bwd(g, a, c, torch.float32))
+    xb, kb, gb = _cut(x, nb, S), _cut(k.float(), nb, S), _cut(y_grad, nb, S)
+    xr, kr = xb.flip(-1), kb.flip(-1)
+    dx = torch.zeros((nb, B, D, S), dtype=torch.float32, device=x.device)
+    dk = torch.zeros((nb, D, S), dtype=torch.float32, device=x.device)
+    for j in range(nb):
+        n = nb - j
+        gx, gk = head_bwd(gb[j:].reshape(n * B, D, S), xb[:n].reshape(n * B, D, S), kb[j])
+        dx[:n] += gx.view(n, B, D, S)
+        dk[j] += gk
+        n = nb - 1 - j
+        if n > 0:
+            gh = _head_to_tail(gb[j + 1:]).reshape(n * B, D, S)
+            gx, gk = head_bwd(gh, xr[:n].reshape(n * B, D, S), kr[j])
+            dx[:n] += gx.view(n, B, D, S).float().flip(-1)
+            dk[j] += gk.flip(-1)
+    dx = dx.movedim(0, -2).reshape(B, D, nb * S)[..., :L].to(x.dtype)
+    return dx, dk.movedim(0, -2).reshape(D, nb * S)[..., :L].contiguous()
+
+
 def fftconv_fwd(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     """y = causal_conv(x, k).  x (B, D, L) float32/bfloat16/float16, k (D, L).
 
@@ -290,6 +366,8 @@ def fftconv_fwd(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     if x.dim() != 3 or k.dim() != 2 or k.shape[0] != x.shape[1] or k.shape[1] != x.shape[2]:
         raise RuntimeError(f"fftconv: x {tuple(x.shape)} and k {tuple(k.shape)} do not match (B,D,L)/(D,L)")
     B, D, L = x.shape
+    if L > fftconv_max_length():
+        return _fftconv_long_fwd(x, k)
     xc = x.contiguous()
     kc = k.contiguous().float()
     y = torch.empty_like(xc)
@@ -306,6 +384,9 @@ def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
     B, D, L = x.shape
     if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
         raise RuntimeError("fftconv_bwd: y_grad must match x in shape and dtype")
+    if L > fftconv_max_length():
+        dx, dk = _fftconv_long_bwd(y_grad, x, k)
+        return dx, dk.to(k_dtype)
     dy = y_grad.contiguous()
     xc = x.contiguous()
     kc = k.contiguous().float()
@@ -328,6 +409,9 @@ def fftconv_residual_fwd(x: torch.Tensor, k: torch.Tensor, omega: torch.Tensor) 
     if omega.numel() != x.shape[1]:
         raise RuntimeError(f"fftconv: omega has {omega.numel()} elements for D={x.shape[1]}")
     B, D, L = x.shape
+    if L > fftconv_max_length():  # blocks, then the skip term in float32
+        y = _fftconv_long_fwd(x, k).float() + x.float() * omega.reshape(-1, 1).float()
+        return y.to(x.dtype)
     xc = x.contiguous()
     kc = k.contiguous().float()
     wc = omega.reshape(-1).contiguous().float()
@@ -347,6 +431,10 @@ def fftconv_residual_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
     B, D, L = x.shape
     if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
         raise RuntimeError("fftconv_bwd: y_grad must match x in shape and dtype")
+    if L > fftconv_max_length():
+        dx, dk = _fftconv_long_bwd(y_grad, x, k)
+        dx = (dx.float() + y_grad.float() * omega.reshape(-1, 1).float()).to(x.dtype)
+        return dx, dk, (y_grad.float() * x.float()).sum(dim=(0, 2))
     dy = y_grad.contiguous()
     xc = x.contiguous()
     kc = k.contiguous().float()

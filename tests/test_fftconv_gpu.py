@@ -257,8 +257,77 @@ def test_autograd_function():
     assert rel_err(xc.grad, wdx) <= 1e-4 and rel_err(kc.grad, wdk) <= 1e-4
 
 
-def test_too_long_rows_fail_loudly():
-    x = torch.zeros(1, 1, 32769, device="cuda")
-    k = torch.zeros(1, 32769, device="cuda")
+def test_too_long_rows_fail_loudly_at_the_c_abi():
+    from megalodon_amd import _lib
+    x = torch.zeros(1, 1, 32776, device="cuda")
+    k = torch.zeros(1, 32776, device="cuda")
+    y = torch.empty_like(x)
     with pytest.raises(RuntimeError, match="exceeds"):
-        ops.fftconv_fwd(x, k)
+        _lib.call("mega_fftconv_fwd", _lib.ptr(x), _lib.i32(_lib.dtype_code(x.dtype)), _lib.ptr(k), _lib.i64(1),
+                  _lib.i64(1), _lib.i64(32776), _lib.ptr(y), _lib.stream_ptr(x.device))
+
+
+def _long_data(B, D, L, dtype, seed):
+    # a kernel that still weighs 2 % at the end of the row, so every block pair contributes
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, D, L, generator=g).to(dtype)
+    k = torch.randn(D, L, generator=g) * torch.exp(-4.0 * torch.arange(L, dtype=torch.float32) / L)
+    dy = torch.randn(B, D, L, generator=g).to(dtype)
+    return x, k, dy
+
+
+@pytest.mark.parametrize("B,D,L", [(1, 2, 32769), (2, 3, 40000), (1, 2, 65536), (1, 2, 70001), (1, 1, 131072)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rows_beyond_one_launch_match_oracle(B, D, L, dtype):
+    """L > 32768: the host cuts rows into blocks (heads and tails of block
+    pairs); forward and backward against the float64 oracle on the whole row."""
+    x, k, dy = _long_data(B, D, L, dtype, L + B)
+    y = ops.fftconv_fwd(x.cuda(), k.cuda())
+    assert y.dtype == dtype and y.shape == x.shape
+    assert rel_err(y, fftconv.fftconv_fwd(x, k)) <= TOL[dtype]
+    dx, dk = ops.fftconv_bwd(dy.cuda(), x.cuda(), k.cuda(), torch.float32)
+    wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
+    assert dx.dtype == dtype and dk.shape == k.shape
+    assert rel_err(dx, wdx) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_residual_autograd_function_beyond_one_launch(dtype):
+    B, D, L = 2, 3, 50000
+    x, k, dy = _long_data(B, D, L, dtype, 77)
+    om = torch.randn(D, 1, generator=torch.Generator().manual_seed(5))
+    xc, kc, oc = (t.cuda().requires_grad_(True) for t in (x, k, om))
+    y = fftconv_residual(xc, kc, oc)
+    y.backward(dy.cuda())
+    x64, k64, o64 = (t.double().requires_grad_(True) for t in (x, k, om))
+    want = fftconv.fftconv_fwd(x64, k64) + x64 * o64
+    want.backward(dy.double())
+    assert y.dtype == dtype
+    assert rel_err(y, want.detach()) <= TOL[dtype]
+    assert rel_err(xc.grad, x64.grad) <= TOL[dtype]
+    assert rel_err(kc.grad, k64.grad) <= TOL[dtype]
+    assert rel_err(oc.grad, o64.grad) <= TOL[dtype]
+
+
+def test_cema_layer_at_twice_the_launch_length():
+    """MultiHeadComplexEMA forward+backward at L = 65536 (fp32): kernel
+    generation, the block-cut convolution and every parameter gradient against
+    the float64 closed form + FFT convolution + autograd."""
+    from megalodon_amd.modules import MultiHeadComplexEMA
+    B, D, N, L = 1, 8, 16, 65536
+    torch.manual_seed(3)
+    m = MultiHeadComplexEMA(D, N).cuda()
+    io = synthetic.cema_inputs(B, D, L, 99)
+    x = io["x"].cuda().requires_grad_(True)
+    out, _ = m(x, None, False)
+    out.backward(io["dy"].cuda())
+    pr = {n_: v.detach().cpu().double().requires_grad_(True) for n_, v in m.named_parameters()}
+    xo = io["x"].double().requires_grad_(True)
+    p, q, g = cema.calc_coeffs(pr["alpha"], pr["delta"], pr["theta"], pr["gamma"], N)
+    want = fftconv.fftconv_fwd(xo, cema.ema_weight_fwd(p, q.log(), g, L)) + xo * pr["omega"]
+    want.backward(io["dy"].double())
+    assert rel_err(out, want.detach()) <= 1e-4
+    assert rel_err(x.grad, xo.grad) <= 1e-4
+    for n_, prm in m.named_parameters():
+        assert rel_err(prm.grad, pr[n_].grad) <= 1e-4, n_

@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 import torch
 
+from conftest import rel_err
 from oracle import cema, fftconv
 
 
@@ -63,3 +64,20 @@ def test_bwd_matches_autograd_over_bruteforce_sum(B, D, L):
             dkb[:, j] += (dyn[:, :, t] * xn[:, :, t - j]).sum(0)
     assert np.allclose(dx.numpy(), dxb, atol=1e-10)
     assert np.allclose(dk.numpy(), dkb, atol=1e-10)
+
+
+@pytest.mark.parametrize("L,nb,S", [(100, 2, 56), (37, 3, 16), (64, 4, 16), (50, 2, 32)])
+def test_long_row_block_decomposition_with_the_oracle_as_one_launch(L, nb, S):
+    """The host-side cutting of rows longer than one launch (heads and tails of
+    block pairs, tails as heads of reversed blocks), with the oracle standing in
+    for the launch: equal to the oracle on the whole row, forward and backward."""
+    from megalodon_amd import extension as ops
+    g = torch.Generator().manual_seed(L)
+    x = torch.randn(2, 3, L, generator=g, dtype=torch.float64)
+    k = torch.randn(3, L, generator=g, dtype=torch.float64)
+    dy = torch.randn(2, 3, L, generator=g, dtype=torch.float64)
+    y = ops._fftconv_long_fwd(x, k, blocks=(nb, S), head=fftconv.fftconv_fwd)
+    assert rel_err(y, fftconv.fftconv_fwd(x, k)) < 1e-6   # the sums over terms are float32
+    dx, dk = ops._fftconv_long_bwd(dy, x, k, blocks=(nb, S), head_bwd=fftconv.fftconv_bwd)
+    wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
+    assert rel_err(dx, wdx) < 1e-6 and rel_err(dk, wdk) < 1e-6
