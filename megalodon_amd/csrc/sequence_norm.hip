@@ -25,7 +25,7 @@ namespace mega {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kTileFeatLast = 128;   // time steps per partial, (B, L, H)
+constexpr int kTileFeatLast = 64;    // time steps per partial, (B, L, H)
 constexpr int kTileLenLast = 2048;   // time steps per partial, (B, H, L)
 
 // (n, mean, M2) <- combination with (n2, mean2, M2_2); M2 = sum (x - mean)^2
@@ -229,9 +229,25 @@ __global__ __launch_bounds__(kThreads) void moments_len_last_kernel(
   }
 }
 
-// Shape of the combination passes: lanes along features, waves along tiles.
-constexpr int kColFeat = kWave;               // features per workgroup
-constexpr int kColSlices = kThreads / kWave;  // tile slices per workgroup
+// Sum of the per-tile step counts of one batch entry, by the whole workgroup
+// (every thread must call it; thread 0 holds the result).
+__device__ __forceinline__ long long block_count(const int* __restrict__ cnt, int tiles, long long* lds) {
+  long long c = 0;
+  for (int t = threadIdx.x; t < tiles; t += kThreads) c += cnt[t];
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) c += __shfl_down(c, o);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  __syncthreads();
+  if (lane == 0) lds[wave] = c;
+  __syncthreads();
+  c = 0;
+  for (int w = 0; w < kThreads / kWave; ++w) c += lds[w];
+  return c;
+}
+
+// Shape of the combination passes: 16 threads along features, 16 along tiles.
+constexpr int kColFeat = 16;                      // neighbouring features (128 bytes of float2) per pass
+constexpr int kColSlices = kThreads / kColFeat;   // tile slices per workgroup
 constexpr int kColAhead = 8;                  // loads issued before their merges
 
 // One workgroup per (b, g): combine the (tile, feature) partial moments.
@@ -242,7 +258,7 @@ __global__ __launch_bounds__(kThreads) void finalize_fwd_kernel(const float2* __
   __shared__ float lds[3 * kThreads / kWave];
   const int g = blockIdx.x;
   const int64_t b = blockIdx.y;
-  const int lane = threadIdx.x % kWave, slice = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kColFeat, slice = threadIdx.x / kColFeat;
   float n = 0.f, m = 0.f, s = 0.f;
   for (int k0 = 0; k0 < D; k0 += kColFeat) {
     const bool live = k0 + lane < D;
@@ -266,11 +282,11 @@ __global__ __launch_bounds__(kThreads) void finalize_fwd_kernel(const float2* __
     const float var = n > 0.f ? s / n : 0.f;
     mean[b * G + g] = m;
     rstd[b * G + g] = 1.f / sqrtf(var + eps);
-    if (g == 0) {
-      int64_t c = 0;
-      for (int t = 0; t < tiles; ++t) c += cnt[b * tiles + t];
-      count[b] = c;
-    }
+  }
+  if (g == 0) {
+    __shared__ long long cl[kThreads / kWave];
+    const long long c = block_count(cnt + b * tiles, tiles, cl);
+    if (threadIdx.x == 0) count[b] = c;
   }
 }
 
@@ -288,7 +304,7 @@ __global__ __launch_bounds__(kThreads) void finalize_bwd_kernel(
   const int g = blockIdx.x;
   const int64_t b = blockIdx.y;
   const float r = rstd[b * G + g];
-  const int lane = threadIdx.x % kWave, slice = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kColFeat, slice = threadIdx.x / kColFeat;
   float A = 0.f, Bs = 0.f;
   for (int k0 = 0; k0 < D; k0 += kColFeat) {
     const bool live = k0 + lane < D;
@@ -323,9 +339,9 @@ __global__ __launch_bounds__(kThreads) void finalize_bwd_kernel(
   }
 }
 
-// The per-feature operator (D == 1): a workgroup owns 64 neighbouring features
-// of one batch entry; wave w walks tiles w, w + 4, ... (eight loads in flight
-// per lane), the four partial results are combined in wave order through LDS.
+// The per-feature operator (D == 1): a workgroup owns 16 neighbouring features
+// of one batch entry; slice w walks tiles w, w + 16, ... (eight loads in flight
+// per thread), the partial results are combined in slice order through LDS.
 
 __global__ __launch_bounds__(kThreads) void finalize_fwd_cols_kernel(const float2* __restrict__ part,
                                                                      const int* __restrict__ cnt, int64_t H, int tiles,
@@ -333,7 +349,7 @@ __global__ __launch_bounds__(kThreads) void finalize_fwd_cols_kernel(const float
                                                                      float* __restrict__ mean,
                                                                      float* __restrict__ rstd) {
   __shared__ float lds[kColSlices][3][kColFeat];
-  const int lane = threadIdx.x % kWave, slice = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kColFeat, slice = threadIdx.x / kColFeat;
   const int64_t h = static_cast<int64_t>(blockIdx.x) * kColFeat + lane;
   const int64_t b = blockIdx.y;
   const bool live = h < H;
@@ -353,15 +369,15 @@ __global__ __launch_bounds__(kThreads) void finalize_fwd_cols_kernel(const float
   }
   lds[slice][0][lane] = n, lds[slice][1][lane] = m, lds[slice][2][lane] = s;
   __syncthreads();
+  if (blockIdx.x == 0) {
+    __shared__ long long cl[kThreads / kWave];
+    const long long c = block_count(cnt + b * tiles, tiles, cl);
+    if (threadIdx.x == 0) count[b] = c;
+  }
   if (slice != 0 || !live) return;
   for (int w = 1; w < kColSlices; ++w) merge(n, m, s, lds[w][0][lane], lds[w][1][lane], lds[w][2][lane]);
   mean[b * H + h] = m;
   rstd[b * H + h] = 1.f / sqrtf((n > 0.f ? s / n : 0.f) + eps);
-  if (h == 0) {
-    int64_t c = 0;
-    for (int t = 0; t < tiles; ++t) c += cnt[b * tiles + t];
-    count[b] = c;
-  }
 }
 
 template <int DT>
@@ -370,7 +386,7 @@ __global__ __launch_bounds__(kThreads) void finalize_bwd_cols_kernel(
     const typename Elem<DT>::type* __restrict__ gamma, int64_t H, int tiles, float2* __restrict__ col,
     float2* __restrict__ coef) {
   __shared__ float lds[kColSlices][2][kColFeat];
-  const int lane = threadIdx.x % kWave, slice = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kColFeat, slice = threadIdx.x / kColFeat;
   const int64_t h = static_cast<int64_t>(blockIdx.x) * kColFeat + lane;
   const int64_t b = blockIdx.y;
   const bool live = h < H;
