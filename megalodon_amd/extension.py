@@ -306,13 +306,6 @@ def _cut(t: torch.Tensor, nb: int, S: int) -> torch.Tensor:
     return t.reshape(*t.shape[:-1], nb, S).movedim(-2, 0).contiguous()
 
 
-def _head_to_tail(h: torch.Tensor) -> torch.Tensor:
-    """h[..., m] -> t[..., S-2-m] for m <= S-2, last entry 0 (its own inverse)."""
-    t = torch.zeros_like(h)
-    t[..., :-1] = h[..., :-1].flip(-1)
-    return t
-
-
 def _fftconv_long_fwd(x: torch.Tensor, k: torch.Tensor, blocks=None, head=None) -> torch.Tensor:
     """`blocks` = (nb, S) and `head` = the one-launch operator; the defaults are
     the library's limits and `fftconv_fwd` (tests pass others)."""
@@ -321,15 +314,15 @@ def _fftconv_long_fwd(x: torch.Tensor, k: torch.Tensor, blocks=None, head=None) 
     head = head or fftconv_fwd
     xb, kb = _cut(x, nb, S), _cut(k.float(), nb, S)
     xr, kr = xb.flip(-1), kb.flip(-1)
-    y = torch.zeros((nb, B, D, S), dtype=torch.float32, device=x.device)
+    y = torch.zeros((B, D, nb, S), dtype=torch.float32, device=x.device)  # the row, block by block
     for j in range(nb):
         n = nb - j
-        y[j:] += head(xb[:n].reshape(n * B, D, S), kb[j]).view(n, B, D, S)
+        y[:, :, j:] += head(xb[:n].reshape(n * B, D, S), kb[j]).view(n, B, D, S).permute(1, 2, 0, 3)
         n = nb - 1 - j
         if n > 0:
-            h = head(xr[:n].reshape(n * B, D, S), kr[j]).view(n, B, D, S)
-            y[j + 1:] += _head_to_tail(h.float())
-    return y.movedim(0, -2).reshape(B, D, nb * S)[..., :L].to(x.dtype)
+            h = head(xr[:n].reshape(n * B, D, S), kr[j]).view(n, B, D, S).permute(1, 2, 0, 3)
+            y[:, :, j + 1:, :S - 1] += h[..., :S - 1].flip(-1)  # tail[t] = h[S-2-t]
+    return y.view(B, D, nb * S)[..., :L].to(x.dtype)
 
 
 def _fftconv_long_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor, blocks=None,
@@ -339,21 +332,22 @@ def _fftconv_long_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor, bl
     head_bwd = head_bwd or (lambda g, a, c: fftconv_bwd(g, a, c, torch.float32))
     xb, kb, gb = _cut(x, nb, S), _cut(k.float(), nb, S), _cut(y_grad, nb, S)
     xr, kr = xb.flip(-1), kb.flip(-1)
-    dx = torch.zeros((nb, B, D, S), dtype=torch.float32, device=x.device)
-    dk = torch.zeros((nb, D, S), dtype=torch.float32, device=x.device)
+    dx = torch.zeros((B, D, nb, S), dtype=torch.float32, device=x.device)
+    dk = torch.zeros((D, nb, S), dtype=torch.float32, device=x.device)
     for j in range(nb):
         n = nb - j
         gx, gk = head_bwd(gb[j:].reshape(n * B, D, S), xb[:n].reshape(n * B, D, S), kb[j])
-        dx[:n] += gx.view(n, B, D, S)
-        dk[j] += gk
+        dx[:, :, :n] += gx.view(n, B, D, S).permute(1, 2, 0, 3)
+        dk[:, j] += gk
         n = nb - 1 - j
         if n > 0:
-            gh = _head_to_tail(gb[j + 1:]).reshape(n * B, D, S)
-            gx, gk = head_bwd(gh, xr[:n].reshape(n * B, D, S), kr[j])
-            dx[:n] += gx.view(n, B, D, S).float().flip(-1)
-            dk[j] += gk.flip(-1)
-    dx = dx.movedim(0, -2).reshape(B, D, nb * S)[..., :L].to(x.dtype)
-    return dx, dk.movedim(0, -2).reshape(D, nb * S)[..., :L].contiguous()
+            # gradient of h from the gradient of the tail: the same index reversal
+            gh = torch.zeros((n, B, D, S), dtype=gb.dtype, device=x.device)
+            gh[..., :S - 1] = gb[j + 1:, ..., :S - 1].flip(-1)
+            gx, gk = head_bwd(gh.reshape(n * B, D, S), xr[:n].reshape(n * B, D, S), kr[j])
+            dx[:, :, :n] += gx.view(n, B, D, S).permute(1, 2, 0, 3).flip(-1)
+            dk[:, j] += gk.flip(-1)
+    return dx.view(B, D, nb * S)[..., :L].to(x.dtype), dk.view(D, nb * S)[..., :L].contiguous()
 
 
 def fftconv_fwd(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
