@@ -81,3 +81,11 @@ def test_long_row_block_decomposition_with_the_oracle_as_one_launch(L, nb, S):
     dx, dk = ops._fftconv_long_bwd(dy, x, k, blocks=(nb, S), head_bwd=fftconv.fftconv_bwd)
     wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
     assert rel_err(dx, wdx) < 1e-6 and rel_err(dk, wdk) < 1e-6
+
+
+def test_long_row_block_sizes_fit_one_launch():
+    from megalodon_amd import extension as ops
+    top = ops.fftconv_max_length()
+    for L in (top + 1, top + 7, 40000, 2 * top, 2 * top + 1, 100003, 8 * top, 8 * top + 5):
+        nb, S = ops._long_blocks(L)
+        assert nb >= 2 and S % 8 == 0 and S <= top and nb * S >= L > (nb - 1) * S
