@@ -34,7 +34,11 @@ __device__ __forceinline__ cf qpow(float a, float phi, int64_t j) {
   const double fr = turns - rint(turns);  // in [-0.5, 0.5]
   float s, c;
   sincospif(2.0f * static_cast<float>(fr), &s, &c);
-  const float mag = static_cast<float>(exp(static_cast<double>(a) * jj));
+  // |q|^j = 2^t, t = a j log2(e): the integer part of t goes into the exponent
+  // exactly, the fraction (|f| <= 0.5, rounded to float: 3e-8) through exp2f
+  const double t = fmax(static_cast<double>(a) * jj * 1.4426950408889634, -1000.0);
+  const double ti = rint(t);
+  const float mag = ldexpf(exp2f(static_cast<float>(t - ti)), static_cast<int>(ti));
   return {mag * c, mag * s};
 }
 
@@ -353,6 +357,30 @@ __global__ __launch_bounds__(kThreads) void ema_weight_bwd_mfma_kernel(
   const bool live = n < N;
   const float la = live ? lq[n].x : 0.f, lphi = live ? lq[n].y : 0.f;
 
+  const int64_t rows = (L + 63) / 64;
+  const int64_t mtiles = (rows + 31) / 32;
+  auto load_tile = [&](int64_t mt, float (*raw)[8]) {
+    const int64_t j0 = (32 * mt + col) * 64 + 8 * g;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int64_t j = j0 + 16 * s;
+      if (j + 8 <= L) {
+        const float4 u = *reinterpret_cast<const float4*>(drow + j);
+        const float4 v = *reinterpret_cast<const float4*>(drow + j + 4);
+        raw[s][0] = u.x; raw[s][1] = u.y; raw[s][2] = u.z; raw[s][3] = u.w;
+        raw[s][4] = v.x; raw[s][5] = v.y; raw[s][6] = v.z; raw[s][7] = v.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) raw[s][e] = j + e < L ? drow[j + e] : 0.f;
+      }
+    }
+  };
+
+  // the first tile's loads fly while the operand below is built (a second
+  // tile in flight per wave costs the third workgroup per CU and runs 6 % slower)
+  float raw[4][8];
+  if (wave < mtiles) load_tile(wave, raw);
+
   // B operand: lane <-> column (kind, n), k = h = 16 s + 8 g + e; real and
   // imaginary parts are the two 32-column tiles.  It is the same for the four
   // waves: wave s builds k-step s and the operand lives in LDS (64 registers
@@ -382,29 +410,8 @@ __global__ __launch_bounds__(kThreads) void ema_weight_bwd_mfma_kernel(
   const cf st1 = qpow(la, lphi, 64), st2 = cmul(st1, st1), st3 = cmul(st2, st1);
   const cf st8 = qpow(la, lphi, 512);
 
-  const int64_t rows = (L + 63) / 64;
-  const int64_t mtiles = (rows + 31) / 32;
   cf s2{0.f, 0.f}, s1{0.f, 0.f};
 
-  auto load_tile = [&](int64_t mt, float (*raw)[8]) {
-    const int64_t j0 = (32 * mt + col) * 64 + 8 * g;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int64_t j = j0 + 16 * s;
-      if (j + 8 <= L) {
-        const float4 u = *reinterpret_cast<const float4*>(drow + j);
-        const float4 v = *reinterpret_cast<const float4*>(drow + j + 4);
-        raw[s][0] = u.x; raw[s][1] = u.y; raw[s][2] = u.z; raw[s][3] = u.w;
-        raw[s][4] = v.x; raw[s][5] = v.y; raw[s][6] = v.z; raw[s][7] = v.w;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) raw[s][e] = j + e < L ? drow[j + e] : 0.f;
-      }
-    }
-  };
-
-  float raw[4][8];
-  if (wave < mtiles) load_tile(wave, raw);
   for (int64_t mt = wave; mt < mtiles; mt += kThreads / kWave) {
     u32x4 ahi[4], alo[4];
 #pragma unroll
