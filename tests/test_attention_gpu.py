@@ -163,3 +163,50 @@ def test_standalone_softmax(shape, causal, dtype):
         assert torch.count_nonzero(torch.triu(y.float(), diagonal=L2 - L1 + 1)) == 0
     y.backward(dy.cuda())
     assert rel_err(xg.grad, xd.grad) <= TOL
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_swift_attention_module_matches_oracle(causal):
+    """SwiftAttention (the reference's fused_attention.py module) forward and
+    backward, bf16, against the float64 oracle; eval mode ignores its dropout."""
+    from megalodon_amd.modules import SwiftAttention
+    B, L, N, H1, H2 = 2, 300, 2, 64, 128
+    g = torch.Generator().manual_seed(11)
+    q, k = (torch.randn(B, L, N, H1, generator=g).bfloat16() / H1 ** 0.25 for _ in range(2))
+    v = torch.randn(B, L, N, H2, generator=g).bfloat16()
+    dy = torch.randn(B, L, N, H2, generator=g).bfloat16()
+    m = SwiftAttention(scale=0.5, dropout=0.3, use_causal_mask=causal).eval()
+    assert "dropout=0.3" in repr(m) and f"causal={causal}" in repr(m)
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    y = m(qc, kc, vc)
+    y.backward(dy.cuda())
+    want, _ = oa.chunk_attention_fwd(q, k, v, 0.5, causal)
+    wq, wk, wv = oa.chunk_attention_bwd(dy, q, k, v, 0.5, causal)
+    assert rel_err(y, want) <= 2e-2
+    assert rel_err(qc.grad, wq) <= 2e-2 and rel_err(kc.grad, wk) <= 2e-2 and rel_err(vc.grad, wv) <= 2e-2
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_softmax_module_matches_torch(causal):
+    """AttentionSoftmax (the reference's attention_softmax.py module) in eval
+    mode: rows of softmax with the bottom-right aligned causal mask, and the
+    gradient of a float64 softmax."""
+    from megalodon_amd.modules import AttentionSoftmax
+    B, N, L1, L2 = 2, 3, 70, 100
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(B, N, L1, L2, generator=g).bfloat16()   # the op takes 16-bit scores
+    dy = torch.randn(B, N, L1, L2, generator=g).bfloat16()
+    m = AttentionSoftmax(dropout=0.5, use_causal_mask=causal).eval()
+    xc = x.cuda().requires_grad_(True)
+    y = m(xc)
+    y.backward(dy.cuda())
+    x64 = x.double().requires_grad_(True)
+    s = x64
+    if causal:
+        r = torch.arange(L1).view(L1, 1)
+        c = torch.arange(L2).view(1, L2)
+        s = x64.masked_fill(c > r + (L2 - L1), float("-inf"))
+    want = torch.softmax(s, dim=-1)
+    want.backward(dy.double())
+    assert rel_err(y, want.detach()) <= 2e-2
+    assert rel_err(xc.grad, x64.grad) <= 2e-2
