@@ -31,6 +31,22 @@ class FFTConvFunc(torch.autograd.Function):
 fftconv = FFTConvFunc.apply
 
 
+def fused_fftconv_fwd(x: torch.Tensor, k: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(y, x_saved, k_saved) with the call pattern of the reference's
+    ``fused_fftconv_fwd(x, k) -> (y, x_f, k_f)`` (fused_ops/fftconv.py:79-93).
+    The two saved tensors are what ``fused_fftconv_bwd`` takes back; here they
+    are x and k themselves (the backward kernel recomputes the transforms on
+    chip), not complex spectra."""
+    return fftconv_fwd(x, k), x, k
+
+
+def fused_fftconv_bwd(y_grad: torch.Tensor, x_saved: torch.Tensor, k_saved: torch.Tensor,
+                      k_dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(dx, dk) from the pair ``fused_fftconv_fwd`` returned
+    (fused_ops/fftconv.py:96-106); dk has dtype ``k_dtype``."""
+    return fftconv_bwd(y_grad, x_saved, k_saved, k_dtype)
+
+
 class FFTConvResidualFunc(torch.autograd.Function):
     """``fftconv(x, k) + x * omega`` as one op: the two lines around the
     convolution in MultiHeadComplexEMA.forward

@@ -331,3 +331,14 @@ def test_cema_layer_at_twice_the_launch_length():
     assert rel_err(x.grad, xo.grad) <= 1e-4
     for n_, prm in m.named_parameters():
         assert rel_err(prm.grad, pr[n_].grad) <= 1e-4, n_
+
+
+def test_fused_fftconv_pair_has_the_reference_call_pattern():
+    """y, a, b = fused_fftconv_fwd(x, k); dx, dk = fused_fftconv_bwd(dy, a, b, k.dtype)."""
+    from megalodon_amd.fused_ops import fused_fftconv_bwd, fused_fftconv_fwd
+    x, k, dy = _data(2, 3, 5000, torch.float32, 8)
+    y, a, b = fused_fftconv_fwd(x.cuda(), k.cuda())
+    dx, dk = fused_fftconv_bwd(dy.cuda(), a, b, k.dtype)
+    wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
+    assert rel_err(y, fftconv.fftconv_fwd(x, k)) <= 1e-4
+    assert dk.dtype == k.dtype and rel_err(dx, wdx) <= 1e-4 and rel_err(dk, wdk) <= 1e-4
