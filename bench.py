@@ -106,10 +106,15 @@ def other_ops(torch, dev, synthetic):
                                               tio["gamma"], tio["beta"], tio["mask"], tG, 1e-5)
     ty, tcount, tmean, tvar, tcm, tcr = fwd()
     ms = dev_ms(fwd, 10)
-    other["timestep_norm_fwd"] = {"ms": ms, "GBps": 4 * tE / ms / 1e6, "frac_hbm": 4 * tE / ms / 1e6 / HBM_PEAK_GBS}
+    # GBps / frac_hbm price the op at its 4E (6E) algorithmic bytes; padding rows
+    # are written (zeros) but never read, so GBps_moved counts them once less
+    live = 1.0 - float(tio["mask"].float().mean()) if tio.get("mask") is not None else 1.0
+    other["timestep_norm_fwd"] = {"ms": ms, "GBps": 4 * tE / ms / 1e6, "frac_hbm": 4 * tE / ms / 1e6 / HBM_PEAK_GBS,
+                                  "unmasked_steps": live, "GBps_moved": (2 + 2 * live) * tE / ms / 1e6}
     ms = dev_ms(lambda: ops.group_timestep_norm_bwd(tio["dy"], tio["dmean"], tio["dvar"], tio["x"], tio["prev_mean"],
                                                     tcount, tcm, tcr, tio["gamma"], tio["mask"], tG), 10)
-    other["timestep_norm_bwd"] = {"ms": ms, "GBps": 6 * tE / ms / 1e6, "frac_hbm": 6 * tE / ms / 1e6 / HBM_PEAK_GBS}
+    other["timestep_norm_bwd"] = {"ms": ms, "GBps": 6 * tE / ms / 1e6, "frac_hbm": 6 * tE / ms / 1e6 / HBM_PEAK_GBS,
+                                  "unmasked_steps": live, "GBps_moved": (2 + 4 * live) * tE / ms / 1e6}
     del tio, ty, tcm, tcr
     aio = {k_: v_.to(dev) for k_, v_ in synthetic.attention_inputs(8, 4096, 4, 256, 2048, 1003).items()}
     pairs = 4096 * 4097 // 2

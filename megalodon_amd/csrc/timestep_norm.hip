@@ -493,11 +493,17 @@ void tsn_fwd_wave_kernel(const TsnParams p, int tiles) {
   const int64_t pass_stride = static_cast<int64_t>(RPW) * p.D;
   const int rows_left = p.L - t0 - lane / LPR;  // pass q is in range iff q * RPW < rows_left
   const typename Elem<DT>::type* xp = static_cast<const typename Elem<DT>::type*>(p.x) + off0;
+  // lane <-> time step for the scan; bit r of `live` says that row r of the
+  // tile is a real, unmasked step.  Padding rows are never read: their
+  // output is zero and they leave the statistics alone.
+  const int t = t0 + lane;
+  const bool valid = t < p.L && (p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0);
+  const unsigned long long live = __ballot(valid);
   uint4 xv[P];
 #pragma unroll
   for (int q = 0; q < P; ++q) {
     xv[q] = make_uint4(0, 0, 0, 0);
-    if (q * RPW < rows_left && col_ok) xv[q] = *reinterpret_cast<const uint4*>(xp + q * pass_stride);
+    if (((live >> (q * RPW + lane / LPR)) & 1) && col_ok) xv[q] = *reinterpret_cast<const uint4*>(xp + q * pass_stride);
   }
   uint4 gmv = make_uint4(0, 0, 0, 0), btv = make_uint4(0, 0, 0, 0);
   if (col_ok) {
@@ -507,8 +513,6 @@ void tsn_fwd_wave_kernel(const TsnParams p, int tiles) {
   const int64_t chain64 = static_cast<int64_t>(b) * p.G + g;
   const Wel prior{static_cast<float>(p.prev_count[b]), ldT<DT>(p.prev_mean, chain64),
                   ldT<DT>(p.prev_var, chain64)};
-  const int t = t0 + lane;
-  const bool valid = t < p.L && (p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0);
 #pragma unroll
   for (int q = 0; q < P; ++q) {
     const int r = q * RPW + lane / LPR;
@@ -740,6 +744,13 @@ void tsn_bwd_kernel(const TsnParams p) {
 
   // everything the tile needs from memory is requested up front: the rows of x
   // and dy, gamma, the saved statistics and the chain's boundary values
+  // bit r of `live`: row r of the tile is a real, unmasked step.  Padding rows
+  // are never read (dx = 0 there and they add nothing to any sum).
+  unsigned long long live;
+  {
+    const int t = t0 + lane;
+    live = __ballot(t < p.L && (p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0));
+  }
   uint4 xv[P], dv[P];
 #pragma unroll
   for (int q = 0; q < P; ++q) {
@@ -747,7 +758,7 @@ void tsn_bwd_kernel(const TsnParams p) {
     const int t = t0 + r;
     xv[q] = make_uint4(0, 0, 0, 0);
     dv[q] = make_uint4(0, 0, 0, 0);
-    if (t < p.L && col_ok) {
+    if (((live >> r) & 1) && col_ok) {
       const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
       xv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.x) + off);
       dv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.dy) + off);
