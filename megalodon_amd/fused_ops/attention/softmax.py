@@ -1,28 +1,19 @@
-"""Standalone attention softmax autograd op (mirror of
-megalodon/modules/fused_ops/attention/softmax.py:9-35)."""
-from typing import Tuple
-
-import torch
-from torch.autograd.function import FunctionCtx
-
-from ... import extension as megalodon_ops
+"""`attention_softmax(x, dropout, use_causal_mask, training) -> y`: row softmax
+of attention scores with the bottom-right aligned causal mask and DropKey, as
+the op of megalodon/modules/fused_ops/attention/softmax.py:9-35.  Backward
+needs y only: a dropped key has probability 0 and so no gradient."""
+from ... import extension as ops
+from .._autograd import fused_op
 
 
-class AttentionSoftmaxFunc(torch.autograd.Function):
-
-    @staticmethod
-    def forward(ctx: FunctionCtx, x: torch.Tensor, dropout: float = 0.0, use_causal_mask: bool = True,
-                training: bool = True) -> torch.Tensor:
-        y = megalodon_ops.attention_softmax_fwd(x, dropout if training else 0.0, use_causal_mask)
-        ctx.save_for_backward(y)
-        ctx.use_causal_mask = use_causal_mask
-        return y
-
-    @staticmethod
-    def backward(ctx: FunctionCtx, y_grad: torch.Tensor) -> Tuple[torch.Tensor, None, None, None]:
-        y, = ctx.saved_tensors
-        x_grad = megalodon_ops.attention_softmax_bwd(y_grad, y, ctx.use_causal_mask)
-        return x_grad, None, None, None
+def _run(x, dropout=0.0, use_causal_mask=True, training=True):
+    y = ops.attention_softmax_fwd(x, dropout if training else 0.0, use_causal_mask)
+    return y, (y,), use_causal_mask
 
 
+def _grad(use_causal_mask, saved, y_grad):
+    return ops.attention_softmax_bwd(y_grad, saved[0], use_causal_mask), None, None, None
+
+
+AttentionSoftmaxFunc = fused_op("AttentionSoftmaxFunc", _run, _grad, doc=__doc__)
 attention_softmax = AttentionSoftmaxFunc.apply

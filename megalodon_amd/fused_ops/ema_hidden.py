@@ -1,35 +1,19 @@
-"""`ema_hidden` autograd op (mirror of megalodon/modules/fused_ops/ema_hidden.py:8-33)."""
-from typing import Optional, Tuple
-
-import torch
-from torch.autograd.function import FunctionCtx
-
-from .. import extension as megalodon_ops
+"""`ema_hidden(x, p, q, hx) -> h`: the EMA state after the last step of x (and
+of a carried state `hx`), as the op of
+megalodon/modules/fused_ops/ema_hidden.py:8-33."""
+from .. import extension as ops
+from ._autograd import fused_op
 
 
-class EMAHiddenFunc(torch.autograd.Function):
-
-    @staticmethod
-    def forward(
-        ctx: FunctionCtx,
-        x: torch.Tensor,
-        p: torch.Tensor,
-        q: torch.Tensor,
-        hx: Optional[torch.Tensor],
-    ) -> torch.Tensor:
-        log_q = q.log()
-        h, v = megalodon_ops.ema_hidden_fwd(x, p, log_q, hx)
-        ctx.save_for_backward(x, p, log_q, hx, v)
-        return h
-
-    @staticmethod
-    def backward(
-        ctx: FunctionCtx,
-        h_grad: torch.Tensor,
-    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
-        x, p, log_q, hx, v = ctx.saved_tensors
-        x_grad, p_grad, q_grad, hx_grad = megalodon_ops.ema_hidden_bwd(h_grad, x, p, log_q, hx, v)
-        return x_grad, p_grad, q_grad, hx_grad
+def _run(x, p, q, hx):
+    log_q = q.log()
+    h, vander = ops.ema_hidden_fwd(x, p, log_q, hx)
+    return h, (x, p, log_q, hx, vander), None
 
 
+def _grad(_, saved, h_grad):
+    return ops.ema_hidden_bwd(h_grad, *saved)  # (dx, dp, dq, dhx)
+
+
+EMAHiddenFunc = fused_op("EMAHiddenFunc", _run, _grad, doc=__doc__)
 ema_hidden = EMAHiddenFunc.apply

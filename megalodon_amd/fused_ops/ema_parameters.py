@@ -1,38 +1,21 @@
-"""`ema_parameters` autograd op (mirror of megalodon/modules/fused_ops/ema_parameters.py:8-35)."""
-from typing import Optional, Tuple
-
-import torch
-from torch.autograd.function import FunctionCtx
-
-from .. import extension as megalodon_ops
-
-
-class EMAParametersFunc(torch.autograd.Function):
-
-    @staticmethod
-    def forward(
-        ctx: FunctionCtx,
-        p: torch.Tensor,
-        q: torch.Tensor,
-        gamma: torch.Tensor,
-        hx: Optional[torch.Tensor],
-        length: int,
-    ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-        log_q = q.log()
-        weight, bias, vander = megalodon_ops.ema_parameters_fwd(p, log_q, gamma, hx, length)
-        ctx.save_for_backward(p, log_q, gamma, hx, vander)
-        return weight, bias
-
-    @staticmethod
-    def backward(
-        ctx: FunctionCtx,
-        weight_grad: torch.Tensor,
-        bias_grad: Optional[torch.Tensor],
-    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor], None]:
-        p, log_q, gamma, hx, vander = ctx.saved_tensors
-        p_grad, q_grad, gamma_grad, hx_grad = megalodon_ops.ema_parameters_bwd(
-            weight_grad, bias_grad, p, log_q, gamma, hx, vander)
-        return p_grad, q_grad, gamma_grad, hx_grad, None
+"""`ema_parameters(p, q, gamma, hx, length) -> (weight, bias)`: the CEMA
+convolution kernel and, with a carried state `hx`, its bias rows, as the op of
+megalodon/modules/fused_ops/ema_parameters.py:8-35.  The entry points work on
+log q; the gradient comes back with respect to q itself."""
+from .. import extension as ops
+from ._autograd import fused_op
 
 
+def _run(p, q, gamma, hx, length):
+    log_q = q.log()
+    weight, bias, vander = ops.ema_parameters_fwd(p, log_q, gamma, hx, length)
+    return (weight, bias), (p, log_q, gamma, hx, vander), None
+
+
+def _grad(_, saved, weight_grad, bias_grad):
+    # (dp, dq, dgamma, dhx) + nothing for `length`
+    return (*ops.ema_parameters_bwd(weight_grad, bias_grad, *saved), None)
+
+
+EMAParametersFunc = fused_op("EMAParametersFunc", _run, _grad, doc=__doc__)
 ema_parameters = EMAParametersFunc.apply

@@ -11,25 +11,20 @@ from torch import nn
 
 from ..fused_ops import cema_kernel, ema_hidden, ema_parameters, fftconv_residual
 
-_r2c = torch.view_as_complex
 
-
+@torch.no_grad()
 def _reset_parameters(alpha, delta, theta, gamma, omega, embed_dim):
-    # delta & alpha
-    nn.init.normal_(alpha, mean=0.0, std=0.2)
-    nn.init.normal_(delta, mean=0.0, std=0.2)
-    idx = torch.randperm(embed_dim)
-    # theta: logit of permuted log-spaced frequencies exp(-i ln(D)/D), i = 1..D
-    freqs = math.log(embed_dim) / embed_dim
-    freqs = torch.exp(torch.arange(1, embed_dim + 1) * -freqs)
-    freqs = freqs[idx].to(theta).view(embed_dim, 1, 1)
-    freqs = torch.log(freqs / (1.0 - freqs))
-    with torch.no_grad():
-        theta.copy_(freqs)
-    # gamma (imaginary part zero at init), omega
-    nn.init.normal_(gamma, mean=0.0, std=1.0)
-    with torch.no_grad():
-        gamma[:, :, 1] = 0.
+    """Initial values as in the reference (:64-98): narrow normal logits for the
+    decay pair; base frequencies sigmoid(theta) = D^(-i/D), i = 1..D in random
+    order (log-spaced between 1/D and 1); real N(0, 1) mixing weights; a
+    truncated normal skip weight."""
+    alpha.normal_(0.0, 0.2)
+    delta.normal_(0.0, 0.2)
+    order = (torch.randperm(embed_dim) + 1).to(torch.float32)
+    base = torch.exp(-order * (math.log(embed_dim) / embed_dim))
+    theta.copy_(torch.logit(base).view(embed_dim, 1, 1))
+    gamma[..., 0].normal_(0.0, 1.0)
+    gamma[..., 1].zero_()
     nn.init.trunc_normal_(omega, mean=0.0, std=0.25, a=-1.0, b=1.0)
 
 
@@ -55,20 +50,17 @@ class MultiHeadComplexEMA(nn.Module):
         _reset_parameters(self.alpha, self.delta, self.theta, self.gamma, self.omega, self.embed_dim)
 
     def _calc_coeffs(self):
+        """(p, q, gamma_hat) in float32: p = sigmoid(alpha) (D, N, 1);
+        q = (1 - p sigmoid(delta)) exp(i n base), n = 1..N, with base =
+        sigmoid(theta) 2 pi / N (D, N, 1) complex; gamma_hat = gamma / sqrt(N)
+        (D, N) complex (:100-117)."""
         self._coeffs = None
-        # D x 1 x 1
-        theta = torch.sigmoid(self.theta.float()) * (2 * math.pi / self.ndim)
-        # 1 x N
-        wavelets = torch.arange(1, self.ndim + 1, dtype=theta.dtype, device=theta.device).view(1, self.ndim)
-        # D x N x 1
-        theta = wavelets.unsqueeze(2) * theta
-        alpha = torch.sigmoid(self.alpha.float())
-        delta = torch.sigmoid(self.delta.float())
-        p = alpha
-        q = torch.polar(1.0 - alpha * delta, theta)
-        # D x N
-        gamma = _r2c(self.gamma.float()) * self.scale
-        return p, q, gamma
+        n_modes = self.ndim
+        p = torch.sigmoid(self.alpha.float())
+        base = torch.sigmoid(self.theta.float()) * (2 * math.pi / n_modes)
+        harmonics = torch.arange(1, n_modes + 1, dtype=base.dtype, device=base.device).view(1, n_modes, 1)
+        q = torch.polar(1.0 - p * torch.sigmoid(self.delta.float()), base * harmonics)
+        return p, q, torch.view_as_complex(self.gamma.float()) * self.scale
 
     def coeffs(self):
         if self.training:

@@ -24,19 +24,21 @@ class RotaryEmbedding(nn.Module):
         self.freqs_cis: Optional[torch.Tensor] = None
 
     @torch.no_grad()
-    def _precompute_until(self, max_positions: int) -> torch.Tensor:
-        assert self.max_positions <= max_positions
-        self.max_positions = max_positions
-        t = torch.arange(max_positions, dtype=torch.float32, device=self.freqs.device)
+    def _table(self, positions: int) -> torch.Tensor:
+        """exp(i t f_j) for t < positions: complex64, (positions, dim / 2)."""
+        t = torch.arange(positions, dtype=torch.float32, device=self.freqs.device)
         angles = torch.outer(t, self.freqs.float())
-        return torch.polar(torch.ones_like(angles), angles)   # complex64, positions x dim / 2
+        return torch.polar(torch.ones_like(angles), angles)
 
     def get_freqs_cis(self, start: int, end: int) -> torch.Tensor:
-        if self.freqs_cis is None:
-            self.freqs_cis = self._precompute_until(self.max_positions)
-        if end > self.freqs_cis.shape[0]:
-            warnings.warn('Extending rotary range from {} to {}'.format(self.max_positions, end))
-            self.freqs_cis = self._precompute_until(end)
+        """Rows start .. end-1 of the table; the table grows (with a warning, as
+        in the reference :36-42) when `end` lies beyond it."""
+        have = 0 if self.freqs_cis is None else self.freqs_cis.shape[0]
+        if end > have:
+            if end > self.max_positions:
+                warnings.warn(f"Extending rotary range from {self.max_positions} to {end}")
+                self.max_positions = end
+            self.freqs_cis = self._table(self.max_positions)
         return self.freqs_cis[start:end]
 
     def forward(self, xq, xk, start: int):
@@ -44,4 +46,4 @@ class RotaryEmbedding(nn.Module):
         return apply_rotary_emb(xq, xk, freqs_cis=freqs_cis, backward=False)
 
     def extra_repr(self) -> str:
-        return 'dim={}, max positions={}, base={:.1f}'.format(self.embed_dim, self.max_positions, self.base)
+        return f"dim={self.embed_dim}, max positions={self.max_positions}, base={self.base:.1f}"
