@@ -201,3 +201,33 @@ def test_non_group_operator(mask):
     want = tn.group_timestep_norm_bwd_autograd(dy, dmean, dvar, x, pc, pm, pv, gamma, beta, m, H, 1e-5)
     for name, a, b_ in zip(["dx", "dprev_mean", "dprev_var", "dgamma", "dbeta"], got, want):
         assert rel_err(a, b_) <= 1e-4, name
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mask", ["trailing", "holes"])
+def test_padding_rows_are_never_read(mask, dtype):
+    """NaN / Inf in x and dy at masked steps: every output agrees with a run with
+    zeros there (masked steps have y = dx = 0, leave the statistics alone and
+    add nothing to the parameter gradients).  Not bit for bit: the order in
+    which a tile combines its predecessors' records varies from run to run."""
+    B, L, H, G = 3, 333, 256, 4
+    x, pc, pm, pv, gamma, beta, m, dy, dmean, dvar = _case(B, L, H, G, 21, dtype, 2, mask)
+    clean_x, clean_dy = x.masked_fill(m.unsqueeze(-1), 0.0), dy.masked_fill(m.unsqueeze(-1), 0.0)
+    junk = torch.where(torch.arange(H) % 2 == 0, float("nan"), float("inf")).to(dtype)
+    dirty_x = torch.where(m.unsqueeze(-1), junk, x)
+    dirty_dy = torch.where(m.unsqueeze(-1), -junk, dy)
+    outs = []
+    for xx, gg in ((clean_x, clean_dy), (dirty_x, dirty_dy)):
+        cx, cpc, cpm, cpv, cg, cb, cm = _cuda(xx, pc, pm, pv, gamma, beta, m)
+        fwd = ops.group_timestep_norm_fwd(cx, cpc, cpm, cpv, cg, cb, cm, G, 1e-5)
+        y, count, mean, var, cummean, cumrstd = fwd
+        bwd = ops.group_timestep_norm_bwd(gg.cuda(), dmean.cuda(), dvar.cuda(), cx, cpm, count, cummean, cumrstd,
+                                          cg, cm, G)
+        outs.append([t.cpu() for t in (*fwd, *bwd)])
+    for a, b_ in zip(*outs):
+        assert torch.isfinite(b_.float()).all()
+        if a.dtype == torch.int64:
+            assert torch.equal(a, b_)
+        else:
+            assert rel_err(b_, a.double()) <= (1e-5 if dtype == torch.float32 else 1e-2)
+    assert (outs[1][0][m] == 0).all() and (outs[1][6][m] == 0).all()   # y and dx at masked steps
