@@ -349,13 +349,20 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
 
   // everything the tile needs from memory is requested up front: the rows, the
   // affine parameters of the last phase and the chain's prior state
+  // bit r of `live`: row r of the tile is a real, unmasked step; padding rows
+  // are never read
+  unsigned long long live;
+  {
+    const int t = t0 + lane;
+    live = __ballot(t < p.L && (p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0));
+  }
   uint4 xv[P];
 #pragma unroll
   for (int q = 0; q < P; ++q) {
     const int r = q * RPP + wave * RPW + lane / LPR;
     const int t = t0 + r;
     xv[q] = make_uint4(0, 0, 0, 0);
-    if (t < p.L && col_ok) {
+    if (((live >> r) & 1) && col_ok) {
       const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
       xv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.x) + off);
     }
