@@ -136,3 +136,22 @@ def test_argument_errors():
         ops.group_sequence_norm_fwd(x, w, w, torch.zeros(2, 7, dtype=torch.bool, device="cuda"), 3, 1e-5)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         ops.group_sequence_norm_fwd(x.cpu(), w.cpu(), w.cpu(), None, 3, 1e-5)
+
+
+@pytest.mark.parametrize("length_last", [False, True])
+@pytest.mark.parametrize("groups", [4, None])
+def test_autograd_wrapper_matches_oracle_autograd(groups, length_last):
+    """fused_ops.sequence_norm through torch.autograd against autograd over the
+    float64 oracle forward: y and the gradients of x, gamma and beta."""
+    from megalodon_amd.fused_ops import sequence_norm
+    B, L, H = 2, 300, 64
+    x, dy, gamma, beta, m = _case(B, L, H, torch.float32, 5, "holes", length_last)
+    cx, cg, cb = (t.cuda().requires_grad_(True) for t in (x, gamma, beta))
+    y = sequence_norm(cx, cg, cb, m.cuda(), groups, 1e-5, length_last)
+    y.backward(dy.cuda())
+    x64, g64, b64 = (t.double().requires_grad_(True) for t in (x, gamma, beta))
+    want, *_ = sn.group_sequence_norm_fwd(x64, g64, b64, m, H if groups is None else groups, 1e-5, length_last)
+    want.backward(dy.double())
+    assert rel_err(y, want.detach()) <= 1e-4
+    for got, ref in ((cx.grad, x64.grad), (cg.grad, g64.grad), (cb.grad, b64.grad)):
+        assert rel_err(got, ref) <= 1e-4
