@@ -109,20 +109,29 @@ int mega_cema_coeffs_bwd(const float* dp, const float* dq, const float* dgamma_h
  *   x, y (B, D, L) of `dtype` (MEGA_F32 / MEGA_BF16 / MEGA_F16);
  *   k (D, L) float32 in the TIME domain (the reference passes rfft(k); here
  *   the transform of k happens inside the kernel and nothing is saved).
- *   float32 rows: arithmetic is float32 throughout; y is rounded once on
- *   store.  bfloat16 / float16 rows with 2048 < L, L % 8 == 0 and 16-byte
- *   aligned x, k, y: the DFT stages run on the matrix cores (fp16 operands,
- *   fp32 accumulation, fp16 between stages, rows pre-scaled by a power of
- *   two), twiddles, the spectral product and all sums in float32; measured
- *   error against a float64 convolution <= 4e-3 of the largest output
- *   (the bfloat16 rounding of y alone is 2e-3).  Other 16-bit rows take the
- *   float32 path.
+ *   Arithmetic is float32 throughout for every dtype (16-bit rows are
+ *   widened on load as the reference does, fftconv.py:37-44; y is rounded
+ *   once on store): error against a float64 convolution ~1e-6 of the largest
+ *   output before that rounding.
+ *   Opt-in: with MEGA_FFTCONV_F16_STAGES set in the environment (to anything
+ *   but "0"; read per call), bfloat16 / float16 rows with 2048 < L,
+ *   L % 8 == 0 and 16-byte aligned x, k, y run their DFT stages on the matrix
+ *   cores (fp16 operands, fp32 accumulation, fp16 between stages, rows
+ *   pre-scaled by a power of two; twiddles, the spectral product and all sums
+ *   in float32): about 3x faster, measured error <= 4e-3 of the largest output
+ *   (y, dx) and 1.1e-3 (dk), i.e. inside the 16-bit bar but not the float32
+ *   one.
  *   L <= mega_fftconv_max_length() (32768); longer rows return
  *   MEGA_ERR_UNSUPPORTED.
- *   The float32 path's first call for a transform size on a device allocates
- *   the twiddle tables and a per-workgroup scratch (kept until process exit)
- *   and synchronises `stream` once; the matrix-core path allocates nothing.
+ *   The float32 engine needs twiddle tables (one per device and transform
+ *   size) and a per-workgroup scratch block (one per device, transform size
+ *   and stream, so launches on different streams never share slots); both are
+ *   kept until process exit.  mega_fftconv_prepare(L, stream) makes them ahead
+ *   of time (it allocates and synchronises `stream` once; not capturable);
+ *   after it, the convolution entry points on that stream only enqueue.
+ *   Without it the first call for a size / stream does the same work itself.
  * ---------------------------------------------------------------------- */
+int mega_fftconv_prepare(int64_t L, void* stream);
 int mega_fftconv_max_length(void);
 int mega_fftconv_fwd(const void* x, int dtype, const float* k, int64_t B,
                      int64_t D, int64_t L, void* y, void* stream);
@@ -261,7 +270,9 @@ int mega_attention_bwd(const void* dy, const void* q, const void* k, const void*
  * pass and takes the spectrum of k (fftconv_fwd(x, k_f) -> (y, x_f),
  * fftconv_bwd(dy, x_f, k_f, k_dtype), megalodon/modules/fused_ops/fftconv.py:
  * 21-28,62-75, csrc/ops/fftconv_kernel.cu:34-164).  This pair does the same for
- * the matrix-core path: the forward also writes the spectra of x and of k (an
+ * the matrix-core path (the fp16-stage engine, opt-in through
+ * MEGA_FFTCONV_F16_STAGES as described at mega_fftconv_fwd; without it
+ * mega_fftconv_spectrum_bytes returns 0): the forward also writes the spectra of x and of k (an
  * opaque fp16 layout with the rows' scales, 16-byte aligned: spec_x takes
  * mega_fftconv_spectrum_bytes(dtype, B, D, L) bytes, spec_k, which depends on
  * the channel only, mega_fftconv_spectrum_bytes(dtype, 1, D, L)), the backward

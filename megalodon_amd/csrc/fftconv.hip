@@ -26,18 +26,27 @@ using namespace fftc;
 
 // ------------------------------ tables --------------------------------------
 constexpr int kMaxDevices = 16;
+struct StreamScratch {
+  hipStream_t stream;
+  float* ptr;
+};
 struct TableCache {
   c32* ptr[kMaxDevices][4] = {};
-  float* scratch[kMaxDevices][4] = {};
   int slots[kMaxDevices][4] = {};
+  // one scratch block per stream that has run this transform size: launches
+  // on different streams of a device may overlap, and a workgroup's slot is
+  // picked by its index alone
+  std::vector<StreamScratch> scratch[kMaxDevices][4];
   std::mutex mu;
 };
 TableCache g_tables;
 
-// Twiddle tables and the per-workgroup scratch slots live for the life of the
-// process (one allocation per device and transform size, made on first use;
-// that first call therefore cannot be captured into a graph).  Scratch is
-// 2*M floats per resident workgroup (at most 2 workgroups per CU).
+// Twiddle tables (one per device and transform size) and the per-workgroup
+// scratch slots (one block per device, transform size and stream) live for the
+// life of the process.  They are made on first use, or ahead of time by
+// mega_fftconv_prepare; making them allocates and, for the tables,
+// synchronises the stream once, so that call cannot be captured into a graph.
+// Scratch is 2*M floats per resident workgroup (at most 2 workgroups per CU).
 template <int LOGM>
 int get_tables(hipStream_t stream, const c32** out, float** scratch, int* slots) {
   using C = Cfg<LOGM>;
@@ -50,11 +59,7 @@ int get_tables(hipStream_t stream, const c32** out, float** scratch, int* slots)
     hipDeviceProp_t prop;
     MEGA_CHECK_HIP(hipGetDeviceProperties(&prop, dev));
     const int per_cu = LOGM == 14 ? 1 : 2;
-    const int nslots = prop.multiProcessorCount * per_cu;
-    float* sc = nullptr;
-    MEGA_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&sc), sizeof(float) * 2 * C::M * nslots));
-    g_tables.scratch[dev][LOGM - 11] = sc;
-    g_tables.slots[dev][LOGM - 11] = nslots;
+    g_tables.slots[dev][LOGM - 11] = prop.multiProcessorCount * per_cu;
     c32* p = nullptr;
     MEGA_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&p), sizeof(c32) * C::TABLE));
     std::vector<c32> host(C::TABLE);
@@ -67,9 +72,17 @@ int get_tables(hipStream_t stream, const c32** out, float** scratch, int* slots)
     }
     slot = p;
   }
+  const int nslots = g_tables.slots[dev][LOGM - 11];
+  float* sc = nullptr;
+  for (const StreamScratch& s : g_tables.scratch[dev][LOGM - 11])
+    if (s.stream == stream) sc = s.ptr;
+  if (sc == nullptr) {
+    MEGA_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&sc), sizeof(float) * 2 * C::M * nslots));
+    g_tables.scratch[dev][LOGM - 11].push_back(StreamScratch{stream, sc});
+  }
   *out = slot;
-  *scratch = g_tables.scratch[dev][LOGM - 11];
-  *slots = g_tables.slots[dev][LOGM - 11];
+  *scratch = sc;
+  *slots = nslots;
   return MEGA_OK;
 }
 
@@ -425,6 +438,15 @@ __global__ __launch_bounds__(kDirectThreads) void direct_conv_kernel(
   }
 }
 
+// The transforms are float32 unless MEGA_FFTCONV_F16_STAGES is set (to anything
+// but "0") in the environment: then 16-bit rows the matrix-core engine can take
+// run its fp16-operand DFT stages (3x faster, error ~1e-3 of the largest
+// output instead of ~1e-6).  Read per call.
+bool f16_stages_enabled() {
+  const char* v = getenv("MEGA_FFTCONV_F16_STAGES");
+  return v != nullptr && !(v[0] == '0' && v[1] == 0);
+}
+
 template <int DT, int MODE>
 int launch_conv(const void* a, const void* b, void* out, int64_t B, int64_t D, int64_t L, int flip,
                 const float* omega, hipStream_t stream) {
@@ -440,8 +462,8 @@ int launch_conv(const void* a, const void* b, void* out, int64_t B, int64_t D, i
     MEGA_CHECK_LAUNCH();
     return MEGA_OK;
   }
-  // 16-bit rows of 16385..32768 samples run their DFT stages on the matrix cores
-  if (fftm::applicable(DT, L, a, b, out) && getenv("MEGA_FFTCONV_VALU") == nullptr)
+  // opt-in: 16-bit rows run their DFT stages on the matrix cores with fp16 operands
+  if (f16_stages_enabled() && fftm::applicable(DT, L, a, b, out))
     return fftm::launch_conv(DT, MODE, a, b, out, B, D, L, flip, omega, stream);
   if (L <= 4096) return launch_fft<11, DT, MODE>(a, b, out, B, D, L, flip, omega, stream);
   if (L <= 8192) return launch_fft<12, DT, MODE>(a, b, out, B, D, L, flip, omega, stream);
@@ -475,6 +497,22 @@ using namespace mega;
 
 extern "C" int mega_fftconv_max_length(void) { return static_cast<int>(kMaxL); }
 
+extern "C" int mega_fftconv_prepare(int64_t L, void* stream) {
+  MEGA_CHECK_ARG(L >= 0, "mega_fftconv_prepare: negative size");
+  if (L > kMaxL)
+    return set_error(MEGA_ERR_UNSUPPORTED, "mega_fftconv_prepare: L=%lld exceeds the supported %lld",
+                     (long long)L, (long long)kMaxL);
+  if (L <= kDirectMaxL) return MEGA_OK;  // the time-domain kernel needs neither tables nor scratch
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const c32* tab = nullptr;
+  float* scratch = nullptr;
+  int slots = 0;
+  if (L <= 4096) return get_tables<11>(s, &tab, &scratch, &slots);
+  if (L <= 8192) return get_tables<12>(s, &tab, &scratch, &slots);
+  if (L <= 16384) return get_tables<13>(s, &tab, &scratch, &slots);
+  return get_tables<14>(s, &tab, &scratch, &slots);
+}
+
 namespace {
 int fftconv_fwd_impl(const char* who, const void* x, int dtype, const float* k, const float* omega,
                      int64_t B, int64_t D, int64_t L, void* y, void* stream) {
@@ -506,7 +544,7 @@ int fftconv_bwd_impl(const char* who, const void* dy, const void* x, int dtype, 
     return MEGA_OK;
   }
   if (fftm::applicable(dtype, L, dy, x, dx) && reinterpret_cast<uintptr_t>(k) % 16 == 0 &&
-      reinterpret_cast<uintptr_t>(dk) % 16 == 0 && getenv("MEGA_FFTCONV_VALU") == nullptr &&
+      reinterpret_cast<uintptr_t>(dk) % 16 == 0 && f16_stages_enabled() &&
       getenv("MEGA_FFTCONV_SPLIT_BWD") == nullptr)
     return fftm::launch_backward(dtype, dy, x, k, dx, dk, B, D, L, omega, s);
   int rc = dispatch_conv<0>(dtype, dy, k, dx, B, D, L, 1, omega, s);
@@ -543,7 +581,7 @@ extern "C" int mega_fftconv_residual_bwd(const void* dy, const void* x, int dtyp
 
 // ---- forward that keeps the spectra of x and k, backward that uses them ----------
 extern "C" int64_t mega_fftconv_spectrum_bytes(int dtype, int64_t B, int64_t D, int64_t L) {
-  if (B <= 0 || D <= 0 || L <= 0 || getenv("MEGA_FFTCONV_VALU") != nullptr) return 0;
+  if (B <= 0 || D <= 0 || L <= 0 || !f16_stages_enabled()) return 0;
   return fftm::spectrum_bytes(dtype, B, D, L);
 }
 

@@ -442,6 +442,15 @@ def fftconv_residual_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
     return dx, dk, dk[:, 0].clone()
 
 
+def fftconv_prepare(L: int, device=None) -> None:
+    """Make the float32 convolution engine's tables and the current stream's
+    scratch block for rows of L samples ahead of time (allocates and
+    synchronises once); later convolution calls on that stream only enqueue."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    with torch.cuda.device(dev):
+        _lib.call("mega_fftconv_prepare", _lib.i64(min(int(L), fftconv_max_length())), _lib.stream_ptr(dev))
+
+
 def fftconv_spectrum_bytes(dtype: torch.dtype, B: int, D: int, L: int) -> int:
     """Bytes of one saved-spectrum buffer for this shape, 0 when the shape does
     not take the saved-spectrum path."""
@@ -485,6 +494,9 @@ def fftconv_residual_bwd_saved(y_grad: torch.Tensor, spec_x: torch.Tensor, spec_
             or spec_k.numel() != fftconv_spectrum_bytes(y_grad.dtype, 1, D, L)):
         raise RuntimeError("fftconv_bwd: the saved spectra do not belong to this shape")
     dy = y_grad.contiguous()
+    if dy.data_ptr() % 16 != 0:
+        # a contiguous view at an odd storage offset: the kernel's 16-byte loads need an aligned row
+        dy = dy.clone(memory_format=torch.contiguous_format)
     wc = omega.reshape(-1).contiguous().float()
     dx = torch.empty_like(dy)
     dk = torch.empty((D, L), dtype=torch.float32, device=dev)

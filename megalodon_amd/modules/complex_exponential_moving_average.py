@@ -77,6 +77,10 @@ class MultiHeadComplexEMA(nn.Module):
     ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
         # B x D x L
         bsz, _, seq_len = x.size()
+        if self.training:
+            # the reference's training forward goes through _calc_coeffs(), which drops the
+            # coefficients cached for evaluation (:100-101,119-125); every branch below does the same
+            self._coeffs = None
         if hx is None and not compute_last_state and self.alpha.is_cuda:
             # no carried state: coefficients and kernel as one autograd node
             # (two launches per direction instead of the coefficient graph)

@@ -123,3 +123,35 @@ def test_layer_split_sequence_equals_whole(dtype, L1, L2):
     p, q, gamma = layer.coeffs()
     want = cema.ema_hidden_fwd(x.cpu(), p.cpu(), q.cpu().log(), None)
     assert rel_err(hw, want) <= TOL
+
+
+def test_cached_coefficients_are_dropped_by_a_training_forward():
+    """eval decode -> parameter update + training forward -> eval decode: the
+    second decode must use the new parameters (the reference's training forward
+    resets the cache through _calc_coeffs, complex_exponential_moving_average.py:100-101,119-125)."""
+    torch.manual_seed(11)
+    D, N, B, L = 5, 16, 2, 40
+    layer = MultiHeadComplexEMA(D, N).cuda()
+    x = torch.randn(B, D, L).cuda()
+    h0 = torch.randn(B, D, N, dtype=torch.complex64).cuda()
+    layer.eval()
+    with torch.no_grad():
+        layer(x, h0, True)                      # fills the evaluation cache
+    assert layer._coeffs is not None
+    layer.train()
+    with torch.no_grad():
+        layer.alpha.add_(0.7)
+        layer.delta.sub_(0.4)
+    layer(x, None, False)[0].sum().backward()   # the no-state training branch
+    assert layer._coeffs is None
+    layer.eval()
+    with torch.no_grad():
+        y, h = layer(x, h0, True)
+    pr = {n_: v.detach().cpu().double() for n_, v in layer.named_parameters()}
+    p, q, g = cema.calc_coeffs(pr["alpha"], pr["delta"], pr["theta"], pr["gamma"], N)
+    x64, h64 = x.cpu().double(), h0.cpu().to(torch.complex128)
+    from oracle import fftconv as offt
+    want = (offt.fftconv_fwd(x64, cema.ema_weight_fwd(p, q.log(), g, L)) + x64 * pr["omega"]
+            + cema.ema_bias_fwd(q.log(), g, h64, L))
+    assert rel_err(y, want) <= TOL
+    assert rel_err(h, cema.ema_hidden_fwd(x64, p, q.log(), h64)) <= TOL

@@ -1,6 +1,10 @@
 """Parity of the HIP causal FFT convolution with the float64 oracle.
-Tolerances: rel err (max|a-b|/max|b|) <= 1e-4 for float32 rows, <= 2e-2 for
-bfloat16 / float16 rows (forward values and both gradients)."""
+Tolerances: rel err (max|a-b|/max|b|) <= 1e-4 for every float32 tensor (rows of
+float32 input, and dk / d omega whatever the input dtype), <= 2e-2 for
+bfloat16 / float16 tensors.  The default engine computes in float32; the
+opt-in matrix-core engine (MEGA_FFTCONV_F16_STAGES=1, fp16 between its DFT
+stages) is tested beside it and holds dk to 5e-3 only, which is why it is not
+the default."""
 import pytest
 import torch
 
@@ -12,6 +16,28 @@ from oracle import cema, fftconv
 
 pytestmark = pytest.mark.gpu
 TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+F16_STAGE_DK = 5e-3   # float32 outputs of the opt-in fp16-stage engine (measured 1.1e-3)
+
+
+@pytest.fixture(params=["fp32", "f16_stages"])
+def engine(request, monkeypatch):
+    """Both convolution engines for 16-bit rows: the default float32 one and the
+    opt-in matrix-core one (the library reads the variable per call)."""
+    if request.param == "f16_stages":
+        monkeypatch.setenv("MEGA_FFTCONV_F16_STAGES", "1")
+    else:
+        monkeypatch.delenv("MEGA_FFTCONV_F16_STAGES", raising=False)
+    return request.param
+
+
+@pytest.fixture
+def f16_stages(monkeypatch):
+    monkeypatch.setenv("MEGA_FFTCONV_F16_STAGES", "1")
+
+
+def f32_tol(engine, dtype):
+    """Bar for a float32 output computed from rows of `dtype`."""
+    return F16_STAGE_DK if (engine == "f16_stages" and dtype != torch.float32) else 1e-4
 
 SHAPES = [
     (1, 3, 1), (2, 3, 31), (2, 5, 50), (1, 4, 2048), (2, 3, 1000),     # direct (time-domain) kernel
@@ -33,7 +59,7 @@ def _data(B, D, L, dtype, seed):
 
 @pytest.mark.parametrize("B,D,L", SHAPES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_fwd_matches_oracle(B, D, L, dtype):
+def test_fwd_matches_oracle(B, D, L, dtype, engine):
     x, k, _ = _data(B, D, L, dtype, 31 * L + B)
     y = ops.fftconv_fwd(x.cuda(), k.cuda())
     assert y.dtype == dtype and y.shape == x.shape
@@ -43,13 +69,13 @@ def test_fwd_matches_oracle(B, D, L, dtype):
 
 @pytest.mark.parametrize("B,D,L", SHAPES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_bwd_matches_oracle(B, D, L, dtype):
+def test_bwd_matches_oracle(B, D, L, dtype, engine):
     x, k, dy = _data(B, D, L, dtype, 17 * L + B)
     dx, dk = ops.fftconv_bwd(dy.cuda(), x.cuda(), k.cuda(), torch.float32)
     assert dx.dtype == dtype and dk.dtype == torch.float32 and dk.shape == k.shape
     wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
     assert rel_err(dx, wdx) <= TOL[dtype]
-    assert rel_err(dk, wdk) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= f32_tol(engine, dtype)
 
 
 RES_SHAPES = [(2, 3, 50), (1, 4, 2048), (2, 3, 4097), (1, 3, 8192), (2, 2, 12345), (2, 3, 32768), (1, 2, 32767),
@@ -58,7 +84,7 @@ RES_SHAPES = [(2, 3, 50), (1, 4, 2048), (2, 3, 4097), (1, 3, 8192), (2, 2, 12345
 
 @pytest.mark.parametrize("B,D,L", RES_SHAPES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_residual_variant_matches_oracle(B, D, L, dtype):
+def test_residual_variant_matches_oracle(B, D, L, dtype, engine):
     """y = fftconv(x, k) + omega x and its three gradients; the expected values
     are the float64 oracle convolution plus the skip term written out."""
     x, k, dy = _data(B, D, L, dtype, 7 * L + B)
@@ -71,14 +97,14 @@ def test_residual_variant_matches_oracle(B, D, L, dtype):
     dx, dk, dw = ops.fftconv_residual_bwd(dy.cuda(), x.cuda(), k.cuda(), omega.cuda())
     wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
     assert rel_err(dx, wdx.double() + w64 * dy.double()) <= TOL[dtype]
-    assert rel_err(dk, wdk) <= TOL[dtype]
-    assert dw.shape == (D,) and rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= f32_tol(engine, dtype)
+    assert dw.shape == (D,) and rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= f32_tol(engine, dtype)
 
 
 @pytest.mark.parametrize("B,D,L", [(1, 3, 32768), (2, 2, 20000), (2, 4, 16384), (1, 8, 8192), (3, 16, 4096),
                                    (2, 8, 2056), (1, 4, 12344)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_saved_spectrum_pair_matches_oracle(B, D, L, dtype):
+def test_saved_spectrum_pair_matches_oracle(B, D, L, dtype, f16_stages):
     """Forward that keeps the spectra of x and k, backward from dy and the two
     buffers alone: same values and gradients as the float64 oracle."""
     x, k, dy = _data(B, D, L, dtype, 13 * L + B)
@@ -90,15 +116,15 @@ def test_saved_spectrum_pair_matches_oracle(B, D, L, dtype):
     dx, dk, dw = ops.fftconv_residual_bwd_saved(dy.cuda(), sx, sk, omega.cuda())
     wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
     assert rel_err(dx, wdx.double() + w64 * dy.double()) <= TOL[dtype]
-    assert rel_err(dk, wdk) <= TOL[dtype]
-    assert rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= F16_STAGE_DK
+    assert rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= F16_STAGE_DK
     # the recomputing pair gives the same forward bits
     assert torch.equal(y, ops.fftconv_residual_fwd(x.cuda(), k.cuda(), omega.cuda()))
 
 
 @pytest.mark.parametrize("B,D,L", [(3, 256, 20000), (2, 1024, 4096), (2, 130, 32768), (4, 520, 9000)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_batch_walking_forward_matches_oracle(B, D, L, dtype):
+def test_batch_walking_forward_matches_oracle(B, D, L, dtype, f16_stages):
     """B > 1 with at least half as many channel groups as compute units: the
     forward that transforms k once per channel group and walks the batch, with
     and without kept spectra, and the backward from those spectra (the
@@ -119,14 +145,14 @@ def test_batch_walking_forward_matches_oracle(B, D, L, dtype):
     dx, dk, dw = ops.fftconv_residual_bwd_saved(dy.cuda(), sx, sk, omega.cuda())
     wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
     assert rel_err(dx, wdx.double() + w64 * dy.double()) <= TOL[dtype]
-    assert rel_err(dk, wdk) <= TOL[dtype]
-    assert rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= F16_STAGE_DK
+    assert rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= F16_STAGE_DK
     # every batch entry on its own (B = 1: the kernel that transforms k per row) gives the same rows
     for b in range(B):
         assert torch.equal(ops.fftconv_residual_fwd(x[b:b + 1].cuda(), k.cuda(), omega.cuda())[0], y1[b])
 
 
-def test_saved_spectrum_pair_at_full_row_count_agrees_with_recomputing_pair():
+def test_saved_spectrum_pair_at_full_row_count_agrees_with_recomputing_pair(f16_stages):
     """Config-1 rows (L = 32768, bf16) over 512 channels and two batch entries:
     the backward from kept spectra and the backward that re-transforms x and k
     see the same fp16 spectra, so they agree far inside the bfloat16 bar."""
@@ -143,7 +169,13 @@ def test_saved_spectrum_pair_at_full_row_count_agrees_with_recomputing_pair():
     assert rel_err(dx, rdx) <= 4e-3 and rel_err(dk, rdk) <= 1e-3 and rel_err(dw, rdw) <= 1e-3
 
 
-def test_saved_spectrum_path_is_refused_outside_its_shapes():
+def test_saved_spectrum_path_is_off_without_the_switch(monkeypatch):
+    monkeypatch.delenv("MEGA_FFTCONV_F16_STAGES", raising=False)
+    assert ops.fftconv_spectrum_bytes(torch.bfloat16, 1, 8, 4096) == 0
+
+
+def test_saved_spectrum_path_is_refused_outside_its_shapes(f16_stages):
+    assert ops.fftconv_spectrum_bytes(torch.bfloat16, 1, 8, 4096) > 0
     assert ops.fftconv_spectrum_bytes(torch.float32, 1, 8, 4096) == 0
     assert ops.fftconv_spectrum_bytes(torch.bfloat16, 1, 8, 2048) == 0
     assert ops.fftconv_spectrum_bytes(torch.bfloat16, 1, 3, 4096) == 0   # 8 rows per pass, D = 3
@@ -153,15 +185,17 @@ def test_saved_spectrum_path_is_refused_outside_its_shapes():
         ops.fftconv_residual_fwd_saving(x, torch.zeros(3, 4096, device="cuda"), torch.zeros(3, device="cuda"))
 
 
-def test_residual_autograd_function_16bit_uses_saved_spectra():
+def test_residual_autograd_function_16bit(engine):
+    """bf16 rows through the autograd node: kept (x, k) on the default engine,
+    kept spectra on the opt-in one."""
     x, k, dy = _data(2, 8, 6000, torch.bfloat16, 3)
     omega = torch.randn(8, 1)
     xg, kg, wg = (t.cuda().requires_grad_() for t in (x, k, omega))
     fftconv_residual(xg, kg, wg).backward(dy.cuda())
     wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
     assert rel_err(xg.grad, wdx.double() + omega.double().view(1, 8, 1) * dy.double()) <= 2e-2
-    assert rel_err(kg.grad, wdk) <= 2e-2
-    assert rel_err(wg.grad.view(-1), (dy.double() * x.double()).sum(dim=(0, 2))) <= 2e-2
+    assert rel_err(kg.grad, wdk) <= f32_tol(engine, torch.bfloat16)
+    assert rel_err(wg.grad.view(-1), (dy.double() * x.double()).sum(dim=(0, 2))) <= f32_tol(engine, torch.bfloat16)
 
 
 def test_residual_autograd_function():
@@ -176,16 +210,16 @@ def test_residual_autograd_function():
 
 
 @pytest.mark.parametrize("B,D,L", [(2, 3, 5000), (1, 5, 2400), (2, 3, 10000), (1, 2, 30000)])
-def test_float16_rows(B, D, L):
+def test_float16_rows(B, D, L, engine):
     x, k, dy = _data(B, D, L, torch.float16, 5)
     y = ops.fftconv_fwd(x.cuda(), k.cuda())
     assert rel_err(y, fftconv.fftconv_fwd(x, k)) <= TOL[torch.float16]
     dx, dk = ops.fftconv_bwd(dy.cuda(), x.cuda(), k.cuda(), torch.float32)
     wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
-    assert rel_err(dx, wdx) <= TOL[torch.float16] and rel_err(dk, wdk) <= TOL[torch.float16]
+    assert rel_err(dx, wdx) <= TOL[torch.float16] and rel_err(dk, wdk) <= f32_tol(engine, torch.float16)
 
 
-def test_rows_of_a_pass_do_not_mix():
+def test_rows_of_a_pass_do_not_mix(f16_stages):
     """Short 16-bit rows share a workgroup pass: a row of zeros between busy
     rows stays exactly zero, and every row equals its single-row result."""
     B, D, L = 1, 8, 4096
@@ -210,7 +244,7 @@ def test_config0_cema_forward_fp32():
     assert rel_err(out, want) <= 1e-4
 
 
-def test_config1_rows_bf16_fwd_bwd_with_ema_kernel():
+def test_config1_rows_bf16_fwd_bwd_with_ema_kernel(engine):
     """BASELINE config 1 row shape (L=32768, ndim=16, x bf16), a slice of the channels."""
     D, N, L = 48, 16, 32768
     prm = synthetic.cema_params(D, N, 1001)
@@ -222,7 +256,7 @@ def test_config1_rows_bf16_fwd_bwd_with_ema_kernel():
     dx, dk = ops.fftconv_bwd(io["dy"].cuda(), io["x"].cuda(), k.cuda(), torch.float32)
     wdx, wdk = fftconv.fftconv_bwd(io["dy"], io["x"], k)
     assert rel_err(dx, wdx) <= 2e-2
-    assert rel_err(dk, wdk) <= 2e-2
+    assert rel_err(dk, wdk) <= f32_tol(engine, torch.bfloat16)
 
 
 def test_full_size_linearity_and_shift_properties():
@@ -278,7 +312,7 @@ def _long_data(B, D, L, dtype, seed):
 
 @pytest.mark.parametrize("B,D,L", [(1, 2, 32769), (2, 3, 40000), (1, 2, 65536), (1, 2, 70001), (1, 1, 131072)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_rows_beyond_one_launch_match_oracle(B, D, L, dtype):
+def test_rows_beyond_one_launch_match_oracle(B, D, L, dtype, engine):
     """L > 32768: the host cuts rows into blocks (heads and tails of block
     pairs); forward and backward against the float64 oracle on the whole row."""
     x, k, dy = _long_data(B, D, L, dtype, L + B)
@@ -289,11 +323,11 @@ def test_rows_beyond_one_launch_match_oracle(B, D, L, dtype):
     wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
     assert dx.dtype == dtype and dk.shape == k.shape
     assert rel_err(dx, wdx) <= TOL[dtype]
-    assert rel_err(dk, wdk) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= f32_tol(engine, dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_residual_autograd_function_beyond_one_launch(dtype):
+def test_residual_autograd_function_beyond_one_launch(dtype, engine):
     B, D, L = 2, 3, 50000
     x, k, dy = _long_data(B, D, L, dtype, 77)
     om = torch.randn(D, 1, generator=torch.Generator().manual_seed(5))
@@ -306,8 +340,8 @@ def test_residual_autograd_function_beyond_one_launch(dtype):
     assert y.dtype == dtype
     assert rel_err(y, want.detach()) <= TOL[dtype]
     assert rel_err(xc.grad, x64.grad) <= TOL[dtype]
-    assert rel_err(kc.grad, k64.grad) <= TOL[dtype]
-    assert rel_err(oc.grad, o64.grad) <= TOL[dtype]
+    assert rel_err(kc.grad, k64.grad) <= f32_tol(engine, dtype)
+    assert rel_err(oc.grad, o64.grad) <= f32_tol(engine, dtype)
 
 
 def test_cema_layer_at_twice_the_launch_length():
