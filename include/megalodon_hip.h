@@ -458,6 +458,33 @@ int mega_group_sequence_norm_bwd(const void* dy, const void* x, const int64_t* c
                                  int64_t H, int64_t num_groups, int length_last, void* dx,
                                  void* dgamma, void* dbeta, void* workspace, void* stream);
 
+/* ------------------------------------------------------------------------
+ * The CEMA layer as a chunked recurrence (no kernel row, no spectra).
+ *
+ * Replaces, for one call of MultiHeadComplexEMA.forward
+ *   (megalodon/modules/complex_exponential_moving_average.py:127-147), the chain
+ *   k, b = ema_parameters(p, q, gamma, hx, L)      (fused_ops/ema_parameters.py:8-35,
+ *                                                    csrc/ops/ema_parameters.cc:17-77)
+ *   out  = fftconv(x, k) + x * omega (+ b)          (fused_ops/fftconv.py:9-50)
+ *   h    = ema_hidden(x, p, q, hx)                  (csrc/ops/ema_hidden.cc:16-62)
+ * which is the recurrence h[t] = q h[t-1] + p x[t], out[t] = Re sum_n gamma_n
+ * h_n[t] + omega x[t] with h[-1] = hx.  The row is processed in chunks of 64
+ * steps as matrix products on the matrix cores (bf16 operand pieces carrying
+ * 16 significant bits, float32 states and accumulation); x is read once and
+ * out written once.
+ *   x, y (B, D, L) of `dtype` (MEGA_BF16 / MEGA_F16), 16-byte aligned, any
+ *   L % 8 == 0 (no upper limit); p (D, N) float32; log_q, gamma (D, N)
+ *   complex64 as mega_ema_weight_fwd takes them, N <= 16; omega (D) float32 or
+ *   null; h0 (B, D, N) complex64 or null (zero state); h_last (B, D, N)
+ *   complex64 or null (not wanted).
+ *   mega_cema_scan_supported(dtype, N, L) tells whether a shape is taken;
+ *   others return MEGA_ERR_UNSUPPORTED (use the kernel-row path then).
+ * ---------------------------------------------------------------------- */
+int mega_cema_scan_supported(int dtype, int64_t N, int64_t L);
+int mega_cema_scan_fwd(const void* x, int dtype, const float* p, const float* log_q,
+                       const float* gamma, const float* omega, const float* h0, int64_t B,
+                       int64_t D, int64_t N, int64_t L, void* y, float* h_last, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

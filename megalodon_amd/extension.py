@@ -508,6 +508,44 @@ def fftconv_residual_bwd_saved(y_grad: torch.Tensor, spec_x: torch.Tensor, spec_
 
 
 # --------------------------------------------------------------------------
+# The CEMA layer as a chunked recurrence (csrc/cema_scan.hip)
+# --------------------------------------------------------------------------
+def cema_scan_supported(x: torch.Tensor, ndim: int) -> bool:
+    """Whether `cema_scan_fwd` takes this input: bfloat16 / float16 rows on the
+    GPU, at most 16 modes, a length that is a multiple of 8."""
+    if not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    fn = _lib.load().mega_cema_scan_supported
+    return bool(fn(_lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(ndim), _lib.i64(x.shape[-1])))
+
+
+def cema_scan_fwd(x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor, gamma: torch.Tensor,
+                  omega: Optional[torch.Tensor], h0: Optional[torch.Tensor] = None,
+                  compute_last_state: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """(out, h_last): ``fftconv(x, k) + x * omega + b`` and, on request, the state
+    after the last step, for k, b = ema_parameters(p, q, gamma, h0, L) -- without
+    forming k (complex_exponential_moving_average.py:127-147).  x (B, D, L)
+    bfloat16 / float16; p (D, N[, 1]) float32; log_q, gamma (D, N[, 1]) complex64."""
+    dev = _require_cuda(x, p, log_q, gamma, omega, h0)
+    B, D, L = x.shape
+    N = p.shape[1]
+    xc = x.contiguous()
+    if xc.data_ptr() % 16 != 0:
+        xc = xc.clone(memory_format=torch.contiguous_format)
+    pc = p.reshape(D, N).contiguous().float()
+    lq, gm = _as_c64(log_q, "log_q").reshape(D, N), _as_c64(gamma, "gamma").reshape(D, N)
+    wc = None if omega is None else omega.reshape(-1).contiguous().float()
+    hc = None if h0 is None else _as_c64(h0, "h0").reshape(B, D, N)
+    y = torch.empty_like(xc)
+    h_last = torch.empty((B, D, N), dtype=torch.complex64, device=dev) if compute_last_state else None
+    with torch.cuda.device(dev):
+        _lib.call("mega_cema_scan_fwd", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)), _lib.ptr(pc),
+                  _lib.ptr(lq), _lib.ptr(gm), _lib.ptr(wc), _lib.ptr(hc), _lib.i64(B), _lib.i64(D), _lib.i64(N),
+                  _lib.i64(L), _lib.ptr(y), _lib.ptr(h_last), _lib.stream_ptr(dev))
+    return y, h_last
+
+
+# --------------------------------------------------------------------------
 # group_timestep_norm (reference: csrc/ops/timestep_norm.cc:621-705)
 # --------------------------------------------------------------------------
 def _tsn_workspace(B, L, D, G, backward, dev):

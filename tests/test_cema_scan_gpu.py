@@ -1,0 +1,80 @@
+"""The chunked-recurrence CEMA kernels against the float64 oracle (closed-form
+kernel + FFT convolution + carried-state bias + last state, and their autograd
+gradients).  Bars: 2e-2 for bfloat16 / float16 tensors, 1e-4 for float32
+tensors (the parameter gradients and the complex last state)."""
+import math
+
+import pytest
+import torch
+
+from conftest import rel_err
+from megalodon_amd import extension as ops
+from oracle import cema as ocema
+from oracle import fftconv as offt
+
+pytestmark = pytest.mark.gpu
+
+
+def _params(D, N, seed):
+    g = torch.Generator().manual_seed(seed)
+    alpha = torch.sigmoid(torch.randn(D, N, 1, generator=g))
+    delta = torch.sigmoid(torch.randn(D, N, 1, generator=g))
+    theta = torch.rand(D, 1, 1, generator=g) * (2 * math.pi / N)
+    q = torch.polar(1.0 - alpha * delta, theta * torch.arange(1, N + 1, dtype=torch.float32).view(1, N, 1))
+    gam = torch.complex(torch.randn(D, N, generator=g), torch.randn(D, N, generator=g)) / math.sqrt(2 * N)
+    omega = torch.randn(D, generator=g)
+    return alpha, q, gam, omega
+
+
+def _oracle_fwd(x, p, q, gam, omega, h0):
+    L = x.shape[-1]
+    lq = q.to(torch.complex128).log()
+    k = ocema.ema_weight_fwd(p.double(), lq, gam.to(torch.complex128), L)
+    want = offt.fftconv_fwd(x.double(), k) + x.double() * omega.double().view(1, -1, 1)
+    if h0 is not None:
+        want = want + ocema.ema_bias_fwd(lq, gam.to(torch.complex128), h0.to(torch.complex128), L)
+    last = ocema.ema_hidden_fwd(x.double(), p.double(), lq, None if h0 is None else h0.to(torch.complex128))
+    return want, last
+
+
+SHAPES = [(1, 2, 16, 8), (2, 3, 16, 64), (1, 3, 16, 72), (2, 2, 5, 1000), (1, 4, 16, 4096), (2, 2, 16, 8200),
+          (1, 3, 16, 16384), (1, 2, 16, 16392), (1, 5, 16, 32768), (1, 2, 16, 40000), (1, 2, 1, 2048),
+          (1, 2, 16, 65536)]
+
+
+@pytest.mark.parametrize("B,D,N,L", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("state", [False, True])
+def test_forward_matches_oracle(B, D, N, L, dtype, state):
+    p, q, gam, omega = _params(D, N, 3 * L + D)
+    g = torch.Generator().manual_seed(L)
+    x = torch.randn(B, D, L, generator=g).to(dtype)
+    h0 = torch.complex(torch.randn(B, D, N, generator=g), torch.randn(B, D, N, generator=g)) if state else None
+    assert ops.cema_scan_supported(x.cuda(), N)
+    y, last = ops.cema_scan_fwd(x.cuda(), p.cuda(), q.log().cuda(), gam.cuda(), omega.cuda(),
+                                None if h0 is None else h0.cuda(), True)
+    want, wlast = _oracle_fwd(x, p, q, gam, omega, h0)
+    assert y.dtype == dtype and y.shape == x.shape
+    assert rel_err(y, want) <= 2e-2
+    # the rounding of y aside, the values carry float32 accuracy: compare before rounding would need
+    # a float32 output, so the last state (complex64, never rounded to 16 bits) stands for it
+    assert last.shape == (B, D, N) and rel_err(last, wlast) <= 1e-4
+
+
+def test_forward_without_skip_term_and_without_last_state():
+    B, D, N, L = 2, 3, 16, 3000
+    p, q, gam, omega = _params(D, N, 5)
+    x = torch.randn(B, D, L, generator=torch.Generator().manual_seed(1)).bfloat16()
+    y, last = ops.cema_scan_fwd(x.cuda(), p.cuda(), q.log().cuda(), gam.cuda(), None)
+    want, _ = _oracle_fwd(x, p, q, gam, torch.zeros(D), None)
+    assert last is None and rel_err(y, want) <= 2e-2
+
+
+def test_unsupported_shapes_are_refused():
+    x = torch.zeros(1, 2, 100, dtype=torch.bfloat16, device="cuda")   # L % 8 != 0
+    assert not ops.cema_scan_supported(x, 16)
+    assert not ops.cema_scan_supported(torch.zeros(1, 2, 64, device="cuda"), 16)   # float32 rows
+    assert not ops.cema_scan_supported(torch.zeros(1, 2, 64, dtype=torch.bfloat16, device="cuda"), 17)
+    p, q, gam, omega = _params(2, 16, 1)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        ops.cema_scan_fwd(x, p.cuda(), q.log().cuda(), gam.cuda(), omega.cuda())
