@@ -485,6 +485,22 @@ int mega_cema_scan_fwd(const void* x, int dtype, const float* p, const float* lo
                        const float* gamma, const float* omega, const float* h0, int64_t B,
                        int64_t D, int64_t N, int64_t L, void* y, float* h_last, void* stream);
 
+/* Backward of mega_cema_scan_fwd without a carried state (the training path):
+ * replaces the chain fftconv_bwd -> (dx, dk), ema_parameters_bwd(dk, ...) ->
+ * (dp, dq, dgamma) and the two elementwise passes of the skip term
+ *   (fused_ops/fftconv.py:53-75, csrc/ops/ema_parameters.cc:80-98,141-156);
+ * dk is never formed.  dy, x, dx (B, D, L) bfloat16, 16-byte aligned,
+ * L % 8 == 0; the parameter gradients come PER ROW, (B, D, N) -- dp float32,
+ * dq and dgamma complex64 in PyTorch's conjugate convention, as
+ * mega_ema_weight_bwd returns them -- and domega (B, D) float32; the caller
+ * sums over B.  mega_cema_scan_bwd_supported(dtype, N, L) tells whether a
+ * shape is taken. */
+int mega_cema_scan_bwd_supported(int dtype, int64_t N, int64_t L);
+int mega_cema_scan_bwd(const void* dy, const void* x, int dtype, const float* p,
+                       const float* log_q, const float* gamma, const float* omega, int64_t B,
+                       int64_t D, int64_t N, int64_t L, void* dx, float* dp, float* dq,
+                       float* dgamma, float* domega, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

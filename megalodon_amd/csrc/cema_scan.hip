@@ -382,6 +382,493 @@ int launch_fwd(const void* x, void* y, const float* p, const cf* log_q, const cf
   return MEGA_OK;
 }
 
+
+// ------------------------------ backward ------------------------------------
+// With c_n = p_n gamma_n and, per mode,
+//   A = sum_{t >= s} dy[t] x[s] q^(t-s),   B = dA / dq
+// the gradients the reference forms from dk (ema_parameters.cc:80-98 after
+// fftconv.py:53-75) are dp = Re(A gamma), dq = conj(B p gamma), dgamma = conj(A p),
+// domega = sum dy x, and dx[s] = sum_{t >= s} k[t-s] dy[t] + omega dy[s].  By chunks, in
+// reverse time (DY[c][i] = dy[64 c + i], XR[c][j'] = x[64 c + 63 - j']):
+//   (G, G')[c]   = Pg DY[c],     Pg = rows (Re, Im)(q^i), then (Re, Im)(i q^(i-1)), i < 64
+//   R[c]  = G[c] + q^64 R[c+1],   R'[c] = G'[c] + 64 q^63 R[c+1] + q^64 R'[c+1]      (scan)
+//   (X, X')[c]   = Pg XR[c]
+//   W  = sum_c X[c] R[c+1],   W' = sum_c (X'[c] R[c+1] + X[c] R'[c+1])
+//   DX[c] = K^T DY[c] + Qd R[c+1],   Qd[j][m] = (Re, -Im)(c_n q_n^(64-j))
+//   M     = sum_c DY[c]^T X[c]   (64 x 64, rows i >= columns j), dkin[l] = sum_j M[j+l][j]
+//   A = sum_l q^l dkin[l] + q W,   B = sum_l l q^(l-1) dkin[l] + W + q W'
+// Segments of 128 chunks are taken from the end of the row to its start; a
+// wave holds one chunk tile of the segment.  The chunk-contracted product M
+// needs operands with chunks along k: the wave parks its DY and X tiles in a
+// private LDS tile and reads them back with the transposing LDS read; the same
+// tile hands out the time-reversed x operand.
+constexpr int kRP = 68;       // floats per row of the reverse-state buffer: (R, R') = 64 + 4
+constexpr int kSP = 72;       // 16-bit elements per row of a wave's staging tile: 64 + 8
+constexpr int kBwdNC = kWaves * 32;  // chunks per segment
+constexpr int kBwdCPS = kBwdNC / kSubs;
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint2 lds_read_tr(const uint16_t* q) {
+  const short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) short4v*)(q));
+  return __builtin_bit_cast(uint2, v);
+}
+
+// LDS of the backward kernel, by byte offset.  The region from kOffR on is reused:
+// tables while the operand blocks are built, the per-wave copies of M at the end.
+constexpr int kOffPg = 0;                                   // 8 blocks x 2 pieces x 64 lanes x 16 B
+constexpr int kOffR = kOffPg + 8 * 2 * kWave * 16;          // (kBwdNC + 1) rows of kRP floats
+constexpr int kOffStage = kOffR + (kBwdNC + 1) * kRP * 4;   // kWaves tiles of 32 x kSP elements
+constexpr int kOffSmall = kOffStage + kWaves * 32 * kSP * 2;
+struct BwdSmall {
+  cf sub_end[kSubs][2][16];
+  cf carry[2][2][16];
+  float pn[16];
+  cf gn[16];
+  float red[kWaves][2][32];
+  float dkin[kT];
+  cf ab[16][2][16];
+};
+constexpr int kBwdLds = kOffSmall + static_cast<int>(sizeof(BwdSmall));
+// build-time tables inside the reused region
+constexpr int kOffQp = kOffR;                               // cf [16][66]
+constexpr int kOffKl = kOffQp + 16 * (kT + 2) * 8;          // float [64]
+constexpr int kOffKQ = kOffKl + kT * 4;                     // 8 blocks x 2 pieces x 64 x 16 B
+static_assert(kOffKQ + 8 * 2 * kWave * 16 <= kOffSmall, "build-time tables must fit the reused region");
+static_assert(kWaves * 3 * 16 * kWave * 4 + kWaves * kT * 4 <= kOffSmall - kOffR, "the copies of M must fit the reused region");
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void cema_scan_bwd_kernel(
+    const void* __restrict__ dy, const void* __restrict__ x, void* __restrict__ dx,
+    const float* __restrict__ p, const cf* __restrict__ log_q, const cf* __restrict__ gamma,
+    const float* __restrict__ omega, float* __restrict__ dp, cf* __restrict__ dq,
+    cf* __restrict__ dgamma, float* __restrict__ domega, int D, int N, int64_t L) {
+  static_assert(XOp<DT>::XP == 1, "the backward kernel takes bfloat16 rows");
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  u32x4* const pg = reinterpret_cast<u32x4*>(smem_raw + kOffPg);      // [blk][piece][lane]
+  float* const rbuf = reinterpret_cast<float*>(smem_raw + kOffR);
+  BwdSmall& sm = *reinterpret_cast<BwdSmall*>(smem_raw + kOffSmall);
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int g = lane >> 5, r = lane & 31;
+  uint16_t* const stage = reinterpret_cast<uint16_t*>(smem_raw + kOffStage) + wave * 32 * kSP;
+  const int64_t row = blockIdx.x;
+  const int d = static_cast<int>(row % D);
+  const uint16_t* dyrow = static_cast<const uint16_t*>(dy) + row * L;
+  const uint16_t* xrow = static_cast<const uint16_t*>(x) + row * L;
+  uint16_t* dxrow = static_cast<uint16_t*>(dx) + row * L;
+  const float wres = omega != nullptr ? omega[d] : 0.f;
+  const int64_t C = (L + kT - 1) / kT;
+  const int64_t seg_last = (C - 1) / kBwdNC * kBwdNC;
+
+  XOp<DT> db[4], xb[4];
+  auto load_tiles = [&](int64_t seg0) {
+    const int64_t chunk = seg0 + wave * 32 + r;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int64_t elem = chunk * kT + 16 * s + 8 * g;
+      db[s].load(dyrow, elem, elem + 8 <= L);
+      xb[s].load(xrow, elem, elem + 8 <= L);
+    }
+  };
+  load_tiles(seg_last);
+
+  // ---- per-row tables and operand blocks -----------------------------------------
+  const int sn = tid & 15, sa = tid >> 4;
+  cf (*qp)[kT + 2] = reinterpret_cast<cf(*)[kT + 2]>(smem_raw + kOffQp);
+  float* klocal = reinterpret_cast<float*>(smem_raw + kOffKl);
+  u32x4* const kq = reinterpret_cast<u32x4*>(smem_raw + kOffKQ);
+  cf lq{0.f, 0.f};
+  if (sn < N) lq = log_q[d * N + sn];
+  {
+    cf v{0.f, 0.f}, q1{0.f, 0.f};
+    if (sn < N) {
+      v = qpow(lq.x, lq.y, 4 * sa);
+      q1 = qpow(lq.x, lq.y, 1);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      qp[sn][4 * sa + e] = v;
+      v = cmul(v, q1);
+    }
+    if (sa == 15) qp[sn][kT] = v;
+    if (tid < 16) {
+      sm.pn[tid] = tid < N ? p[d * N + tid] : 0.f;
+      sm.gn[tid] = tid < N ? gamma[d * N + tid] : cf{0.f, 0.f};
+      sm.carry[0][0][tid] = cf{0.f, 0.f};
+      sm.carry[0][1][tid] = cf{0.f, 0.f};
+    }
+  }
+  // scan multipliers: over one chunk (q^64, 64 q^63) and over a sub-segment of CPS chunks
+  cf qT{0.f, 0.f}, qTd{0.f, 0.f}, qS{0.f, 0.f}, qSd{0.f, 0.f};
+  if (sn < N) {
+    qT = qpow(lq.x, lq.y, kT);
+    const cf a = qpow(lq.x, lq.y, kT - 1);
+    qTd = cf{kT * a.x, kT * a.y};
+    qS = qpow(lq.x, lq.y, kT * kBwdCPS);
+    const cf b = qpow(lq.x, lq.y, kT * kBwdCPS - 1);
+    qSd = cf{(kT * kBwdCPS) * b.x, (kT * kBwdCPS) * b.y};
+  }
+  __syncthreads();
+  if (tid < kT) {
+    float acc = 0.f;
+#pragma unroll
+    for (int n = 0; n < 16; ++n) {
+      const cf c = cmul(cf{sm.pn[n] * sm.gn[n].x, sm.pn[n] * sm.gn[n].y}, qp[n][tid]);
+      acc += c.x;
+    }
+    klocal[tid] = acc;
+  }
+  __syncthreads();
+  // blocks 0..7: Pg (kind = b >> 2, k-step s = b & 3); 8..11: K^T by offset 16 (b - 8);
+  // 12..15: Qd (row tile jt = (b - 12) >> 1, k-step s2 = (b - 12) & 1)
+  for (int item = tid; item < 16 * kWave; item += kThreads) {
+    const int blk = item >> 6, ln = item & 63, rr = ln & 31, gg = ln >> 5;
+    float v[8];
+    if (blk < 8) {
+      const int kind = blk >> 2, s = blk & 3, n = rr >> 1, part = rr & 1;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int i = 16 * s + 8 * gg + e;
+        cf w = qp[n][kind ? (i > 0 ? i - 1 : 0) : i];
+        const float sc = kind ? static_cast<float>(i) : 1.f;
+        v[e] = sc * (part ? w.y : w.x);
+      }
+    } else if (blk < 12) {
+      const int o = 16 * (blk - 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int lag = o - rr + 8 * gg + e;
+        v[e] = lag >= 0 ? klocal[lag] : 0.f;
+      }
+    } else {
+      const int jt = (blk - 12) >> 1, s2 = (blk - 12) & 1, j = 32 * jt + rr;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int m = 16 * s2 + 8 * gg + e, n = m >> 1;
+        const cf c = cf{sm.pn[n] * sm.gn[n].x, sm.pn[n] * sm.gn[n].y};
+        const cf w = cmul(c, qp[n][kT - j]);
+        v[e] = (m & 1) ? -w.y : w.x;
+      }
+    }
+    u32x4 hi, lo;
+    split8(v, hi, lo);
+    u32x4* dst = blk < 8 ? pg + (blk * 2) * kWave : kq + ((blk - 8) * 2) * kWave;
+    dst[ln] = hi;
+    dst[kWave + ln] = lo;
+  }
+  __syncthreads();
+  u32x4 KQ[8][2];
+#pragma unroll
+  for (int b = 0; b < 8; ++b) {
+    KQ[b][0] = kq[(b * 2) * kWave + lane];
+    KQ[b][1] = kq[(b * 2 + 1) * kWave + lane];
+  }
+  __syncthreads();  // the tables' region becomes the reverse-state buffer and the staging tiles
+
+  floatx16 macc[3];  // M tiles (0,0), (1,0), (1,1) over this wave's chunks
+#pragma unroll
+  for (int t = 0; t < 3; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) macc[t][i] = 0.f;
+  cf wacc[8], wdacc[8];  // W, W' of modes n = 4 qd + 2 g + b at index 2 qd + b, over this lane's chunks
+#pragma unroll
+  for (int i = 0; i < 8; ++i) wacc[i] = wdacc[i] = cf{0.f, 0.f};
+
+  // transposing read of a staged tile: row tile tt (32 time steps), k-step ks (16 chunks)
+  const int tr_base = (8 * g + ((lane & 15) >> 2)) * kSP + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  auto read_tr = [&](int tt, int ks) {
+    const uint16_t* q = stage + tr_base + 16 * ks * kSP + 32 * tt;
+    const uint2 lo = lds_read_tr(q), hi = lds_read_tr(q + 4 * kSP);
+    return u32x4{lo.x, lo.y, hi.x, hi.y};
+  };
+
+  int cur = 0;
+  for (int64_t seg0 = seg_last; seg0 >= 0; seg0 -= kBwdNC) {
+    const int nc = static_cast<int>(C - seg0 < kBwdNC ? C - seg0 : kBwdNC);
+    const int c0 = wave * 32;
+    const bool on = c0 < nc;
+    // ---- (G, G') = Pg DY -------------------------------------------------------------
+    if (on) {
+#pragma unroll
+      for (int kind = 0; kind < 2; ++kind) {
+        floatx16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const u32x4 a[2] = {pg[((kind * 4 + s) * 2) * kWave + lane], pg[((kind * 4 + s) * 2 + 1) * kWave + lane]};
+          acc = mma_split<1>(a, db[s].pc, acc);
+        }
+        float* dst = rbuf + (c0 + r) * kRP + 32 * kind + 4 * g;
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd)
+          *reinterpret_cast<float4*>(dst + 8 * qd) =
+              make_float4(acc[4 * qd], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3]);
+      }
+    }
+    lds_barrier();
+    // ---- reverse scan over the chunks of the segment ------------------------------------
+    {
+      float* col = rbuf + 2 * sn;
+      cf e{0.f, 0.f}, ed{0.f, 0.f};
+#pragma unroll 4
+      for (int i = kBwdCPS - 1; i >= 0; --i) {
+        const int c = sa * kBwdCPS + i;
+        if (c < nc) {
+          const float2 gv = *reinterpret_cast<const float2*>(col + c * kRP);
+          const float2 gd = *reinterpret_cast<const float2*>(col + c * kRP + 32);
+          const cf nd = cadd(cf{gd.x, gd.y}, cadd(cmul(qTd, e), cmul(qT, ed)));
+          e = cadd(cf{gv.x, gv.y}, cmul(qT, e));
+          ed = nd;
+        }
+      }
+      sm.sub_end[sa][0][sn] = e;
+      sm.sub_end[sa][1][sn] = ed;
+      lds_barrier();
+      const cf cin0 = sm.carry[cur][0][sn], cind0 = sm.carry[cur][1][sn];
+      cf h = cin0, hd = cind0;
+      for (int s = kSubs - 1; s > sa; --s) {
+        const cf nd = cadd(sm.sub_end[s][1][sn], cadd(cmul(qSd, h), cmul(qS, hd)));
+        h = cadd(sm.sub_end[s][0][sn], cmul(qS, h));
+        hd = nd;
+      }
+      if (sa == kSubs - 1) {  // the state after the segment's last chunk
+        *reinterpret_cast<float2*>(col + nc * kRP) = make_float2(cin0.x, cin0.y);
+        *reinterpret_cast<float2*>(col + nc * kRP + 32) = make_float2(cind0.x, cind0.y);
+      }
+#pragma unroll 4
+      for (int i = kBwdCPS - 1; i >= 0; --i) {
+        const int c = sa * kBwdCPS + i;
+        if (c < nc) {
+          const float2 gv = *reinterpret_cast<const float2*>(col + c * kRP);
+          const float2 gd = *reinterpret_cast<const float2*>(col + c * kRP + 32);
+          const cf nd = cadd(cf{gd.x, gd.y}, cadd(cmul(qTd, h), cmul(qT, hd)));
+          h = cadd(cf{gv.x, gv.y}, cmul(qT, h));
+          hd = nd;
+          *reinterpret_cast<float2*>(col + c * kRP) = make_float2(h.x, h.y);
+          *reinterpret_cast<float2*>(col + c * kRP + 32) = make_float2(hd.x, hd.y);
+        }
+      }
+      if (sa == 0) {
+        sm.carry[cur ^ 1][0][sn] = h;
+        sm.carry[cur ^ 1][1][sn] = hd;
+      }
+    }
+    lds_barrier();
+    if (on) {
+      // ---- the wave's private tile: DY parked and read back with chunks along k ----------
+      uint16_t* mine = stage + r * kSP + 8 * g;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) *reinterpret_cast<u32x4*>(mine + 16 * s) = db[s].pc[0];
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      u32x4 dyt[2][2];
+#pragma unroll
+      for (int it = 0; it < 2; ++it)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) dyt[it][ks] = read_tr(it, ks);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int s = 0; s < 4; ++s) *reinterpret_cast<u32x4*>(mine + 16 * s) = xb[s].pc[0];
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      // M += DY^T X over the tile's 32 chunks
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const u32x4 xt = read_tr(jt, ks);
+          if (jt == 0) macc[0] = mfma_bf16(dyt[0][ks], xt, macc[0]);
+          macc[1 + jt] = mfma_bf16(dyt[1][ks], xt, macc[1 + jt]);
+        }
+      // time-reversed x as an operand: steps 63 - (16 s + 8 g + e)
+      u32x4 xr[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(stage + r * kSP + 56 - 16 * s - 8 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) xr[s][e] = __builtin_amdgcn_alignbit(v[3 - e], v[3 - e], 16);
+      }
+      // ---- (X, X') = Pg XR, then W += X R[c+1], W' += X' R[c+1] + X R'[c+1] ---------------
+      floatx16 xacc[2];
+#pragma unroll
+      for (int kind = 0; kind < 2; ++kind) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) xacc[kind][i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const u32x4 a[2] = {pg[((kind * 4 + s) * 2) * kWave + lane], pg[((kind * 4 + s) * 2 + 1) * kWave + lane]};
+          xacc[kind] = mma_split<1>(a, &xr[s], xacc[kind]);
+        }
+      }
+      const float* rnext = rbuf + (c0 + r + 1) * kRP + 4 * g;
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const float4 rv = *reinterpret_cast<const float4*>(rnext + 8 * qd);
+        const float4 rd = *reinterpret_cast<const float4*>(rnext + 32 + 8 * qd);
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const cf xv{xacc[0][4 * qd + 2 * b], xacc[0][4 * qd + 2 * b + 1]};
+          const cf xd{xacc[1][4 * qd + 2 * b], xacc[1][4 * qd + 2 * b + 1]};
+          const cf rr_ = b ? cf{rv.z, rv.w} : cf{rv.x, rv.y};
+          const cf rdd = b ? cf{rd.z, rd.w} : cf{rd.x, rd.y};
+          wacc[2 * qd + b] = cadd(wacc[2 * qd + b], cmul(xv, rr_));
+          wdacc[2 * qd + b] = cadd(wdacc[2 * qd + b], cadd(cmul(xd, rr_), cmul(xv, rdd)));
+        }
+      }
+      // ---- DX = K^T DY + Qd R[c+1] (+ omega dy), written from the accumulators ---------------
+      u32x4 hb[2][2];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const float* src = rbuf + (c0 + r + 1) * kRP + 16 * s2 + 8 * g;
+        const float4 u = *reinterpret_cast<const float4*>(src);
+        const float4 w = *reinterpret_cast<const float4*>(src + 4);
+        const float v[8] = {u.x, u.y, u.z, u.w, w.x, w.y, w.z, w.w};
+        split8(v, hb[s2][0], hb[s2][1]);
+      }
+      const int64_t chunk = seg0 + c0 + r;
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt) {
+        floatx16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int s = 2 * jt; s < 4; ++s) acc = mma_split<1>(KQ[s - 2 * jt], db[s].pc, acc);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          acc = mfma_bf16(KQ[4 + 2 * jt + s2][0], hb[s2][0], acc);
+          acc = mfma_bf16(KQ[4 + 2 * jt + s2][1], hb[s2][0], acc);
+          acc = mfma_bf16(KQ[4 + 2 * jt + s2][0], hb[s2][1], acc);
+        }
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr) {
+          float oct[8];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            oct[e] = acc[8 * pr + e];
+            oct[4 + e] = acc[8 * pr + 4 + e];
+            half_swap(oct[e], oct[4 + e]);
+          }
+          const int s = 2 * jt + pr;
+          float gv[8];
+          db[s].values(gv);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) oct[e] = fmaf(wres, gv[e], oct[e]);
+          const int64_t elem = chunk * kT + 16 * s + 8 * g;
+          if (elem + 8 <= L) *reinterpret_cast<uint4*>(dxrow + elem) = pack8<DT>(oct);
+        }
+      }
+    }
+    cur ^= 1;
+    if (seg0 > 0) {
+      load_tiles(seg0 - kBwdNC);
+      lds_barrier();  // the next segment's (G, G') overwrite the rows read above
+    }
+  }
+
+  // ---- reductions over the workgroup --------------------------------------------------------
+  // W, W': over the 32 lanes (chunks) of a half wave, then over the waves
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    wacc[i].x = group_sum<32>(wacc[i].x);
+    wacc[i].y = group_sum<32>(wacc[i].y);
+    wdacc[i].x = group_sum<32>(wdacc[i].x);
+    wdacc[i].y = group_sum<32>(wdacc[i].y);
+  }
+  if (r == 0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      sm.red[wave][g][4 * i] = wacc[i].x;
+      sm.red[wave][g][4 * i + 1] = wacc[i].y;
+      sm.red[wave][g][4 * i + 2] = wdacc[i].x;
+      sm.red[wave][g][4 * i + 3] = wdacc[i].y;
+    }
+  }
+  __syncthreads();  // every wave is done with the state buffer and its staging tile
+  float* mcopy = reinterpret_cast<float*>(smem_raw + kOffR);  // [wave][tile][register][lane]
+#pragma unroll
+  for (int t = 0; t < 3; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mcopy[((wave * 3 + t) * 16 + i) * kWave + lane] = macc[t][i];
+  __syncthreads();
+  float* dpart = mcopy + kWaves * 3 * 16 * kWave;  // [wave][l]
+  {
+    // dkin[l] = sum_j M[j + l][j]: thread (l, wave copy) walks the l-th diagonal of its copy
+    const int l = tid & 63, wv = tid >> 6;
+    float acc = 0.f;
+    for (int j = 0; j + l < kT; ++j) {
+      const int i = j + l, t = (i >> 5) + (j >> 5), ii = i & 31;
+      const int reg = 4 * (ii >> 3) + (ii & 3), ln = 32 * ((ii >> 2) & 1) + (j & 31);
+      acc += mcopy[((wv * 3 + t) * 16 + reg) * kWave + ln];
+    }
+    dpart[wv * kT + l] = acc;
+  }
+  __syncthreads();
+  if (tid < kT) sm.dkin[tid] = (dpart[tid] + dpart[kT + tid]) + (dpart[2 * kT + tid] + dpart[3 * kT + tid]);
+  __syncthreads();
+  {
+    // A_in = sum_l q^l dkin[l], B_in = sum_l l q^(l-1) dkin[l]: thread (n, a) takes l = 4 a .. 4 a + 3
+    cf ain{0.f, 0.f}, bin{0.f, 0.f};
+    if (sn < N) {
+      const cf q1 = qpow(lq.x, lq.y, 1);
+      cf v = qpow(lq.x, lq.y, 4 * sa);
+      cf u = sa > 0 ? qpow(lq.x, lq.y, 4 * sa - 1) : cf{0.f, 0.f};  // q^(l-1); the l = 0 term is zero
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int l = 4 * sa + e;
+        const float dk = sm.dkin[l];
+        ain.x = fmaf(dk, v.x, ain.x);
+        ain.y = fmaf(dk, v.y, ain.y);
+        const float dl = dk * static_cast<float>(l);
+        bin.x = fmaf(dl, u.x, bin.x);
+        bin.y = fmaf(dl, u.y, bin.y);
+        u = (l == 0) ? cf{1.f, 0.f} : cmul(u, q1);
+        v = cmul(v, q1);
+      }
+    }
+    sm.ab[sa][0][sn] = ain;
+    sm.ab[sa][1][sn] = bin;
+  }
+  __syncthreads();
+  if (tid < N) {
+    const int n = tid;
+    cf ain{0.f, 0.f}, bin{0.f, 0.f};
+    for (int a = 0; a < 16; ++a) {
+      ain = cadd(ain, sm.ab[a][0][n]);
+      bin = cadd(bin, sm.ab[a][1][n]);
+    }
+    // mode n sits in half g = (n >> 1) & 1 at index 2 (n >> 2) + (n & 1)
+    const int hg = (n >> 1) & 1, idx = 2 * (n >> 2) + (n & 1);
+    cf w{0.f, 0.f}, wd{0.f, 0.f};
+    for (int wv = 0; wv < kWaves; ++wv) {
+      w.x += sm.red[wv][hg][4 * idx];
+      w.y += sm.red[wv][hg][4 * idx + 1];
+      wd.x += sm.red[wv][hg][4 * idx + 2];
+      wd.y += sm.red[wv][hg][4 * idx + 3];
+    }
+    const cf q1 = qpow(lq.x, lq.y, 1);
+    const cf A = cadd(ain, cmul(q1, w));
+    const cf Bq = cadd(cadd(bin, w), cmul(q1, wd));
+    const cf gm = sm.gn[n];
+    const float pp = sm.pn[n];
+    dp[row * N + n] = A.x * gm.x - A.y * gm.y;
+    const cf t = cmul(Bq, cf{pp * gm.x, pp * gm.y});
+    dq[row * N + n] = cf{t.x, -t.y};
+    dgamma[row * N + n] = cf{A.x * pp, -A.y * pp};
+  }
+  if (tid == 0) domega[row] = sm.dkin[0];
+}
+
+int launch_bwd(const void* dy, const void* x, void* dx, const float* p, const cf* log_q,
+               const cf* gamma, const float* omega, float* dp, cf* dq, cf* dgamma, float* domega,
+               int64_t B, int64_t D, int64_t N, int64_t L, hipStream_t stream) {
+  MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&cema_scan_bwd_kernel<MEGA_BF16>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds));
+  cema_scan_bwd_kernel<MEGA_BF16><<<dim3(static_cast<unsigned>(B * D)), kThreads, kBwdLds, stream>>>(
+      dy, x, dx, p, log_q, gamma, omega, dp, dq, dgamma, domega, static_cast<int>(D),
+      static_cast<int>(N), L);
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
+}
+
 }  // namespace
 }  // namespace mega
 
@@ -413,4 +900,28 @@ extern "C" int mega_cema_scan_fwd(const void* x, int dtype, const float* p, cons
   cf* hl = reinterpret_cast<cf*>(h_last);
   if (dtype == MEGA_BF16) return launch_fwd<MEGA_BF16, 2>(x, y, p, lq, gm, omega, h0c, hl, B, D, N, L, s);
   return launch_fwd<MEGA_F16, 1>(x, y, p, lq, gm, omega, h0c, hl, B, D, N, L, s);
+}
+
+extern "C" int mega_cema_scan_bwd_supported(int dtype, int64_t N, int64_t L) {
+  return dtype == MEGA_BF16 && N >= 1 && N <= 16 && L >= 8 && L % 8 == 0;
+}
+
+extern "C" int mega_cema_scan_bwd(const void* dy, const void* x, int dtype, const float* p,
+                                  const float* log_q, const float* gamma, const float* omega,
+                                  int64_t B, int64_t D, int64_t N, int64_t L, void* dx, float* dp,
+                                  float* dq, float* dgamma, float* domega, void* stream) {
+  const char* who = "mega_cema_scan_bwd";
+  MEGA_CHECK_ARG(dy && x && p && log_q && gamma && dx && dp && dq && dgamma && domega, "%s: null pointer", who);
+  MEGA_CHECK_ARG(B >= 0 && D >= 0 && L >= 0, "%s: negative size", who);
+  MEGA_CHECK_ARG(B * D <= 0x7fffffff, "%s: too many rows", who);
+  if (!mega_cema_scan_bwd_supported(dtype, N, L))
+    return set_error(MEGA_ERR_UNSUPPORTED,
+                     "%s: needs bfloat16 rows, N <= 16 and L a multiple of 8 (dtype %d, N %lld, L %lld)", who,
+                     dtype, (long long)N, (long long)L);
+  const auto al = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  MEGA_CHECK_ARG(al(dy) && al(x) && al(dx), "%s: dy, x and dx must be 16-byte aligned", who);
+  if (B == 0 || D == 0) return MEGA_OK;
+  return launch_bwd(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
+                    omega, dp, reinterpret_cast<cf*>(dq), reinterpret_cast<cf*>(dgamma), domega, B, D, N, L,
+                    static_cast<hipStream_t>(stream));
 }

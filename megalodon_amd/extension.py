@@ -545,6 +545,49 @@ def cema_scan_fwd(x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor, gamma: 
     return y, h_last
 
 
+def cema_scan_bwd_supported(x: torch.Tensor, ndim: int) -> bool:
+    """Whether `cema_scan_bwd` takes this input (bfloat16 rows; otherwise as the forward)."""
+    if not x.is_cuda or x.dim() != 3 or x.dtype != torch.bfloat16:
+        return False
+    fn = _lib.load().mega_cema_scan_bwd_supported
+    return bool(fn(_lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(ndim), _lib.i64(x.shape[-1])))
+
+
+def cema_scan_bwd(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor,
+                  gamma: torch.Tensor, omega: Optional[torch.Tensor]):
+    """(dx, dp, dq, dgamma, domega) of ``cema_scan_fwd(x, p, log_q, gamma, omega)[0]``
+    (no carried state): dp (D, N) float32, dq and dgamma (D, N) complex64 in
+    the convention of ``ema_parameters_bwd`` (gradient w.r.t. q, conjugated),
+    domega (D,) float32."""
+    dev = _require_cuda(y_grad, x, p, log_q, gamma, omega)
+    B, D, L = x.shape
+    N = p.shape[1]
+    if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
+        raise RuntimeError("cema_scan_bwd: y_grad must match x in shape and dtype")
+
+    def aligned(t):
+        t = t.contiguous()
+        return t if t.data_ptr() % 16 == 0 else t.clone(memory_format=torch.contiguous_format)
+
+    dy, xc = aligned(y_grad), aligned(x)
+    pc = p.reshape(D, N).contiguous().float()
+    lq, gm = _as_c64(log_q, "log_q").reshape(D, N), _as_c64(gamma, "gamma").reshape(D, N)
+    wc = None if omega is None else omega.reshape(-1).contiguous().float()
+    dx = torch.empty_like(xc)
+    dp = torch.empty((B, D, N), dtype=torch.float32, device=dev)
+    dq = torch.empty((B, D, N), dtype=torch.complex64, device=dev)
+    dg = torch.empty((B, D, N), dtype=torch.complex64, device=dev)
+    dw = torch.empty((B, D), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_cema_scan_bwd", _lib.ptr(dy), _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
+                  _lib.ptr(pc), _lib.ptr(lq), _lib.ptr(gm), _lib.ptr(wc), _lib.i64(B), _lib.i64(D), _lib.i64(N),
+                  _lib.i64(L), _lib.ptr(dx), _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg), _lib.ptr(dw),
+                  _lib.stream_ptr(dev))
+    if B == 1:
+        return dx, dp[0], dq[0], dg[0], dw[0]
+    return dx, dp.sum(0), dq.sum(0), dg.sum(0), dw.sum(0)
+
+
 # --------------------------------------------------------------------------
 # group_timestep_norm (reference: csrc/ops/timestep_norm.cc:621-705)
 # --------------------------------------------------------------------------
