@@ -1,0 +1,44 @@
+"""The CEMA layer without a carried state as one autograd node over its raw
+parameters: the lines
+    p, q, gamma = self.coeffs()
+    k, b = ema_parameters(p, q, gamma, None, L)
+    out = fftconv(x, k) + x * self.omega
+of megalodon/modules/complex_exponential_moving_average.py:127-147, evaluated
+as a chunked recurrence (csrc/cema_scan.hip): two launches forward
+(coefficients, recurrence), two backward; neither the kernel row k nor dk nor
+any spectrum exists."""
+from typing import Tuple
+
+import torch
+from torch.autograd.function import FunctionCtx
+
+from .. import extension as megalodon_ops
+
+
+class CEMAScanFunc(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx: FunctionCtx, x: torch.Tensor, alpha: torch.Tensor, delta: torch.Tensor, theta: torch.Tensor,
+                gamma: torch.Tensor, omega: torch.Tensor) -> torch.Tensor:
+        p, log_q, gamma_hat = megalodon_ops.cema_coeffs_fwd(alpha, delta, theta, gamma)
+        y, _ = megalodon_ops.cema_scan_fwd(x, p, log_q, gamma_hat, omega)
+        ctx.save_for_backward(x, alpha, delta, theta, p, log_q, gamma_hat, omega)
+        return y
+
+    @staticmethod
+    def backward(ctx: FunctionCtx, y_grad: torch.Tensor) -> Tuple[torch.Tensor, ...]:
+        x, alpha, delta, theta, p, log_q, gamma_hat, omega = ctx.saved_tensors
+        dx, dp, dq, dg, dw = megalodon_ops.cema_scan_bwd(y_grad, x, p, log_q, gamma_hat, omega)
+        dalpha, ddelta, dtheta, dgamma = megalodon_ops.cema_coeffs_bwd(dp, dq, dg, alpha, delta, theta)
+        return dx, dalpha, ddelta, dtheta, dgamma, dw.to(omega.dtype).view_as(omega)
+
+
+cema_scan = CEMAScanFunc.apply
+
+
+def cema_scan_applicable(x: torch.Tensor, ndim: int, needs_grad: bool) -> bool:
+    """The recurrence kernels take bfloat16 / float16 rows of a length that is a
+    multiple of 8 with at most 16 modes; the backward kernel bfloat16 only."""
+    if needs_grad:
+        return megalodon_ops.cema_scan_bwd_supported(x, ndim)
+    return megalodon_ops.cema_scan_supported(x, ndim)

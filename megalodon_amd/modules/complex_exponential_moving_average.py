@@ -2,14 +2,20 @@
 (megalodon/modules/complex_exponential_moving_average.py:42-150), minus the
 `megalodon.distributed` look-ups: model-parallel world size is 1, so
 ``dim_per_partition == embed_dim`` and the theta permutation is drawn locally
-instead of being broadcast (:21-26)."""
+instead of being broadcast (:21-26).  16-bit inputs on the GPU run the layer as
+a chunked recurrence (fused_ops/cema_scan.py); MEGA_CEMA_FFT=1 in the
+environment keeps them on the kernel-row + FFT-convolution operators that
+float32 inputs use."""
 from typing import Optional, Tuple
 import math
+import os
 
 import torch
 from torch import nn
 
-from ..fused_ops import cema_kernel, ema_hidden, ema_parameters, fftconv_residual
+from .. import extension as megalodon_ops
+from ..fused_ops import (cema_kernel, cema_scan, cema_scan_applicable, ema_hidden, ema_parameters,
+                         fftconv_residual)
 
 
 @torch.no_grad()
@@ -81,7 +87,20 @@ class MultiHeadComplexEMA(nn.Module):
             # the reference's training forward goes through _calc_coeffs(), which drops the
             # coefficients cached for evaluation (:100-101,119-125); every branch below does the same
             self._coeffs = None
-        if hx is None and not compute_last_state and self.alpha.is_cuda:
+        stateless = hx is None and not compute_last_state
+        needs_grad = torch.is_grad_enabled() and (x.requires_grad or self.alpha.requires_grad
+                                                  or (hx is not None and hx.requires_grad))
+        if self.alpha.is_cuda and os.environ.get("MEGA_CEMA_FFT") is None:
+            # 16-bit rows: the layer as a chunked recurrence on the matrix cores (no kernel
+            # row, no transform); with a carried state only where no gradient is wanted
+            if stateless and cema_scan_applicable(x, self.ndim, needs_grad):
+                out = cema_scan(x, self.alpha.float(), self.delta.float(), self.theta.float(), self.gamma.float(),
+                                self.omega)
+                return out, None
+            if not stateless and not needs_grad and cema_scan_applicable(x, self.ndim, False):
+                p, q, gamma = self.coeffs()
+                return megalodon_ops.cema_scan_fwd(x, p, q.log(), gamma, self.omega, hx, compute_last_state)
+        if stateless and self.alpha.is_cuda:
             # no carried state: coefficients and kernel as one autograd node
             # (two launches per direction instead of the coefficient graph)
             k, b = cema_kernel(self.alpha.float(), self.delta.float(), self.theta.float(), self.gamma.float(),
