@@ -190,6 +190,27 @@ int mega_group_timestep_norm_fwd(const void* x, int dtype, const int64_t* prev_c
                                  float* cummean, float* cumrstd, void* workspace,
                                  void* stream);
 
+/* The forward above for callers that cannot allocate (code under graph
+ * capture, serving loops, harnesses that forbid it).  No counterpart in the
+ * reference, whose operators allocate their own scratch (torch::empty in
+ * timestep_norm_kernel.cu:1542-1565).  Same arguments without `workspace`: the
+ * tickets, per-tile counts and look-back records live in a static device
+ * array of mega_group_timestep_norm_static_scratch_bytes() (2 MiB) per GPU,
+ * held until the process ends.  Shapes whose
+ * mega_group_timestep_norm_workspace_bytes(B, L, D, G, 0) exceeds it return
+ * MEGA_ERR_UNSUPPORTED.  The call allocates and frees nothing and clears what
+ * it needs itself with a kernel; all calls on one GPU share the one array, so
+ * two calls that overlap on a GPU (different streams, different threads) race
+ * -- serialise them. */
+int64_t mega_group_timestep_norm_static_scratch_bytes(void);
+int mega_group_timestep_norm_fwd_static(const void* x, int dtype, const int64_t* prev_count,
+                                        const void* prev_mean, const void* prev_var,
+                                        const void* gamma, const void* beta,
+                                        const uint8_t* padding_mask, int64_t B, int64_t L,
+                                        int64_t D, int64_t G, double eps, void* y, int64_t* count,
+                                        void* mean, void* var, float* cummean, float* cumrstd,
+                                        void* stream);
+
 /* Replaces group_timestep_norm_bwd(dy, dmean, dvar, x, prev_mean, count,
  *   cummean, cumrstd, gamma, padding_mask?, num_groups)
  *   -> (dx, dprev_mean, dprev_var, dgamma, dbeta)

@@ -29,6 +29,8 @@
 // cost 190 us in tickets alone.)
 #include "common.hpp"
 
+#include <mutex>
+
 #include <algorithm>
 
 namespace mega {
@@ -1233,4 +1235,58 @@ extern "C" int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, c
     case MEGA_BF16: return tsn_bwd_impl<MEGA_BF16>(p, dgamma, dbeta, workspace, s);
     default: return tsn_bwd_impl<MEGA_F16>(p, dgamma, dbeta, workspace, s);
   }
+}
+
+// ---- forward without a caller workspace: a static device buffer ---------------------
+// Callers that may not allocate (graph capture, serving loops) get the
+// forward's scratch (tickets, per-tile counts, look-back records) from a
+// file-scope device array instead of a workspace argument.  Each GPU holds its
+// own copy of the array until the process ends; `scratch` itself is only the
+// host-side name of the symbol, so its device address is looked up once per
+// device and that pointer is what the kernels receive.
+constexpr int64_t kStaticScratchBytes = 2 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kScratchDevices = 64;
+void* g_scratch_ptr[kScratchDevices] = {};
+std::mutex g_scratch_mu;
+
+int static_scratch(void** out) {
+  int dev = 0;
+  MEGA_CHECK_HIP(hipGetDevice(&dev));
+  MEGA_CHECK_ARG(dev >= 0 && dev < kScratchDevices, "device index %d not supported", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    MEGA_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MEGA_OK;
+}
+}  // namespace
+
+extern "C" int64_t mega_group_timestep_norm_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int mega_group_timestep_norm_fwd_static(const void* x, int dtype, const int64_t* prev_count,
+                                                   const void* prev_mean, const void* prev_var,
+                                                   const void* gamma, const void* beta,
+                                                   const uint8_t* padding_mask, int64_t B, int64_t L,
+                                                   int64_t D, int64_t G, double eps, void* y,
+                                                   int64_t* count, void* mean, void* var,
+                                                   float* cummean, float* cumrstd, void* stream) {
+  int rc = check_dims("mega_group_timestep_norm_fwd_static", B, L, D, G);
+  if (rc != MEGA_OK) return rc;
+  const int64_t need = mega_group_timestep_norm_workspace_bytes(B, L, D, G, 0);
+  if (need > kStaticScratchBytes)
+    return set_error(MEGA_ERR_UNSUPPORTED,
+                     "mega_group_timestep_norm_fwd_static: this shape needs %lld bytes of scratch, the static "
+                     "buffer holds %lld; use mega_group_timestep_norm_fwd with a workspace",
+                     (long long)need, (long long)kStaticScratchBytes);
+  void* ptr = nullptr;
+  rc = static_scratch(&ptr);
+  if (rc != MEGA_OK) return rc;
+  return mega_group_timestep_norm_fwd(x, dtype, prev_count, prev_mean, prev_var, gamma, beta, padding_mask,
+                                      B, L, D, G, eps, y, count, mean, var, cummean, cumrstd, ptr, stream);
 }
