@@ -59,10 +59,40 @@ __device__ __forceinline__ void lds_barrier() {
 // a <-> b between the two halves of the wave (v_permlane32_swap_b32): afterwards
 // the low half holds (its own a, the high half's a), the high half (the low
 // half's b, its own b).  Written as inline assembly: the compiler's builtin
-// returned the first result for both outputs here.  The s_nop covers the wait
-// states the instruction needs after a vector write of its operands.
+// returned the first result for both outputs here.  The compiler does not
+// see what the assembly reads, so it guards none of the hazards: the s_nop
+// covers the wait states after a vector write of an operand, and operands
+// that come out of an MFMA must first pass through an ordinary vector
+// instruction (`settle`), which the compiler does schedule behind the MFMA.
 __device__ __forceinline__ void half_swap(float& a, float& b) {
   asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void half_swap(uint32_t& a, uint32_t& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+// two floats -> one word of two 16-bit elements of type DT
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  if (DT == MEGA_BF16) return pack_bf16x2(lo, hi);
+  return static_cast<uint32_t>(float_to_f16_bits(lo)) | (static_cast<uint32_t>(float_to_f16_bits(hi)) << 16);
+}
+// An accumulator tile (lane <-> chunk, register 4 qd + e <-> step 8 qd + 4 g + e of a 32-step
+// row tile) rounded to 16 bits and regrouped so that the lane of half g holds the 8
+// consecutive steps 16 pr + 8 g .. + 7: the rounding is the ordinary vector instruction
+// that separates the MFMA from the swaps (see half_swap).
+template <int DT>
+__device__ __forceinline__ uint4 octet_of(const floatx16& acc, int pr) {
+  uint32_t a0 = pack2<DT>(acc[8 * pr], acc[8 * pr + 1]), a1 = pack2<DT>(acc[8 * pr + 2], acc[8 * pr + 3]);
+  uint32_t b0 = pack2<DT>(acc[8 * pr + 4], acc[8 * pr + 5]), b1 = pack2<DT>(acc[8 * pr + 6], acc[8 * pr + 7]);
+  half_swap(a0, b0);
+  half_swap(a1, b1);
+  return make_uint4(a0, a1, b0, b1);
+}
+// 1.0f the optimiser cannot see through
+__device__ __forceinline__ float opaque_one() {
+  float one = 1.0f;
+  asm volatile("" : "+v"(one));
+  return one;
 }
 
 // Eight consecutive steps of a row as a matrix operand: XP bf16 pieces whose sum
@@ -116,257 +146,339 @@ template <int NT>
 struct FwdSmem {
   static constexpr int NC = kWaves * NT * 32;  // chunks per segment
   cf qp[16][kT + 2];                           // q_n^e, e = 0 .. 64
-  float klocal[kT];                            // k[0 .. 63]
+  float klocal[kT];                            // k[0 .. 63] (+ omega at lag 0)
   float pn[16];
   cf gn[16];
-  cf sub_end[kSubs][16];
+  cf sub_end[kSubs][16];                       // local end state of each sub-segment (4 per wave)
+  cf wave_end[2][kWaves][16];                  // local end state of each wave's 4 sub-segments, by item parity
+  float wave_cin[kWaves][32];                  // state in front of each wave's first chunk
   cf carry[2][16];
+  cf pw[12][16];                               // q^(4 k), q^(16 k) (k < 4), q, q^64, q^(64 CPS), q^(256 CPS)
   u32x4 aop[kFwdBlocks][2][kWave];
-  float H[(NC + 1) * kHP];                     // row 0: state before the segment, row 1 + c: after chunk c
+  float H[(NC + 1) * kHP];                     // row 1 + c: state after chunk c of the segment
 };
 
+// LDS traffic of one wave is processed in order: a wave that has written rows
+// and waits for its own LDS operations can read what its other lanes wrote.
+__device__ __forceinline__ void wave_sync() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
 template <int DT, int NT>
-__global__ __launch_bounds__(kThreads) void cema_scan_fwd_kernel(
+__global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
     const void* __restrict__ x, void* __restrict__ y, const float* __restrict__ p,
     const cf* __restrict__ log_q, const cf* __restrict__ gamma, const float* __restrict__ omega,
-    const cf* __restrict__ h0, cf* __restrict__ h_last, int D, int N, int64_t L) {
+    const cf* __restrict__ h0, cf* __restrict__ h_last, int64_t rows, int D, int N, int64_t L) {
   using Smem = FwdSmem<NT>;
   constexpr int NC = Smem::NC, CPS = NC / kSubs, XP = XOp<DT>::XP;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int g = lane >> 5, r = lane & 31;
-  const int64_t row = blockIdx.x;
-  const int d = static_cast<int>(row % D);
-  const uint16_t* xrow = static_cast<const uint16_t*>(x) + row * L;
-  uint16_t* yrow = static_cast<uint16_t*>(y) + row * L;
-  const float wres = omega != nullptr ? omega[d] : 0.f;
+  // scan roles: mode sn; sub-segment sa = 4 wave + sl of CPS chunks, inside the wave's own tiles
+  const int sn = tid & 15, sa = tid >> 4, sl = sa & 3;
   const int64_t C = (L + kT - 1) / kT;
 
-  // the first segment's rows are requested before the tables are built
-  XOp<DT> xb[NT][4];
-  auto load_tiles = [&](int64_t seg0) {
+  // The workgroup walks (row, segment) items: rows blockIdx.x, + gridDim.x, ...,
+  // the segments of a row in time order.  The x tiles of the next item and the
+  // parameters of the next row are requested ahead (two register sets for the
+  // tiles, swapped by taking the item body twice per loop turn).
+  auto load_tiles = [&](XOp<DT> (&t)[NT][4], int64_t row, int64_t seg0) {
+    const uint16_t* xrow = static_cast<const uint16_t*>(x) + row * L;
 #pragma unroll
     for (int ctl = 0; ctl < NT; ++ctl) {
       const int64_t chunk = seg0 + (wave * NT + ctl) * 32 + r;
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const int64_t elem = chunk * kT + 16 * s + 8 * g;
-        xb[ctl][s].load(xrow, elem, elem + 8 <= L);
+        t[ctl][s].load(xrow, elem, row < rows && elem + 8 <= L);
       }
     }
   };
-  load_tiles(0);
+  struct RowParams {
+    cf lq, gv, hv;
+    float pv, w;
+  };
+  auto fetch_params = [&](int64_t row) {
+    RowParams rp{cf{0.f, 0.f}, cf{0.f, 0.f}, cf{0.f, 0.f}, 0.f, 0.f};
+    if (row < rows) {
+      const int d = static_cast<int>(row % D);
+      if (sn < N) {
+        rp.lq = log_q[d * N + sn];
+        rp.gv = gamma[d * N + sn];
+        rp.pv = p[d * N + sn];
+        if (h0 != nullptr && tid < 16) rp.hv = h0[row * N + sn];
+      }
+      if (omega != nullptr) rp.w = omega[d];
+    }
+    return rp;
+  };
 
-  // ---- per-row tables ---------------------------------------------------------
-  const int sn = tid & 15, sa = tid >> 4;  // mode, and: power group here, sub-segment in the scan
-  {
-    cf v{0.f, 0.f}, q1{0.f, 0.f};
-    if (sn < N) {
-      const cf lq = log_q[d * N + sn];
-      v = qpow(lq.x, lq.y, 4 * sa);
-      q1 = qpow(lq.x, lq.y, 1);
+  cf qT{0.f, 0.f}, qS{0.f, 0.f}, qW{0.f, 0.f};
+  int cur = 0, par = 0;
+  RowParams rp = fetch_params(blockIdx.x);
+
+  // tables, operand blocks and scan multipliers of a row's channel, from the
+  // parameters fetched ahead; then the next row's parameters are requested
+  auto setup_row = [&](int64_t row) {
+    // the few powers that are evaluated directly (phase reduced in float64): 12 per mode;
+    // everything else is a product of two of them and a short chain of multiplications
+    cf direct{0.f, 0.f};
+    if (tid < 12 * 16 && sn < N) {
+      const int k = tid >> 4;
+      const int e = k < 4 ? 4 * k
+                          : (k < 8 ? 16 * (k - 4) : (k == 8 ? 1 : (k == 9 ? kT : (k == 10 ? kT * CPS : 4 * kT * CPS))));
+      direct = qpow(rp.lq.x, rp.lq.y, e);
     }
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      sm.qp[sn][4 * sa + e] = v;
-      v = cmul(v, q1);
-    }
-    if (sa == 15) sm.qp[sn][kT] = v;
+    __syncthreads();  // every wave is done with the previous row's tables and carried state
+    if (tid < 12 * 16) sm.pw[tid >> 4][sn] = direct;
     if (tid < 16) {
-      sm.pn[tid] = tid < N ? p[d * N + tid] : 0.f;
-      sm.gn[tid] = tid < N ? gamma[d * N + tid] : cf{0.f, 0.f};
-      sm.carry[0][tid] = (h0 != nullptr && tid < N) ? h0[row * N + tid] : cf{0.f, 0.f};
+      sm.pn[tid] = rp.pv;
+      sm.gn[tid] = rp.gv;
+      sm.carry[0][tid] = rp.hv;
     }
-  }
-  // q^64 and q^(64 CPS) for the scan
-  cf qT{0.f, 0.f}, qS{0.f, 0.f};
-  if (sn < N) {
-    const cf lq = log_q[d * N + sn];
-    qT = qpow(lq.x, lq.y, kT);
-    qS = qpow(lq.x, lq.y, kT * CPS);
-  }
-  __syncthreads();
-  if (tid < kT) {
-    float acc = 0.f;
-#pragma unroll
-    for (int n = 0; n < 16; ++n) {
-      const cf c = cmul(cf{sm.pn[n] * sm.gn[n].x, sm.pn[n] * sm.gn[n].y}, sm.qp[n][tid]);
-      acc += c.x;
-    }
-    sm.klocal[tid] = acc;
-  }
-  __syncthreads();
-  for (int item = tid; item < kFwdBlocks * kWave; item += kThreads) {
-    const int blk = item >> 6, ln = item & 63, rr = ln & 31, gg = ln >> 5;
-    float v[8];
-    if (blk < 4) {
-      const int n = rr >> 1, part = rr & 1;
-      const float pp = sm.pn[n];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const cf w = sm.qp[n][kT - 1 - (16 * blk + 8 * gg + e)];
-        v[e] = pp * (part ? w.y : w.x);
-      }
-    } else if (blk < 8) {
-      const int o = 16 * (blk - 5);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int lag = o + rr - 8 * gg - e;
-        v[e] = lag >= 0 ? sm.klocal[lag] : 0.f;
-      }
-    } else {
-      const int it = (blk - 8) >> 1, s2 = (blk - 8) & 1, i = 32 * it + rr;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int m = 16 * s2 + 8 * gg + e, n = m >> 1;
-        const cf w = cmul(sm.gn[n], sm.qp[n][i + 1]);
-        v[e] = (m & 1) ? -w.y : w.x;
-      }
-    }
-    u32x4 hi, lo;
-    split8(v, hi, lo);
-    sm.aop[blk][0][ln] = hi;
-    sm.aop[blk][1][ln] = lo;
-  }
-  __syncthreads();
-  u32x4 A[kFwdBlocks][2];
-#pragma unroll
-  for (int b = 0; b < kFwdBlocks; ++b) {
-    A[b][0] = sm.aop[b][0][lane];
-    A[b][1] = sm.aop[b][1][lane];
-  }
-
-  int cur = 0;
-  for (int64_t seg0 = 0; seg0 < C; seg0 += NC) {
-    const int nc = static_cast<int>(C - seg0 < NC ? C - seg0 : NC);
-    // ---- local states S = P X ---------------------------------------------------
-#pragma unroll
-    for (int ctl = 0; ctl < NT; ++ctl) {
-      const int c0 = (wave * NT + ctl) * 32;
-      if (c0 < nc) {
-        floatx16 acc;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) acc = mma_split<XP>(A[s], xb[ctl][s].pc, acc);
-        float* dst = sm.H + (1 + c0 + r) * kHP + 4 * g;
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd)
-          *reinterpret_cast<float4*>(dst + 8 * qd) =
-              make_float4(acc[4 * qd], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3]);
-      }
-    }
-    lds_barrier();
-    // ---- scan over the chunks of the segment --------------------------------------
+    cur = 0;
+    __syncthreads();
     {
-      float* col = sm.H + kHP + 2 * sn;  // state column n of row 1 + c
-      cf h{0.f, 0.f};
-#pragma unroll 4
-      for (int i = 0; i < CPS; ++i) {
-        const int c = sa * CPS + i;
-        if (c < nc) {
-          const float2 s = *reinterpret_cast<const float2*>(col + c * kHP);
-          h = cadd(cmul(qT, h), cf{s.x, s.y});
-        }
+      // q^(4 sa + e), e < 4, and this mode's share of k at those lags, summed over the
+      // 16 modes (the 16 lanes of a row): the skip term omega x rides on k[0]
+      cf v = cmul(sm.pw[sa & 3][sn], sm.pw[4 + (sa >> 2)][sn]);
+      const cf q1 = sm.pw[8][sn];
+      const cf c{rp.pv * rp.gv.x, rp.pv * rp.gv.y};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        sm.qp[sn][4 * sa + e] = v;
+        const float kl = group_sum<16>(c.x * v.x - c.y * v.y);
+        if (sn == 0) sm.klocal[4 * sa + e] = (sa == 0 && e == 0) ? kl + rp.w : kl;
+        v = cmul(v, q1);
       }
-      sm.sub_end[sa][sn] = h;
-      lds_barrier();
-      cf cin = sm.carry[cur][sn];
-      for (int s = 0; s < sa; ++s) cin = cadd(cmul(qS, cin), sm.sub_end[s][sn]);
-      if (sa == 0) *reinterpret_cast<float2*>(sm.H + 2 * sn) = make_float2(cin.x, cin.y);
-      h = cin;
-#pragma unroll 4
-      for (int i = 0; i < CPS; ++i) {
-        const int c = sa * CPS + i;
-        if (c < nc) {
-          const float2 s = *reinterpret_cast<const float2*>(col + c * kHP);
-          h = cadd(cmul(qT, h), cf{s.x, s.y});
-          *reinterpret_cast<float2*>(col + c * kHP) = make_float2(h.x, h.y);
-        }
-      }
-      if (sa == kSubs - 1) sm.carry[cur ^ 1][sn] = h;
+      if (sa == 15) sm.qp[sn][kT] = sm.pw[9][sn];
+      qT = sm.pw[9][sn];
+      qS = sm.pw[10][sn];
+      qW = sm.pw[11][sn];
     }
-    lds_barrier();
-    // ---- Y = K X + Q H[c-1] (+ omega x), written from the accumulators ---------------
+    const RowParams next_rp = fetch_params(row + gridDim.x);
+    __syncthreads();
+    for (int item = tid; item < kFwdBlocks * kWave; item += kThreads) {
+      const int blk = item >> 6, ln = item & 63, rr = ln & 31, gg = ln >> 5;
+      float v[8];
+      if (blk < 4) {
+        const int n = rr >> 1, part = rr & 1;
+        const float pp = sm.pn[n];
 #pragma unroll
-    for (int ctl = 0; ctl < NT; ++ctl) {
-      const int c0 = (wave * NT + ctl) * 32;
-      if (c0 < nc) {
-        u32x4 hb[2][2];
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          const float* src = sm.H + (c0 + r) * kHP + 16 * s2 + 8 * g;
-          const float4 u = *reinterpret_cast<const float4*>(src);
-          const float4 w = *reinterpret_cast<const float4*>(src + 4);
-          const float v[8] = {u.x, u.y, u.z, u.w, w.x, w.y, w.z, w.w};
-          split8(v, hb[s2][0], hb[s2][1]);
+        for (int e = 0; e < 8; ++e) {
+          const cf w = sm.qp[n][kT - 1 - (16 * blk + 8 * gg + e)];
+          v[e] = pp * (part ? w.y : w.x);
         }
-        const int64_t chunk = seg0 + c0 + r;
+      } else if (blk < 8) {
+        const int o = 16 * (blk - 5);
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
+        for (int e = 0; e < 8; ++e) {
+          const int lag = o + rr - 8 * gg - e;
+          v[e] = lag >= 0 ? sm.klocal[lag] : 0.f;
+        }
+      } else {
+        const int it = (blk - 8) >> 1, s2 = (blk - 8) & 1, i = 32 * it + rr;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int m = 16 * s2 + 8 * gg + e, n = m >> 1;
+          const cf w = cmul(sm.gn[n], sm.qp[n][i + 1]);
+          v[e] = (m & 1) ? -w.y : w.x;
+        }
+      }
+      u32x4 hi, lo;
+      split8(v, hi, lo);
+      sm.aop[blk][0][ln] = hi;
+      sm.aop[blk][1][ln] = lo;
+    }
+    __syncthreads();
+    rp = next_rp;
+  };
+  // The operand blocks stay in LDS and are read where a phase needs them (P for the local
+  // states, K and Q for the outputs): held in registers across the whole item they cost
+  // 96 registers and spill.
+  auto load_block = [&](int b, u32x4* dst) {
+    dst[0] = sm.aop[b][0][lane];
+    dst[1] = sm.aop[b][1][lane];
+  };
+
+  // One (row, segment) item.  The item's x tiles were requested by the previous item (or
+  // the prologue); everything that reads them -- the local states and the K X part of the
+  // outputs -- comes first, then the same registers are reloaded with the next item's tiles
+  // while the scan and the state part of the outputs run.
+  XOp<DT> xb[NT][4];
+  auto item = [&](int64_t row, int64_t seg0) {
+    if (seg0 == 0) setup_row(row);
+    uint16_t* yrow = static_cast<uint16_t*>(y) + row * L;
+    const int nc = static_cast<int>(C - seg0 < NC ? C - seg0 : NC);
+    floatx16 yacc[NT][2];
+    // ---- local states S = P X, into this wave's own rows of the state buffer ----------
+    {
+      u32x4 P[4][2];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) load_block(s, P[s]);
+#pragma unroll
+      for (int ctl = 0; ctl < NT; ++ctl) {
+        const int c0 = (wave * NT + ctl) * 32;
+        if (c0 < nc) {
           floatx16 acc;
 #pragma unroll
           for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
-          for (int s = 0; s < 2 + 2 * it; ++s) acc = mma_split<XP>(A[5 + 2 * it - s], xb[ctl][s].pc, acc);
+          for (int s = 0; s < 4; ++s) acc = mma_split<XP>(P[s], xb[ctl][s].pc, acc);
+          float* dst = sm.H + (1 + c0 + r) * kHP + 4 * g;
+#pragma unroll
+          for (int qd = 0; qd < 4; ++qd)
+            *reinterpret_cast<float4*>(dst + 8 * qd) =
+                make_float4(acc[4 * qd], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3]);
+        }
+      }
+    }
+    // ---- the within-chunk part of the outputs, K X (omega x included: K carries omega on
+    //      its diagonal); the accumulators wait for the state part ------------------------
+    {
+      u32x4 K[4][2];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) load_block(4 + b, K[b]);
+#pragma unroll
+      for (int ctl = 0; ctl < NT; ++ctl)
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) yacc[ctl][it][i] = 0.f;
+          if ((wave * NT + ctl) * 32 < nc) {
+#pragma unroll
+            for (int s = 0; s < 2 + 2 * it; ++s)
+              yacc[ctl][it] = mma_split<XP>(K[1 + 2 * it - s], xb[ctl][s].pc, yacc[ctl][it]);
+          }
+        }
+    }
+    {
+      int64_t nrow = row, nseg = seg0 + NC;
+      if (nseg >= C) {
+        nrow = row + gridDim.x;
+        nseg = 0;
+      }
+      load_tiles(xb, nrow, nseg);
+    }
+    wave_sync();
+    // ---- scan over the chunks of the segment: a sub-segment per 16 lanes, the wave's four
+    //      sub-segments are its own chunks; one workgroup barrier hands over the waves' ends -----
+    {
+      float* col = sm.H + kHP + 2 * sn;  // state column n of row 1 + c
+      float2 sv[CPS];                    // the sub-segment's local states, kept for the second pass
+#pragma unroll
+      for (int i = 0; i < CPS; ++i) {
+        const int c = sa * CPS + i;
+        sv[i] = c < nc ? *reinterpret_cast<const float2*>(col + c * kHP) : make_float2(0.f, 0.f);
+      }
+      cf h{0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < CPS; ++i) h = cadd(cmul(qT, h), cf{sv[i].x, sv[i].y});
+      sm.sub_end[sa][sn] = h;
+      wave_sync();
+      if (sl == 3) {
+        cf e = sm.sub_end[sa - 3][sn];
+        e = cadd(cmul(qS, e), sm.sub_end[sa - 2][sn]);
+        e = cadd(cmul(qS, e), sm.sub_end[sa - 1][sn]);
+        sm.wave_end[par][wave][sn] = cadd(cmul(qS, e), h);
+      }
+      lds_barrier();
+      cf cin = sm.carry[cur][sn];
+#pragma unroll
+      for (int w = 0; w < kWaves - 1; ++w) {
+        const cf e = sm.wave_end[par][w][sn];
+        if (w < wave) cin = cadd(cmul(qW, cin), e);
+      }
+      if (sa == kSubs - 1) sm.carry[cur ^ 1][sn] = cadd(cmul(qW, cin), sm.wave_end[par][kWaves - 1][sn]);
+      if (sl == 0) *reinterpret_cast<float2*>(sm.wave_cin[wave] + 2 * sn) = make_float2(cin.x, cin.y);
+#pragma unroll
+      for (int s = 0; s < 3; ++s) {
+        const cf e = sm.sub_end[4 * wave + s][sn];
+        if (s < sl) cin = cadd(cmul(qS, cin), e);
+      }
+      h = cin;
+#pragma unroll
+      for (int i = 0; i < CPS; ++i) {
+        const int c = sa * CPS + i;
+        h = cadd(cmul(qT, h), cf{sv[i].x, sv[i].y});
+        if (c < nc) *reinterpret_cast<float2*>(col + c * kHP) = make_float2(h.x, h.y);
+      }
+    }
+    wave_sync();
+    // ---- the state part of the outputs, Q H[c-1], and the stores ------------------------------
+    {
+      u32x4 Q[4][2];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) load_block(8 + b, Q[b]);
+#pragma unroll
+      for (int ctl = 0; ctl < NT; ++ctl) {
+        const int c0 = (wave * NT + ctl) * 32;
+        if (c0 < nc) {
+          u32x4 hb[2][2];
+          // the state in front of chunk c0 + r: the previous row of the buffer, or, for the
+          // wave's first chunk, what the scan left in wave_cin
+          const float* hrow = (ctl == 0 && r == 0) ? sm.wave_cin[wave] : sm.H + (c0 + r) * kHP;
 #pragma unroll
           for (int s2 = 0; s2 < 2; ++s2) {
-            acc = mfma_bf16(A[8 + 2 * it + s2][0], hb[s2][0], acc);
-            acc = mfma_bf16(A[8 + 2 * it + s2][1], hb[s2][0], acc);
-            acc = mfma_bf16(A[8 + 2 * it + s2][0], hb[s2][1], acc);
+            const float* src = hrow + 16 * s2 + 8 * g;
+            const float4 u = *reinterpret_cast<const float4*>(src);
+            const float4 w = *reinterpret_cast<const float4*>(src + 4);
+            const float v[8] = {u.x, u.y, u.z, u.w, w.x, w.y, w.z, w.w};
+            split8(v, hb[s2][0], hb[s2][1]);
           }
+          const int64_t chunk = seg0 + c0 + r;
 #pragma unroll
-          for (int pr = 0; pr < 2; ++pr) {
-            float oct[8];
+          for (int it = 0; it < 2; ++it) {
+            floatx16 acc = yacc[ctl][it];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              oct[e] = acc[8 * pr + e];
-              oct[4 + e] = acc[8 * pr + 4 + e];
-              half_swap(oct[e], oct[4 + e]);
+            for (int s2 = 0; s2 < 2; ++s2) {
+              acc = mfma_bf16(Q[2 * it + s2][0], hb[s2][0], acc);
+              acc = mfma_bf16(Q[2 * it + s2][1], hb[s2][0], acc);
+              acc = mfma_bf16(Q[2 * it + s2][0], hb[s2][1], acc);
             }
-            const int s = 2 * it + pr;
-            float xv[8];
-            xb[ctl][s].values(xv);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) oct[e] = fmaf(wres, xv[e], oct[e]);
-            const int64_t elem = chunk * kT + 16 * s + 8 * g;
-            if (elem + 8 <= L) *reinterpret_cast<uint4*>(yrow + elem) = pack8<DT>(oct);
+            for (int pr = 0; pr < 2; ++pr) {
+              const uint4 oct = octet_of<DT>(acc, pr);
+              const int64_t elem = chunk * kT + 16 * (2 * it + pr) + 8 * g;
+              if (elem + 8 <= L) *reinterpret_cast<uint4*>(yrow + elem) = oct;
+            }
           }
         }
       }
     }
     cur ^= 1;
-    if (seg0 + NC < C) {
-      load_tiles(seg0 + NC);
-      lds_barrier();  // the next segment's local states overwrite the rows read above
-    }
-  }
-
-  if (h_last != nullptr) {
-    __syncthreads();
-    if (tid < N) {
-      // state after step L - 1: the last chunk may be partial
-      const int64_t seg_last = (C - 1) / NC * NC;
-      const int rem = static_cast<int>(L - (C - 1) * kT);  // 1 .. 64 steps in the last chunk
-      // row C - 1 - seg_last of the state buffer is H[C-2], the next one H[C-1]
-      const float* prev = sm.H + static_cast<int>(C - 1 - seg_last) * kHP + 2 * tid;
-      cf h;
-      if (rem == kT) {
-        h = cf{prev[kHP], prev[kHP + 1]};
-      } else {
-        h = cmul(sm.qp[tid][rem], cf{prev[0], prev[1]});
-        const float pp = sm.pn[tid];
-        for (int j = 0; j < rem; ++j) {
-          const float xv = Elem<DT>::load(xrow + (C - 1) * kT + j) * pp;
-          const cf w = sm.qp[tid][rem - 1 - j];
-          h.x = fmaf(xv, w.x, h.x);
-          h.y = fmaf(xv, w.y, h.y);
+    par ^= 1;
+    if (seg0 + NC >= C && h_last != nullptr) {
+      // the row's last segment: the state after step L - 1 (the last chunk may be partial)
+      lds_barrier();
+      if (tid < N) {
+        const uint16_t* xrow = static_cast<const uint16_t*>(x) + row * L;
+        const int rem = static_cast<int>(L - (C - 1) * kT);  // 1 .. 64 steps in the last chunk
+        const int cl = static_cast<int>(C - 1 - seg0);       // the last chunk inside this segment
+        cf h;
+        if (rem == kT) {
+          const float* lastrow = sm.H + (1 + cl) * kHP + 2 * tid;
+          h = cf{lastrow[0], lastrow[1]};
+        } else {
+          // H[C-2]: the row in front of the last chunk, or the wave's carried-in state
+          const float* prev = (cl % (NT * 32) == 0) ? sm.wave_cin[cl / (NT * 32)] + 2 * tid
+                                                    : sm.H + cl * kHP + 2 * tid;
+          h = cmul(sm.qp[tid][rem], cf{prev[0], prev[1]});
+          const float pp = sm.pn[tid];
+          for (int j = 0; j < rem; ++j) {
+            const float xv = Elem<DT>::load(xrow + (C - 1) * kT + j) * pp;
+            const cf w = sm.qp[tid][rem - 1 - j];
+            h.x = fmaf(xv, w.x, h.x);
+            h.y = fmaf(xv, w.y, h.y);
+          }
         }
+        h_last[row * N + tid] = h;
       }
-      h_last[row * N + tid] = h;
     }
-  }
+  };
+
+  load_tiles(xb, blockIdx.x, 0);
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x)
+    for (int64_t seg0 = 0; seg0 < C; seg0 += NC) item(row, seg0);
 }
 
 template <int DT, int NT>
@@ -376,8 +488,13 @@ int launch_fwd(const void* x, void* y, const float* p, const cf* log_q, const cf
   const size_t lds = sizeof(FwdSmem<NT>);
   MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&cema_scan_fwd_kernel<DT, NT>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-  cema_scan_fwd_kernel<DT, NT><<<dim3(static_cast<unsigned>(B * D)), kThreads, lds, stream>>>(
-      x, y, p, log_q, gamma, omega, h0, h_last, static_cast<int>(D), static_cast<int>(N), L);
+  int dev = 0, cus = 0;
+  MEGA_CHECK_HIP(hipGetDevice(&dev));
+  MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  const int64_t rows = B * D, slots = 2 * static_cast<int64_t>(cus);  // two workgroups fit a compute unit
+  const unsigned grid = static_cast<unsigned>(rows < slots ? rows : slots);
+  cema_scan_fwd_kernel<DT, NT><<<dim3(grid), kThreads, lds, stream>>>(
+      x, y, p, log_q, gamma, omega, h0, h_last, rows, static_cast<int>(D), static_cast<int>(N), L);
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
 }
@@ -459,6 +576,7 @@ __global__ __launch_bounds__(kThreads) void cema_scan_bwd_kernel(
   const float wres = omega != nullptr ? omega[d] : 0.f;
   const int64_t C = (L + kT - 1) / kT;
   const int64_t seg_last = (C - 1) / kBwdNC * kBwdNC;
+  const float one = opaque_one();
 
   XOp<DT> db[4], xb[4];
   auto load_tiles = [&](int64_t seg0) {
@@ -699,11 +817,15 @@ __global__ __launch_bounds__(kThreads) void cema_scan_bwd_kernel(
           xacc[kind] = mma_split<1>(a, &xr[s], xacc[kind]);
         }
       }
+      // chunks past the end of the row have X = 0, but their rows of the state buffer were
+      // never written and may hold anything: they are taken as zero
       const float* rnext = rbuf + (c0 + r + 1) * kRP + 4 * g;
+      const bool live = c0 + r < nc;
+      const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
-        const float4 rv = *reinterpret_cast<const float4*>(rnext + 8 * qd);
-        const float4 rd = *reinterpret_cast<const float4*>(rnext + 32 + 8 * qd);
+        const float4 rv = live ? *reinterpret_cast<const float4*>(rnext + 8 * qd) : zero4;
+        const float4 rd = live ? *reinterpret_cast<const float4*>(rnext + 32 + 8 * qd) : zero4;
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
           const cf xv{xacc[0][4 * qd + 2 * b], xacc[0][4 * qd + 2 * b + 1]};
@@ -743,8 +865,8 @@ __global__ __launch_bounds__(kThreads) void cema_scan_bwd_kernel(
           float oct[8];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            oct[e] = acc[8 * pr + e];
-            oct[4 + e] = acc[8 * pr + 4 + e];
+            oct[e] = acc[8 * pr + e] * one;
+            oct[4 + e] = acc[8 * pr + 4 + e] * one;
             half_swap(oct[e], oct[4 + e]);
           }
           const int s = 2 * jt + pr;
