@@ -88,6 +88,13 @@ __device__ __forceinline__ uint4 octet_of(const floatx16& acc, int pr) {
   half_swap(a1, b1);
   return make_uint4(a0, a1, b0, b1);
 }
+// Makes a lane-derived value opaque to the optimiser.  Offsets, masks and converted indices
+// depend only on the lane, not on the row: left alone they are hoisted out of the persistent
+// row loop into hundreds of spilled registers; recomputing them per item is cheaper.
+__device__ __forceinline__ int opaque(int v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
 // 1.0f the optimiser cannot see through
 __device__ __forceinline__ float opaque_one() {
   float one = 1.0f;
@@ -511,18 +518,20 @@ int launch_fwd(const void* x, void* y, const float* p, const cf* log_q, const cf
 //   R[c]  = G[c] + q^64 R[c+1],   R'[c] = G'[c] + 64 q^63 R[c+1] + q^64 R'[c+1]      (scan)
 //   (X, X')[c]   = Pg XR[c]
 //   W  = sum_c X[c] R[c+1],   W' = sum_c (X'[c] R[c+1] + X[c] R'[c+1])
-//   DX[c] = K^T DY[c] + Qd R[c+1],   Qd[j][m] = (Re, -Im)(c_n q_n^(64-j))
+//   DX[c] = K^T DY[c] + Qd R[c+1],   Qd[j][m] = (Re, -Im)(c_n q_n^(64-j)),  omega on the diagonal of K
 //   M     = sum_c DY[c]^T X[c]   (64 x 64, rows i >= columns j), dkin[l] = sum_j M[j+l][j]
 //   A = sum_l q^l dkin[l] + q W,   B = sum_l l q^(l-1) dkin[l] + W + q W'
 // Segments of 128 chunks are taken from the end of the row to its start; a
 // wave holds one chunk tile of the segment.  The chunk-contracted product M
 // needs operands with chunks along k: the wave parks its DY and X tiles in a
 // private LDS tile and reads them back with the transposing LDS read; the same
-// tile hands out the time-reversed x operand.
+// tile hands out the time-reversed x operand.  Everything that reads the dy
+// and x tiles comes before the scan, so the next item's tiles load under it.
 constexpr int kRP = 68;       // floats per row of the reverse-state buffer: (R, R') = 64 + 4
 constexpr int kSP = 72;       // 16-bit elements per row of a wave's staging tile: 64 + 8
 constexpr int kBwdNC = kWaves * 32;  // chunks per segment
 constexpr int kBwdCPS = kBwdNC / kSubs;
+constexpr int kBwdBlocks = 16;  // Pg 0..7 (kind, k-step), K^T 8..11 (by offset), Qd 12..15 (row tile, k-step)
 
 typedef short short4v __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint2 lds_read_tr(const uint16_t* q) {
@@ -531,263 +540,323 @@ __device__ __forceinline__ uint2 lds_read_tr(const uint16_t* q) {
   return __builtin_bit_cast(uint2, v);
 }
 
-// LDS of the backward kernel, by byte offset.  The region from kOffR on is reused:
-// tables while the operand blocks are built, the per-wave copies of M at the end.
-constexpr int kOffPg = 0;                                   // 8 blocks x 2 pieces x 64 lanes x 16 B
-constexpr int kOffR = kOffPg + 8 * 2 * kWave * 16;          // (kBwdNC + 1) rows of kRP floats
-constexpr int kOffStage = kOffR + (kBwdNC + 1) * kRP * 4;   // kWaves tiles of 32 x kSP elements
-constexpr int kOffSmall = kOffStage + kWaves * 32 * kSP * 2;
-struct BwdSmall {
-  cf sub_end[kSubs][2][16];
-  cf carry[2][2][16];
+struct BwdSmem {
+  u32x4 aop[kBwdBlocks][2][kWave];       // operand blocks, two pieces
+  // row c: (R, R') at the start of chunk c of the segment.  A wave's own 32 rows double as its
+  // private tile for the parked dy / x data before they are written; between rows the buffer
+  // holds the power table (setup) and the reduction scratch (finish).
+  float R[kBwdNC * kRP];
+  float klocal[kT];
   float pn[16];
   cf gn[16];
+  cf pw[14][16];                         // powers evaluated directly (see setup_row)
+  cf sub_end[kSubs][2][16];              // local (R, R') at the start of each sub-segment
+  cf wave_end[2][kWaves][2][16];         // the same for each wave's four sub-segments, by item parity
+  float wave_cin[kWaves][64];            // (R, R') behind each wave's last chunk
+  cf carry[2][2][16];
   float red[kWaves][2][32];
+  float dpart[kWaves][kT];
   float dkin[kT];
-  cf ab[16][2][16];
 };
-constexpr int kBwdLds = kOffSmall + static_cast<int>(sizeof(BwdSmall));
-// build-time tables inside the reused region
-constexpr int kOffQp = kOffR;                               // cf [16][66]
-constexpr int kOffKl = kOffQp + 16 * (kT + 2) * 8;          // float [64]
-constexpr int kOffKQ = kOffKl + kT * 4;                     // 8 blocks x 2 pieces x 64 x 16 B
-static_assert(kOffKQ + 8 * 2 * kWave * 16 <= kOffSmall, "build-time tables must fit the reused region");
-static_assert(kWaves * 3 * 16 * kWave * 4 + kWaves * kT * 4 <= kOffSmall - kOffR, "the copies of M must fit the reused region");
+static_assert(sizeof(cf) * 16 * (kT + 2) + sizeof(cf) * 16 * 2 * 16 <= sizeof(float) * kBwdNC * kRP,
+              "the power table and the final partial sums live in the state buffer");
+static_assert(32 * kSP * 2 <= 32 * kRP * 4 && 16 * kWave * 4 <= 32 * kRP * 4,
+              "a wave's parked tile and one accumulator tile fit its own rows of the state buffer");
+static_assert(sizeof(BwdSmem) <= 80 * 1024, "two workgroups per compute unit");
+
+// (h, h') <- (g, g') + [[m, 0], [md, m]] (h, h'): one step of the reverse scan, over a chunk
+// (m = q^64, md = 64 q^63), a sub-segment or a wave's chunks (the same form with larger powers)
+__device__ __forceinline__ void rstep(cf& h, cf& hd, cf g, cf gd, cf m, cf md) {
+  const cf nd = cadd(gd, cadd(cmul(md, h), cmul(m, hd)));
+  h = cadd(g, cmul(m, h));
+  hd = nd;
+}
 
 template <int DT>
-__global__ __launch_bounds__(kThreads) void cema_scan_bwd_kernel(
+__global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
     const void* __restrict__ dy, const void* __restrict__ x, void* __restrict__ dx,
     const float* __restrict__ p, const cf* __restrict__ log_q, const cf* __restrict__ gamma,
     const float* __restrict__ omega, float* __restrict__ dp, cf* __restrict__ dq,
-    cf* __restrict__ dgamma, float* __restrict__ domega, int D, int N, int64_t L) {
+    cf* __restrict__ dgamma, float* __restrict__ domega, int64_t rows, int D, int N, int64_t L) {
   static_assert(XOp<DT>::XP == 1, "the backward kernel takes bfloat16 rows");
+  constexpr int NC = kBwdNC, CPS = kBwdCPS;
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  u32x4* const pg = reinterpret_cast<u32x4*>(smem_raw + kOffPg);      // [blk][piece][lane]
-  float* const rbuf = reinterpret_cast<float*>(smem_raw + kOffR);
-  BwdSmall& sm = *reinterpret_cast<BwdSmall*>(smem_raw + kOffSmall);
-  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-  const int g = lane >> 5, r = lane & 31;
-  uint16_t* const stage = reinterpret_cast<uint16_t*>(smem_raw + kOffStage) + wave * 32 * kSP;
-  const int64_t row = blockIdx.x;
-  const int d = static_cast<int>(row % D);
-  const uint16_t* dyrow = static_cast<const uint16_t*>(dy) + row * L;
-  const uint16_t* xrow = static_cast<const uint16_t*>(x) + row * L;
-  uint16_t* dxrow = static_cast<uint16_t*>(dx) + row * L;
-  const float wres = omega != nullptr ? omega[d] : 0.f;
+  BwdSmem& sm = *reinterpret_cast<BwdSmem*>(smem_raw);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  // lane-derived indices, re-derived from an opaque thread id wherever a phase starts
+#define MEGA_LANE_IDS                                                          \
+  const int tid = opaque(threadIdx.x) & (kThreads - 1), lane = tid & (kWave - 1); \
+  const int g = lane >> 5, r = lane & 31, sn = tid & 15, sa = tid >> 4, sl = sa & 3; \
+  (void)g; (void)r; (void)sn; (void)sa; (void)sl; (void)lane;                   \
+  float* const myrows = sm.R + wave * 32 * kRP;                                \
+  uint16_t* const stage = reinterpret_cast<uint16_t*>(myrows);                 \
+  (void)stage
+  cf (*qp)[kT + 2] = reinterpret_cast<cf(*)[kT + 2]>(sm.R);                 // setup and finish only
+  cf (*ab)[2][16] = reinterpret_cast<cf(*)[2][16]>(sm.R + 2 * 16 * (kT + 2));  // finish only, behind the table
   const int64_t C = (L + kT - 1) / kT;
-  const int64_t seg_last = (C - 1) / kBwdNC * kBwdNC;
-  const float one = opaque_one();
+  const int64_t seg_last = (C - 1) / NC * NC;
 
   XOp<DT> db[4], xb[4];
-  auto load_tiles = [&](int64_t seg0) {
+  auto load_tiles = [&](int64_t row, int64_t seg0) {
+    MEGA_LANE_IDS;
+    const uint16_t* dyrow = static_cast<const uint16_t*>(dy) + row * L;
+    const uint16_t* xrow = static_cast<const uint16_t*>(x) + row * L;
     const int64_t chunk = seg0 + wave * 32 + r;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int64_t elem = chunk * kT + 16 * s + 8 * g;
-      db[s].load(dyrow, elem, elem + 8 <= L);
-      xb[s].load(xrow, elem, elem + 8 <= L);
+      const bool on = row < rows && elem + 8 <= L;
+      db[s].load(dyrow, elem, on);
+      xb[s].load(xrow, elem, on);
     }
   };
-  load_tiles(seg_last);
+  struct RowParams {
+    cf lq, gv;
+    float pv, w;
+  };
+  auto fetch_params = [&](int64_t row) {
+    MEGA_LANE_IDS;
+    RowParams rp{cf{0.f, 0.f}, cf{0.f, 0.f}, 0.f, 0.f};
+    if (row < rows) {
+      const int d = static_cast<int>(row % D);
+      if (sn < N) {
+        rp.lq = log_q[d * N + sn];
+        rp.gv = gamma[d * N + sn];
+        rp.pv = p[d * N + sn];
+      }
+      if (omega != nullptr) rp.w = omega[d];
+    }
+    return rp;
+  };
+  auto load_block = [&](int b, u32x4* dst, int lane) {
+    dst[0] = sm.aop[b][0][lane];
+    dst[1] = sm.aop[b][1][lane];
+  };
 
-  // ---- per-row tables and operand blocks -----------------------------------------
-  const int sn = tid & 15, sa = tid >> 4;
-  cf (*qp)[kT + 2] = reinterpret_cast<cf(*)[kT + 2]>(smem_raw + kOffQp);
-  float* klocal = reinterpret_cast<float*>(smem_raw + kOffKl);
-  u32x4* const kq = reinterpret_cast<u32x4*>(smem_raw + kOffKQ);
-  cf lq{0.f, 0.f};
-  if (sn < N) lq = log_q[d * N + sn];
-  {
-    cf v{0.f, 0.f}, q1{0.f, 0.f};
-    if (sn < N) {
-      v = qpow(lq.x, lq.y, 4 * sa);
-      q1 = qpow(lq.x, lq.y, 1);
+  // scan multipliers of this thread's mode: over a chunk, a sub-segment, a wave's chunks
+  cf qT{0.f, 0.f}, qTd{0.f, 0.f}, q1{0.f, 0.f};
+  int cur = 0, par = 0;
+  RowParams rp = fetch_params(blockIdx.x);
+
+
+  // per-row accumulators
+  floatx16 macc[3];      // M tiles (0,0), (1,0), (1,1) over this wave's chunks
+  cf wacc[8], wdacc[8];  // W, W' of modes n = 4 qd + 2 g + b at index 2 qd + b, over this lane's chunks
+
+  auto setup_row = [&](int64_t row) {
+    MEGA_LANE_IDS;
+    // powers evaluated directly (phase reduced in float64), 14 per mode: q^(4 k), q^(16 k)
+    // (k < 4), q, q^64, q^(64 CPS), q^(64 CPS - 1), q^(256 CPS), q^(256 CPS - 1)
+    cf direct{0.f, 0.f};
+    if (tid < 14 * 16 && sn < N) {
+      const int k = tid >> 4;
+      const int tab[6] = {1, kT, kT * CPS, kT * CPS - 1, 4 * kT * CPS, 4 * kT * CPS - 1};
+      const int e = k < 4 ? 4 * k : (k < 8 ? 16 * (k - 4) : tab[k - 8]);
+      direct = qpow(rp.lq.x, rp.lq.y, e);
     }
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      qp[sn][4 * sa + e] = v;
-      v = cmul(v, q1);
-    }
-    if (sa == 15) qp[sn][kT] = v;
+    __syncthreads();  // every wave is done with the previous row's tables and reductions
+    if (tid < 14 * 16) sm.pw[tid >> 4][sn] = direct;
     if (tid < 16) {
-      sm.pn[tid] = tid < N ? p[d * N + tid] : 0.f;
-      sm.gn[tid] = tid < N ? gamma[d * N + tid] : cf{0.f, 0.f};
+      sm.pn[tid] = rp.pv;
+      sm.gn[tid] = rp.gv;
       sm.carry[0][0][tid] = cf{0.f, 0.f};
       sm.carry[0][1][tid] = cf{0.f, 0.f};
     }
-  }
-  // scan multipliers: over one chunk (q^64, 64 q^63) and over a sub-segment of CPS chunks
-  cf qT{0.f, 0.f}, qTd{0.f, 0.f}, qS{0.f, 0.f}, qSd{0.f, 0.f};
-  if (sn < N) {
-    qT = qpow(lq.x, lq.y, kT);
-    const cf a = qpow(lq.x, lq.y, kT - 1);
-    qTd = cf{kT * a.x, kT * a.y};
-    qS = qpow(lq.x, lq.y, kT * kBwdCPS);
-    const cf b = qpow(lq.x, lq.y, kT * kBwdCPS - 1);
-    qSd = cf{(kT * kBwdCPS) * b.x, (kT * kBwdCPS) * b.y};
-  }
-  __syncthreads();
-  if (tid < kT) {
-    float acc = 0.f;
+    cur = 0;
+    __syncthreads();
+    {
+      cf v = cmul(sm.pw[sa & 3][sn], sm.pw[4 + (sa >> 2)][sn]);
+      q1 = sm.pw[8][sn];
+      const cf c{rp.pv * rp.gv.x, rp.pv * rp.gv.y};
 #pragma unroll
-    for (int n = 0; n < 16; ++n) {
-      const cf c = cmul(cf{sm.pn[n] * sm.gn[n].x, sm.pn[n] * sm.gn[n].y}, qp[n][tid]);
-      acc += c.x;
+      for (int e = 0; e < 4; ++e) {
+        qp[sn][4 * sa + e] = v;
+        const float kl = group_sum<16>(c.x * v.x - c.y * v.y);
+        if (sn == 0) sm.klocal[4 * sa + e] = (sa == 0 && e == 0) ? kl + rp.w : kl;  // omega on the diagonal
+        v = cmul(v, q1);
+      }
+      if (sa == 15) qp[sn][kT] = sm.pw[9][sn];
+      qT = sm.pw[9][sn];
     }
-    klocal[tid] = acc;
-  }
-  __syncthreads();
-  // blocks 0..7: Pg (kind = b >> 2, k-step s = b & 3); 8..11: K^T by offset 16 (b - 8);
-  // 12..15: Qd (row tile jt = (b - 12) >> 1, k-step s2 = (b - 12) & 1)
-  for (int item = tid; item < 16 * kWave; item += kThreads) {
-    const int blk = item >> 6, ln = item & 63, rr = ln & 31, gg = ln >> 5;
-    float v[8];
-    if (blk < 8) {
-      const int kind = blk >> 2, s = blk & 3, n = rr >> 1, part = rr & 1;
+    __syncthreads();
+    // 64 q^63
+    qTd = cf{kT * qp[sn][kT - 1].x, kT * qp[sn][kT - 1].y};
+    for (int item = tid; item < kBwdBlocks * kWave; item += kThreads) {
+      const int blk = item >> 6, ln = item & 63, rr = ln & 31, gg = ln >> 5;
+      float v[8];
+      if (blk < 8) {
+        const int kind = blk >> 2, s = blk & 3, n = rr >> 1, part = rr & 1;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int i = 16 * s + 8 * gg + e;
-        cf w = qp[n][kind ? (i > 0 ? i - 1 : 0) : i];
-        const float sc = kind ? static_cast<float>(i) : 1.f;
-        v[e] = sc * (part ? w.y : w.x);
-      }
-    } else if (blk < 12) {
-      const int o = 16 * (blk - 8);
+        for (int e = 0; e < 8; ++e) {
+          const int i = 16 * s + 8 * gg + e;
+          const cf w = qp[n][kind ? (i > 0 ? i - 1 : 0) : i];
+          const float sc = kind ? static_cast<float>(i) : 1.f;
+          v[e] = sc * (part ? w.y : w.x);
+        }
+      } else if (blk < 12) {
+        const int o = 16 * (blk - 8);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int lag = o - rr + 8 * gg + e;
-        v[e] = lag >= 0 ? klocal[lag] : 0.f;
-      }
-    } else {
-      const int jt = (blk - 12) >> 1, s2 = (blk - 12) & 1, j = 32 * jt + rr;
+        for (int e = 0; e < 8; ++e) {
+          const int lag = o - rr + 8 * gg + e;
+          v[e] = lag >= 0 ? sm.klocal[lag] : 0.f;
+        }
+      } else {
+        const int jt = (blk - 12) >> 1, s2 = (blk - 12) & 1, j = 32 * jt + rr;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int m = 16 * s2 + 8 * gg + e, n = m >> 1;
-        const cf c = cf{sm.pn[n] * sm.gn[n].x, sm.pn[n] * sm.gn[n].y};
-        const cf w = cmul(c, qp[n][kT - j]);
-        v[e] = (m & 1) ? -w.y : w.x;
+        for (int e = 0; e < 8; ++e) {
+          const int m = 16 * s2 + 8 * gg + e, n = m >> 1;
+          const cf c = cf{sm.pn[n] * sm.gn[n].x, sm.pn[n] * sm.gn[n].y};
+          const cf w = cmul(c, qp[n][kT - j]);
+          v[e] = (m & 1) ? -w.y : w.x;
+        }
       }
+      u32x4 hi, lo;
+      split8(v, hi, lo);
+      sm.aop[blk][0][ln] = hi;
+      sm.aop[blk][1][ln] = lo;
     }
-    u32x4 hi, lo;
-    split8(v, hi, lo);
-    u32x4* dst = blk < 8 ? pg + (blk * 2) * kWave : kq + ((blk - 8) * 2) * kWave;
-    dst[ln] = hi;
-    dst[kWave + ln] = lo;
-  }
-  __syncthreads();
-  u32x4 KQ[8][2];
 #pragma unroll
-  for (int b = 0; b < 8; ++b) {
-    KQ[b][0] = kq[(b * 2) * kWave + lane];
-    KQ[b][1] = kq[(b * 2 + 1) * kWave + lane];
-  }
-  __syncthreads();  // the tables' region becomes the reverse-state buffer and the staging tiles
-
-  floatx16 macc[3];  // M tiles (0,0), (1,0), (1,1) over this wave's chunks
+    for (int t = 0; t < 3; ++t)
 #pragma unroll
-  for (int t = 0; t < 3; ++t)
+      for (int i = 0; i < 16; ++i) macc[t][i] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) macc[t][i] = 0.f;
-  cf wacc[8], wdacc[8];  // W, W' of modes n = 4 qd + 2 g + b at index 2 qd + b, over this lane's chunks
-#pragma unroll
-  for (int i = 0; i < 8; ++i) wacc[i] = wdacc[i] = cf{0.f, 0.f};
-
-  // transposing read of a staged tile: row tile tt (32 time steps), k-step ks (16 chunks)
-  const int tr_base = (8 * g + ((lane & 15) >> 2)) * kSP + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-  auto read_tr = [&](int tt, int ks) {
-    const uint16_t* q = stage + tr_base + 16 * ks * kSP + 32 * tt;
-    const uint2 lo = lds_read_tr(q), hi = lds_read_tr(q + 4 * kSP);
-    return u32x4{lo.x, lo.y, hi.x, hi.y};
+    for (int i = 0; i < 8; ++i) wacc[i] = wdacc[i] = cf{0.f, 0.f};
+    __syncthreads();
+    rp = fetch_params(row + gridDim.x);
   };
 
-  int cur = 0;
-  for (int64_t seg0 = seg_last; seg0 >= 0; seg0 -= kBwdNC) {
-    const int nc = static_cast<int>(C - seg0 < kBwdNC ? C - seg0 : kBwdNC);
+  // the row's reductions and its five gradient outputs
+  auto finish_row = [&](int64_t row) {
+    MEGA_LANE_IDS;
+    // W, W': over the 32 lanes (chunks) of a half wave, then over the waves
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      wacc[i].x = group_sum<32>(wacc[i].x);
+      wacc[i].y = group_sum<32>(wacc[i].y);
+      wdacc[i].x = group_sum<32>(wdacc[i].x);
+      wdacc[i].y = group_sum<32>(wdacc[i].y);
+    }
+    if (r == 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        sm.red[wave][g][4 * i] = wacc[i].x;
+        sm.red[wave][g][4 * i + 1] = wacc[i].y;
+        sm.red[wave][g][4 * i + 2] = wdacc[i].x;
+        sm.red[wave][g][4 * i + 3] = wdacc[i].y;
+      }
+    }
+    // dkin[l] = sum_j M[j + l][j]: each wave sums the diagonals of its own M, one tile at a
+    // time through its own rows of the state buffer ([register][lane]); lane = lag l
+    {
+      float acc = 0.f;
+      const int l = lane;
+#pragma unroll
+      for (int t = 0; t < 3; ++t) {
+        wave_sync();
+#pragma unroll
+        for (int i = 0; i < 16; ++i) myrows[i * kWave + lane] = macc[t][i];
+        wave_sync();
+        // tile t holds rows i = 32 (t > 0) + ii, columns j = 32 (t > 1) + jj
+        const int i0 = t > 0 ? 32 : 0, j0 = t > 1 ? 32 : 0;
+        for (int jj = 0; jj < 32; ++jj) {
+          const int ii = j0 + jj + l - i0;  // row inside the tile of the entry on diagonal l
+          if (ii >= 0 && ii < 32) acc += myrows[(4 * (ii >> 3) + (ii & 3)) * kWave + 32 * ((ii >> 2) & 1) + jj];
+        }
+      }
+      sm.dpart[wave][l] = acc;
+    }
+    __syncthreads();  // every wave is done with the state buffer: it takes the power table again
+    if (tid < kT) sm.dkin[tid] = (sm.dpart[0][tid] + sm.dpart[1][tid]) + (sm.dpart[2][tid] + sm.dpart[3][tid]);
+    {
+      cf v = cmul(sm.pw[sa & 3][sn], sm.pw[4 + (sa >> 2)][sn]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        qp[sn][4 * sa + e] = v;
+        v = cmul(v, q1);
+      }
+    }
+    __syncthreads();
+    {
+      // A_in = sum_l q^l dkin[l], B_in = sum_l l q^(l-1) dkin[l]: thread (n, a) takes l = 4 a .. 4 a + 3
+      cf ain{0.f, 0.f}, bin{0.f, 0.f};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int l = 4 * sa + e;
+        const float dk = sm.dkin[l];
+        const cf v = qp[sn][l];
+        ain.x = fmaf(dk, v.x, ain.x);
+        ain.y = fmaf(dk, v.y, ain.y);
+        if (l > 0) {
+          const cf u = qp[sn][l - 1];
+          const float dl = dk * static_cast<float>(l);
+          bin.x = fmaf(dl, u.x, bin.x);
+          bin.y = fmaf(dl, u.y, bin.y);
+        }
+      }
+      ab[sa][0][sn] = ain;
+      ab[sa][1][sn] = bin;
+    }
+    __syncthreads();
+    if (tid < N) {
+      const int n = tid;
+      cf ain{0.f, 0.f}, bin{0.f, 0.f};
+      for (int a = 0; a < 16; ++a) {
+        ain = cadd(ain, ab[a][0][n]);
+        bin = cadd(bin, ab[a][1][n]);
+      }
+      // mode n sits in half g = (n >> 1) & 1 at index 2 (n >> 2) + (n & 1)
+      const int hg = (n >> 1) & 1, idx = 2 * (n >> 2) + (n & 1);
+      cf w{0.f, 0.f}, wd{0.f, 0.f};
+      for (int wv = 0; wv < kWaves; ++wv) {
+        w.x += sm.red[wv][hg][4 * idx];
+        w.y += sm.red[wv][hg][4 * idx + 1];
+        wd.x += sm.red[wv][hg][4 * idx + 2];
+        wd.y += sm.red[wv][hg][4 * idx + 3];
+      }
+      const cf qq = sm.pw[8][n];
+      const cf A = cadd(ain, cmul(qq, w));
+      const cf Bq = cadd(cadd(bin, w), cmul(qq, wd));
+      const cf gm = sm.gn[n];
+      const float pp = sm.pn[n];
+      dp[row * N + n] = A.x * gm.x - A.y * gm.y;
+      const cf t = cmul(Bq, cf{pp * gm.x, pp * gm.y});
+      dq[row * N + n] = cf{t.x, -t.y};
+      dgamma[row * N + n] = cf{A.x * pp, -A.y * pp};
+    }
+    // the skip term sat on the diagonal of K, not in M: domega = sum dy x = dkin[0]
+    if (tid == 0) domega[row] = sm.dkin[0];
+  };
+
+  auto item = [&](int64_t row, int64_t seg0) {
+    MEGA_LANE_IDS;
+    // transposing read of the parked tile: row tile tt (32 time steps), k-step ks (16 chunks)
+    const int tr_base = (8 * g + ((lane & 15) >> 2)) * kSP + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    auto read_tr = [&](int tt, int ks) {
+      const uint16_t* q = stage + tr_base + 16 * ks * kSP + 32 * tt;
+      const uint2 lo = lds_read_tr(q), hi = lds_read_tr(q + 4 * kSP);
+      return u32x4{lo.x, lo.y, hi.x, hi.y};
+    };
+    if (seg0 == seg_last) setup_row(row);
+    uint16_t* dxrow = static_cast<uint16_t*>(dx) + row * L;
+    const int nc = static_cast<int>(C - seg0 < NC ? C - seg0 : NC);
     const int c0 = wave * 32;
     const bool on = c0 < nc;
-    // ---- (G, G') = Pg DY -------------------------------------------------------------
-    if (on) {
-#pragma unroll
-      for (int kind = 0; kind < 2; ++kind) {
-        floatx16 acc;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const u32x4 a[2] = {pg[((kind * 4 + s) * 2) * kWave + lane], pg[((kind * 4 + s) * 2 + 1) * kWave + lane]};
-          acc = mma_split<1>(a, db[s].pc, acc);
-        }
-        float* dst = rbuf + (c0 + r) * kRP + 32 * kind + 4 * g;
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd)
-          *reinterpret_cast<float4*>(dst + 8 * qd) =
-              make_float4(acc[4 * qd], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3]);
-      }
-    }
-    lds_barrier();
-    // ---- reverse scan over the chunks of the segment ------------------------------------
-    {
-      float* col = rbuf + 2 * sn;
-      cf e{0.f, 0.f}, ed{0.f, 0.f};
-#pragma unroll 4
-      for (int i = kBwdCPS - 1; i >= 0; --i) {
-        const int c = sa * kBwdCPS + i;
-        if (c < nc) {
-          const float2 gv = *reinterpret_cast<const float2*>(col + c * kRP);
-          const float2 gd = *reinterpret_cast<const float2*>(col + c * kRP + 32);
-          const cf nd = cadd(cf{gd.x, gd.y}, cadd(cmul(qTd, e), cmul(qT, ed)));
-          e = cadd(cf{gv.x, gv.y}, cmul(qT, e));
-          ed = nd;
-        }
-      }
-      sm.sub_end[sa][0][sn] = e;
-      sm.sub_end[sa][1][sn] = ed;
-      lds_barrier();
-      const cf cin0 = sm.carry[cur][0][sn], cind0 = sm.carry[cur][1][sn];
-      cf h = cin0, hd = cind0;
-      for (int s = kSubs - 1; s > sa; --s) {
-        const cf nd = cadd(sm.sub_end[s][1][sn], cadd(cmul(qSd, h), cmul(qS, hd)));
-        h = cadd(sm.sub_end[s][0][sn], cmul(qS, h));
-        hd = nd;
-      }
-      if (sa == kSubs - 1) {  // the state after the segment's last chunk
-        *reinterpret_cast<float2*>(col + nc * kRP) = make_float2(cin0.x, cin0.y);
-        *reinterpret_cast<float2*>(col + nc * kRP + 32) = make_float2(cind0.x, cind0.y);
-      }
-#pragma unroll 4
-      for (int i = kBwdCPS - 1; i >= 0; --i) {
-        const int c = sa * kBwdCPS + i;
-        if (c < nc) {
-          const float2 gv = *reinterpret_cast<const float2*>(col + c * kRP);
-          const float2 gd = *reinterpret_cast<const float2*>(col + c * kRP + 32);
-          const cf nd = cadd(cf{gd.x, gd.y}, cadd(cmul(qTd, h), cmul(qT, hd)));
-          h = cadd(cf{gv.x, gv.y}, cmul(qT, h));
-          hd = nd;
-          *reinterpret_cast<float2*>(col + c * kRP) = make_float2(h.x, h.y);
-          *reinterpret_cast<float2*>(col + c * kRP + 32) = make_float2(hd.x, hd.y);
-        }
-      }
-      if (sa == 0) {
-        sm.carry[cur ^ 1][0][sn] = h;
-        sm.carry[cur ^ 1][1][sn] = hd;
-      }
-    }
-    lds_barrier();
+    u32x4 xr[4];  // time-reversed x as an operand: steps 63 - (16 s + 8 g + e)
     if (on) {
       // ---- the wave's private tile: DY parked and read back with chunks along k ----------
       uint16_t* mine = stage + r * kSP + 8 * g;
 #pragma unroll
       for (int s = 0; s < 4; ++s) *reinterpret_cast<u32x4*>(mine + 16 * s) = db[s].pc[0];
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wave_sync();
       u32x4 dyt[2][2];
 #pragma unroll
       for (int it = 0; it < 2; ++it)
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) dyt[it][ks] = read_tr(it, ks);
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wave_sync();
 #pragma unroll
       for (int s = 0; s < 4; ++s) *reinterpret_cast<u32x4*>(mine + 16 * s) = xb[s].pc[0];
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wave_sync();
       // M += DY^T X over the tile's 32 chunks
 #pragma unroll
       for (int jt = 0; jt < 2; ++jt)
@@ -797,52 +866,140 @@ __global__ __launch_bounds__(kThreads) void cema_scan_bwd_kernel(
           if (jt == 0) macc[0] = mfma_bf16(dyt[0][ks], xt, macc[0]);
           macc[1 + jt] = mfma_bf16(dyt[1][ks], xt, macc[1 + jt]);
         }
-      // time-reversed x as an operand: steps 63 - (16 s + 8 g + e)
-      u32x4 xr[4];
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const u32x4 v = *reinterpret_cast<const u32x4*>(stage + r * kSP + 56 - 16 * s - 8 * g);
 #pragma unroll
         for (int e = 0; e < 4; ++e) xr[s][e] = __builtin_amdgcn_alignbit(v[3 - e], v[3 - e], 16);
       }
-      // ---- (X, X') = Pg XR, then W += X R[c+1], W' += X' R[c+1] + X R'[c+1] ---------------
-      floatx16 xacc[2];
+      wave_sync();  // the tile has been read: its place takes the wave's rows of (G, G')
+      // ---- (G, G') = Pg DY, into this wave's own rows of the state buffer ----------------
 #pragma unroll
       for (int kind = 0; kind < 2; ++kind) {
+        floatx16 acc;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) xacc[kind][i] = 0.f;
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-          const u32x4 a[2] = {pg[((kind * 4 + s) * 2) * kWave + lane], pg[((kind * 4 + s) * 2 + 1) * kWave + lane]};
-          xacc[kind] = mma_split<1>(a, &xr[s], xacc[kind]);
+          u32x4 a[2];
+          load_block(kind * 4 + s, a, lane);
+          acc = mma_split<1>(a, db[s].pc, acc);
+        }
+        float* dst = myrows + r * kRP + 32 * kind + 4 * g;
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd)
+          *reinterpret_cast<float4*>(dst + 8 * qd) =
+              make_float4(acc[4 * qd], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3]);
+      }
+    }
+    wave_sync();
+    // ---- reverse scan over the chunks of the segment; a wave's four sub-segments are its own
+    //      chunks, one workgroup barrier hands over the waves' ends ---------------------------------
+    {
+      float* col = sm.R + 2 * sn;
+      float2 gv[CPS], gd[CPS];
+#pragma unroll
+      for (int i = 0; i < CPS; ++i) {
+        const int c = sa * CPS + i;
+        const bool live = c < nc;
+        gv[i] = live ? *reinterpret_cast<const float2*>(col + c * kRP) : make_float2(0.f, 0.f);
+        gd[i] = live ? *reinterpret_cast<const float2*>(col + c * kRP + 32) : make_float2(0.f, 0.f);
+      }
+      cf e{0.f, 0.f}, ed{0.f, 0.f};
+#pragma unroll
+      for (int i = CPS - 1; i >= 0; --i) rstep(e, ed, cf{gv[i].x, gv[i].y}, cf{gd[i].x, gd[i].y}, qT, qTd);
+      sm.sub_end[sa][0][sn] = e;
+      sm.sub_end[sa][1][sn] = ed;
+      wave_sync();
+      // multipliers over a sub-segment and over a wave's chunks
+      const cf qS = sm.pw[10][sn], qW = sm.pw[12][sn];
+      const cf qSd{(kT * CPS) * sm.pw[11][sn].x, (kT * CPS) * sm.pw[11][sn].y};
+      const cf qWd{(4 * kT * CPS) * sm.pw[13][sn].x, (4 * kT * CPS) * sm.pw[13][sn].y};
+      if (sl == 0) {
+        // the wave's chunks from zero: sub-segments 3, 2, 1, then this one
+        cf h = sm.sub_end[sa + 3][0][sn], hd = sm.sub_end[sa + 3][1][sn];
+        rstep(h, hd, sm.sub_end[sa + 2][0][sn], sm.sub_end[sa + 2][1][sn], qS, qSd);
+        rstep(h, hd, sm.sub_end[sa + 1][0][sn], sm.sub_end[sa + 1][1][sn], qS, qSd);
+        rstep(h, hd, e, ed, qS, qSd);
+        sm.wave_end[par][wave][0][sn] = h;
+        sm.wave_end[par][wave][1][sn] = hd;
+      }
+      lds_barrier();
+      cf h = sm.carry[cur][0][sn], hd = sm.carry[cur][1][sn];
+#pragma unroll
+      for (int w = kWaves - 1; w >= 1; --w) {
+        const cf we = sm.wave_end[par][w][0][sn], wed = sm.wave_end[par][w][1][sn];
+        if (w > wave) rstep(h, hd, we, wed, qW, qWd);
+      }
+      if (sa == 0) {
+        // through wave 0's chunks too: the state at the start of the segment, the next item's carry
+        cf ch = h, chd = hd;
+        rstep(ch, chd, sm.wave_end[par][0][0][sn], sm.wave_end[par][0][1][sn], qW, qWd);
+        sm.carry[cur ^ 1][0][sn] = ch;
+        sm.carry[cur ^ 1][1][sn] = chd;
+      }
+      if (sl == 3) {  // (R, R') behind the wave's last chunk
+        *reinterpret_cast<float2*>(sm.wave_cin[wave] + 2 * sn) = make_float2(h.x, h.y);
+        *reinterpret_cast<float2*>(sm.wave_cin[wave] + 32 + 2 * sn) = make_float2(hd.x, hd.y);
+      }
+#pragma unroll
+      for (int s = 3; s >= 1; --s) {
+        const cf se = sm.sub_end[4 * wave + s][0][sn], sed = sm.sub_end[4 * wave + s][1][sn];
+        if (s > sl) rstep(h, hd, se, sed, qS, qSd);
+      }
+#pragma unroll
+      for (int i = CPS - 1; i >= 0; --i) {
+        const int c = sa * CPS + i;
+        rstep(h, hd, cf{gv[i].x, gv[i].y}, cf{gd[i].x, gd[i].y}, qT, qTd);
+        if (c < nc) {
+          *reinterpret_cast<float2*>(col + c * kRP) = make_float2(h.x, h.y);
+          *reinterpret_cast<float2*>(col + c * kRP + 32) = make_float2(hd.x, hd.y);
         }
       }
-      // chunks past the end of the row have X = 0, but their rows of the state buffer were
-      // never written and may hold anything: they are taken as zero
-      const float* rnext = rbuf + (c0 + r + 1) * kRP + 4 * g;
+    }
+    wave_sync();
+    if (on) {
+      // (R, R')[c + 1]: the next row of the buffer, or, for the wave's last chunk, wave_cin;
+      // chunks past the end of the row have X = 0 and DY = 0, their rows may hold anything
       const bool live = c0 + r < nc;
+      const float* rnext = (r == 31) ? sm.wave_cin[wave] : myrows + (r + 1) * kRP;
       const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      // ---- (X, X') = Pg XR;  W += X R[c+1], W' += X' R[c+1] + X R'[c+1] ---------------------------
+      {
+        floatx16 xacc[2];
 #pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        const float4 rv = live ? *reinterpret_cast<const float4*>(rnext + 8 * qd) : zero4;
-        const float4 rd = live ? *reinterpret_cast<const float4*>(rnext + 32 + 8 * qd) : zero4;
+        for (int kind = 0; kind < 2; ++kind) {
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-          const cf xv{xacc[0][4 * qd + 2 * b], xacc[0][4 * qd + 2 * b + 1]};
-          const cf xd{xacc[1][4 * qd + 2 * b], xacc[1][4 * qd + 2 * b + 1]};
-          const cf rr_ = b ? cf{rv.z, rv.w} : cf{rv.x, rv.y};
-          const cf rdd = b ? cf{rd.z, rd.w} : cf{rd.x, rd.y};
-          wacc[2 * qd + b] = cadd(wacc[2 * qd + b], cmul(xv, rr_));
-          wdacc[2 * qd + b] = cadd(wdacc[2 * qd + b], cadd(cmul(xd, rr_), cmul(xv, rdd)));
+          for (int i = 0; i < 16; ++i) xacc[kind][i] = 0.f;
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            u32x4 a[2];
+            load_block(kind * 4 + s, a, lane);
+            xacc[kind] = mma_split<1>(a, &xr[s], xacc[kind]);
+          }
+        }
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const float4 rv = live ? *reinterpret_cast<const float4*>(rnext + 4 * g + 8 * qd) : zero4;
+          const float4 rd = live ? *reinterpret_cast<const float4*>(rnext + 32 + 4 * g + 8 * qd) : zero4;
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            const cf xv{xacc[0][4 * qd + 2 * b], xacc[0][4 * qd + 2 * b + 1]};
+            const cf xd{xacc[1][4 * qd + 2 * b], xacc[1][4 * qd + 2 * b + 1]};
+            const cf rr_ = b ? cf{rv.z, rv.w} : cf{rv.x, rv.y};
+            const cf rdd = b ? cf{rd.z, rd.w} : cf{rd.x, rd.y};
+            wacc[2 * qd + b] = cadd(wacc[2 * qd + b], cmul(xv, rr_));
+            wdacc[2 * qd + b] = cadd(wdacc[2 * qd + b], cadd(cmul(xd, rr_), cmul(xv, rdd)));
+          }
         }
       }
-      // ---- DX = K^T DY + Qd R[c+1] (+ omega dy), written from the accumulators ---------------
+      // ---- DX = K^T DY + Qd R[c+1] (omega dy included: K carries omega on its diagonal) -------------
       u32x4 hb[2][2];
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        const float* src = rbuf + (c0 + r + 1) * kRP + 16 * s2 + 8 * g;
-        const float4 u = *reinterpret_cast<const float4*>(src);
-        const float4 w = *reinterpret_cast<const float4*>(src + 4);
+        const float* src = rnext + 16 * s2 + 8 * g;
+        const float4 u = live ? *reinterpret_cast<const float4*>(src) : zero4;
+        const float4 w = live ? *reinterpret_cast<const float4*>(src + 4) : zero4;
         const float v[8] = {u.x, u.y, u.z, u.w, w.x, w.y, w.z, w.w};
         split8(v, hb[s2][0], hb[s2][1]);
       }
@@ -853,139 +1010,60 @@ __global__ __launch_bounds__(kThreads) void cema_scan_bwd_kernel(
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
-        for (int s = 2 * jt; s < 4; ++s) acc = mma_split<1>(KQ[s - 2 * jt], db[s].pc, acc);
+        for (int s = 2 * jt; s < 4; ++s) {
+          u32x4 a[2];
+          load_block(8 + s - 2 * jt, a, lane);
+          acc = mma_split<1>(a, db[s].pc, acc);
+        }
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
-          acc = mfma_bf16(KQ[4 + 2 * jt + s2][0], hb[s2][0], acc);
-          acc = mfma_bf16(KQ[4 + 2 * jt + s2][1], hb[s2][0], acc);
-          acc = mfma_bf16(KQ[4 + 2 * jt + s2][0], hb[s2][1], acc);
+          u32x4 a[2];
+          load_block(12 + 2 * jt + s2, a, lane);
+          acc = mfma_bf16(a[0], hb[s2][0], acc);
+          acc = mfma_bf16(a[1], hb[s2][0], acc);
+          acc = mfma_bf16(a[0], hb[s2][1], acc);
         }
 #pragma unroll
         for (int pr = 0; pr < 2; ++pr) {
-          float oct[8];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            oct[e] = acc[8 * pr + e] * one;
-            oct[4 + e] = acc[8 * pr + 4 + e] * one;
-            half_swap(oct[e], oct[4 + e]);
-          }
-          const int s = 2 * jt + pr;
-          float gv[8];
-          db[s].values(gv);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) oct[e] = fmaf(wres, gv[e], oct[e]);
-          const int64_t elem = chunk * kT + 16 * s + 8 * g;
-          if (elem + 8 <= L) *reinterpret_cast<uint4*>(dxrow + elem) = pack8<DT>(oct);
+          const uint4 oct = octet_of<DT>(acc, pr);
+          const int64_t elem = chunk * kT + 16 * (2 * jt + pr) + 8 * g;
+          if (elem + 8 <= L) *reinterpret_cast<uint4*>(dxrow + elem) = oct;
         }
       }
     }
     cur ^= 1;
-    if (seg0 > 0) {
-      load_tiles(seg0 - kBwdNC);
-      lds_barrier();  // the next segment's (G, G') overwrite the rows read above
-    }
-  }
-
-  // ---- reductions over the workgroup --------------------------------------------------------
-  // W, W': over the 32 lanes (chunks) of a half wave, then over the waves
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    wacc[i].x = group_sum<32>(wacc[i].x);
-    wacc[i].y = group_sum<32>(wacc[i].y);
-    wdacc[i].x = group_sum<32>(wdacc[i].x);
-    wdacc[i].y = group_sum<32>(wdacc[i].y);
-  }
-  if (r == 0) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      sm.red[wave][g][4 * i] = wacc[i].x;
-      sm.red[wave][g][4 * i + 1] = wacc[i].y;
-      sm.red[wave][g][4 * i + 2] = wdacc[i].x;
-      sm.red[wave][g][4 * i + 3] = wdacc[i].y;
-    }
-  }
-  __syncthreads();  // every wave is done with the state buffer and its staging tile
-  float* mcopy = reinterpret_cast<float*>(smem_raw + kOffR);  // [wave][tile][register][lane]
-#pragma unroll
-  for (int t = 0; t < 3; ++t)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) mcopy[((wave * 3 + t) * 16 + i) * kWave + lane] = macc[t][i];
-  __syncthreads();
-  float* dpart = mcopy + kWaves * 3 * 16 * kWave;  // [wave][l]
-  {
-    // dkin[l] = sum_j M[j + l][j]: thread (l, wave copy) walks the l-th diagonal of its copy
-    const int l = tid & 63, wv = tid >> 6;
-    float acc = 0.f;
-    for (int j = 0; j + l < kT; ++j) {
-      const int i = j + l, t = (i >> 5) + (j >> 5), ii = i & 31;
-      const int reg = 4 * (ii >> 3) + (ii & 3), ln = 32 * ((ii >> 2) & 1) + (j & 31);
-      acc += mcopy[((wv * 3 + t) * 16 + reg) * kWave + ln];
-    }
-    dpart[wv * kT + l] = acc;
-  }
-  __syncthreads();
-  if (tid < kT) sm.dkin[tid] = (dpart[tid] + dpart[kT + tid]) + (dpart[2 * kT + tid] + dpart[3 * kT + tid]);
-  __syncthreads();
-  {
-    // A_in = sum_l q^l dkin[l], B_in = sum_l l q^(l-1) dkin[l]: thread (n, a) takes l = 4 a .. 4 a + 3
-    cf ain{0.f, 0.f}, bin{0.f, 0.f};
-    if (sn < N) {
-      const cf q1 = qpow(lq.x, lq.y, 1);
-      cf v = qpow(lq.x, lq.y, 4 * sa);
-      cf u = sa > 0 ? qpow(lq.x, lq.y, 4 * sa - 1) : cf{0.f, 0.f};  // q^(l-1); the l = 0 term is zero
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int l = 4 * sa + e;
-        const float dk = sm.dkin[l];
-        ain.x = fmaf(dk, v.x, ain.x);
-        ain.y = fmaf(dk, v.y, ain.y);
-        const float dl = dk * static_cast<float>(l);
-        bin.x = fmaf(dl, u.x, bin.x);
-        bin.y = fmaf(dl, u.y, bin.y);
-        u = (l == 0) ? cf{1.f, 0.f} : cmul(u, q1);
-        v = cmul(v, q1);
+    par ^= 1;
+    if (seg0 == 0) finish_row(row);
+    // the next item's tiles
+    {
+      int64_t nrow = row, nseg = seg0 - NC;
+      if (nseg < 0) {
+        nrow = row + gridDim.x;
+        nseg = seg_last;
       }
+      load_tiles(nrow, nseg);
     }
-    sm.ab[sa][0][sn] = ain;
-    sm.ab[sa][1][sn] = bin;
-  }
-  __syncthreads();
-  if (tid < N) {
-    const int n = tid;
-    cf ain{0.f, 0.f}, bin{0.f, 0.f};
-    for (int a = 0; a < 16; ++a) {
-      ain = cadd(ain, sm.ab[a][0][n]);
-      bin = cadd(bin, sm.ab[a][1][n]);
-    }
-    // mode n sits in half g = (n >> 1) & 1 at index 2 (n >> 2) + (n & 1)
-    const int hg = (n >> 1) & 1, idx = 2 * (n >> 2) + (n & 1);
-    cf w{0.f, 0.f}, wd{0.f, 0.f};
-    for (int wv = 0; wv < kWaves; ++wv) {
-      w.x += sm.red[wv][hg][4 * idx];
-      w.y += sm.red[wv][hg][4 * idx + 1];
-      wd.x += sm.red[wv][hg][4 * idx + 2];
-      wd.y += sm.red[wv][hg][4 * idx + 3];
-    }
-    const cf q1 = qpow(lq.x, lq.y, 1);
-    const cf A = cadd(ain, cmul(q1, w));
-    const cf Bq = cadd(cadd(bin, w), cmul(q1, wd));
-    const cf gm = sm.gn[n];
-    const float pp = sm.pn[n];
-    dp[row * N + n] = A.x * gm.x - A.y * gm.y;
-    const cf t = cmul(Bq, cf{pp * gm.x, pp * gm.y});
-    dq[row * N + n] = cf{t.x, -t.y};
-    dgamma[row * N + n] = cf{A.x * pp, -A.y * pp};
-  }
-  if (tid == 0) domega[row] = sm.dkin[0];
+  };
+
+  load_tiles(blockIdx.x, seg_last);
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x)
+    for (int64_t seg0 = seg_last; seg0 >= 0; seg0 -= NC) item(row, seg0);
+#undef MEGA_LANE_IDS
 }
 
 int launch_bwd(const void* dy, const void* x, void* dx, const float* p, const cf* log_q,
                const cf* gamma, const float* omega, float* dp, cf* dq, cf* dgamma, float* domega,
                int64_t B, int64_t D, int64_t N, int64_t L, hipStream_t stream) {
+  const int lds = static_cast<int>(sizeof(BwdSmem));
   MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&cema_scan_bwd_kernel<MEGA_BF16>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds));
-  cema_scan_bwd_kernel<MEGA_BF16><<<dim3(static_cast<unsigned>(B * D)), kThreads, kBwdLds, stream>>>(
-      dy, x, dx, p, log_q, gamma, omega, dp, dq, dgamma, domega, static_cast<int>(D),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  int dev = 0, cus = 0;
+  MEGA_CHECK_HIP(hipGetDevice(&dev));
+  MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  const int64_t rows = B * D, slots = 2 * static_cast<int64_t>(cus);  // two workgroups fit a compute unit
+  const unsigned grid = static_cast<unsigned>(rows < slots ? rows : slots);
+  cema_scan_bwd_kernel<MEGA_BF16><<<dim3(grid), kThreads, lds, stream>>>(
+      dy, x, dx, p, log_q, gamma, omega, dp, dq, dgamma, domega, rows, static_cast<int>(D),
       static_cast<int>(N), L);
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
