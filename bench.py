@@ -1,15 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the Megalodon fused-op hot path on one MI355X.
 
-A step is one CEMA layer forward+backward at the 7B layer width (BASELINE
-config 1): k = ema_parameters(p, q, gamma) -> y = fftconv(x, k) + x*omega, then
-backward through both ops to dx, d(alpha, delta, theta, gamma, omega), with
-B=1, L=32768, D=4096, ndim=16, x and the upstream gradient in bf16.  The
-convolution's DFT stages run on the matrix cores (fp16 operands, fp32
-accumulation; twiddles, the spectral product and every sum in fp32); the same
-step through the all-fp32 VALU convolution engine is timed beside it
-("fp32_fft_engine").  Inputs are synthetic, seeded, and resident in HBM before
-the timed region.  Prints one JSON line.
+Headline (`value`): one full Megalodon-7B-style block, forward + backward, at
+L = 32768 (BASELINE config 4: D=4096, EMA ndim 16, z 1024, value 8192, 4 heads,
+chunk 4096, FFN 11008 SwiGLU, bf16 weights and activations, fp32 norm / EMA
+state), in tokens/s.  A step is one forward + backward of the block on
+synthetic, seeded inputs that are resident in HBM before the timed region.
+
+Beside it, in the same JSON line:
+  roofline      the dominant kernel of the CEMA + convolution sub-layer
+                (config 1: B=1, L=32768, D=4096, ndim=16, x / dy bf16), timed
+                live with device events on the launch stream
+  cema_layer    the config-1 step (layer forward + backward) on the default
+                path (chunked recurrence on the matrix cores, float32-equivalent
+                arithmetic) and on the two FFT-convolution engines
+  other_ops     TimestepNorm (config 2) and chunk attention (config 3)
+  cpu_baseline  the block on the host cores through the reference's CPU
+                formulation, on a bounded sample; per-op baselines in cpu_ops
+Prints one JSON line.
 """
 import argparse
 import json
@@ -22,82 +30,267 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
-# HBM bytes one forward convolution launch moves at config 1 (1.11e9 of them the spectra kept for the backward): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from
-# two rocprofv3 --pmc passes of this script, the factors being what the same counters read for a plain
-# copy of 2^30 bytes (--copy-calibration).  A measured constant: counters cannot be read from in here.
-FFTCONV_TRAFFIC_BYTES = 2.49e9
+# HBM bytes one backward launch of the CEMA recurrence moves at config 1: FETCH_SIZE x 2.0 +
+# WRITE_SIZE x 1.0 from two rocprofv3 --pmc passes of this script (--cema-only --copy-calibration),
+# the factors being what the same counters read for a plain copy of 2^30 bytes.  A measured
+# constant (profiles/cema_scan_config1_hbm_traffic.txt): counters cannot be read from in here.
+CEMA_BWD_TRAFFIC_BYTES = None
+
+CFG4 = dict(model_dim=4096, z_dim=1024, value_dim=8192, num_heads=4, cema_ndim=16, chunk_size=4096,
+            ffn_hidden_dim=11008, norm_num_groups=32)
 
 
-def cpu_baseline(B, D, N, L, seed, budget_s=25.0):
-    """The same step on the host cores through the reference's CPU formulation:
-    ema_parameters by the C/OpenMP restatement of its C++ loop nest, the
-    convolution by torch.fft on CPU tensors (which is the reference's CPU
-    path), on a bounded slice of the channels (every loop nest is linear in D).
-    """
+def host_cores():
+    env = os.environ.get("OMP_NUM_THREADS")
+    return int(env) if env else min(os.cpu_count() or 1, 16)
+
+
+# --------------------------------------------------------------------------- CPU baselines
+def _timed(fn, budget_s, max_reps=3):
+    t0 = time.perf_counter()
+    fn()
+    one = time.perf_counter() - t0
+    reps = max(1, min(max_reps, int(budget_s / max(one, 1e-3)) - 1))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    return (time.perf_counter() - t0) / reps, reps
+
+
+def cpu_cema(B, D, N, L, seed, cores, budget_s=12.0):
+    """Config 1 through the reference's CPU formulation: ema_parameters by the
+    C/OpenMP restatement of its loop nest (csrc/ops/ema_parameters.cc), the
+    convolution by torch.fft on CPU tensors (fused_ops/fftconv.py:30-75)."""
     import torch
     from megalodon_amd import synthetic
-    from oracle import native, fftconv as offt
-
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16) if os.environ.get("OMP_NUM_THREADS") is None else int(os.environ["OMP_NUM_THREADS"])
-    torch.set_num_threads(cores)
-    os.environ.setdefault("OMP_NUM_THREADS", str(cores))
+    from oracle import native
     lib = native.port()
-    Ds = 512
+    Ds = 256
     prm = synthetic.cema_params(D, N, seed)
     io = synthetic.cema_inputs(B, Ds, L, seed, torch.bfloat16)
-    p, lq, g = prm["p"][:Ds], prm["q"][:Ds].log(), prm["gamma"][:Ds]
-    om = prm["omega"][:Ds]
+    p, lq, g, om = prm["p"][:Ds], prm["q"][:Ds].log(), prm["gamma"][:Ds], prm["omega"][:Ds]
 
     def step():
         k = native.ema_weight_fwd(lib, "oracle_", p, lq, g, L)
         x = io["x"].float()
-        L_ = x.shape[-1]
-        n = 2 * (L_ if (L_ & (L_ - 1)) == 0 else (1 << L_.bit_length()))
+        n = 2 * (L if (L & (L - 1)) == 0 else (1 << L.bit_length()))
         x_f = torch.fft.rfft(x, n=n)
         k_f = torch.fft.rfft(k, n=n, norm="forward")
-        y = torch.fft.irfft(x_f * k_f, n=n, norm="forward")[..., :L_].to(torch.bfloat16)
+        y = torch.fft.irfft(x_f * k_f, n=n, norm="forward")[..., :L].to(torch.bfloat16)
         out = y + io["x"] * om
         dy = io["dy"].float()
         dy_f = torch.fft.rfft(dy.flip(dims=(-1,)), n=n)
-        dx = torch.fft.irfft(dy_f * k_f, n=n, norm="forward")[..., :L_].flip(dims=(-1,)).to(torch.bfloat16)
-        dk = torch.fft.irfft((dy_f * x_f).sum(dim=0), n=n)[..., :L_].flip(dims=(-1,))
+        dx = torch.fft.irfft(dy_f * k_f, n=n, norm="forward")[..., :L].flip(dims=(-1,)).to(torch.bfloat16)
+        dk = torch.fft.irfft((dy_f * x_f).sum(dim=0), n=n)[..., :L].flip(dims=(-1,))
         dx = dx + io["dy"] * om
         dom = (io["dy"].float() * x).sum(dim=(0, 2))
-        grads = native.ema_weight_bwd(lib, "oracle_", dk, p, lq, g)
-        return out, dx, dom, grads
+        return out, dx, dom, native.ema_weight_bwd(lib, "oracle_", dk, p, lq, g)
 
-    t0 = time.perf_counter()
-    step()
-    one = time.perf_counter() - t0
-    reps = max(1, min(5, int(budget_s / max(one, 1e-3)) - 1))
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        step()
-    dt = (time.perf_counter() - t0) / reps
-    tokens_per_s = B * L / (dt * D / Ds)
-    return {
-        "value": tokens_per_s, "unit": "tokens/s", "cores": cores, "kind": "port",
-        "sample": f"{Ds} of {D} channels, {reps} rep(s) of the full fwd+bwd step at L={L}, "
-                  f"{dt:.3f} s each, scaled by D/{Ds}",
-    }
+    dt, reps = _timed(step, budget_s)
+    return {"value": B * L / (dt * D / Ds), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{Ds} of {D} channels, {reps} rep(s) of the fwd+bwd step at L={L}, {dt:.2f} s each, "
+                      f"scaled by D/{Ds}"}
 
 
-def other_ops(torch, dev, synthetic):
-    """TimestepNorm (config 2), chunk attention (config 3) and one block (config 4),
-    timed with device events; reported beside the config-1 step."""
-    def dev_ms(fn, n):
+def cpu_timestep_norm(cores, budget_s=12.0):
+    """Config 2 through the C/OpenMP restatement of GroupTimestepNormCPUFwd/Bwd
+    (csrc/ops/timestep_norm.cc:218-450; the scan runs over the batch only, as there)."""
+    import torch
+    from megalodon_amd import synthetic
+    from oracle import native
+    lib = native.port()
+    B, L, D, G = 4, 8192, 4096, 32
+    Ls = 2048
+    io = {k: (v[:, :Ls].contiguous() if v.dim() >= 2 and v.shape[1] == L else v)
+          for k, v in synthetic.timestep_norm_inputs(B, L, D, G, 1002).items()}
+    f = {k: (v.float() if v.is_floating_point() else v) for k, v in io.items()}
+
+    def step():
+        y, count, mean, var, cm, cr = native.group_timestep_norm_fwd(
+            lib, "oracle_", f["x"], f["prev_count"], f["prev_mean"], f["prev_var"], f["gamma"], f["beta"],
+            f["mask"], G, 1e-5)
+        native.group_timestep_norm_bwd(lib, "oracle_", f["dy"], f["dmean"], f["dvar"], f["x"], f["prev_mean"],
+                                       count, cm, cr, f["gamma"], f["mask"], G)
+
+    dt, reps = _timed(step, budget_s)
+    return {"value": B * Ls / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"first {Ls} of {L} steps of all {B} sequences (the loop nest is linear in L), "
+                      f"{reps} rep(s), {dt:.2f} s each"}
+
+
+def cpu_attention(cores, budget_s=12.0):
+    """Config 3 through the reference's unfused branch: matmul + causal mask +
+    float32 softmax + matmul, backward by autograd
+    (modules/moving_average_gated_attention.py:116-129)."""
+    import torch
+    from megalodon_amd import synthetic
+    C, H1, H2 = 4096, 256, 2048
+    io = synthetic.attention_inputs(1, C, 1, H1, H2, 1003)
+    q, k, v = (io[n].float().transpose(1, 2).requires_grad_(True) for n in ("q", "k", "v"))
+    dy = io["dy"].float().transpose(1, 2)
+    mask = torch.full((C, C), float("-inf")).triu(1)
+
+    def step():
+        for t in (q, k, v):
+            t.grad = None
+        s = torch.matmul(q, k.transpose(2, 3)) + mask
+        out = torch.matmul(torch.softmax(s, dim=-1, dtype=torch.float32), v)
+        out.backward(dy)
+
+    dt, reps = _timed(step, budget_s)
+    pairs = 32  # 8 chunks x 4 heads
+    return {"value": 32768 / (dt * pairs), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"1 of {pairs} (chunk, head) pairs (they are independent), {reps} rep(s), {dt:.2f} s each, "
+                      f"scaled by {pairs}"}
+
+
+def cpu_block(cores, budget_s=25.0):
+    """Config 4 on the host: the float64 composition of the oracles (TimestepNorm
+    closed form, CEMA kernel + torch.fft convolution, matmul + softmax attention,
+    F.linear projections), forward + backward by autograd, on a prefix of the
+    sequence (every stage but attention is linear in L; attention is cheaper per
+    token below one chunk, so the figure flatters the CPU)."""
+    import torch
+    from oracle import block as oblock
+    Ls = 256
+    g = torch.Generator().manual_seed(1004)
+    D, Z, H, F_ = CFG4["model_dim"], CFG4["z_dim"], CFG4["value_dim"], CFG4["ffn_hidden_dim"]
+    N = CFG4["cema_ndim"]
+    r = lambda *s: (torch.randn(*s, generator=g, dtype=torch.float64) * 0.02).requires_grad_(True)
+    p = {"mega.timenorm.weight": r(D), "mega.timenorm.bias": r(D), "mega.cema.alpha": r(D, N, 1),
+         "mega.cema.delta": r(D, N, 1), "mega.cema.theta": r(D, 1, 1), "mega.cema.gamma": r(D, N, 2),
+         "mega.cema.omega": r(D, 1), "mega.rmsnorm.weight": r(D), "mega.wz.weight": r(Z, D), "mega.wz.bias": r(Z),
+         "mega.wv.weight": r(H, D), "mega.wv.bias": r(H), "mega.wr.weight": r(H, D), "mega.wr.bias": r(H),
+         "mega.wh1.weight": r(D, D), "mega.wh1.bias": r(D), "mega.wh2.weight": r(D, H), "mega.gamma": r(2, Z),
+         "mega.beta": r(2, Z), "nffn.norm.weight": r(D), "nffn.norm.bias": r(D), "nffn.fc1.weight": r(F_, D),
+         "nffn.fc2.weight": r(D, F_), "nffn.fc3.weight": r(F_, D)}
+    x = (torch.rand(1, Ls, D, generator=g, dtype=torch.float64) * 2 - 1).requires_grad_(True)
+    dy = torch.randn(1, Ls, D, generator=g, dtype=torch.float64)
+
+    def step():
+        for t in list(p.values()) + [x]:
+            t.grad = None
+        out = oblock.mega_block_forward(p, x, num_heads=CFG4["num_heads"], ndim=N, chunk_size=CFG4["chunk_size"],
+                                        groups=CFG4["norm_num_groups"])
+        out.backward(dy)
+
+    dt, reps = _timed(step, budget_s, max_reps=2)
+    return {"value": Ls / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"the first {Ls} of 32768 tokens through the float64 oracle of the block "
+                      f"(oracle/block.py), {reps} rep(s), {dt:.2f} s each"}
+
+
+# --------------------------------------------------------------------------- GPU legs
+def dev_ms(torch, fn, n):
+    fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(n):
         fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(n):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / n
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / n
 
-    from megalodon_amd import extension as ops
+
+def block_leg(torch, dev, steps, warmup):
+    from megalodon_amd.modules import MegaBlock
+    torch.manual_seed(1004)
+    blk = MegaBlock(**CFG4).to(dev).bfloat16()
+    gb = torch.Generator().manual_seed(1004)
+    bx = (torch.rand(1, 32768, 4096, generator=gb) * 2 - 1).bfloat16().to(dev).requires_grad_(True)
+    bdy = torch.randn(1, 32768, 4096, generator=gb).bfloat16().to(dev)
+
+    def step():
+        bx.grad = None
+        for prm in blk.parameters():
+            prm.grad = None
+        o, _ = blk(bx)
+        o.backward(bdy)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    del blk, bx, bdy
+    torch.cuda.empty_cache()
+    return dt
+
+
+def cema_leg(torch, dev, steps, warmup, copy_calibration):
+    """Config 1: layer forward + backward; per-kernel device times of the default path."""
+    from megalodon_amd import _lib, synthetic
+    from megalodon_amd.modules import MultiHeadComplexEMA
+    B, D, N, L, seed = 1, 4096, 16, 32768, 1001
+    layer = MultiHeadComplexEMA(D, N).to(dev).train()
+    io = synthetic.cema_inputs(B, D, L, seed, torch.bfloat16)
+    x = io["x"].to(dev).requires_grad_(True)
+    dy = io["dy"].to(dev)
+
+    def step():
+        x.grad = None
+        for prm in layer.parameters():
+            prm.grad = None
+        out, _ = layer(x, None, False)
+        out.backward(dy)
+
+    def timed(n):
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    for _ in range(warmup):
+        step()
+    log = {"mega_cema_scan_fwd": [], "mega_cema_scan_bwd": [], "mega_cema_coeffs_fwd": [], "mega_cema_coeffs_bwd": []}
+    _lib.set_event_log(log)
+    dt = timed(steps)
+    _lib.set_event_log(None)
+    avg = {k: (sum(a.elapsed_time(b) for a, b in v) / max(1, len(v))) for k, v in log.items()}
+    E = B * D * L
+    res = {"ms_per_step": dt * 1e3, "tokens_per_s": B * L / dt,
+           "GBps_on_10E": 10 * E / dt / 1e9, "frac_hbm_on_10E": 10 * E / dt / 1e9 / HBM_PEAK_GBS,
+           "kernels_ms": avg,
+           "scan_fwd_GBps": 4 * E / (avg["mega_cema_scan_fwd"] * 1e-3) / 1e9,
+           "scan_bwd_GBps": 6 * E / (avg["mega_cema_scan_bwd"] * 1e-3) / 1e9}
+    # the same step on the FFT-convolution operators: float32 transforms, then the fp16-stage engine
+    n_alt = max(1, min(5, steps))
+    os.environ["MEGA_CEMA_FFT"] = "1"
+    try:
+        res["fft_conv_fp32_engine"] = {"ms_per_step": timed(n_alt) * 1e3, "steps": n_alt}
+        os.environ["MEGA_FFTCONV_F16_STAGES"] = "1"
+        res["fft_conv_f16_stage_engine"] = {"ms_per_step": timed(n_alt) * 1e3, "steps": n_alt}
+    finally:
+        os.environ.pop("MEGA_CEMA_FFT", None)
+        os.environ.pop("MEGA_FFTCONV_F16_STAGES", None)
+    if copy_calibration:
+        src = torch.ones(1 << 29, dtype=torch.bfloat16, device=dev)
+        dst = torch.empty_like(src)
+        torch.mul(src, 1.0, out=dst)  # reads 2^30 bytes, writes 2^30 bytes
+        torch.cuda.synchronize()
+        del src, dst
+    roofline = {
+        "bound": "hbm",
+        "kernel": "cema_scan_bwd_kernel<bf16> (one launch = backward of the CEMA layer for all B*D rows: dx and the "
+                  "gradients of p, q, gamma, omega from dy and x; the longest kernel of the config-1 step)",
+        "achieved": res["scan_bwd_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": res["scan_bwd_GBps"] / HBM_PEAK_GBS, "traffic": CEMA_BWD_TRAFFIC_BYTES,
+        "algorithmic_bytes": 6 * E,
+    }
+    return res, roofline
+
+
+def other_ops(torch, dev):
+    """TimestepNorm (config 2) and chunk attention (config 3), timed with device events."""
+    from megalodon_amd import extension as ops, synthetic
     other = {}
     tB, tL, tD, tG = 4, 8192, 4096, 32
     tio = {k_: v_.to(dev) for k_, v_ in synthetic.timestep_norm_inputs(tB, tL, tD, tG, 1002).items()}
@@ -105,14 +298,15 @@ def other_ops(torch, dev, synthetic):
     fwd = lambda: ops.group_timestep_norm_fwd(tio["x"], tio["prev_count"], tio["prev_mean"], tio["prev_var"],
                                               tio["gamma"], tio["beta"], tio["mask"], tG, 1e-5)
     ty, tcount, tmean, tvar, tcm, tcr = fwd()
-    ms = dev_ms(fwd, 10)
-    # GBps / frac_hbm price the op at its 4E (6E) algorithmic bytes; padding rows
-    # are written (zeros) but never read, so GBps_moved counts them once less
-    live = 1.0 - float(tio["mask"].float().mean()) if tio.get("mask") is not None else 1.0
+    ms = dev_ms(torch, fwd, 10)
+    # GBps / frac_hbm price the op at its 4E (6E) algorithmic bytes; padding rows are written
+    # (zeros) but never read, so GBps_moved counts them once less
+    live = 1.0 - float(tio["mask"].float().mean())
     other["timestep_norm_fwd"] = {"ms": ms, "GBps": 4 * tE / ms / 1e6, "frac_hbm": 4 * tE / ms / 1e6 / HBM_PEAK_GBS,
                                   "unmasked_steps": live, "GBps_moved": (2 + 2 * live) * tE / ms / 1e6}
-    ms = dev_ms(lambda: ops.group_timestep_norm_bwd(tio["dy"], tio["dmean"], tio["dvar"], tio["x"], tio["prev_mean"],
-                                                    tcount, tcm, tcr, tio["gamma"], tio["mask"], tG), 10)
+    ms = dev_ms(torch, lambda: ops.group_timestep_norm_bwd(tio["dy"], tio["dmean"], tio["dvar"], tio["x"],
+                                                           tio["prev_mean"], tcount, tcm, tcr, tio["gamma"],
+                                                           tio["mask"], tG), 10)
     other["timestep_norm_bwd"] = {"ms": ms, "GBps": 6 * tE / ms / 1e6, "frac_hbm": 6 * tE / ms / 1e6 / HBM_PEAK_GBS,
                                   "unmasked_steps": live, "GBps_moved": (2 + 4 * live) * tE / ms / 1e6}
     del tio, ty, tcm, tcr
@@ -120,38 +314,11 @@ def other_ops(torch, dev, synthetic):
     pairs = 4096 * 4097 // 2
     f_fwd, f_bwd = 2 * pairs * (256 + 2048) * 32, 2 * pairs * (2 * 256 + 2 * 2048) * 32
     ay, aw = ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True)
-    ms = dev_ms(lambda: ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True), 3)
+    ms = dev_ms(torch, lambda: ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True), 5)
     other["attention_fwd"] = {"ms": ms, "TFLOPs": f_fwd / ms / 1e9, "frac_mfma_bf16": f_fwd / ms / 1e9 / 2516.6}
-    ms = dev_ms(lambda: ops.attention_bwd(aio["dy"], aio["q"], aio["k"], aio["v"], aw, 1.0, True), 3)
+    ms = dev_ms(torch, lambda: ops.attention_bwd(aio["dy"], aio["q"], aio["k"], aio["v"], aw, 1.0, True), 5)
     other["attention_bwd"] = {"ms": ms, "TFLOPs": f_bwd / ms / 1e9, "frac_mfma_bf16": f_bwd / ms / 1e9 / 2516.6}
     del aio, ay, aw
-    torch.cuda.empty_cache()
-
-    # config 4: one full 7B-style block forward+backward (random init std 0.02, bf16)
-    from megalodon_amd.modules import MegaBlock
-    torch.manual_seed(1004)
-    blk = MegaBlock(model_dim=4096, z_dim=1024, value_dim=8192, num_heads=4, cema_ndim=16, chunk_size=4096,
-                    ffn_hidden_dim=11008, norm_num_groups=32).to(dev).bfloat16()
-    gb = torch.Generator().manual_seed(1004)
-    bx = (torch.rand(1, 32768, 4096, generator=gb) * 2 - 1).bfloat16().to(dev).requires_grad_(True)
-    bdy = torch.randn(1, 32768, 4096, generator=gb).bfloat16().to(dev)
-
-    def block_step():
-        bx.grad = None
-        for prm in blk.parameters():
-            prm.grad = None
-        o, _ = blk(bx)
-        o.backward(bdy)
-
-    block_step()
-    torch.cuda.synchronize()
-    tb0 = time.perf_counter()
-    for _ in range(3):
-        block_step()
-    torch.cuda.synchronize()
-    bms = (time.perf_counter() - tb0) / 3 * 1e3
-    other["block_config4_fwd_bwd"] = {"ms": bms, "tokens_per_s": 32768 / (bms * 1e-3)}
-    del blk, bx, bdy
     torch.cuda.empty_cache()
     return other
 
@@ -162,8 +329,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--skip-other-ops", action="store_true",
-                    help="time only the config-1 step (short runs under a profiler)")
+    ap.add_argument("--cema-only", action="store_true",
+                    help="time only the config-1 layer step (short runs under a profiler)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain elementwise copy of 1 GiB in, 1 GiB out "
                          "(reference point for scaling FETCH_SIZE / WRITE_SIZE counters)")
@@ -175,8 +342,7 @@ def main():
         sys.exit(2)
 
     import torch
-    from megalodon_amd import _lib, synthetic
-    from megalodon_amd.modules import MultiHeadComplexEMA
+    from megalodon_amd import _lib
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -184,112 +350,44 @@ def main():
     _lib.load()  # fails loudly when the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    B, D, N, L, seed = 1, 4096, 16, 32768, 1001
 
-    layer = MultiHeadComplexEMA(D, N).to(dev)
-    layer.train()
-    io = synthetic.cema_inputs(B, D, L, seed, torch.bfloat16)
-    x = io["x"].to(dev).requires_grad_(True)
-    dy = io["dy"].to(dev)
+    cema, roofline = cema_leg(torch, dev, args.steps, args.warmup, args.copy_calibration)
+    if args.cema_only:
+        print(json.dumps({"cema_layer": cema, "roofline": roofline}), flush=True)
+        return
+    other = other_ops(torch, dev)
+    dt = block_leg(torch, dev, args.steps, args.warmup)
 
-    def step():
-        x.grad = None
-        for prm in layer.parameters():
-            prm.grad = None
-        out, _ = layer(x, None, False)
-        out.backward(dy.to(out.dtype))
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-
-    log = {"mega_fftconv_residual_fwd_saving": [], "mega_fftconv_residual_bwd_saved": [],
-           "mega_ema_weight_fwd": [], "mega_ema_weight_bwd": []}
-    _lib.set_event_log(log)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    _lib.set_event_log(None)
-
-    def avg_ms(name):
-        ev = log[name]
-        return sum(a.elapsed_time(b) for a, b in ev) / max(1, len(ev))
-
-    E = B * D * L
-    ms_step = dt / args.steps * 1e3
-    conv_ms = avg_ms("mega_fftconv_residual_fwd_saving")  # one launch of the convolution kernel
-    conv_bytes = 8 * E  # x 2E + k 4E in, y 2E out (bf16 rows, fp32 kernel); the saved spectra are not counted
-    achieved = conv_bytes / (conv_ms * 1e-3) / 1e9
-    kernels = {
-        "fftconv_fwd_ms": conv_ms,
-        "fftconv_bwd_ms": avg_ms("mega_fftconv_residual_bwd_saved"),
-        "ema_weight_fwd_ms": avg_ms("mega_ema_weight_fwd"),
-        "ema_weight_bwd_ms": avg_ms("mega_ema_weight_bwd"),
-    }
-    # dy 2E in, dx 2E + dk 4E out; x and k are not read again (their spectra are: not counted)
-    kernels["fftconv_bwd_GBps"] = 8 * E / (kernels["fftconv_bwd_ms"] * 1e-3) / 1e9
-    kernels["ema_weight_fwd_GBps"] = 4 * E / (kernels["ema_weight_fwd_ms"] * 1e-3) / 1e9
-    kernels["ema_weight_bwd_GBps"] = 4 * E / (kernels["ema_weight_bwd_ms"] * 1e-3) / 1e9
-
-    # the same step with every FFT butterfly in fp32 on the vector ALUs
-    fp32_engine = None
-    if not args.skip_other_ops:
-        os.environ["MEGA_FFTCONV_VALU"] = "1"
-        try:
-            step()
-            torch.cuda.synchronize()
-            n32 = max(1, min(5, args.steps))
-            t1 = time.perf_counter()
-            for _ in range(n32):
-                step()
-            torch.cuda.synchronize()
-            dt32 = (time.perf_counter() - t1) / n32
-        finally:
-            os.environ.pop("MEGA_FFTCONV_VALU", None)
-        fp32_engine = {"ms_per_step": dt32 * 1e3, "tokens_per_s": B * L / dt32, "steps": n32}
-
-    if args.copy_calibration:
-        src = torch.ones(1 << 29, dtype=torch.bfloat16, device=dev)
-        dst = torch.empty_like(src)
-        torch.mul(src, 1.0, out=dst)  # reads 2^30 bytes, writes 2^30 bytes
-        torch.cuda.synchronize()
-        del src, dst
-
-    other = {}
-    if not args.skip_other_ops:
-        other = other_ops(torch, dev, synthetic)
     result = {
         "metric": "Megalodon layer fwd+bwd tokens/s at L=32K, 1 GPU; CEMA+FFT-conv HBM GB/s (% peak)",
-        "value": B * L / (dt / args.steps),
+        "value": 32768 / dt,
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_step,
+        "ms_per_step": dt * 1e3,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16*f16+f32",
+        "dtype": "bf16 (fp32 accumulation; CEMA recurrence, norm statistics and softmax in fp32)",
         "data": "synthetic",
-        "config": {"workload": "configs[1]: CEMA + causal FFT convolution forward+backward, "
-                               "B=1 L=32768 D=4096 ndim=16, x/dy bf16, k/dk fp32; DFT stages fp16 operands "
-                               "with fp32 accumulation on the matrix cores, everything else fp32",
-                   "global_batch": B, "seq_len": L},
-        "roofline": {
-            "bound": "hbm", "kernel": "fftconv_mfma_kernel<bf16, MODE=0> (one launch = forward conv of all rows, skip term "
-                                      "included, spectra of x and k kept for the backward launch)",
-            "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": FFTCONV_TRAFFIC_BYTES,
-        },
-        "kernels": kernels,
-        "fp32_fft_engine": fp32_engine,
+        "config": {"workload": "configs[4]: one Megalodon-7B-style block forward+backward, B=1 L=32768 D=4096, "
+                               "EMA ndim 16, z 1024, value 8192, 4 heads, chunk 4096, FFN 11008 SwiGLU, bf16 weights "
+                               "and activations, fp32 norm / EMA parameters; TimestepNorm -> CEMA -> gated chunk "
+                               "attention -> normalized FFN",
+                   "global_batch": 1, "seq_len": 32768},
+        "roofline": roofline,
+        "cema_layer": cema,
         "other_ops": other,
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(B, D, N, L, seed)
+        cores = host_cores()
+        torch.set_num_threads(cores)
+        os.environ.setdefault("OMP_NUM_THREADS", str(cores))
+        result["cpu_baseline"] = cpu_block(cores)
+        result["cpu_ops"] = {"cema_conv_config1": cpu_cema(1, 4096, 16, 32768, 1001, cores),
+                             "timestep_norm_config2": cpu_timestep_norm(cores),
+                             "attention_config3": cpu_attention(cores)}
     print(json.dumps(result), flush=True)
 
 
