@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # WRITE_SIZE x 1.0 from two rocprofv3 --pmc passes of this script (--cema-only --copy-calibration),
 # the factors being what the same counters read for a plain copy of 2^30 bytes.  A measured
 # constant (profiles/cema_scan_config1_hbm_traffic.txt): counters cannot be read from in here.
-CEMA_BWD_TRAFFIC_BYTES = None
+CEMA_BWD_TRAFFIC_BYTES = 8.097e8
 
 CFG4 = dict(model_dim=4096, z_dim=1024, value_dim=8192, num_heads=4, cema_ndim=16, chunk_size=4096,
             ffn_hidden_dim=11008, norm_num_groups=32)
