@@ -745,25 +745,35 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
         sm.red[wave][g][4 * i + 3] = wdacc[i].y;
       }
     }
-    // dkin[l] = sum_j M[j + l][j]: each wave sums the diagonals of its own M, one tile at a
-    // time through its own rows of the state buffer ([register][lane]); lane = lag l
+    // dkin[l] = sum_j M[j + l][j]: each wave sums the diagonals of its own M, one 32 x 32 tile
+    // at a time through its own rows of the state buffer ([i][j], pitch 33).  Lane t takes the
+    // diagonal d = t - 31 of a tile, sum_j tile[j + d][j]; it belongs to lag d in the tiles
+    // (0,0), (1,1) (only d >= 0 is asked for) and to lag 32 + d in the tile (1,0).
     {
-      float acc = 0.f;
-      const int l = lane;
+      const int d = lane - 31, jlo = d < 0 ? -d : 0, jhi = d > 0 ? 32 - d : 32;
+      float same = 0.f, cross = 0.f;
 #pragma unroll
       for (int t = 0; t < 3; ++t) {
         wave_sync();
 #pragma unroll
-        for (int i = 0; i < 16; ++i) myrows[i * kWave + lane] = macc[t][i];
+        for (int i = 0; i < 16; ++i) myrows[(8 * (i >> 2) + 4 * g + (i & 3)) * 33 + r] = macc[t][i];
         wave_sync();
-        // tile t holds rows i = 32 (t > 0) + ii, columns j = 32 (t > 1) + jj
-        const int i0 = t > 0 ? 32 : 0, j0 = t > 1 ? 32 : 0;
-        for (int jj = 0; jj < 32; ++jj) {
-          const int ii = j0 + jj + l - i0;  // row inside the tile of the entry on diagonal l
-          if (ii >= 0 && ii < 32) acc += myrows[(4 * (ii >> 3) + (ii & 3)) * kWave + 32 * ((ii >> 2) & 1) + jj];
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+          const float v = myrows[(j < jlo || j >= jhi) ? 0 : d * 33 + j * 34];
+          acc += (j < jlo || j >= jhi) ? 0.f : v;
         }
+        if (t == 1) cross = acc; else same += acc;
       }
-      sm.dpart[wave][l] = acc;
+      wave_sync();
+      myrows[lane] = same;
+      myrows[64 + lane] = cross;
+      wave_sync();
+      // lag l: same[d = l] (l <= 31) + cross[d = l - 32] (l >= 1)
+      float v = lane >= 1 ? myrows[64 + lane - 1] : 0.f;
+      if (lane <= 31) v += myrows[31 + lane];
+      sm.dpart[wave][lane] = v;
     }
     __syncthreads();  // every wave is done with the state buffer: it takes the power table again
     if (tid < kT) sm.dkin[tid] = (sm.dpart[0][tid] + sm.dpart[1][tid]) + (sm.dpart[2][tid] + sm.dpart[3][tid]);
