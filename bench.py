@@ -310,6 +310,22 @@ def other_ops(torch, dev):
     other["timestep_norm_bwd"] = {"ms": ms, "GBps": 6 * tE / ms / 1e6, "frac_hbm": 6 * tE / ms / 1e6 / HBM_PEAK_GBS,
                                   "unmasked_steps": live, "GBps_moved": (2 + 4 * live) * tE / ms / 1e6}
     del tio, ty, tcm, tcr
+    # what a kernel that only moves the same streams reaches: one read + one write stream of 2E
+    # bytes each (the forward passes), two reads + one write (the backward passes)
+    a = torch.empty(2 * tE, dtype=torch.uint8, device=dev).random_()
+    b = torch.empty_like(a).random_()
+    ceiling = {}
+    for name, second, streams in (("read1_write1", None, 2), ("read2_write1", b, 3)):
+        best = None
+        for wgs in (2048, 4096, 8192, 16384, 32768):
+            for nt in (False, True):
+                ms = dev_ms(torch, lambda: ops.stream_copy(a, second, wgs, nt), 10)
+                if best is None or ms < best[0]:
+                    best = (ms, wgs, nt)
+        ceiling[name] = {"ms": best[0], "GBps": streams * 2 * tE / best[0] / 1e6,
+                         "frac_hbm": streams * 2 * tE / best[0] / 1e6 / HBM_PEAK_GBS, "workgroups": best[1], "nontemporal": best[2]}
+    other["stream_copy_ceiling"] = ceiling
+    del a, b
     aio = {k_: v_.to(dev) for k_, v_ in synthetic.attention_inputs(8, 4096, 4, 256, 2048, 1003).items()}
     pairs = 4096 * 4097 // 2
     f_fwd, f_bwd = 2 * pairs * (256 + 2048) * 32, 2 * pairs * (2 * 256 + 2 * 2048) * 32

@@ -32,6 +32,7 @@ extern "C" {
 #define MEGA_ERR_INVALID_ARG 1
 #define MEGA_ERR_UNSUPPORTED 2
 #define MEGA_ERR_HIP 3
+#define MEGA_ERR_TIMEOUT 4   /* a bounded device-side wait ran out (mega_group_timestep_norm_status) */
 
 /* element types of activation tensors (x, y, dy, dx, q, k, v ...) */
 #define MEGA_F32 0
@@ -226,6 +227,23 @@ int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, const void* 
                                  int64_t D, int64_t G, void* dx, void* dprev_mean,
                                  void* dprev_var, void* dgamma, void* dbeta,
                                  void* workspace, void* stream);
+
+/* The tiled kernels above hand running statistics from tile to tile through
+ * records in `workspace`; a tile polls for its predecessors' records at most a
+ * fixed number of times (a couple of seconds), then sets a status word in the
+ * workspace, continues with NaN in place of the missing value and exits, so a
+ * launch always drains.  No counterpart in the reference, whose kernels scan a
+ * sequence inside one thread block (timestep_norm_kernel.cu:1288-1325).
+ * mega_group_timestep_norm_status waits for `stream`, reads the status word of
+ * the last forward or backward launch that used `workspace` (NULL: the static
+ * buffer of mega_group_timestep_norm_fwd_static on the current device) and
+ * returns MEGA_OK or MEGA_ERR_TIMEOUT.
+ * mega_test_timestep_norm_lookback is a test hook for the launches that
+ * follow it: `spin_limit` polls per wait (<= 0: the default) and a tile index
+ * that publishes no record (-1: none), which makes its successors run into
+ * the limit without any kernel hanging. */
+int mega_group_timestep_norm_status(const void* workspace, void* stream);
+void mega_test_timestep_norm_lookback(long long spin_limit, int mute_tile);
 
 /* ------------------------------------------------------------------------
  * Chunk attention (causal inside each chunk), fused fp32 softmax.
@@ -521,6 +539,18 @@ int mega_cema_scan_bwd(const void* dy, const void* x, int dtype, const float* p,
                        const float* log_q, const float* gamma, const float* omega, int64_t B,
                        int64_t D, int64_t N, int64_t L, void* dx, float* dp, float* dq,
                        float* dgamma, float* domega, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Streaming reference kernel for measurements (no counterpart in the
+ * reference): out = a (b == NULL) or out = a XOR b over `bytes` bytes
+ * (multiple of 16, operands 16-byte aligned), grid-stride with `workgroups`
+ * workgroups of 256 lanes, 16-byte accesses, eight loads per lane in flight,
+ * with nontemporal accesses if `nontemporal` is non-zero.
+ * Its rate is the practical ceiling the HBM-bound operators are compared with
+ * next to the published peak.
+ * ---------------------------------------------------------------------- */
+int mega_bench_stream_copy(const void* a, const void* b, void* out, int64_t bytes,
+                           int workgroups, int nontemporal, void* stream);
 
 #ifdef __cplusplus
 }

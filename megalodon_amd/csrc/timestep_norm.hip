@@ -29,6 +29,7 @@
 // cost 190 us in tickets alone.)
 #include "common.hpp"
 
+#include <atomic>
 #include <mutex>
 
 #include <algorithm>
@@ -40,6 +41,7 @@ constexpr int kTL = 64;        // timesteps per tile = lanes per wavefront
 constexpr int kThreads = 256;  // 4 wavefronts
 constexpr int kWaves = kThreads / kWave;
 constexpr int kTicketStride = 16;  // ints between ticket counters: one 64-byte line each
+constexpr int kStatusSlot = 1;     // the status word lives in the unused part of the first ticket's line
 
 struct TsnParams {
   const void* x;
@@ -65,9 +67,24 @@ struct TsnParams {
   int* ticket;             // one counter per chain, kTicketStride ints apart (the per-wave forward kernel uses the first)
   const int* nbefore;      // (B, NT+1) unmasked steps before tile j
   unsigned long long* rec; // per (chain, tile) records
+  unsigned int* status;    // one word: bit 0 = a look-back wait ran into spin_limit
+  long long spin_limit;    // polls of one record before a wait is given up
+  int mute_tile;           // test hook: this tile index publishes nothing (-1: none)
   int B, L, D, G, Dg, NT;
   float eps;
 };
+
+// A wait for another tile's record is bounded: tiles of a chain start in time
+// order, so in a healthy launch the record arrives within the predecessor's own
+// run time.  A wave that has polled spin_limit times sets bit 0 of the status
+// word, takes NaN as the missing value (every output that depends on it shows
+// it) and goes on, so the grid always drains;
+// mega_group_timestep_norm_status reports the word to the host.
+constexpr long long kDefaultSpinLimit = 1ll << 22;  // >= 2 s of polling on this part
+constexpr unsigned int kStatusGaveUp = 1u;
+__device__ __forceinline__ void give_up(const TsnParams& p) {
+  __hip_atomic_fetch_or(p.status, kStatusGaveUp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // ---- 64-bit record words: two floats published together -------------------------
 // A word that nobody has written yet holds kEmpty (all ones).  A published word
@@ -223,6 +240,7 @@ __global__ void tsn_prep_kernel(int* ticket, int n_tickets, unsigned long long* 
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t i = gid; i < rec_words; i += stride) rec[i] = kEmpty;
   for (int64_t i = gid; i < n_tickets; i += stride) ticket[i * kTicketStride] = 0;
+  if (gid == 0) ticket[kStatusSlot] = 0;  // the status word of this launch
   // block b (< B) also builds nbefore[b][0..NT]: thread i counts the unmasked
   // steps of tiles i per .. i per + per - 1, a block-wide exclusive scan turns
   // the counts into starting values
@@ -273,6 +291,9 @@ __global__ void tsn_prep_kernel(int* ticket, int n_tickets, unsigned long long* 
   }
 }
 
+// the serial kernels never wait: their launches only reset the workspace's status word
+__global__ void tsn_clear_status_kernel(int* ticket) { ticket[kStatusSlot] = 0; }
+
 // ------------------------------ forward ---------------------------------------
 constexpr int kFwdWords = 2;  // aggregate (u, v), inclusive prefix (u, v)
 
@@ -291,6 +312,7 @@ __device__ __forceinline__ Wel fwd_lookback(const TsnParams& p, int b, int g, in
     if (lane < kWin) {
       if (idx >= 0) {
         const unsigned long long* r = rec + static_cast<int64_t>(idx) * kFwdWords;
+        long long polls = 0;
         while (true) {
           // both words in one round trip: the aggregate counts only if the
           // inclusive prefix is not there yet
@@ -305,6 +327,12 @@ __device__ __forceinline__ Wel fwd_lookback(const TsnParams& p, int b, int g, in
           if (fa) {
             kind = 1;
             val = Wel{static_cast<float>(nb[idx + 1] - nb[idx]), au, av};
+            break;
+          }
+          if (++polls >= p.spin_limit) {
+            give_up(p);
+            kind = 2;
+            val = Wel{prior.n + static_cast<float>(nb[idx + 1]), __builtin_nanf(""), __builtin_nanf("")};
             break;
           }
           __builtin_amdgcn_s_sleep(2);
@@ -410,11 +438,11 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
     }
     unsigned long long* rec = p.rec + (chain64 * p.NT + j) * kFwdWords;
     const Wel agg{__shfl(me.n, 63, 64), __shfl(me.u, 63, 64), __shfl(me.v, 63, 64)};
-    if (lane == 0 && j + 1 < p.NT) {
+    if (lane == 0 && j + 1 < p.NT && j != p.mute_tile) {
       put_pair(rec + 0, agg.u, agg.v);
     }
     const Wel prefix = j == 0 ? prior : fwd_lookback(p, b, g, j, lane, prior);
-    if (lane == 0 && j + 1 < p.NT) {
+    if (lane == 0 && j + 1 < p.NT && j != p.mute_tile) {
       const Wel inc = wel_merge(prefix, agg);
       put_pair(rec + 1, inc.u, inc.v);
     }
@@ -563,11 +591,11 @@ void tsn_fwd_wave_kernel(const TsnParams p, int tiles) {
   }
   unsigned long long* rec = p.rec + (chain64 * p.NT + j) * kFwdWords;
   const Wel agg{__shfl(me.n, 63, 64), __shfl(me.u, 63, 64), __shfl(me.v, 63, 64)};
-  if (lane == 0 && j + 1 < p.NT) {
+  if (lane == 0 && j + 1 < p.NT && j != p.mute_tile) {
     put_pair(rec + 0, agg.u, agg.v);
   }
   const Wel prefix = j == 0 ? prior : fwd_lookback(p, b, g, j, lane, prior);
-  if (lane == 0 && j + 1 < p.NT) {
+  if (lane == 0 && j + 1 < p.NT && j != p.mute_tile) {
     const Wel inc = wel_merge(prefix, agg);
     put_pair(rec + 1, inc.u, inc.v);
   }
@@ -683,6 +711,7 @@ __device__ __forceinline__ State2 bwd_lookahead(const TsnParams& p, int64_t chai
     if (lane < kWin) {
       if (idx < p.NT) {
         const unsigned long long* r = rec + static_cast<int64_t>(idx) * kBwdWords;
+        long long polls = 0;
         while (true) {
           // all three words in one round trip
           float a, e, bu, bv, ug, vg;
@@ -696,6 +725,12 @@ __device__ __forceinline__ State2 bwd_lookahead(const TsnParams& p, int64_t chai
           if (f0 & f1) {
             kind = 1;
             val = Aff{a, e, bu, bv};
+            break;
+          }
+          if (++polls >= p.spin_limit) {
+            give_up(p);
+            kind = 2;
+            sv = State2{__builtin_nanf(""), __builtin_nanf("")};
             break;
           }
           __builtin_amdgcn_s_sleep(2);
@@ -850,7 +885,7 @@ void tsn_bwd_kernel(const TsnParams p) {
       if (lane + d < 64) inc = aff_compose(inc, o);
     }
     unsigned long long* rec = p.rec + (chain64 * p.NT + j) * kBwdWords;
-    if (lane == 0 && j > 0) {
+    if (lane == 0 && j > 0 && j != p.mute_tile) {
       put_pair(rec + 0, inc.a, inc.e);
       put_pair(rec + 1, inc.bu, inc.bv);
     }
@@ -862,7 +897,7 @@ void tsn_bwd_kernel(const TsnParams p) {
     if (lane == 0) {
       const State2 sout = aff_apply(inc, sin);
       if (j > 0) {
-        put_pair(rec + 2, sout.ug, sout.vg);
+        if (j != p.mute_tile) put_pair(rec + 2, sout.ug, sout.vg);
       } else {
         stT<DT>(p.mean, chain64, sout.ug);
         stT<DT>(p.var, chain64, sout.vg);
@@ -1054,6 +1089,11 @@ __global__ __launch_bounds__(kPgWaves * 64) void tsn_param_grad_kernel(
 // ------------------------------ host side --------------------------------------
 inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
+// Test hooks (mega_test_timestep_norm_lookback): the poll limit of the look-back
+// waits and a tile index that publishes no record, for the launches that follow.
+std::atomic<long long> g_spin_limit{kDefaultSpinLimit};
+std::atomic<int> g_mute_tile{-1};
+
 struct WsLayout {
   int64_t ticket_off, nbefore_off, rec_off, rec_words, part_off, total;
 };
@@ -1115,6 +1155,9 @@ int tsn_fwd_impl(TsnParams p, void* workspace, hipStream_t s) {
     const WsLayout w = ws_layout(p.B, p.L, p.D, p.G, kFwdWords, false);
     char* ws = static_cast<char*>(workspace);
     p.ticket = reinterpret_cast<int*>(ws + w.ticket_off);
+    p.status = reinterpret_cast<unsigned int*>(p.ticket + kStatusSlot);
+    p.spin_limit = g_spin_limit.load();
+    p.mute_tile = g_mute_tile.load();
     int* nbefore = reinterpret_cast<int*>(ws + w.nbefore_off);
     p.nbefore = nbefore;
     p.rec = reinterpret_cast<unsigned long long*>(ws + w.rec_off);
@@ -1124,6 +1167,7 @@ int tsn_fwd_impl(TsnParams p, void* workspace, hipStream_t s) {
     MEGA_CHECK_LAUNCH();
     return launch_fast<DT, true>(p, static_cast<int64_t>(p.B) * p.G * NT, s);
   }
+  tsn_clear_status_kernel<<<1, 1, 0, s>>>(static_cast<int*>(workspace));
   tsn_fwd_serial_kernel<DT><<<p.B * p.G, kWave, 0, s>>>(p);
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
@@ -1139,6 +1183,9 @@ int tsn_bwd_impl(TsnParams p, void* dgamma, void* dbeta, void* workspace, hipStr
   int rows;
   if (fast_path_ok(DT, p.D, p.Dg, p.x, p.y, p.dy) && fast_path_ok(DT, p.D, p.Dg, p.gamma, nullptr, nullptr)) {
     p.ticket = reinterpret_cast<int*>(ws + w.ticket_off);
+    p.status = reinterpret_cast<unsigned int*>(p.ticket + kStatusSlot);
+    p.spin_limit = g_spin_limit.load();
+    p.mute_tile = g_mute_tile.load();
     int* nbefore = reinterpret_cast<int*>(ws + w.nbefore_off);
     p.nbefore = nbefore;
     p.rec = reinterpret_cast<unsigned long long*>(ws + w.rec_off);
@@ -1150,6 +1197,7 @@ int tsn_bwd_impl(TsnParams p, void* dgamma, void* dbeta, void* workspace, hipStr
     if (rc != MEGA_OK) return rc;
     rows = static_cast<int>(p.B * NT);
   } else {
+    tsn_clear_status_kernel<<<1, 1, 0, s>>>(static_cast<int*>(workspace));
     tsn_bwd_serial_kernel<DT><<<p.B * p.G, kWave, 0, s>>>(p);
     MEGA_CHECK_LAUNCH();
     rows = p.B;
@@ -1237,6 +1285,13 @@ extern "C" int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, c
   }
 }
 
+// Test hook: look-back poll limit (<= 0 restores the default) and a tile index
+// that publishes no record (-1: none) for the launches that follow.
+extern "C" void mega_test_timestep_norm_lookback(long long spin_limit, int mute_tile) {
+  g_spin_limit.store(spin_limit > 0 ? spin_limit : kDefaultSpinLimit);
+  g_mute_tile.store(mute_tile);
+}
+
 // ---- forward without a caller workspace: a static device buffer ---------------------
 // Callers that may not allocate (graph capture, serving loops) get the
 // forward's scratch (tickets, per-tile counts, look-back records) from a
@@ -1266,6 +1321,32 @@ int static_scratch(void** out) {
   return MEGA_OK;
 }
 }  // namespace
+
+// Status of the last fast-path launch that used `workspace`: waits for the
+// stream, reads the launch's status word and returns MEGA_OK, or
+// MEGA_ERR_TIMEOUT when a look-back wait was given up (the outputs that
+// depended on the missing record are NaN).  The serial kernels never wait.
+// A null `workspace` means the static buffer of mega_group_timestep_norm_fwd_static
+// on the current device.
+extern "C" int mega_group_timestep_norm_status(const void* workspace, void* stream) {
+  if (workspace == nullptr) {
+    void* ptr = nullptr;
+    const int rc = static_scratch(&ptr);
+    if (rc != MEGA_OK) return rc;
+    workspace = ptr;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  unsigned int word = 0;
+  MEGA_CHECK_HIP(hipMemcpyAsync(&word, static_cast<const int*>(workspace) + kStatusSlot, sizeof(word),
+                                hipMemcpyDeviceToHost, s));
+  MEGA_CHECK_HIP(hipStreamSynchronize(s));
+  if (word & kStatusGaveUp)
+    return set_error(MEGA_ERR_TIMEOUT,
+                     "TimestepNorm: a tile gave up waiting for an earlier tile's record after %lld polls; "
+                     "the outputs that depend on it are NaN",
+                     g_spin_limit.load());
+  return MEGA_OK;
+}
 
 extern "C" int64_t mega_group_timestep_norm_static_scratch_bytes(void) { return kStaticScratchBytes; }
 

@@ -355,7 +355,12 @@ def fftconv_fwd(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
 
     Differs from the reference's ``fftconv_fwd(x, k_f) -> (y, x_f)`` in taking
     the time-domain kernel and returning no saved spectrum: backward recomputes
-    it (1 GiB of ``x_f`` is not kept alive between forward and backward)."""
+    it (1 GiB of ``x_f`` is not kept alive between forward and backward).
+
+    With a complex ``k`` the call is the reference's own: ``fftconv_fwd(x, k_f)
+    -> (y, x_f)`` (see ``_fftconv_fwd_spectral``)."""
+    if k.is_complex():
+        return _fftconv_fwd_spectral(x, k)
     dev = _require_cuda(x, k)
     if x.dim() != 3 or k.dim() != 2 or k.shape[0] != x.shape[1] or k.shape[1] != x.shape[2]:
         raise RuntimeError(f"fftconv: x {tuple(x.shape)} and k {tuple(k.shape)} do not match (B,D,L)/(D,L)")
@@ -373,7 +378,11 @@ def fftconv_fwd(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
 
 def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
                 k_dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
-    """(dx, dk) with dk of dtype ``k_dtype`` (fftconv.py:53-75)."""
+    """(dx, dk) with dk of dtype ``k_dtype`` (fftconv.py:53-75).  With complex
+    ``x`` and ``k`` the call is the reference's ``fftconv_bwd(y_grad, x_f, k_f,
+    k_dtype)``."""
+    if x.is_complex() or k.is_complex():
+        return _fftconv_bwd_spectral(y_grad, x, k, k_dtype)
     dev = _require_cuda(y_grad, x, k)
     B, D, L = x.shape
     if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
@@ -391,6 +400,39 @@ def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
                   _lib.ptr(kc), _lib.i64(B), _lib.i64(D), _lib.i64(L), _lib.ptr(dx), _lib.ptr(dk),
                   _lib.stream_ptr(dev))
     return dx, dk.to(k_dtype)
+
+
+# The reference's operator signatures (megalodon/csrc/ops/fftconv.cc:10-19,
+# called from fused_ops/fftconv.py:79-106): the kernel arrives as the spectrum
+# k_f = rfft(k, n=2M) (D, M+1), M = L rounded up to a power of two, unnormalised,
+# and the forward hands back x_f = rfft(x, n=2M) (B, D, M+1) complex64 for the
+# backward to keep.  The convolution kernels here work from the time-domain rows,
+# so a spectrum is taken back to its row once on entry (exact up to float32
+# rounding: the row was zero padded to 2M before it was transformed, so its first
+# L samples are the row) and x_f is produced for the caller as the reference does.
+def _spectrum_to_row(s: torch.Tensor, L: int, what: str) -> torch.Tensor:
+    M = 1 << max(0, (L - 1).bit_length())
+    if not s.is_complex() or s.shape[-1] != M + 1:
+        raise RuntimeError(f"fftconv: {what} must be the complex spectrum of {M + 1} bins of rows of length {L}, "
+                           f"got {tuple(s.shape)} {s.dtype}")
+    return torch.fft.irfft(s.to(torch.complex64), n=2 * M)[..., :L].contiguous()
+
+
+def _fftconv_fwd_spectral(x: torch.Tensor, k_f: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    _require_cuda(x, k_f)
+    L = x.shape[-1]
+    M = 1 << max(0, (L - 1).bit_length())
+    y = fftconv_fwd(x, _spectrum_to_row(k_f, L, "k_f"))
+    x_f = rfft(x, False) if 32 <= M <= 16384 else torch.fft.rfft(x.float(), n=2 * M)
+    return y, x_f
+
+
+def _fftconv_bwd_spectral(y_grad: torch.Tensor, x_f: torch.Tensor, k_f: torch.Tensor,
+                          k_dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    _require_cuda(y_grad, x_f, k_f)
+    L = y_grad.shape[-1]
+    x = _spectrum_to_row(x_f, L, "x_f").to(y_grad.dtype)
+    return fftconv_bwd(y_grad, x, _spectrum_to_row(k_f, L, "k_f"), k_dtype)
 
 
 def fftconv_residual_fwd(x: torch.Tensor, k: torch.Tensor, omega: torch.Tensor) -> torch.Tensor:
@@ -591,11 +633,39 @@ def cema_scan_bwd(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, log_q:
 # --------------------------------------------------------------------------
 # group_timestep_norm (reference: csrc/ops/timestep_norm.cc:621-705)
 # --------------------------------------------------------------------------
+# One workspace per (device, stream, direction), grown on demand and kept: no
+# allocation sits in the operator after its first call, and launches on
+# different streams never share one (each call clears what it uses itself).
+_tsn_ws_cache = {}
+
+
 def _tsn_workspace(B, L, D, G, backward, dev):
     fn = _lib.load().mega_group_timestep_norm_workspace_bytes
     fn.restype = _lib.ctypes.c_int64
     nbytes = int(fn(_lib.i64(B), _lib.i64(L), _lib.i64(D), _lib.i64(G), _lib.i32(1 if backward else 0)))
-    return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(dev).cuda_stream, bool(backward))
+    ws = _tsn_ws_cache.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        _tsn_ws_cache[key] = ws
+    return ws
+
+
+def timestep_norm_status(device=None) -> None:
+    """Waits for the current stream of `device` and raises RuntimeError if a tile
+    of the last group_timestep_norm_fwd / _bwd launched on it gave up waiting for
+    an earlier tile's statistics (its outputs are NaN then).  The kernels bound
+    that wait themselves, so a launch always finishes; this call says whether
+    one of them ran into the bound."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    with torch.cuda.device(dev):
+        for backward in (False, True):
+            ws = _tsn_ws_cache.get((idx, stream, backward))
+            if ws is not None:
+                _lib.call("mega_group_timestep_norm_status", _lib.ptr(ws), _lib.stream_ptr(dev))
 
 
 def _mask_bytes(padding_mask):
@@ -687,6 +757,23 @@ def group_timestep_norm_bwd(
                   _lib.ptr(dpm), _lib.ptr(dpv), _lib.ptr(dg), _lib.ptr(db), _lib.ptr(ws),
                   _lib.stream_ptr(dev))
     return dx, dpm, dpv, dg, db
+
+
+def stream_copy(a: torch.Tensor, b: Optional[torch.Tensor] = None, workgroups: int = 8192,
+                nontemporal: bool = False) -> torch.Tensor:
+    """out = a (or a XOR b, bytewise) through the library's streaming reference
+    kernel: the rate a kernel reaches that only moves an operator's bytes."""
+    dev = _require_cuda(a, b)
+    ac = a.contiguous()
+    out = torch.empty_like(ac)
+    nbytes = ac.numel() * ac.element_size()
+    if b is not None and (b.shape != a.shape or b.dtype != a.dtype):
+        raise RuntimeError("stream_copy: b must match a")
+    bc = None if b is None else b.contiguous()
+    with torch.cuda.device(dev):
+        _lib.call("mega_bench_stream_copy", _lib.ptr(ac), _lib.ptr(bc), _lib.ptr(out), _lib.i64(nbytes),
+                  _lib.i32(int(workgroups)), _lib.i32(1 if nontemporal else 0), _lib.stream_ptr(dev))
+    return out
 
 
 # --------------------------------------------------------------------------

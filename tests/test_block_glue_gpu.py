@@ -183,3 +183,15 @@ def test_linear_with_residual_inside_the_gemm():
     # a layer with bias keeps the separate add
     lb = Linear(256, 384, bias=True).cuda().bfloat16()
     assert rel_err(lb(x, residual=r), F.linear(x64, lb.weight.double(), lb.bias.double()) + r64) <= 2e-2
+
+
+@pytest.mark.parametrize("nbytes", [16, 4096 + 16, 3 * 1024 * 1024 + 48])
+@pytest.mark.parametrize("two", [False, True])
+def test_stream_copy_reference_kernel(nbytes, two):
+    from megalodon_amd import extension as ops
+    a = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
+    b = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") if two else None
+    for wgs in (1, 7, 512):
+        for nt in (False, True):
+            out = ops.stream_copy(a, b, wgs, nt)
+            assert torch.equal(out, a ^ b if two else a)

@@ -376,3 +376,43 @@ def test_fused_fftconv_pair_has_the_reference_call_pattern():
     wdx, wdk = fftconv.fftconv_bwd(dy, x, k)
     assert rel_err(y, fftconv.fftconv_fwd(x, k)) <= 1e-4
     assert dk.dtype == k.dtype and rel_err(dx, wdx) <= 1e-4 and rel_err(dk, wdk) <= 1e-4
+
+
+# The reference's own call pattern (fused_ops/fftconv.py:79-106): the kernel goes
+# in as a spectrum, the forward returns (y, x_f), the backward takes the two
+# spectra and the kernel's dtype.  Only the import line of that file changes.
+def _reference_style_fwd(x, k):
+    L = x.size(-1)
+    N = L if (L & (L - 1)) == 0 else (1 << L.bit_length())
+    if k.dtype in (torch.float32, torch.float64):
+        k_f = torch.fft.rfft(k, 2 * N)
+    else:
+        k_f = ops.rfft(k, False)
+    y, x_f = ops.fftconv_fwd(x, k_f)
+    return y, x_f, k_f
+
+
+@pytest.mark.parametrize("B,D,L", [(2, 3, 32), (2, 3, 1000), (1, 4, 4096), (2, 2, 6001), (1, 3, 16384)])
+@pytest.mark.parametrize("dtype,k_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.float32),
+                                           (torch.float16, torch.float16)])
+def test_reference_call_pattern_with_spectra(B, D, L, dtype, k_dtype):
+    x, k, dy = _data(B, D, L, dtype, 17 * L + D)
+    k = k.to(k_dtype)
+    N = 1 << (L - 1).bit_length()
+    y, x_f, k_f = _reference_style_fwd(x.cuda(), k.cuda())
+    assert y.dtype == dtype and y.shape == x.shape
+    assert x_f.shape == (B, D, N + 1) and x_f.dtype == torch.complex64 and k_f.shape == (D, N + 1)
+    want_xf = torch.fft.rfft(x.double(), n=2 * N)
+    assert rel_err(x_f, want_xf) <= 1e-4
+    assert rel_err(y, fftconv.fftconv_fwd(x.double(), k.double())) <= TOL[dtype]
+    dx, dk = ops.fftconv_bwd(dy.cuda(), x_f, k_f, k_dtype)
+    wdx, wdk = fftconv.fftconv_bwd(dy.double(), x.double(), k.double())
+    assert dx.dtype == dtype and dk.dtype == k_dtype and dk.shape == (D, L)
+    assert rel_err(dx, wdx) <= TOL[dtype]
+    assert rel_err(dk, wdk) <= TOL[k_dtype]
+
+
+def test_spectral_signature_rejects_wrong_bin_count():
+    x = torch.zeros(1, 2, 100, device="cuda")
+    with pytest.raises(RuntimeError, match="129 bins"):
+        ops.fftconv_fwd(x, torch.zeros(2, 101, dtype=torch.complex64, device="cuda"))

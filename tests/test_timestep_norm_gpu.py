@@ -231,3 +231,38 @@ def test_padding_rows_are_never_read(mask, dtype):
         else:
             assert rel_err(b_, a.double()) <= (1e-5 if dtype == torch.float32 else 1e-2)
     assert (outs[1][0][m] == 0).all() and (outs[1][6][m] == 0).all()   # y and dx at masked steps
+
+
+# A tile's wait for its predecessors' records is bounded.  The host forces the
+# condition (one tile index publishes nothing, the poll limit is tiny): every
+# kernel still exits, the status call reports the timeout, the outputs that
+# depended on the missing record are NaN, and the next ordinary launch on the
+# same workspace is clean again.
+@pytest.mark.parametrize("H,G", [(256, 2), (1024, 2)])      # per-wave tiles / one workgroup per tile
+def test_lookback_wait_is_bounded(H, G):
+    from megalodon_amd import _lib
+    B, L = 2, 64 * 6
+    x, pc, pm, pv, gamma, beta, _, dy, dmean, dvar = _case(B, L, H, G, 3, torch.bfloat16, mask=None)
+    args = _cuda(x, pc, pm, pv, gamma, beta)
+    good = ops.group_timestep_norm_fwd(*args, None, G, 1e-5)
+    ops.timestep_norm_status()
+    hook = _lib.load().mega_test_timestep_norm_lookback
+    hook.restype = None
+    try:
+        hook(_lib.ctypes.c_longlong(500), _lib.ctypes.c_int(2))
+        y = ops.group_timestep_norm_fwd(*args, None, G, 1e-5)[0]
+        with pytest.raises(RuntimeError, match="gave up waiting"):
+            ops.timestep_norm_status()
+        assert torch.equal(y[:, :64 * 3], good[0][:, :64 * 3])        # tiles 0..2 never needed tile 2's record
+        assert torch.isnan(y[:, 64 * 3:].float()).all()               # tiles 3.. did
+        dxm = ops.group_timestep_norm_bwd(*_cuda(dy, dmean, dvar, x, pm), good[1], good[4], good[5],
+                                          args[4], None, G)[0]
+        with pytest.raises(RuntimeError, match="gave up waiting"):
+            ops.timestep_norm_status()
+        assert torch.isnan(dxm[:, :64 * 2].float()).all()             # the backward runs from the end
+    finally:
+        hook(_lib.ctypes.c_longlong(0), _lib.ctypes.c_int(-1))
+    again = ops.group_timestep_norm_fwd(*args, None, G, 1e-5)
+    dx = ops.group_timestep_norm_bwd(*_cuda(dy, dmean, dvar, x, pm), again[1], again[4], again[5], args[4], None, G)[0]
+    ops.timestep_norm_status()
+    assert torch.equal(again[0], good[0]) and torch.isfinite(dx.float()).all()
