@@ -560,7 +560,7 @@ struct BwdSmem {
 };
 static_assert(sizeof(cf) * 16 * (kT + 2) + sizeof(cf) * 16 * 2 * 16 <= sizeof(float) * kBwdNC * kRP,
               "the power table and the final partial sums live in the state buffer");
-static_assert(32 * kSP * 2 <= 32 * kRP * 4 && 16 * kWave * 4 <= 32 * kRP * 4,
+static_assert(32 * kSP * 2 <= 32 * kRP * 4 && 16 * kWave * 4 <= 32 * kRP * 4 && kWave * 33 <= 32 * kRP,
               "a wave's parked tile and one accumulator tile fit its own rows of the state buffer");
 static_assert(sizeof(BwdSmem) <= 80 * 1024, "two workgroups per compute unit");
 
@@ -728,52 +728,64 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
   // the row's reductions and its five gradient outputs
   auto finish_row = [&](int64_t row) {
     MEGA_LANE_IDS;
-    // W, W': over the 32 lanes (chunks) of a half wave, then over the waves
+    // W, W': over the 32 lanes (chunks) of a half wave, then over the waves.  A lane holds 32
+    // partial sums (8 modes x (W, W') x (re, im)) and each half of the wave its own 8 modes: the
+    // wave transposes them through its rows of the state buffer ([lane][value], pitch 33), and
+    // lane (g, t) adds up value t of half g.
+    wave_sync();
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      wacc[i].x = group_sum<32>(wacc[i].x);
-      wacc[i].y = group_sum<32>(wacc[i].y);
-      wdacc[i].x = group_sum<32>(wdacc[i].x);
-      wdacc[i].y = group_sum<32>(wdacc[i].y);
+      float* dst = myrows + lane * 33 + 4 * i;
+      dst[0] = wacc[i].x;
+      dst[1] = wacc[i].y;
+      dst[2] = wdacc[i].x;
+      dst[3] = wdacc[i].y;
     }
-    if (r == 0) {
+    wave_sync();
+    {
+      float part[32];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        sm.red[wave][g][4 * i] = wacc[i].x;
-        sm.red[wave][g][4 * i + 1] = wacc[i].y;
-        sm.red[wave][g][4 * i + 2] = wdacc[i].x;
-        sm.red[wave][g][4 * i + 3] = wdacc[i].y;
-      }
+      for (int j = 0; j < 32; ++j) part[j] = myrows[(32 * g + j) * 33 + r];
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < 32; ++j) acc += part[j];
+      sm.red[wave][g][r] = acc;
     }
     // dkin[l] = sum_j M[j + l][j]: each wave sums the diagonals of its own M, one 32 x 32 tile
-    // at a time through its own rows of the state buffer ([i][j], pitch 33).  Lane t takes the
-    // diagonal d = t - 31 of a tile, sum_j tile[j + d][j]; it belongs to lag d in the tiles
-    // (0,0), (1,1) (only d >= 0 is asked for) and to lag 32 + d in the tile (1,0).
+    // at a time through its own rows of the state buffer ([i][j], pitch 33).  Lane (g, t) walks
+    // the wrapped diagonal tile[(j + t) mod 32][j] over its 16 columns j = 16 g .. 16 g + 15:
+    // the part with j + t < 32 belongs to the diagonal d = t, the rest to d = t - 32.  The tiles
+    // (0,0) and (1,1) hold the same lags d >= 0 (their d < 0 is not asked for) and are added
+    // first; the tile (1,0) holds lag 32 + d for both signs of d.
     {
-      const int d = lane - 31, jlo = d < 0 ? -d : 0, jhi = d > 0 ? 32 - d : 32;
-      float same = 0.f, cross = 0.f;
+      float lo[2], hi[2];
 #pragma unroll
-      for (int t = 0; t < 3; ++t) {
+      for (int t = 0; t < 2; ++t) {
         wave_sync();
 #pragma unroll
-        for (int i = 0; i < 16; ++i) myrows[(8 * (i >> 2) + 4 * g + (i & 3)) * 33 + r] = macc[t][i];
+        for (int i = 0; i < 16; ++i)
+          myrows[(8 * (i >> 2) + 4 * g + (i & 3)) * 33 + r] = t == 0 ? macc[0][i] + macc[2][i] : macc[1][i];
         wave_sync();
-        float acc = 0.f;
+        float v[16];
 #pragma unroll
-        for (int j = 0; j < 32; ++j) {
-          const float v = myrows[(j < jlo || j >= jhi) ? 0 : d * 33 + j * 34];
-          acc += (j < jlo || j >= jhi) ? 0.f : v;
+        for (int jj = 0; jj < 16; ++jj) {
+          const int j = 16 * g + jj;
+          v[jj] = myrows[((j + r) & 31) * 33 + j];
         }
-        if (t == 1) cross = acc; else same += acc;
+        lo[t] = hi[t] = 0.f;
+#pragma unroll
+        for (int jj = 0; jj < 16; ++jj) {
+          const bool below = 16 * g + jj + r < 32;
+          lo[t] += below ? v[jj] : 0.f;
+          hi[t] += below ? 0.f : v[jj];
+        }
       }
-      wave_sync();
-      myrows[lane] = same;
-      myrows[64 + lane] = cross;
-      wave_sync();
-      // lag l: same[d = l] (l <= 31) + cross[d = l - 32] (l >= 1)
-      float v = lane >= 1 ? myrows[64 + lane - 1] : 0.f;
-      if (lane <= 31) v += myrows[31 + lane];
-      sm.dpart[wave][lane] = v;
+      // the two halves of the wave took different columns
+      const float same = lo[0] + __shfl_xor(lo[0], 32, 64);
+      const float cross_lo = lo[1] + __shfl_xor(lo[1], 32, 64);
+      const float cross_hi = hi[1] + __shfl_xor(hi[1], 32, 64);
+      // lag l <= 31: same[d = l] + cross[d = l - 32]; lag l >= 32: cross[d = l - 32]
+      sm.dpart[wave][lane] = g == 0 ? same + cross_hi : cross_lo;
     }
     __syncthreads();  // every wave is done with the state buffer: it takes the power table again
     if (tid < kT) sm.dkin[tid] = (sm.dpart[0][tid] + sm.dpart[1][tid]) + (sm.dpart[2][tid] + sm.dpart[3][tid]);
