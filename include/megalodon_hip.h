@@ -252,8 +252,12 @@ void mega_test_timestep_norm_lookback(long long spin_limit, int mute_tile);
  *   reference: megalodon/csrc/ops/attention_kernel.cu:40-133,261-281,
  *              megalodon/csrc/softmax.cuh:86-131, binding attention.cc:28.
  *   q (B, L1, NH, H1), k (B, L2, NH, H1), v (B, L2, NH, H2), y (B, L1, NH, H2),
- *   w (B, NH, L1, L2), all of `dtype` (MEGA_BF16 or MEGA_F16), contiguous; B
- *   counts chunks (the module views (batch, L) as (batch*L/chunk, chunk)).
+ *   w (B, NH, L1, L2), all of `dtype`, contiguous; B counts chunks (the
+ *   module views (batch, L) as (batch*L/chunk, chunk)).  MEGA_BF16 / MEGA_F16
+ *   run on the matrix cores and are what follows describes; MEGA_F32
+ *   (attention_kernel.cu:269-281 dispatches over it too) keeps float32 storage
+ *   and arithmetic on the vector ALUs, writes every row of w to its end, and
+ *   needs twice the workspace bytes the size query returns.
  *   S = scale * q k^T rounded to `dtype`; with `causal` row r keeps columns
  *   0 .. L2 - L1 + r (L2 >= L1 required: cached keys / values in front of the
  *   chunk, softmax.cuh:99-100), all columns otherwise; P = softmax in fp32,

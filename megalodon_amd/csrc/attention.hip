@@ -21,11 +21,23 @@
 // A key/value prefix (L2 > L1, cached keys in front of the chunk) shifts the
 // diagonal by L2 - L1 columns in every one of these rules.
 #include "common.hpp"
+#include "dropkey.hpp"
 
 #include <algorithm>
 #include <cstdlib>
 
 namespace mega {
+
+// float32 tensors: attention_f32.hip
+int attention_f32_fwd(const float* q, const float* k, const float* v, int64_t B, int64_t L1, int64_t L2,
+                      int64_t NH, int64_t H1, int64_t H2, float scale, int causal, const DropKey* drop,
+                      float* y, float* w, hipStream_t s);
+int attention_f32_bwd(const float* dy, const float* q, const float* k, const float* v, const float* w,
+                      int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1, int64_t H2, float scale,
+                      int causal, float* dq, float* dk, float* dv, float* dp, hipStream_t s);
+int softmax_f32_fwd(float* x, int64_t Z, int64_t L1, int64_t L2, int causal, const DropKey* drop, hipStream_t s);
+int softmax_f32_bwd(const float* y, float* dy, int64_t Z, int64_t L1, int64_t L2, int causal, hipStream_t s);
+
 namespace {
 
 constexpr int kTile = 256;     // workgroup tile (M and N)
@@ -459,29 +471,6 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
   }  // work item
 }
 
-// ---- DropKey (softmax.cuh:135-196) ----------------------------------------------
-// With probability `p` a key is taken out of a row (its score becomes -inf)
-// before the softmax; the survivors are not rescaled, and the backward needs no
-// mask because a dropped key has probability 0.  The reference draws from
-// curand's Philox stream of the thread that holds the element; here the draw of
-// element (row i, column j) is a pure function of its position, so it does not
-// depend on the kernel flavour or the element type: Philox4x32-10 with counter
-// (j / 4, i, offset_lo, offset_hi) and key (seed_lo, seed_hi) gives four words,
-// element j takes word j % 4, u = (word >> 8) * 2^-24, dropped iff u < p.
-// i counts rows over all matrices (i = matrix * L1 + r < 2^32).
-struct DropKey {
-  float p;
-  uint32_t seed_lo, seed_hi, off_lo, off_hi;
-};
-
-// drops[e] for the four columns 4 * quad .. 4 * quad + 3 of row i
-__device__ __forceinline__ void dropkey_quad(const DropKey& dk, uint32_t i, uint32_t quad, bool* drops) {
-  uint32_t w[4];
-  philox4x32_10(quad, i, dk.off_lo, dk.off_hi, dk.seed_lo, dk.seed_hi, w);
-#pragma unroll
-  for (int e = 0; e < 4; ++e) drops[e] = static_cast<float>(w[e] >> 8) * 0x1p-24f < dk.p;
-}
-
 // ---- causal softmax over rows (in place), one wavefront per row ---------------
 // `coff` < 0: every row keeps all L2 columns.  `coff` = L2 - L1 >= 0 (causal,
 // bottom-right aligned, softmax.cuh:99-100): row r keeps columns [0, n) with
@@ -761,8 +750,7 @@ AttnWs attn_ws(int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1, int64_
 
 int check_attn(const char* who, int dtype, int64_t B, int64_t L1, int64_t L2, int64_t NH,
                int64_t H1, int64_t H2, int causal) {
-  if (dtype != MEGA_BF16 && dtype != MEGA_F16)
-    return set_error(MEGA_ERR_UNSUPPORTED, "%s: only bfloat16 / float16 tensors are supported", who);
+  MEGA_CHECK_ARG(valid_dtype(dtype), "%s: unknown dtype %d", who, dtype);
   MEGA_CHECK_ARG(B >= 0 && L1 >= 0 && L2 >= 0 && NH >= 1 && H1 >= 1 && H2 >= 1, "%s: bad sizes", who);
   MEGA_CHECK_ARG(B * NH <= 65535, "%s: batch * heads exceeds 65535", who);
   MEGA_CHECK_ARG(L1 <= (1 << 24) && L2 <= (1 << 24), "%s: sequence too long", who);
@@ -874,6 +862,10 @@ static int attention_fwd_entry(const char* who, const void* q, const void* k, co
   MEGA_CHECK_ARG(q && k && v && y && w && workspace, "%s: null pointer", who);
   MEGA_CHECK_ARG(L2 >= 1, "%s: no keys", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MEGA_F32)
+    return attention_f32_fwd(static_cast<const float*>(q), static_cast<const float*>(k),
+                             static_cast<const float*>(v), B, L1, L2, NH, H1, H2, (float)scale, causal, drop,
+                             static_cast<float*>(y), static_cast<float*>(w), s);
   auto u = [](const void* p) { return static_cast<const uint16_t*>(p); };
   auto m = [](void* p) { return static_cast<uint16_t*>(p); };
   if (dtype == MEGA_BF16)
@@ -915,6 +907,12 @@ extern "C" int mega_attention_bwd(const void* dy, const void* q, const void* k, 
                  "mega_attention_bwd: null pointer");
   MEGA_CHECK_ARG(L1 >= 1 && L2 >= 1, "mega_attention_bwd: empty sequence");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MEGA_F32)
+    return attention_f32_bwd(static_cast<const float*>(dy), static_cast<const float*>(q),
+                             static_cast<const float*>(k), static_cast<const float*>(v),
+                             static_cast<const float*>(w), B, L1, L2, NH, H1, H2, (float)scale, causal,
+                             static_cast<float*>(dq), static_cast<float*>(dk), static_cast<float*>(dv),
+                             static_cast<float*>(workspace), s);
   auto u = [](const void* p) { return static_cast<const uint16_t*>(p); };
   auto m = [](void* p) { return static_cast<uint16_t*>(p); };
   if (dtype == MEGA_BF16)
@@ -926,8 +924,7 @@ extern "C" int mega_attention_bwd(const void* dy, const void* q, const void* k, 
 
 // ---- standalone causal softmax ---------------------------------------------------
 static int check_softmax(const char* who, int dtype, int64_t Z, int64_t L1, int64_t L2, int causal) {
-  if (dtype != MEGA_BF16 && dtype != MEGA_F16)
-    return set_error(MEGA_ERR_UNSUPPORTED, "%s: only bfloat16 / float16 tensors are supported", who);
+  MEGA_CHECK_ARG(valid_dtype(dtype), "%s: unknown dtype %d", who, dtype);
   MEGA_CHECK_ARG(Z >= 0 && L1 >= 0 && L2 >= 0, "%s: bad sizes", who);
   MEGA_CHECK_ARG(Z <= 65535, "%s: more than 65535 matrices", who);
   MEGA_CHECK_ARG(L1 <= (1 << 24) && L2 <= (1 << 24), "%s: rows too long", who);
@@ -941,6 +938,7 @@ static int softmax_fwd_entry(const char* who, void* x, int dtype, int64_t Z, int
   if (rc != MEGA_OK) return rc;
   MEGA_CHECK_ARG(x != nullptr || Z * L1 * L2 == 0, "%s: null pointer", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MEGA_F32) return softmax_f32_fwd(static_cast<float*>(x), Z, L1, L2, causal, drop, s);
   if (dtype == MEGA_BF16)
     return launch_softmax<MEGA_BF16>(nullptr, static_cast<uint16_t*>(x), Z, L1, L2, causal, s, 1, drop);
   return launch_softmax<MEGA_F16>(nullptr, static_cast<uint16_t*>(x), Z, L1, L2, causal, s, 1, drop);
@@ -970,6 +968,8 @@ extern "C" int mega_attention_softmax_bwd(const void* y, void* dy, int dtype, in
                  "mega_attention_softmax_bwd: null pointer");
   if (Z * L1 * L2 == 0) return MEGA_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MEGA_F32)
+    return softmax_f32_bwd(static_cast<const float*>(y), static_cast<float*>(dy), Z, L1, L2, causal, s);
   if (dtype == MEGA_BF16)
     return launch_softmax<MEGA_BF16>(static_cast<const uint16_t*>(y), static_cast<uint16_t*>(dy), Z, L1,
                                      L2, causal, s, 1);

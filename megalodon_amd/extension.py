@@ -779,12 +779,13 @@ def stream_copy(a: torch.Tensor, b: Optional[torch.Tensor] = None, workgroups: i
 # --------------------------------------------------------------------------
 # attention (reference: csrc/ops/attention.cc:28-29, attention_kernel.cu:261-303)
 # --------------------------------------------------------------------------
-def _attn_workspace(B, L1, L2, NH, H1, H2, backward, dev):
+def _attn_workspace(B, L1, L2, NH, H1, H2, backward, dev, wide=False):
+    # `wide`: float32 tensors need twice the bytes of the 16-bit layout the size query describes
     fn = _lib.load().mega_attention_workspace_bytes
     fn.restype = _lib.ctypes.c_int64
     nbytes = int(fn(_lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH), _lib.i64(H1), _lib.i64(H2),
                     _lib.i32(1 if backward else 0)))
-    return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    return torch.empty(nbytes * (2 if wide else 1), dtype=torch.uint8, device=dev)
 
 
 def _attn_dims(q, k, v):
@@ -826,7 +827,7 @@ def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: floa
         qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
         y = torch.empty((B, L1, NH, H2), dtype=v.dtype, device=dev)
         w = torch.empty((B, NH, L1, L2), dtype=v.dtype, device=dev)
-        ws = _attn_workspace(B, L1, L2, NH, H1, H2, False, dev)
+        ws = _attn_workspace(B, L1, L2, NH, H1, H2, False, dev, q.dtype == torch.float32)
         seed, offset = dropkey_philox_state(dev, L2)
         with torch.cuda.device(dev):
             _lib.call("mega_attention_dropkey_fwd", _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc),
@@ -838,7 +839,7 @@ def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: floa
     qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
     y = torch.empty((B, L1, NH, H2), dtype=v.dtype, device=dev)
     w = torch.empty((B, NH, L1, L2), dtype=v.dtype, device=dev)
-    ws = _attn_workspace(B, L1, L2, NH, H1, H2, False, dev)
+    ws = _attn_workspace(B, L1, L2, NH, H1, H2, False, dev, q.dtype == torch.float32)
     with torch.cuda.device(dev):
         _lib.call("mega_attention_fwd", _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc),
                   _lib.i32(_lib.dtype_code(q.dtype)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH),
@@ -856,7 +857,7 @@ def attention_bwd(y_grad: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: tor
         raise RuntimeError("attention_bwd: w / y_grad shapes do not match q, k, v")
     qc, kc, vc, dy, wc = q.contiguous(), k.contiguous(), v.contiguous(), y_grad.contiguous(), w.contiguous()
     dq, dk, dv = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc)
-    ws = _attn_workspace(B, L1, L2, NH, H1, H2, True, dev)
+    ws = _attn_workspace(B, L1, L2, NH, H1, H2, True, dev, q.dtype == torch.float32)
     with torch.cuda.device(dev):
         _lib.call("mega_attention_bwd", _lib.ptr(dy), _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc), _lib.ptr(wc),
                   _lib.i32(_lib.dtype_code(q.dtype)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH),
@@ -875,7 +876,7 @@ def _softmax_dims(x: torch.Tensor):
 
 def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool) -> torch.Tensor:
     """y = softmax(x) over the last axis (float32 inside), rows masked causally
-    (bottom-right aligned) when asked; x (..., L1, L2) bfloat16 / float16
+    (bottom-right aligned) when asked; x (..., L1, L2) bfloat16 / float16 / float32
     (attention_softmax_kernel.cu:96-108)."""
     dev = _require_cuda(x)
     if not 0.0 <= dropout <= 1.0:

@@ -13,6 +13,7 @@ from oracle import attention as oa
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
+TOL_F32 = 1e-4   # float32 tensors (the vector-ALU flavour of the operator)
 
 
 def _run(B, L1, L2, NH, H1, H2, causal, dtype, seed, scale=1.0):
@@ -21,9 +22,10 @@ def _run(B, L1, L2, NH, H1, H2, causal, dtype, seed, scale=1.0):
     k = (torch.randn(B, L2, NH, H1, generator=g) / H1 ** 0.5).to(dtype)
     v = (torch.randn(B, L2, NH, H2, generator=g) / H2 ** 0.5).to(dtype)
     dy = torch.randn(B, L1, NH, H2, generator=g).to(dtype)
+    TOL = TOL_F32 if dtype == torch.float32 else globals()["TOL"]
     y, w = ops.attention_fwd(q.cuda(), k.cuda(), v.cuda(), scale, 0.0, causal)
     wy, wp = oa.chunk_attention_fwd(q, k, v, scale, causal)
-    assert y.shape == (B, L1, NH, H2) and w.shape == (B, NH, L1, L2) and y.dtype == dtype
+    assert y.shape == (B, L1, NH, H2) and w.shape == (B, NH, L1, L2) and y.dtype == dtype and w.dtype == dtype
     assert rel_err(y, wy) <= TOL
     if causal:
         # compare the probabilities on and below the diagonal (blocks right of the diagonal block are not written)
@@ -61,6 +63,28 @@ def test_causal_with_key_value_prefix(B, L1, L2, NH, H1, H2, dtype):
     """L2 > L1: row r attends to keys 0 .. L2 - L1 + r (bottom-right aligned
     mask), forward values, probabilities and all three gradients."""
     _run(B, L1, L2, NH, H1, H2, True, dtype, seed=L1 + L2)
+
+
+@pytest.mark.parametrize("B,L1,L2,NH,H1,H2,causal", [
+    (2, 256, 256, 2, 64, 128, True),     # whole 64 x 64 tiles
+    (2, 100, 131, 3, 32, 72, True),      # ragged in every dimension, key/value prefix
+    (1, 300, 300, 1, 16, 24, False),     # every row sees every key
+    (1, 1, 40, 1, 16, 16, True),         # one new query
+    (1, 520, 1000, 2, 32, 64, True),     # several row tiles, prefix of 480 keys
+])
+def test_float32_tensors(B, L1, L2, NH, H1, H2, causal):
+    """The reference dispatches the operator over float32 too
+    (attention_kernel.cu:269-281); here float32 q, k, v keep float32 storage and
+    arithmetic: y, w and the three gradients within 1e-4 of the oracle, and w
+    holds exact zeros above the diagonal."""
+    _run(B, L1, L2, NH, H1, H2, causal, torch.float32, seed=L1 + 2 * L2, scale=0.8)
+    if causal:
+        g = torch.Generator().manual_seed(1)
+        q = torch.randn(B, L1, NH, H1, generator=g).cuda()
+        k = torch.randn(B, L2, NH, H1, generator=g).cuda()
+        v = torch.randn(B, L2, NH, H2, generator=g).cuda()
+        _, w = ops.attention_fwd(q, k, v, 1.0, 0.0, True)
+        assert torch.count_nonzero(torch.triu(w, diagonal=L2 - L1 + 1)) == 0
 
 
 def test_causal_with_fewer_keys_than_queries_fails_loudly():
@@ -129,11 +153,11 @@ def test_unsupported_cases_fail_loudly():
     q = torch.zeros(1, 8, 1, 8, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match=r"\[0, 1\]"):
         ops.attention_fwd(q, q, q, 1.0, 1.5, True)   # not a probability
-    with pytest.raises(RuntimeError, match="bfloat16"):
-        ops.attention_fwd(q.float(), q.float(), q.float(), 1.0, 0.0, True)
+    with pytest.raises(RuntimeError, match="float64"):
+        ops.attention_fwd(q.double(), q.double(), q.double(), 1.0, 0.0, True)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("shape,causal", [
     ((2, 3, 300, 300), True), ((1, 2, 100, 260), True), ((4, 64, 512), False), ((1, 1, 1, 40), True),
     ((2, 1, 50, 4100), False),   # rows longer than the register-resident kernels take
@@ -157,12 +181,13 @@ def test_standalone_softmax(shape, causal, dtype):
     want.backward(dy.double())
     xg = x.cuda().requires_grad_(True)
     y = attention_softmax(xg, 0.0, causal, True)
+    tol = TOL_F32 if dtype == torch.float32 else TOL
     assert y.dtype == dtype and y.shape == x.shape
-    assert rel_err(y, want.detach()) <= TOL
+    assert rel_err(y, want.detach()) <= tol
     if causal:
         assert torch.count_nonzero(torch.triu(y.float(), diagonal=L2 - L1 + 1)) == 0
     y.backward(dy.cuda())
-    assert rel_err(xg.grad, xd.grad) <= TOL
+    assert rel_err(xg.grad, xd.grad) <= tol
 
 
 @pytest.mark.parametrize("causal", [True, False])
