@@ -597,17 +597,24 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
   const int64_t seg_last = (C - 1) / NC * NC;
 
   XOp<DT> db[4], xb[4];
-  auto load_tiles = [&](int64_t row, int64_t seg0) {
+  auto load_dy = [&](int64_t row, int64_t seg0) {
     MEGA_LANE_IDS;
     const uint16_t* dyrow = static_cast<const uint16_t*>(dy) + row * L;
+    const int64_t chunk = seg0 + wave * 32 + r;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int64_t elem = chunk * kT + 16 * s + 8 * g;
+      db[s].load(dyrow, elem, row < rows && elem + 8 <= L);
+    }
+  };
+  auto load_x = [&](int64_t row, int64_t seg0) {
+    MEGA_LANE_IDS;
     const uint16_t* xrow = static_cast<const uint16_t*>(x) + row * L;
     const int64_t chunk = seg0 + wave * 32 + r;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int64_t elem = chunk * kT + 16 * s + 8 * g;
-      const bool on = row < rows && elem + 8 <= L;
-      db[s].load(dyrow, elem, on);
-      xb[s].load(xrow, elem, on);
+      xb[s].load(xrow, elem, row < rows && elem + 8 <= L);
     }
   };
   struct RowParams {
@@ -864,37 +871,51 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
     const int c0 = wave * 32;
     const bool on = c0 < nc;
     u32x4 xr[4];  // time-reversed x as an operand: steps 63 - (16 s + 8 g + e)
+    // the next item of this workgroup: its x tile is requested as soon as this item's has been
+    // consumed, its dy tile at the end of the item
+    int64_t nrow = row, nseg = seg0 - NC;
+    if (nseg < 0) {
+      nrow = row + gridDim.x;
+      nseg = seg_last;
+    }
     if (on) {
-      // ---- the wave's private tile: DY parked and read back with chunks along k ----------
+      // ---- the wave's private tile: X parked first (it arrived an item ago), read back with
+      //      chunks along k and time-reversed; then DY, whose loads were issued last ------------
       uint16_t* mine = stage + r * kSP + 8 * g;
-#pragma unroll
-      for (int s = 0; s < 4; ++s) *reinterpret_cast<u32x4*>(mine + 16 * s) = db[s].pc[0];
-      wave_sync();
-      u32x4 dyt[2][2];
-#pragma unroll
-      for (int it = 0; it < 2; ++it)
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) dyt[it][ks] = read_tr(it, ks);
-      wave_sync();
 #pragma unroll
       for (int s = 0; s < 4; ++s) *reinterpret_cast<u32x4*>(mine + 16 * s) = xb[s].pc[0];
       wave_sync();
-      // M += DY^T X over the tile's 32 chunks
+      u32x4 xt[2][2];
 #pragma unroll
       for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-          const u32x4 xt = read_tr(jt, ks);
-          if (jt == 0) macc[0] = mfma_bf16(dyt[0][ks], xt, macc[0]);
-          macc[1 + jt] = mfma_bf16(dyt[1][ks], xt, macc[1 + jt]);
-        }
+        for (int ks = 0; ks < 2; ++ks) xt[jt][ks] = read_tr(jt, ks);
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const u32x4 v = *reinterpret_cast<const u32x4*>(stage + r * kSP + 56 - 16 * s - 8 * g);
 #pragma unroll
         for (int e = 0; e < 4; ++e) xr[s][e] = __builtin_amdgcn_alignbit(v[3 - e], v[3 - e], 16);
       }
+      wave_sync();
+#pragma unroll
+      for (int s = 0; s < 4; ++s) *reinterpret_cast<u32x4*>(mine + 16 * s) = db[s].pc[0];
+      wave_sync();
+      // M += DY^T X over the tile's 32 chunks
+#pragma unroll
+      for (int it = 0; it < 2; ++it)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const u32x4 dyt = read_tr(it, ks);
+          if (it == 0) macc[0] = mfma_bf16(dyt, xt[0][ks], macc[0]);
+          if (it == 1) {
+            macc[1] = mfma_bf16(dyt, xt[0][ks], macc[1]);
+            macc[2] = mfma_bf16(dyt, xt[1][ks], macc[2]);
+          }
+        }
       wave_sync();  // the tile has been read: its place takes the wave's rows of (G, G')
+    }
+    load_x(nrow, nseg);
+    if (on) {
       // ---- (G, G') = Pg DY, into this wave's own rows of the state buffer ----------------
 #pragma unroll
       for (int kind = 0; kind < 2; ++kind) {
@@ -1056,18 +1077,11 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
     cur ^= 1;
     par ^= 1;
     if (seg0 == 0) finish_row(row);
-    // the next item's tiles
-    {
-      int64_t nrow = row, nseg = seg0 - NC;
-      if (nseg < 0) {
-        nrow = row + gridDim.x;
-        nseg = seg_last;
-      }
-      load_tiles(nrow, nseg);
-    }
+    load_dy(nrow, nseg);
   };
 
-  load_tiles(blockIdx.x, seg_last);
+  load_x(blockIdx.x, seg_last);
+  load_dy(blockIdx.x, seg_last);
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x)
     for (int64_t seg0 = seg_last; seg0 >= 0; seg0 -= NC) item(row, seg0);
 #undef MEGA_LANE_IDS
