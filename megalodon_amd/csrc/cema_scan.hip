@@ -596,7 +596,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
   const int64_t C = (L + kT - 1) / kT;
   const int64_t seg_last = (C - 1) / NC * NC;
 
-  XOp<DT> db[4], xb[4];
+  XOp<DT> db[4], xb[4], dn[4];  // dn: the next item's dy tile on its way
   auto load_dy = [&](int64_t row, int64_t seg0) {
     MEGA_LANE_IDS;
     const uint16_t* dyrow = static_cast<const uint16_t*>(dy) + row * L;
@@ -604,7 +604,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int64_t elem = chunk * kT + 16 * s + 8 * g;
-      db[s].load(dyrow, elem, row < rows && elem + 8 <= L);
+      dn[s].load(dyrow, elem, row < rows && elem + 8 <= L);
     }
   };
   auto load_x = [&](int64_t row, int64_t seg0) {
@@ -936,6 +936,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
       }
     }
     wave_sync();
+    load_dy(nrow, nseg);
     // ---- reverse scan over the chunks of the segment; a wave's four sub-segments are its own
     //      chunks, one workgroup barrier hands over the waves' ends ---------------------------------
     {
@@ -1077,11 +1078,14 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
     cur ^= 1;
     par ^= 1;
     if (seg0 == 0) finish_row(row);
-    load_dy(nrow, nseg);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) db[s] = dn[s];
   };
 
   load_x(blockIdx.x, seg_last);
   load_dy(blockIdx.x, seg_last);
+#pragma unroll
+  for (int s = 0; s < 4; ++s) db[s] = dn[s];
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x)
     for (int64_t seg0 = seg_last; seg0 >= 0; seg0 -= NC) item(row, seg0);
 #undef MEGA_LANE_IDS
