@@ -946,8 +946,10 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
       for (int i = 0; i < CPS; ++i) {
         const int c = sa * CPS + i;
         const bool live = c < nc;
-        gv[i] = live ? *reinterpret_cast<const float2*>(col + c * kRP) : make_float2(0.f, 0.f);
-        gd[i] = live ? *reinterpret_cast<const float2*>(col + c * kRP + 32) : make_float2(0.f, 0.f);
+        const float2 a0 = *reinterpret_cast<const float2*>(col + c * kRP);
+        const float2 b0 = *reinterpret_cast<const float2*>(col + c * kRP + 32);
+        gv[i] = live ? a0 : make_float2(0.f, 0.f);
+        gd[i] = live ? b0 : make_float2(0.f, 0.f);
       }
       cf e{0.f, 0.f}, ed{0.f, 0.f};
 #pragma unroll
@@ -1024,8 +1026,12 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
         }
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
-          const float4 rv = live ? *reinterpret_cast<const float4*>(rnext + 4 * g + 8 * qd) : zero4;
-          const float4 rd = live ? *reinterpret_cast<const float4*>(rnext + 32 + 4 * g + 8 * qd) : zero4;
+          // loaded whatever the row holds, then masked: a conditional load is split into
+          // single-word reads under an execution mask
+          const float4 rv0 = *reinterpret_cast<const float4*>(rnext + 4 * g + 8 * qd);
+          const float4 rd0 = *reinterpret_cast<const float4*>(rnext + 32 + 4 * g + 8 * qd);
+          const float4 rv = live ? rv0 : zero4;
+          const float4 rd = live ? rd0 : zero4;
 #pragma unroll
           for (int b = 0; b < 2; ++b) {
             const cf xv{xacc[0][4 * qd + 2 * b], xacc[0][4 * qd + 2 * b + 1]};
@@ -1042,8 +1048,10 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         const float* src = rnext + 16 * s2 + 8 * g;
-        const float4 u = live ? *reinterpret_cast<const float4*>(src) : zero4;
-        const float4 w = live ? *reinterpret_cast<const float4*>(src + 4) : zero4;
+        const float4 u0 = *reinterpret_cast<const float4*>(src);
+        const float4 w0 = *reinterpret_cast<const float4*>(src + 4);
+        const float4 u = live ? u0 : zero4;
+        const float4 w = live ? w0 : zero4;
         const float v[8] = {u.x, u.y, u.z, u.w, w.x, w.y, w.z, w.w};
         split8(v, hb[s2][0], hb[s2][1]);
       }
