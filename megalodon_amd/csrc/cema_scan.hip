@@ -280,7 +280,8 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int lag = o + rr - 8 * gg - e;
-          v[e] = lag >= 0 ? sm.klocal[lag] : 0.f;
+          const float kv = sm.klocal[lag >= 0 ? lag : 0];  // read, then masked: no branch around the load
+          v[e] = lag >= 0 ? kv : 0.f;
         }
       } else {
         const int it = (blk - 8) >> 1, s2 = (blk - 8) & 1, i = 32 * it + rr;
@@ -375,7 +376,8 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
 #pragma unroll
       for (int i = 0; i < CPS; ++i) {
         const int c = sa * CPS + i;
-        sv[i] = c < nc ? *reinterpret_cast<const float2*>(col + c * kHP) : make_float2(0.f, 0.f);
+        const float2 s0 = *reinterpret_cast<const float2*>(col + c * kHP);  // read, then masked
+        sv[i] = c < nc ? s0 : make_float2(0.f, 0.f);
       }
       cf h{0.f, 0.f};
 #pragma unroll
@@ -705,7 +707,8 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int lag = o - rr + 8 * gg + e;
-          v[e] = lag >= 0 ? sm.klocal[lag] : 0.f;
+          const float kv = sm.klocal[lag >= 0 ? lag : 0];  // read, then masked: no branch around the load
+          v[e] = lag >= 0 ? kv : 0.f;
         }
       } else {
         const int jt = (blk - 12) >> 1, s2 = (blk - 12) & 1, j = 32 * jt + rr;
