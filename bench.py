@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # WRITE_SIZE x 1.0 from two rocprofv3 --pmc passes of this script (--cema-only --copy-calibration),
 # the factors being what the same counters read for a plain copy of 2^30 bytes.  A measured
 # constant (profiles/cema_scan_config1_hbm_traffic.txt): counters cannot be read from in here.
-CEMA_BWD_TRAFFIC_BYTES = 8.097e8
+CEMA_BWD_TRAFFIC_BYTES = 8.091e8
 
 CFG4 = dict(model_dim=4096, z_dim=1024, value_dim=8192, num_heads=4, cema_ndim=16, chunk_size=4096,
             ffn_hidden_dim=11008, norm_num_groups=32)
@@ -65,7 +65,7 @@ def cpu_cema(B, D, N, L, seed, cores, budget_s=12.0):
     from megalodon_amd import synthetic
     from oracle import native
     lib = native.port()
-    Ds = 256
+    Ds = 1024
     prm = synthetic.cema_params(D, N, seed)
     io = synthetic.cema_inputs(B, Ds, L, seed, torch.bfloat16)
     p, lq, g, om = prm["p"][:Ds], prm["q"][:Ds].log(), prm["gamma"][:Ds], prm["omega"][:Ds]
@@ -100,7 +100,7 @@ def cpu_timestep_norm(cores, budget_s=12.0):
     from oracle import native
     lib = native.port()
     B, L, D, G = 4, 8192, 4096, 32
-    Ls = 2048
+    Ls = L
     io = {k: (v[:, :Ls].contiguous() if v.dim() >= 2 and v.shape[1] == L else v)
           for k, v in synthetic.timestep_norm_inputs(B, L, D, G, 1002).items()}
     f = {k: (v.float() if v.is_floating_point() else v) for k, v in io.items()}
@@ -112,10 +112,9 @@ def cpu_timestep_norm(cores, budget_s=12.0):
         native.group_timestep_norm_bwd(lib, "oracle_", f["dy"], f["dmean"], f["dvar"], f["x"], f["prev_mean"],
                                        count, cm, cr, f["gamma"], f["mask"], G)
 
-    dt, reps = _timed(step, budget_s)
+    dt, reps = _timed(step, budget_s, max_reps=30)
     return {"value": B * Ls / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"first {Ls} of {L} steps of all {B} sequences (the loop nest is linear in L), "
-                      f"{reps} rep(s), {dt:.2f} s each"}
+            "sample": f"the whole config (all {Ls} steps of all {B} sequences), {reps} rep(s), {dt:.2f} s each"}
 
 
 def cpu_attention(cores, budget_s=12.0):
@@ -137,7 +136,7 @@ def cpu_attention(cores, budget_s=12.0):
         out = torch.matmul(torch.softmax(s, dim=-1, dtype=torch.float32), v)
         out.backward(dy)
 
-    dt, reps = _timed(step, budget_s)
+    dt, reps = _timed(step, budget_s, max_reps=30)
     pairs = 32  # 8 chunks x 4 heads
     return {"value": 32768 / (dt * pairs), "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": f"1 of {pairs} (chunk, head) pairs (they are independent), {reps} rep(s), {dt:.2f} s each, "
@@ -152,7 +151,7 @@ def cpu_block(cores, budget_s=25.0):
     token below one chunk, so the figure flatters the CPU)."""
     import torch
     from oracle import block as oblock
-    Ls = 256
+    Ls = 1024
     g = torch.Generator().manual_seed(1004)
     D, Z, H, F_ = CFG4["model_dim"], CFG4["z_dim"], CFG4["value_dim"], CFG4["ffn_hidden_dim"]
     N = CFG4["cema_ndim"]
@@ -174,7 +173,7 @@ def cpu_block(cores, budget_s=25.0):
                                         groups=CFG4["norm_num_groups"])
         out.backward(dy)
 
-    dt, reps = _timed(step, budget_s, max_reps=2)
+    dt, reps = _timed(step, budget_s, max_reps=3)
     return {"value": Ls / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": f"the first {Ls} of 32768 tokens through the float64 oracle of the block "
                       f"(oracle/block.py), {reps} rep(s), {dt:.2f} s each"}
