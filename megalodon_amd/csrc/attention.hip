@@ -12,7 +12,7 @@
 // Differences in execution: the reference runs full-square cuBLAS GEMMs and a
 // full-row softmax; here every product is one hand-written MFMA GEMM
 // (v_mfma_f32_32x32x16, 256x256 workgroup tile, eight wavefronts of 128x64,
-// double-buffered LDS staging of 32-wide k slabs) that skips the tiles above
+// LDS staging of 32-wide k slabs in four buffers, one barrier per two slabs) that skips the tiles above
 // the causal diagonal and the k-ranges where P / dS are structurally zero, so
 // causal attention costs half the flops and half the P traffic.  Operands whose
 // reduction index is not the contiguous one (V, dY, K, Q, P, dS in the
@@ -338,9 +338,10 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
       for (int j = 0; j < JN; ++j) acc[i][j] = Mma<DT>::run(fb[j], fa[i], acc[i][j]);
   };
 
-  // One step per slab, one barrier per step, placed between the two k-steps:
-  //   first half:  read the second fragment set of slab cur, write slab cur+1
-  //                to the other LDS buffer, 16 MFMAs on the first set,
+  // One step per slab; the barrier (every step with two LDS buffers, every second step with
+  // four) sits between the two k-steps:
+  //   first half:  read the second fragment set of slab cur, write slab cur + AHEAD
+  //                to its LDS buffer, 16 MFMAs on the first set,
   //   barrier,
   //   second half: read the first fragment set of slab cur+1, request slab
   //                cur+3, 16 MFMAs on the second set.
