@@ -20,8 +20,9 @@
 // bf16 is exact, fp16 x is split into two exact bf16 pieces; the states are
 // float32 and split the same way; accumulation is float32.
 //
-// One workgroup of four waves owns a row; a segment of 256 chunks (16384
-// steps) is resident at a time: wave w holds chunk tiles 2 w, 2 w + 1 of it.
+// One workgroup of four waves owns a row; a segment of 128 NT chunks is
+// resident at a time: wave w holds chunk tiles NT w .. NT w + NT - 1 of it
+// (NT = 1 is what the entry point launches: 8192 steps per segment).
 #include "common.hpp"
 #include "cema_pow.hpp"
 
@@ -1149,7 +1150,8 @@ extern "C" int mega_cema_scan_fwd(const void* x, int dtype, const float* p, cons
   const cf* gm = reinterpret_cast<const cf*>(gamma);
   const cf* h0c = reinterpret_cast<const cf*>(h0);
   cf* hl = reinterpret_cast<cf*>(h_last);
-  if (dtype == MEGA_BF16) return launch_fwd<MEGA_BF16, 2>(x, y, p, lq, gm, omega, h0c, hl, B, D, N, L, s);
+  // one chunk tile per wave (segments of 128 chunks) measured 5 % faster than two for bfloat16 rows as well
+  if (dtype == MEGA_BF16) return launch_fwd<MEGA_BF16, 1>(x, y, p, lq, gm, omega, h0c, hl, B, D, N, L, s);
   return launch_fwd<MEGA_F16, 1>(x, y, p, lq, gm, omega, h0c, hl, B, D, N, L, s);
 }
 
