@@ -12,7 +12,7 @@
 // Differences in execution: the reference runs full-square cuBLAS GEMMs and a
 // full-row softmax; here every product is one hand-written MFMA GEMM
 // (v_mfma_f32_32x32x16, 256x256 workgroup tile, eight wavefronts of 128x64,
-// LDS staging of 32-wide k slabs in four buffers, one barrier per two slabs) that skips the tiles above
+// double-buffered LDS staging of 32-wide k slabs) that skips the tiles above
 // the causal diagonal and the k-ranges where P / dS are structurally zero, so
 // causal attention costs half the flops and half the P traffic.  Operands whose
 // reduction index is not the contiguous one (V, dY, K, Q, P, dS in the
@@ -61,10 +61,6 @@ constexpr int kEpiPitch = 128 + 8;  // epilogue staging pitch (elements) of a wa
 constexpr size_t kGemmLds =
     sizeof(uint16_t) * (4 * 128 * kEpiPitch > 2 * 2 * kOperandElems ? 4 * 128 * kEpiPitch
                                                                      : 2 * 2 * kOperandElems);
-// eight-wave form: four slab buffers (one workgroup barrier per two slabs) or the epilogue staging
-constexpr size_t kGemmLds8 =
-    sizeof(uint16_t) * (8 * 128 * (64 + 8) > 4 * 2 * kOperandElems ? 8 * 128 * (64 + 8) : 4 * 2 * kOperandElems);
-static_assert(kGemmLds8 <= 160 * 1024, "the eight-wave form fills one compute unit's LDS");
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -165,13 +161,6 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
   constexpr int JN = W8 ? 2 : 4;                   // 32-column blocks per wave
   constexpr int NL = W8 ? 2 : 4;                   // 16-byte chunks per thread, operand and slab
   constexpr int EP = W8 ? 64 + 8 : kEpiPitch;      // staging pitch
-  // LDS slab buffers.  Two: slab s + 1 is written while slab s is read, one workgroup barrier per
-  // slab.  Four (eight-wave form): slab s + 2 is written while slab s is read, and a barrier after
-  // every second slab is enough -- a buffer written in step s was last read in step s - 2, and
-  // the slab read in the second half of step s was written in step s - 1; in both cases a
-  // barrier of an odd step lies between.
-  constexpr int NBUF = W8 ? 4 : 2;
-  constexpr int AHEAD = NBUF / 2;  // slabs between the one being read and the one being written
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int wm = W8 ? wave >> 2 : wave >> 1, wn = W8 ? wave & 3 : wave & 1;
 
@@ -290,8 +279,8 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
   const int st_a = TA ? (tid >> 5) * kPitchT + (tid & 31) * 8 : ((tid & 3) * kChunkPitch + (tid >> 2)) * 8;
   const int st_b = TB ? (tid >> 5) * kPitchT + (tid & 31) * 8 : ((tid & 3) * kChunkPitch + (tid >> 2)) * 8;
   auto sstore = [&](const u32x4* qa, const u32x4* qb, int s) {
-    uint16_t* sa = smem + (s & (NBUF - 1)) * 2 * kOperand + st_a;
-    uint16_t* sb = smem + (s & (NBUF - 1)) * 2 * kOperand + kOperand + st_b;
+    uint16_t* sa = smem + (s & 1) * 2 * kOperand + st_a;
+    uint16_t* sb = smem + (s & 1) * 2 * kOperand + kOperand + st_b;
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
       *reinterpret_cast<u32x4*>(sa + i * (TA ? (T / 32) * kPitchT : (T / 4) * 8)) = qa[i];
@@ -338,10 +327,9 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
       for (int j = 0; j < JN; ++j) acc[i][j] = Mma<DT>::run(fb[j], fa[i], acc[i][j]);
   };
 
-  // One step per slab; the barrier (every step with two LDS buffers, every second step with
-  // four) sits between the two k-steps:
-  //   first half:  read the second fragment set of slab cur, write slab cur + AHEAD
-  //                to its LDS buffer, 16 MFMAs on the first set,
+  // One step per slab, one barrier per step, placed between the two k-steps:
+  //   first half:  read the second fragment set of slab cur, write slab cur+1
+  //                to the other LDS buffer, 16 MFMAs on the first set,
   //   barrier,
   //   second half: read the first fragment set of slab cur+1, request slab
   //                cur+3, 16 MFMAs on the second set.
@@ -365,8 +353,8 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
 #define MEGA_GEMM_STEP(R, CA, CB, NA, NB)                                  \
   {                                                                        \
     const int cur = it + (R);                                              \
-    fread(fa1, fb1, 1, cur & (NBUF - 1));                                  \
-    sstore(NA, NB, cur + AHEAD);                                           \
+    fread(fa1, fb1, 1, cur & 1);                                           \
+    sstore(NA, NB, cur + 1);                                               \
     mma(fa0, fb0);                                                         \
     _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
       MEGA_SGB(0x008, 1);                                                  \
@@ -378,8 +366,8 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
     }                                                                      \
     if (kRest > 0) MEGA_SGB(0x008, kRest);                                 \
     __builtin_amdgcn_sched_barrier(0);                                     \
-    if (NBUF == 2 || ((R) & 1)) lds_barrier();                             \
-    fread(fa0, fb0, 0, (cur + 1) & (NBUF - 1));                            \
+    lds_barrier();                                                         \
+    fread(fa0, fb0, 0, (cur + 1) & 1);                                     \
     gload(CA, CB, cur + RING);                                             \
     mma(fa1, fb1);                                                         \
     _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
@@ -399,23 +387,21 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
     gload(ra2, rb2, 2);
     if constexpr (RING == 4) gload(ra3, rb3, 3);
     sstore(ra0, rb0, 0);
-    if constexpr (NBUF == 4) sstore(ra1, rb1, 1);
     lds_barrier();
     fread(fa0, fb0, 0, 0);
     // ring slot R held slab cur, already written to LDS, so it is free for
     // slab cur + kRing
     int it = 0;
     if constexpr (RING == 4) {
-      // step R reloads ring slot R (slab cur + 4) and writes the slot of slab cur + 2 to LDS
       for (; it + 4 <= nslab; it += 4) {
-        MEGA_GEMM_STEP(0, ra0, rb0, ra2, rb2)
-        MEGA_GEMM_STEP(1, ra1, rb1, ra3, rb3)
-        MEGA_GEMM_STEP(2, ra2, rb2, ra0, rb0)
-        MEGA_GEMM_STEP(3, ra3, rb3, ra1, rb1)
+        MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
+        MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
+        MEGA_GEMM_STEP(2, ra2, rb2, ra3, rb3)
+        MEGA_GEMM_STEP(3, ra3, rb3, ra0, rb0)
       }
-      if (it < nslab) MEGA_GEMM_STEP(0, ra0, rb0, ra2, rb2)
-      if (it + 1 < nslab) MEGA_GEMM_STEP(1, ra1, rb1, ra3, rb3)
-      if (it + 2 < nslab) MEGA_GEMM_STEP(2, ra2, rb2, ra0, rb0)
+      if (it < nslab) MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
+      if (it + 1 < nslab) MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
+      if (it + 2 < nslab) MEGA_GEMM_STEP(2, ra2, rb2, ra3, rb3)
     } else {
       for (; it + kRing <= nslab; it += kRing) {
         MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
@@ -728,7 +714,7 @@ int launch_gemm_t(const GemmParams& p, int batch, hipStream_t s) {
   // comparison.
   const char* w4 = getenv("MEGA_GEMM_W4");
   if (fast && !(w4 != nullptr && w4[0] == '1')) {
-    const size_t lds8 = kGemmLds8;
+    const size_t lds8 = sizeof(uint16_t) * 8 * 128 * (64 + 8) > lds ? sizeof(uint16_t) * 8 * 128 * (64 + 8) : lds;
     MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, true, TA, TB, true>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds8));
     gemm_kernel<DT, true, TA, TB, true><<<grid, 2 * kThreads, lds8, s>>>(q);
