@@ -416,3 +416,14 @@ def test_spectral_signature_rejects_wrong_bin_count():
     x = torch.zeros(1, 2, 100, device="cuda")
     with pytest.raises(RuntimeError, match="129 bins"):
         ops.fftconv_fwd(x, torch.zeros(2, 101, dtype=torch.complex64, device="cuda"))
+
+
+def test_prepare_makes_tables_and_scratch_ahead_of_the_first_call():
+    """fftconv_prepare(L) does the float32 engine's first-use allocation; the convolution that
+    follows on the same stream gives the oracle's result (the call itself then allocates nothing)."""
+    B, D, L = 1, 2, 5000
+    ops.fftconv_prepare(L)
+    x, k, _ = _data(B, D, L, torch.float32, 99)
+    y = ops.fftconv_fwd(x.cuda(), k.cuda())
+    assert rel_err(y, fftconv.fftconv_fwd(x.double(), k.double())) <= 1e-4
+    ops.fftconv_prepare(10 ** 6)          # longer rows are cut into launches of the maximum length: prepared too
