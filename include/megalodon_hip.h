@@ -515,8 +515,9 @@ int mega_group_sequence_norm_bwd(const void* dy, const void* x, const int64_t* c
  * steps as matrix products on the matrix cores (bf16 operand pieces carrying
  * 16 significant bits, float32 states and accumulation); x is read once and
  * out written once.
- *   x, y (B, D, L) of `dtype` (MEGA_BF16 / MEGA_F16), 16-byte aligned, any
- *   L % 8 == 0 (no upper limit); p (D, N) float32; log_q, gamma (D, N)
+ *   x, y (B, D, L) of `dtype` (MEGA_BF16, MEGA_F16 or MEGA_F32; float32 rows
+ *   enter the products with their 16 leading bits, y is written in float32),
+ *   16-byte aligned, any L % 8 == 0 (no upper limit); p (D, N) float32; log_q, gamma (D, N)
  *   complex64 as mega_ema_weight_fwd takes them, N <= 16; omega (D) float32 or
  *   null; h0 (B, D, N) complex64 or null (zero state); h_last (B, D, N)
  *   complex64 or null (not wanted).

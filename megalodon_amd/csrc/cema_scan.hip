@@ -135,6 +135,23 @@ template <> struct XOp<MEGA_F16> {
   }
 };
 
+// float32 rows: the two leading bf16 pieces (16 significant bits, what the parameter matrices
+// carry as well); the rest, 2^-17 of a value, is left out
+template <> struct XOp<MEGA_F32> {
+  static constexpr int XP = 2;
+  u32x4 pc[2];
+  __device__ __forceinline__ void load(const void* row, int64_t elem, bool on) {
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+    if (on) {
+      const float4* src = reinterpret_cast<const float4*>(static_cast<const float*>(row) + elem);
+      a = src[0];
+      b = src[1];
+    }
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    split8(v, pc[0], pc[1]);
+  }
+};
+
 // acc += (A_hi + A_lo) * x with the lo * lo term of a two-piece x left out
 template <int XP>
 __device__ __forceinline__ floatx16 mma_split(const u32x4* a, const u32x4* x, floatx16 acc) {
@@ -190,7 +207,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
   // parameters of the next row are requested ahead (two register sets for the
   // tiles, swapped by taking the item body twice per loop turn).
   auto load_tiles = [&](XOp<DT> (&t)[NT][4], int64_t row, int64_t seg0) {
-    const uint16_t* xrow = static_cast<const uint16_t*>(x) + row * L;
+    const typename Elem<DT>::type* xrow = static_cast<const typename Elem<DT>::type*>(x) + row * L;
 #pragma unroll
     for (int ctl = 0; ctl < NT; ++ctl) {
       const int64_t chunk = seg0 + (wave * NT + ctl) * 32 + r;
@@ -316,7 +333,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
   XOp<DT> xb[NT][4];
   auto item = [&](int64_t row, int64_t seg0) {
     if (seg0 == 0) setup_row(row);
-    uint16_t* yrow = static_cast<uint16_t*>(y) + row * L;
+    typename Elem<DT>::type* yrow = static_cast<typename Elem<DT>::type*>(y) + row * L;
     const int nc = static_cast<int>(C - seg0 < NC ? C - seg0 : NC);
     floatx16 yacc[NT][2];
     // ---- local states S = P X, into this wave's own rows of the state buffer ----------
@@ -447,9 +464,21 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
             }
 #pragma unroll
             for (int pr = 0; pr < 2; ++pr) {
-              const uint4 oct = octet_of<DT>(acc, pr);
-              const int64_t elem = chunk * kT + 16 * (2 * it + pr) + 8 * g;
-              if (elem + 8 <= L) *reinterpret_cast<uint4*>(yrow + elem) = oct;
+              if constexpr (DT == MEGA_F32) {
+                // registers 8 pr + 4 h + e hold the steps 16 pr + 8 h + 4 g + e: two 16-byte stores
+                // per lane, no exchange between the halves of the wave
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                  const int64_t elem = chunk * kT + 16 * (2 * it + pr) + 8 * h + 4 * g;
+                  if (elem + 4 <= L)
+                    *reinterpret_cast<float4*>(yrow + elem) = make_float4(acc[8 * pr + 4 * h], acc[8 * pr + 4 * h + 1],
+                                                                          acc[8 * pr + 4 * h + 2], acc[8 * pr + 4 * h + 3]);
+                }
+              } else {
+                const uint4 oct = octet_of<DT>(acc, pr);
+                const int64_t elem = chunk * kT + 16 * (2 * it + pr) + 8 * g;
+                if (elem + 8 <= L) *reinterpret_cast<uint4*>(yrow + elem) = oct;
+              }
             }
           }
         }
@@ -461,7 +490,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
       // the row's last segment: the state after step L - 1 (the last chunk may be partial)
       lds_barrier();
       if (tid < N) {
-        const uint16_t* xrow = static_cast<const uint16_t*>(x) + row * L;
+        const typename Elem<DT>::type* xrow = static_cast<const typename Elem<DT>::type*>(x) + row * L;
         const int rem = static_cast<int>(L - (C - 1) * kT);  // 1 .. 64 steps in the last chunk
         const int cl = static_cast<int>(C - 1 - seg0);       // the last chunk inside this segment
         cf h;
@@ -1127,7 +1156,7 @@ int launch_bwd(const void* dy, const void* x, void* dx, const float* p, const cf
 using namespace mega;
 
 extern "C" int mega_cema_scan_supported(int dtype, int64_t N, int64_t L) {
-  return (dtype == MEGA_BF16 || dtype == MEGA_F16) && N >= 1 && N <= 16 && L >= 8 && L % 8 == 0;
+  return valid_dtype(dtype) && N >= 1 && N <= 16 && L >= 8 && L % 8 == 0;
 }
 
 extern "C" int mega_cema_scan_fwd(const void* x, int dtype, const float* p, const float* log_q,
@@ -1140,7 +1169,7 @@ extern "C" int mega_cema_scan_fwd(const void* x, int dtype, const float* p, cons
   MEGA_CHECK_ARG(B * D <= 0x7fffffff, "%s: too many rows", who);
   if (!mega_cema_scan_supported(dtype, N, L))
     return set_error(MEGA_ERR_UNSUPPORTED,
-                     "%s: needs bfloat16 / float16 rows, N <= 16 and L a multiple of 8 (dtype %d, N %lld, L %lld)",
+                     "%s: needs N <= 16 and L a multiple of 8 (dtype %d, N %lld, L %lld)",
                      who, dtype, (long long)N, (long long)L);
   MEGA_CHECK_ARG(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0,
                  "%s: x and y must be 16-byte aligned", who);
@@ -1152,6 +1181,7 @@ extern "C" int mega_cema_scan_fwd(const void* x, int dtype, const float* p, cons
   cf* hl = reinterpret_cast<cf*>(h_last);
   // one chunk tile per wave (segments of 128 chunks) measured 5 % faster than two for bfloat16 rows as well
   if (dtype == MEGA_BF16) return launch_fwd<MEGA_BF16, 1>(x, y, p, lq, gm, omega, h0c, hl, B, D, N, L, s);
+  if (dtype == MEGA_F32) return launch_fwd<MEGA_F32, 1>(x, y, p, lq, gm, omega, h0c, hl, B, D, N, L, s);
   return launch_fwd<MEGA_F16, 1>(x, y, p, lq, gm, omega, h0c, hl, B, D, N, L, s);
 }
 

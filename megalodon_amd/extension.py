@@ -553,9 +553,9 @@ def fftconv_residual_bwd_saved(y_grad: torch.Tensor, spec_x: torch.Tensor, spec_
 # The CEMA layer as a chunked recurrence (csrc/cema_scan.hip)
 # --------------------------------------------------------------------------
 def cema_scan_supported(x: torch.Tensor, ndim: int) -> bool:
-    """Whether `cema_scan_fwd` takes this input: bfloat16 / float16 rows on the
-    GPU, at most 16 modes, a length that is a multiple of 8."""
-    if not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float16):
+    """Whether `cema_scan_fwd` takes this input: bfloat16 / float16 / float32 rows
+    on the GPU, at most 16 modes, a length that is a multiple of 8."""
+    if not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
         return False
     fn = _lib.load().mega_cema_scan_supported
     return bool(fn(_lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(ndim), _lib.i64(x.shape[-1])))
@@ -567,7 +567,9 @@ def cema_scan_fwd(x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor, gamma: 
     """(out, h_last): ``fftconv(x, k) + x * omega + b`` and, on request, the state
     after the last step, for k, b = ema_parameters(p, q, gamma, h0, L) -- without
     forming k (complex_exponential_moving_average.py:127-147).  x (B, D, L)
-    bfloat16 / float16; p (D, N[, 1]) float32; log_q, gamma (D, N[, 1]) complex64."""
+    bfloat16 / float16 / float32 (float32 rows enter the products with their 16
+    leading bits, the precision the parameter matrices carry too: 1e-5 of the
+    output's scale); p (D, N[, 1]) float32; log_q, gamma (D, N[, 1]) complex64."""
     dev = _require_cuda(x, p, log_q, gamma, omega, h0)
     B, D, L = x.shape
     N = p.shape[1]

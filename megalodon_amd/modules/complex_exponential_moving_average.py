@@ -2,10 +2,11 @@
 (megalodon/modules/complex_exponential_moving_average.py:42-150), minus the
 `megalodon.distributed` look-ups: model-parallel world size is 1, so
 ``dim_per_partition == embed_dim`` and the theta permutation is drawn locally
-instead of being broadcast (:21-26).  16-bit inputs on the GPU run the layer as
-a chunked recurrence (fused_ops/cema_scan.py); MEGA_CEMA_FFT=1 in the
-environment keeps them on the kernel-row + FFT-convolution operators that
-float32 inputs use."""
+instead of being broadcast (:21-26).  On the GPU the layer runs as a chunked
+recurrence (fused_ops/cema_scan.py) wherever its kernels take the case --
+bfloat16 rows with gradients, every dtype without; MEGA_CEMA_FFT=1 in the
+environment keeps everything on the kernel-row + FFT-convolution operators
+that the remaining cases (float32 / float16 training, odd lengths) use."""
 from typing import Optional, Tuple
 import math
 import os
@@ -91,8 +92,9 @@ class MultiHeadComplexEMA(nn.Module):
         needs_grad = torch.is_grad_enabled() and (x.requires_grad or self.alpha.requires_grad
                                                   or (hx is not None and hx.requires_grad))
         if self.alpha.is_cuda and os.environ.get("MEGA_CEMA_FFT") is None:
-            # 16-bit rows: the layer as a chunked recurrence on the matrix cores (no kernel
-            # row, no transform); with a carried state only where no gradient is wanted
+            # the layer as a chunked recurrence on the matrix cores (no kernel row, no
+            # transform, any length in one launch): bfloat16 rows with or without gradients,
+            # float16 / float32 rows and carried states where no gradient is wanted
             if stateless and cema_scan_applicable(x, self.ndim, needs_grad):
                 out = cema_scan(x, self.alpha.float(), self.delta.float(), self.theta.float(), self.gamma.float(),
                                 self.omega)
