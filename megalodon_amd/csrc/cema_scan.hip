@@ -1043,39 +1043,8 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
       const bool live = c0 + r < nc;
       const float* rnext = (r == 31) ? sm.wave_cin[wave] : myrows + (r + 1) * kRP;
       const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-      // ---- (X, X') = Pg XR;  W += X R[c+1], W' += X' R[c+1] + X R'[c+1] ---------------------------
-      {
-        floatx16 xacc[2];
-#pragma unroll
-        for (int kind = 0; kind < 2; ++kind) {
-#pragma unroll
-          for (int i = 0; i < 16; ++i) xacc[kind][i] = 0.f;
-#pragma unroll
-          for (int s = 0; s < 4; ++s) {
-            u32x4 a[2];
-            load_block(kind * 4 + s, a, lane);
-            xacc[kind] = mma_split<1>(a, &xr[s], xacc[kind]);
-          }
-        }
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          // loaded whatever the row holds, then masked: a conditional load is split into
-          // single-word reads under an execution mask
-          const float4 rv0 = *reinterpret_cast<const float4*>(rnext + 4 * g + 8 * qd);
-          const float4 rd0 = *reinterpret_cast<const float4*>(rnext + 32 + 4 * g + 8 * qd);
-          const float4 rv = live ? rv0 : zero4;
-          const float4 rd = live ? rd0 : zero4;
-#pragma unroll
-          for (int b = 0; b < 2; ++b) {
-            const cf xv{xacc[0][4 * qd + 2 * b], xacc[0][4 * qd + 2 * b + 1]};
-            const cf xd{xacc[1][4 * qd + 2 * b], xacc[1][4 * qd + 2 * b + 1]};
-            const cf rr_ = b ? cf{rv.z, rv.w} : cf{rv.x, rv.y};
-            const cf rdd = b ? cf{rd.z, rd.w} : cf{rd.x, rd.y};
-            wacc[2 * qd + b] = cadd(wacc[2 * qd + b], cmul(xv, rr_));
-            wdacc[2 * qd + b] = cadd(wdacc[2 * qd + b], cadd(cmul(xd, rr_), cmul(xv, rdd)));
-          }
-        }
-      }
+      // the stores of dX go out first: they have the (X, X') products and the next item's
+      // staging to retire under before the next loads are issued behind them
       // ---- DX = K^T DY + Qd R[c+1] (omega dy included: K carries omega on its diagonal) -------------
       u32x4 hb[2][2];
 #pragma unroll
@@ -1113,6 +1082,39 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
           const uint4 oct = octet_of<DT>(acc, pr);
           const int64_t elem = chunk * kT + 16 * (2 * jt + pr) + 8 * g;
           if (elem + 8 <= L) *reinterpret_cast<uint4*>(dxrow + elem) = oct;
+        }
+      }
+      // ---- (X, X') = Pg XR;  W += X R[c+1], W' += X' R[c+1] + X R'[c+1] ---------------------------
+      {
+        floatx16 xacc[2];
+#pragma unroll
+        for (int kind = 0; kind < 2; ++kind) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) xacc[kind][i] = 0.f;
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            u32x4 a[2];
+            load_block(kind * 4 + s, a, lane);
+            xacc[kind] = mma_split<1>(a, &xr[s], xacc[kind]);
+          }
+        }
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          // loaded whatever the row holds, then masked: a conditional load is split into
+          // single-word reads under an execution mask
+          const float4 rv0 = *reinterpret_cast<const float4*>(rnext + 4 * g + 8 * qd);
+          const float4 rd0 = *reinterpret_cast<const float4*>(rnext + 32 + 4 * g + 8 * qd);
+          const float4 rv = live ? rv0 : zero4;
+          const float4 rd = live ? rd0 : zero4;
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            const cf xv{xacc[0][4 * qd + 2 * b], xacc[0][4 * qd + 2 * b + 1]};
+            const cf xd{xacc[1][4 * qd + 2 * b], xacc[1][4 * qd + 2 * b + 1]};
+            const cf rr_ = b ? cf{rv.z, rv.w} : cf{rv.x, rv.y};
+            const cf rdd = b ? cf{rd.z, rd.w} : cf{rd.x, rd.y};
+            wacc[2 * qd + b] = cadd(wacc[2 * qd + b], cmul(xv, rr_));
+            wdacc[2 * qd + b] = cadd(wdacc[2 * qd + b], cadd(cmul(xd, rr_), cmul(xv, rdd)));
+          }
         }
       }
     }
