@@ -590,11 +590,18 @@ def cema_scan_fwd(x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor, gamma: 
 
 
 def cema_scan_bwd_supported(x: torch.Tensor, ndim: int) -> bool:
-    """Whether `cema_scan_bwd` takes this input (bfloat16 rows; otherwise as the forward)."""
-    if not x.is_cuda or x.dim() != 3 or x.dtype != torch.bfloat16:
+    """Whether `cema_scan_bwd` takes this input: bfloat16 rows in one launch, float16
+    rows as three launches on their bfloat16 pieces; otherwise as the forward."""
+    if not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float16):
         return False
     fn = _lib.load().mega_cema_scan_bwd_supported
-    return bool(fn(_lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(ndim), _lib.i64(x.shape[-1])))
+    return bool(fn(_lib.i32(_lib.dtype_code(torch.bfloat16)), _lib.i64(ndim), _lib.i64(x.shape[-1])))
+
+
+def _bf16_pieces(t: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """A float16 tensor as the sum of two bfloat16 tensors, exactly (11 significant bits = 8 + 3)."""
+    hi = t.to(torch.bfloat16)
+    return hi, (t.float() - hi.float()).to(torch.bfloat16)
 
 
 def cema_scan_bwd(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor,
@@ -608,6 +615,15 @@ def cema_scan_bwd(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, log_q:
     N = p.shape[1]
     if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
         raise RuntimeError("cema_scan_bwd: y_grad must match x in shape and dtype")
+    if x.dtype == torch.float16:
+        # the backward is linear in y_grad and, for the parameter gradients, in x as well: the
+        # bfloat16 kernel on (hi, hi), (lo, hi) and (hi, lo) pieces; lo x lo is 2^-16 of the result
+        gh, gl = _bf16_pieces(y_grad)
+        xh, xl = _bf16_pieces(x)
+        dx1, *g1 = cema_scan_bwd(gh, xh, p, log_q, gamma, omega)
+        dx2, *g2 = cema_scan_bwd(gl, xh, p, log_q, gamma, omega)
+        _, *g3 = cema_scan_bwd(gh, xl, p, log_q, gamma, omega)
+        return ((dx1.float() + dx2.float()).to(torch.float16), *[a + b + c for a, b, c in zip(g1, g2, g3)])
 
     def aligned(t):
         t = t.contiguous()

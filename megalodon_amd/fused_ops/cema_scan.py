@@ -38,7 +38,8 @@ cema_scan = CEMAScanFunc.apply
 
 def cema_scan_applicable(x: torch.Tensor, ndim: int, needs_grad: bool) -> bool:
     """The recurrence kernels take bfloat16 / float16 / float32 rows of a length that
-    is a multiple of 8 with at most 16 modes; the backward kernel bfloat16 only."""
+    is a multiple of 8 with at most 16 modes; the backward bfloat16 rows, and float16
+    rows through their bfloat16 pieces."""
     if needs_grad:
         return megalodon_ops.cema_scan_bwd_supported(x, ndim)
     return megalodon_ops.cema_scan_supported(x, ndim)

@@ -4,9 +4,9 @@
 ``dim_per_partition == embed_dim`` and the theta permutation is drawn locally
 instead of being broadcast (:21-26).  On the GPU the layer runs as a chunked
 recurrence (fused_ops/cema_scan.py) wherever its kernels take the case --
-bfloat16 rows with gradients, every dtype without; MEGA_CEMA_FFT=1 in the
-environment keeps everything on the kernel-row + FFT-convolution operators
-that the remaining cases (float32 / float16 training, odd lengths) use."""
+bfloat16 / float16 rows with gradients, every dtype without; MEGA_CEMA_FFT=1
+in the environment keeps everything on the kernel-row + FFT-convolution
+operators that the remaining cases (float32 training, odd lengths) use."""
 from typing import Optional, Tuple
 import math
 import os
@@ -93,8 +93,8 @@ class MultiHeadComplexEMA(nn.Module):
                                                   or (hx is not None and hx.requires_grad))
         if self.alpha.is_cuda and os.environ.get("MEGA_CEMA_FFT") is None:
             # the layer as a chunked recurrence on the matrix cores (no kernel row, no
-            # transform, any length in one launch): bfloat16 rows with or without gradients,
-            # float16 / float32 rows and carried states where no gradient is wanted
+            # transform, any length in one launch): bfloat16 / float16 rows with or without
+            # gradients, float32 rows and carried states where no gradient is wanted
             if stateless and cema_scan_applicable(x, self.ndim, needs_grad):
                 out = cema_scan(x, self.alpha.float(), self.delta.float(), self.theta.float(), self.gamma.float(),
                                 self.omega)

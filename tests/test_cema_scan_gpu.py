@@ -75,6 +75,7 @@ def test_unsupported_shapes_are_refused():
     assert not ops.cema_scan_supported(x, 16)
     assert ops.cema_scan_supported(torch.zeros(1, 2, 64, device="cuda"), 16)       # float32 rows: forward only
     assert not ops.cema_scan_bwd_supported(torch.zeros(1, 2, 64, device="cuda"), 16)
+    assert ops.cema_scan_bwd_supported(torch.zeros(1, 2, 64, dtype=torch.float16, device="cuda"), 16)
     assert not ops.cema_scan_supported(torch.zeros(1, 2, 64, dtype=torch.bfloat16, device="cuda"), 17)
     p, q, gam, omega = _params(2, 16, 1)
     with pytest.raises(RuntimeError, match="multiple of 8"):
@@ -86,18 +87,19 @@ BWD_SHAPES = [(1, 2, 16, 8), (2, 3, 16, 64), (1, 3, 16, 72), (2, 2, 5, 1000), (1
 
 
 @pytest.mark.parametrize("B,D,N,L", BWD_SHAPES)
-def test_backward_matches_oracle(B, D, N, L):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_backward_matches_oracle(B, D, N, L, dtype):
     p, q, gam, omega = _params(D, N, 5 * L + D)
     g = torch.Generator().manual_seed(L + 1)
-    x = torch.randn(B, D, L, generator=g).bfloat16()
-    dy = torch.randn(B, D, L, generator=g).bfloat16()
+    x = torch.randn(B, D, L, generator=g).to(dtype)
+    dy = torch.randn(B, D, L, generator=g).to(dtype)
     assert ops.cema_scan_bwd_supported(x.cuda(), N)
     dx, dp, dq, dg, dw = ops.cema_scan_bwd(dy.cuda(), x.cuda(), p.cuda(), q.log().cuda(), gam.cuda(), omega.cuda())
     lq = q.to(torch.complex128).log()
     k = ocema.ema_weight_fwd(p.double(), lq, gam.to(torch.complex128), L)
     wdx, wdk = offt.fftconv_bwd(dy.double(), x.double(), k)
     wdp, wdq, wdg = ocema.ema_weight_bwd(wdk, p.double(), lq, gam.to(torch.complex128))
-    assert dx.dtype == torch.bfloat16
+    assert dx.dtype == dtype
     assert rel_err(dx, wdx + dy.double() * omega.double().view(1, D, 1)) <= 2e-2
     assert rel_err(dp, wdp.reshape(D, N)) <= 1e-4
     assert rel_err(dq, wdq.reshape(D, N)) <= 1e-4
