@@ -545,6 +545,17 @@ int mega_cema_scan_bwd(const void* dy, const void* x, int dtype, const float* p,
                        int64_t D, int64_t N, int64_t L, void* dx, float* dp, float* dq,
                        float* dgamma, float* domega, void* stream);
 
+/* mega_cema_scan_bwd on bfloat16 dy and x with dx written in float32, or not at
+ * all when `dx` is NULL.  The backward is linear in dy and, for the parameter
+ * gradients, in x: a caller with float16 or float32 tensors (the reference's
+ * operators take them, fused_ops/fftconv.py:37-44 upcasts to float32) runs
+ * this on the bfloat16 pieces of dy and x and adds the results up
+ * (extension.py:cema_scan_bwd does). */
+int mega_cema_scan_bwd_wide(const void* dy, const void* x, const float* p, const float* log_q,
+                            const float* gamma, const float* omega, int64_t B, int64_t D,
+                            int64_t N, int64_t L, float* dx, float* dp, float* dq, float* dgamma,
+                            float* domega, void* stream);
+
 /* ------------------------------------------------------------------------
  * Streaming reference kernel for measurements (no counterpart in the
  * reference): out = a (b == NULL) or out = a XOR b over `bytes` bytes

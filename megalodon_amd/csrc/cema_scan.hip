@@ -26,6 +26,8 @@
 #include "common.hpp"
 #include "cema_pow.hpp"
 
+#include <type_traits>
+
 namespace mega {
 namespace {
 
@@ -604,7 +606,9 @@ __device__ __forceinline__ void rstep(cf& h, cf& hd, cf g, cf gd, cf m, cf md) {
   hd = nd;
 }
 
-template <int DT>
+// DX32: dx is written in float32 (or, with a null pointer, not at all) instead of the rows'
+// own type -- for callers that add up the backward of several bfloat16 pieces of one tensor.
+template <int DT, bool DX32>
 __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
     const void* __restrict__ dy, const void* __restrict__ x, void* __restrict__ dx,
     const float* __restrict__ p, const cf* __restrict__ log_q, const cf* __restrict__ gamma,
@@ -899,7 +903,8 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
       return u32x4{lo.x, lo.y, hi.x, hi.y};
     };
     if (seg0 == seg_last) setup_row(row);
-    uint16_t* dxrow = static_cast<uint16_t*>(dx) + row * L;
+    using dx_t = typename std::conditional<DX32, float, uint16_t>::type;
+    dx_t* dxrow = static_cast<dx_t*>(dx) + row * L;
     const int nc = static_cast<int>(C - seg0 < NC ? C - seg0 : NC);
     const int c0 = wave * 32;
     const bool on = c0 < nc;
@@ -1079,9 +1084,20 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
         }
 #pragma unroll
         for (int pr = 0; pr < 2; ++pr) {
-          const uint4 oct = octet_of<DT>(acc, pr);
-          const int64_t elem = chunk * kT + 16 * (2 * jt + pr) + 8 * g;
-          if (elem + 8 <= L) *reinterpret_cast<uint4*>(dxrow + elem) = oct;
+          if constexpr (DX32) {
+            // registers 8 pr + 4 h + e hold the steps 16 pr + 8 h + 4 g + e
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              const int64_t elem = chunk * kT + 16 * (2 * jt + pr) + 8 * h + 4 * g;
+              if (dx != nullptr && elem + 4 <= L)
+                *reinterpret_cast<float4*>(dxrow + elem) = make_float4(acc[8 * pr + 4 * h], acc[8 * pr + 4 * h + 1],
+                                                                       acc[8 * pr + 4 * h + 2], acc[8 * pr + 4 * h + 3]);
+            }
+          } else {
+            const uint4 oct = octet_of<DT>(acc, pr);
+            const int64_t elem = chunk * kT + 16 * (2 * jt + pr) + 8 * g;
+            if (elem + 8 <= L) *reinterpret_cast<uint4*>(dxrow + elem) = oct;
+          }
         }
       }
       // ---- (X, X') = Pg XR;  W += X R[c+1], W' += X' R[c+1] + X R'[c+1] ---------------------------
@@ -1134,18 +1150,19 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
 #undef MEGA_LANE_IDS
 }
 
+template <bool DX32>
 int launch_bwd(const void* dy, const void* x, void* dx, const float* p, const cf* log_q,
                const cf* gamma, const float* omega, float* dp, cf* dq, cf* dgamma, float* domega,
                int64_t B, int64_t D, int64_t N, int64_t L, hipStream_t stream) {
   const int lds = static_cast<int>(sizeof(BwdSmem));
-  MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&cema_scan_bwd_kernel<MEGA_BF16>),
+  MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&cema_scan_bwd_kernel<MEGA_BF16, DX32>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, lds));
   int dev = 0, cus = 0;
   MEGA_CHECK_HIP(hipGetDevice(&dev));
   MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
   const int64_t rows = B * D, slots = 2 * static_cast<int64_t>(cus);  // two workgroups fit a compute unit
   const unsigned grid = static_cast<unsigned>(rows < slots ? rows : slots);
-  cema_scan_bwd_kernel<MEGA_BF16><<<dim3(grid), kThreads, lds, stream>>>(
+  cema_scan_bwd_kernel<MEGA_BF16, DX32><<<dim3(grid), kThreads, lds, stream>>>(
       dy, x, dx, p, log_q, gamma, omega, dp, dq, dgamma, domega, rows, static_cast<int>(D),
       static_cast<int>(N), L);
   MEGA_CHECK_LAUNCH();
@@ -1206,7 +1223,26 @@ extern "C" int mega_cema_scan_bwd(const void* dy, const void* x, int dtype, cons
   const auto al = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
   MEGA_CHECK_ARG(al(dy) && al(x) && al(dx), "%s: dy, x and dx must be 16-byte aligned", who);
   if (B == 0 || D == 0) return MEGA_OK;
-  return launch_bwd(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
-                    omega, dp, reinterpret_cast<cf*>(dq), reinterpret_cast<cf*>(dgamma), domega, B, D, N, L,
-                    static_cast<hipStream_t>(stream));
+  return launch_bwd<false>(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
+                           omega, dp, reinterpret_cast<cf*>(dq), reinterpret_cast<cf*>(dgamma), domega, B, D, N, L,
+                           static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mega_cema_scan_bwd_wide(const void* dy, const void* x, const float* p, const float* log_q,
+                                       const float* gamma, const float* omega, int64_t B, int64_t D,
+                                       int64_t N, int64_t L, float* dx, float* dp, float* dq, float* dgamma,
+                                       float* domega, void* stream) {
+  const char* who = "mega_cema_scan_bwd_wide";
+  MEGA_CHECK_ARG(dy && x && p && log_q && gamma && dp && dq && dgamma && domega, "%s: null pointer", who);
+  MEGA_CHECK_ARG(B >= 0 && D >= 0 && L >= 0, "%s: negative size", who);
+  MEGA_CHECK_ARG(B * D <= 0x7fffffff, "%s: too many rows", who);
+  if (!mega_cema_scan_bwd_supported(MEGA_BF16, N, L))
+    return set_error(MEGA_ERR_UNSUPPORTED, "%s: needs N <= 16 and L a multiple of 8 (N %lld, L %lld)", who,
+                     (long long)N, (long long)L);
+  const auto al = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  MEGA_CHECK_ARG(al(dy) && al(x) && al(dx), "%s: dy, x and dx must be 16-byte aligned", who);
+  if (B == 0 || D == 0) return MEGA_OK;
+  return launch_bwd<true>(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
+                          omega, dp, reinterpret_cast<cf*>(dq), reinterpret_cast<cf*>(dgamma), domega, B, D, N, L,
+                          static_cast<hipStream_t>(stream));
 }
