@@ -106,3 +106,42 @@ def test_backward_matches_oracle(B, D, N, L, dtype):
     assert rel_err(dq, wdq.reshape(D, N)) <= 1e-4
     assert rel_err(dg, wdg.reshape(D, N)) <= 1e-4
     assert rel_err(dw, (dy.double() * x.double()).sum(dim=(0, 2))) <= 1e-4
+
+
+@pytest.mark.parametrize("decay", ["slow", "fast", "mixed"])
+def test_extreme_decay_rates(decay):
+    """|q| within 1e-4 of 1 (states that sum ten thousand steps), |q| near 0 (powers that
+    underflow inside a chunk) and both in one channel, forward with last state and backward."""
+    B, D, N, L = 1, 3, 16, 16384
+    g = torch.Generator().manual_seed(11)
+    if decay == "slow":
+        mag = 1.0 - 1e-4 * (1.0 + torch.rand(D, N, 1, generator=g))
+    elif decay == "fast":
+        mag = 1e-3 * (1.0 + torch.rand(D, N, 1, generator=g))
+    else:
+        mag = torch.where(torch.rand(D, N, 1, generator=g) < 0.5, torch.full((D, N, 1), 0.9999), torch.full((D, N, 1), 0.01))
+    theta = torch.rand(D, 1, 1, generator=g) * (2 * math.pi / N)
+    q = torch.polar(mag, theta * torch.arange(1, N + 1, dtype=torch.float32).view(1, N, 1))
+    p = torch.rand(D, N, 1, generator=g)
+    gam = torch.complex(torch.randn(D, N, generator=g), torch.randn(D, N, generator=g)) / math.sqrt(2 * N)
+    omega = torch.randn(D, generator=g)
+    x = torch.randn(B, D, L, generator=g).bfloat16()
+    dy = torch.randn(B, D, L, generator=g).bfloat16()
+    # The operators take log q, as the reference's do (fused_ops/ema_parameters.py:19 passes
+    # q.log() in complex64).  Near |q| = 1 the float32 logarithm of the float32 q is itself
+    # off by 6e-4 of the decay rate, so the oracle gets the same log q the kernel gets.
+    lq32 = q.log()
+    lq = lq32.to(torch.complex128)
+    y, last = ops.cema_scan_fwd(x.cuda(), p.cuda(), lq32.cuda(), gam.cuda(), omega.cuda(), None, True)
+    k = ocema.ema_weight_fwd(p.double(), lq, gam.to(torch.complex128), L)
+    want = offt.fftconv_fwd(x.double(), k) + x.double() * omega.double().view(1, -1, 1)
+    wlast = ocema.ema_hidden_fwd(x.double(), p.double(), lq, None)
+    assert rel_err(y, want) <= 2e-2 and rel_err(last, wlast) <= 1e-4
+    dx, dp, dq, dg, dw = ops.cema_scan_bwd(dy.cuda(), x.cuda(), p.cuda(), lq32.cuda(), gam.cuda(), omega.cuda())
+    k = ocema.ema_weight_fwd(p.double(), lq, gam.to(torch.complex128), L)
+    wdx, wdk = offt.fftconv_bwd(dy.double(), x.double(), k)
+    wdp, wdq, wdg = ocema.ema_weight_bwd(wdk, p.double(), lq, gam.to(torch.complex128))
+    assert rel_err(dx, wdx + dy.double() * omega.double().view(1, D, 1)) <= 2e-2
+    assert rel_err(dp, wdp.reshape(D, N)) <= 1e-4
+    assert rel_err(dq, wdq.reshape(D, N)) <= 1e-4
+    assert rel_err(dg, wdg.reshape(D, N)) <= 1e-4
