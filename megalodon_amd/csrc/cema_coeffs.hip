@@ -36,7 +36,9 @@ __global__ __launch_bounds__(kThreads) void cema_coeffs_fwd_kernel(
   const float a = sigmoidf(alpha[i]), d = sigmoidf(delta[i]), t = sigmoidf(theta[ch]);
   const float scale = sqrtf(1.f / static_cast<float>(N));
   p[i] = a;
-  log_q[2 * i] = logf(1.f - a * d);
+  // log |q| = log(1 - a d) without forming 1 - a d: rounded to float32 that difference loses
+  // the decay rate's low bits when a d is small (6e-4 of it at a d = 1e-4)
+  log_q[2 * i] = log1pf(-a * d);
   log_q[2 * i + 1] = static_cast<float>(n + 1) * (t * (6.283185307179586f / static_cast<float>(N)));
   gamma_hat[2 * i] = gamma[2 * i] * scale;
   gamma_hat[2 * i + 1] = gamma[2 * i + 1] * scale;
