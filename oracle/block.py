@@ -5,6 +5,13 @@ megalodon/modules/normalized_feedforward_network.py:75-94,
 megalodon/model/mega.py:79-88 and the `weight + 1` norm convention of
 megalodon/modules/layer_norm.py:31,59.  `p` maps the parameter names of
 `megalodon_amd.modules.MegaBlock.named_parameters()` to float64 tensors.
+
+Test infrastructure only.  Pinned by tests/test_oracle_block.py: `_rms` against
+torch.nn.functional.rms_norm, `rotary` against explicit plane rotations, the
+wiring by special cases that a mis-routed tensor fails (zero fc2, zero wh1 /
+wh2, rmsnorm weight -1, causality) and the whole block with all gradients by an
+independent restatement from other primitives (EMA recurrence,
+scaled_dot_product_attention, brute-force prefix statistics).
 """
 from __future__ import annotations
 
