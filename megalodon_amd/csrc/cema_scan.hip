@@ -172,7 +172,6 @@ constexpr int kFwdBlocks = 12;
 template <int NT>
 struct FwdSmem {
   static constexpr int NC = kWaves * NT * 32;  // chunks per segment
-  cf qp[16][kT + 2];                           // q_n^e, e = 0 .. 64
   float klocal[kT];                            // k[0 .. 63] (+ omega at lag 0)
   float pn[16];
   cf gn[16];
@@ -182,15 +181,18 @@ struct FwdSmem {
   cf carry[2][16];
   cf pw[12][16];                               // q^(4 k), q^(16 k) (k < 4), q, q^64, q^(64 CPS), q^(256 CPS)
   u32x4 aop[kFwdBlocks][2][kWave];
-  float H[(NC + 1) * kHP];                     // row 1 + c: state after chunk c of the segment
+  // row 1 + c: state after chunk c of the segment; while a row is set up the buffer holds the
+  // power table q_n^e, e = 0 .. 64 (16 x 66 complex), from which the operand blocks are built
+  float H[(NC + 1) * kHP];
 };
+static_assert(sizeof(cf) * 16 * (kT + 2) <= sizeof(float) * (kWaves * 32 + 1) * kHP, "the power table fits the state buffer");
 
 // LDS traffic of one wave is processed in order: a wave that has written rows
 // and waits for its own LDS operations can read what its other lanes wrote.
 __device__ __forceinline__ void wave_sync() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 template <int DT, int NT>
-__global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
+__global__ __launch_bounds__(kThreads, NT == 1 ? 3 : 2) void cema_scan_fwd_kernel(
     const void* __restrict__ x, void* __restrict__ y, const float* __restrict__ p,
     const cf* __restrict__ log_q, const cf* __restrict__ gamma, const float* __restrict__ omega,
     const cf* __restrict__ h0, cf* __restrict__ h_last, int64_t rows, int D, int N, int64_t L) {
@@ -198,6 +200,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
   constexpr int NC = Smem::NC, CPS = NC / kSubs, XP = XOp<DT>::XP;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
+  cf (*qp)[kT + 2] = reinterpret_cast<cf(*)[kT + 2]>(sm.H);  // while a row is set up
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int g = lane >> 5, r = lane & 31;
   // scan roles: mode sn; sub-segment sa = 4 wave + sl of CPS chunks, inside the wave's own tiles
@@ -272,12 +275,12 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
       const cf c{rp.pv * rp.gv.x, rp.pv * rp.gv.y};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        sm.qp[sn][4 * sa + e] = v;
+        qp[sn][4 * sa + e] = v;
         const float kl = group_sum<16>(c.x * v.x - c.y * v.y);
         if (sn == 0) sm.klocal[4 * sa + e] = (sa == 0 && e == 0) ? kl + rp.w : kl;
         v = cmul(v, q1);
       }
-      if (sa == 15) sm.qp[sn][kT] = sm.pw[9][sn];
+      if (sa == 15) qp[sn][kT] = sm.pw[9][sn];
       qT = sm.pw[9][sn];
       qS = sm.pw[10][sn];
       qW = sm.pw[11][sn];
@@ -292,7 +295,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
         const float pp = sm.pn[n];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const cf w = sm.qp[n][kT - 1 - (16 * blk + 8 * gg + e)];
+          const cf w = qp[n][kT - 1 - (16 * blk + 8 * gg + e)];
           v[e] = pp * (part ? w.y : w.x);
         }
       } else if (blk < 8) {
@@ -308,7 +311,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int m = 16 * s2 + 8 * gg + e, n = m >> 1;
-          const cf w = cmul(sm.gn[n], sm.qp[n][i + 1]);
+          const cf w = cmul(sm.gn[n], qp[n][i + 1]);
           v[e] = (m & 1) ? -w.y : w.x;
         }
       }
@@ -503,13 +506,15 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_fwd_kernel(
           // H[C-2]: the row in front of the last chunk, or the wave's carried-in state
           const float* prev = (cl % (NT * 32) == 0) ? sm.wave_cin[cl / (NT * 32)] + 2 * tid
                                                     : sm.H + cl * kHP + 2 * tid;
-          h = cmul(sm.qp[tid][rem], cf{prev[0], prev[1]});
+          // the recurrence itself over the last chunk's steps (the power table has made way for
+          // the states by now): h <- q h + p x
+          h = cf{prev[0], prev[1]};
+          const cf q1 = sm.pw[8][tid];
           const float pp = sm.pn[tid];
           for (int j = 0; j < rem; ++j) {
             const float xv = Elem<DT>::load(xrow + (C - 1) * kT + j) * pp;
-            const cf w = sm.qp[tid][rem - 1 - j];
-            h.x = fmaf(xv, w.x, h.x);
-            h.y = fmaf(xv, w.y, h.y);
+            h = cmul(q1, h);
+            h.x += xv;
           }
         }
         h_last[row * N + tid] = h;
@@ -532,7 +537,7 @@ int launch_fwd(const void* x, void* y, const float* p, const cf* log_q, const cf
   int dev = 0, cus = 0;
   MEGA_CHECK_HIP(hipGetDevice(&dev));
   MEGA_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  const int64_t rows = B * D, slots = 2 * static_cast<int64_t>(cus);  // two workgroups fit a compute unit
+  const int64_t rows = B * D, slots = (NT == 1 ? 3 : 2) * static_cast<int64_t>(cus);  // workgroups that fit a compute unit
   const unsigned grid = static_cast<unsigned>(rows < slots ? rows : slots);
   cema_scan_fwd_kernel<DT, NT><<<dim3(grid), kThreads, lds, stream>>>(
       x, y, p, log_q, gamma, omega, h0, h_last, rows, static_cast<int>(D), static_cast<int>(N), L);
