@@ -471,6 +471,282 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
   }  // work item
 }
 
+// ---- the same product with the operand slabs sent from memory straight into LDS ------
+// Eight waves of 128 x 64 as above, aligned operands only.  `global_load_lds_dwordx4`
+// writes the 64 lanes' 16-byte pieces to 1 KB of consecutive LDS (base in M0), so no slab
+// passes through registers: no register ring, no LDS store instructions.  The LDS image
+// is dense and the swizzle that keeps fragment reads off each other's banks is applied
+// on the memory side -- which chunk a lane fetches:
+//   k-contiguous operand: a slab is 256 rows of 64 bytes; 1 KB = 16 rows; the chunk at
+//       position c of row r holds k chunk c ^ ((r >> 2) & 3) (16-byte reads go sixteen lanes at
+//       a time over 64 banks: sixteen consecutive rows of one k chunk then cover sixteen different
+//       16-byte bank groups; with (r >> 1) & 3, enough for eight lanes over 32 banks, half of the
+//       LDS cycles were bank conflicts);
+//   k-major operand: a slab is 32 rows of k, 512 bytes each; 1 KB = 2 rows; the chunk at
+//       position c of row k holds m chunk c ^ ((k & 3) << 2) (the four rows of k that a
+//       transposing read touches lie 64 bytes apart, as with the padded rows above).
+// Four slab buffers: slab s + 4 is requested into the buffer of slab s right after the
+// barrier that ends the reads of slab s; three slabs are in flight while one is read.
+constexpr int kStages = 4;
+constexpr int kDmaOperand = kTile * kSlab;   // elements of an operand slab (16 KB)
+constexpr int kDmaStage = 2 * kDmaOperand;   // A, then B
+constexpr size_t kDmaLds = sizeof(uint16_t) * (8 * 128 * (64 + 8) > kStages * kDmaStage ? 8 * 128 * (64 + 8)
+                                                                                         : kStages * kDmaStage);
+
+// One request: lane l's 16 bytes at base + offset go to LDS bytes lds_dst + 16 l .. + 15
+// (lds_dst wave-uniform).  Written as assembly so that the compiler does not see a vector
+// memory instruction that writes LDS: it would put a wait for every request in flight in
+// front of the transposing LDS reads.  The waits for these requests are the explicit
+// `s_waitcnt vmcnt` below.  M0 is reserved: the compiler keeps nothing in it across statements.
+__device__ __forceinline__ void load_to_lds16(const void* base, uint32_t offset, uint32_t lds_dst) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(offset), "s"(base), "s"(lds_dst));
+}
+
+template <int DT, bool TA, bool TB>
+__global__ __launch_bounds__(2 * kThreads) void gemm_dma_kernel(const GemmParams p) {
+  extern __shared__ __align__(16) uint16_t smem[];
+  constexpr int JN = 2, NL = 2, EP = 64 + 8;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wm = wave >> 2, wn = wave & 3;
+  // work items as in gemm_kernel
+  const int G = static_cast<int>(gridDim.x), lin = static_cast<int>(blockIdx.x);
+  int it_lo, it_hi, it_step;
+  if (G % kXcds == 0) {
+    const int xcd = lin % kXcds;
+    it_lo = static_cast<int>(static_cast<int64_t>(p.items) * xcd / kXcds) + lin / kXcds;
+    it_hi = static_cast<int>(static_cast<int64_t>(p.items) * (xcd + 1) / kXcds);
+    it_step = G / kXcds;
+  } else {
+    it_lo = lin;
+    it_hi = p.items;
+    it_step = G;
+  }
+  for (int item = it_lo; item < it_hi; item += it_step) {
+  const int zz = item / p.per_batch;
+  const int rem = item % p.per_batch;
+  int nt, mt_first, mt_second = -1;
+  if (p.tri_out) {
+    int t = rem, m = 0;
+    while (true) {
+      const int cnt = min(p.nt_count, (m * kTile + (kTile - 1) + p.off) / kTile + 1);
+      if (t < cnt) break;
+      t -= cnt;
+      ++m;
+    }
+    mt_first = m;
+    nt = t;
+  } else if (p.k_mode) {
+    nt = rem % p.nt_count;
+    const int pr = rem / p.nt_count;
+    mt_first = p.mt_count - 1 - pr;
+    if (mt_first != pr) mt_second = pr;
+  } else {
+    nt = rem % p.nt_count;
+    mt_first = rem / p.nt_count;
+  }
+  const int z0 = zz / p.nh, z1 = zz % p.nh;
+  const uint16_t* A = p.A + z0 * p.sa0 + z1 * p.sa1;
+  const uint16_t* B = p.B + z0 * p.sb0 + z1 * p.sb1;
+  uint16_t* C = p.C + z0 * p.sc0 + z1 * p.sc1;
+  for (int half = 0; half < 2; ++half) {
+  const int mt = half == 0 ? mt_first : mt_second;
+  if (mt < 0) break;
+  const int m0 = mt * kTile, n0 = nt * kTile;
+  int kb = 0, ke = p.K;
+  if (p.k_mode == 1) ke = min(p.K, ((mt + 1) * kTile + p.off + kSlab - 1) / kSlab * kSlab);
+  if (p.k_mode == 2) kb = min(p.K, max(0, mt * kTile - p.off) / kSlab * kSlab);
+  const int nslab = (ke - kb + kSlab - 1) / kSlab;
+
+  floatx16 acc[4][JN];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < JN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // memory side: wave w sends the 1 KB pieces w and w + 8 of each operand slab; lane l
+  // of piece pc fetches what belongs at position l of the piece (addresses clamped into
+  // the matrix, so every lane always loads)
+  uint32_t offa[NL], offb[NL];
+#pragma unroll
+  for (int i = 0; i < NL; ++i) {
+    const int pc = wave + 8 * i;
+    const int krow = 2 * pc + (lane >> 5), cm = (lane & 31) ^ ((krow & 3) << 2);  // k-major piece
+    const int row = 16 * pc + (lane >> 2), ck = (lane & 3) ^ ((lane >> 4) & 3);   // k-contiguous piece
+    if (TA) offa[i] = static_cast<uint32_t>(((kb + krow) * p.lda + min(m0 + cm * 8, p.M - 8)) * 2);
+    else offa[i] = static_cast<uint32_t>((static_cast<int64_t>(min(m0 + row, p.M - 1)) * p.lda + kb + ck * 8) * 2);
+    if (TB) offb[i] = static_cast<uint32_t>(((kb + krow) * p.ldb + min(n0 + cm * 8, p.N - 8)) * 2);
+    else offb[i] = static_cast<uint32_t>((static_cast<int64_t>(min(n0 + row, p.N - 1)) * p.ldb + kb + ck * 8) * 2);
+  }
+  const uint32_t stepa = static_cast<uint32_t>((TA ? p.lda : 1) * kSlab * 2);
+  const uint32_t stepb = static_cast<uint32_t>((TB ? p.ldb : 1) * kSlab * 2);
+  const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)(smem))) + wave * 1024);
+  // request number n of a slab: n = 0, 2 the two pieces of A, n = 1, 3 those of B
+  auto request_one = [&](int s, int stage, int n) {
+    const uint32_t sc = static_cast<uint32_t>(min(s, nslab - 1));
+    const uint32_t dst = lds_wave + static_cast<uint32_t>(stage * kDmaStage + (n >> 1) * 8 * 512 + (n & 1) * kDmaOperand) * 2;
+    if (n & 1) load_to_lds16(B, offb[n >> 1] + sc * stepb, dst);
+    else load_to_lds16(A, offa[n >> 1] + sc * stepa, dst);
+  };
+  auto request = [&](int s, int stage) {
+#pragma unroll
+    for (int n = 0; n < 2 * NL; ++n) request_one(s, stage, n);
+  };
+
+  // fragment side: k-step `set` of a slab takes k = 16 g + 8 set + e for lane half g
+  const int g = lane >> 5, r = lane & 31;
+  const int ta_a = (lane & 15) >> 2, ta_h = (lane >> 4) & 1, ta_b = lane & 3;
+  int fra[4], frb[JN];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (TA) fra[i] = (16 * g + ta_a) * kTile + (((wm * 16 + 4 * i + 2 * ta_h + (ta_b >> 1)) ^ (ta_a << 2)) * 8) + 4 * (ta_b & 1);
+    else fra[i] = (wm * 128 + 32 * i + r) * kSlab + (((2 * g) ^ ((r >> 2) & 3)) * 8);
+  }
+#pragma unroll
+  for (int j = 0; j < JN; ++j) {
+    if (TB) frb[j] = kDmaOperand + (16 * g + ta_a) * kTile + (((wn * 8 + 4 * j + 2 * ta_h + (ta_b >> 1)) ^ (ta_a << 2)) * 8) + 4 * (ta_b & 1);
+    else frb[j] = kDmaOperand + (wn * 64 + 32 * j + r) * kSlab + (((2 * g) ^ ((r >> 2) & 3)) * 8);
+  }
+  u32x4 fa0[4], fb0[JN], fa1[4], fb1[JN];
+  auto fread = [&](u32x4* fa, u32x4* fb, int set, int stage) {
+    const uint16_t* base = smem + stage * kDmaStage;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (TA) {
+        const uint16_t* q = base + fra[i] + set * 8 * kTile;
+        const uint2 lo = lds_read_tr(q), hi = lds_read_tr(q + 4 * kTile);
+        fa[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+      } else {
+        // chunk 2 g + set sits at position (2 g + set) ^ swizzle = ((2 g) ^ swizzle) ^ set
+        fa[i] = *reinterpret_cast<const u32x4*>(base + (fra[i] ^ (set * 8)));
+      }
+      if (i < JN) {
+        if (TB) {
+          const uint16_t* q = base + frb[i] + set * 8 * kTile;
+          const uint2 lo = lds_read_tr(q), hi = lds_read_tr(q + 4 * kTile);
+          fb[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        } else {
+          fb[i] = *reinterpret_cast<const u32x4*>(base + (frb[i] ^ (set * 8)));
+        }
+      }
+    }
+  };
+  // products lo .. hi - 1 of a k-step, numbered 2 i + j
+  auto mma = [&](const u32x4* fa, const u32x4* fb, int lo, int hi) {
+#pragma unroll
+    for (int n = 0; n < 4 * JN; ++n)
+      if (n >= lo && n < hi) acc[n >> 1][n & 1] = Mma<DT>::run(fb[n & 1], fa[n >> 1], acc[n >> 1][n & 1]);
+  };
+
+  // One step per slab, one barrier per step, placed between the two k-steps:
+  //   first half:  read the second fragment set of slab cur; 8 MFMAs on the first set;
+  //   wait until this wave's pieces of slab cur + 1 have landed (at most the 8 requests of
+  //   slabs cur + 2, cur + 3 still in flight) and its fragment reads have returned; barrier;
+  //   second half: read the first fragment set of slab cur + 1, request slab cur + 4 into
+  //                the buffer slab cur has just left, 8 MFMAs on the second set.
+#define MEGA_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+  constexpr int kFragReads = (TA ? 2 : 1) + (TB ? JN / 2 : (JN + 3) / 4);
+#define MEGA_DMA_STEP(R)                                                   \
+  {                                                                        \
+    const int cur = it + (R);                                              \
+    fread(fa1, fb1, 1, (R));                                               \
+    mma(fa0, fb0, 0, 8);                                                   \
+    _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
+      MEGA_SGB(0x008, 1);                                                  \
+      MEGA_SGB(0x100, kFragReads);                                         \
+    }                                                                      \
+    MEGA_SGB(0x008, 4 * JN - 4);                                           \
+    __builtin_amdgcn_sched_barrier(0);                                     \
+    asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory"); \
+    fread(fa0, fb0, 0, ((R) + 1) & 3);                                     \
+    mma(fa1, fb1, 0, 4);                                                   \
+    _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
+      MEGA_SGB(0x008, 1);                                                  \
+      MEGA_SGB(0x100, kFragReads);                                         \
+    }                                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                     \
+    _Pragma("unroll") for (int n = 0; n < 2 * NL; ++n) {                   \
+      request_one(cur + kStages, (R), n);                                  \
+      mma(fa1, fb1, 4 + n, 5 + n);                                         \
+      __builtin_amdgcn_sched_barrier(0);                                   \
+    }                                                                      \
+  }
+  if (nslab > 0) {
+    request(0, 0);
+    request(1, 1);
+    request(2, 2);
+    request(3, 3);
+    asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+    fread(fa0, fb0, 0, 0);
+    int it = 0;
+    for (; it + 4 <= nslab; it += 4) {
+      MEGA_DMA_STEP(0)
+      MEGA_DMA_STEP(1)
+      MEGA_DMA_STEP(2)
+      MEGA_DMA_STEP(3)
+    }
+    if (it < nslab) MEGA_DMA_STEP(0)
+    if (it + 1 < nslab) MEGA_DMA_STEP(1)
+    if (it + 2 < nslab) MEGA_DMA_STEP(2)
+    // nothing may land in the buffers once they hold the output tiles
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  }
+#undef MEGA_DMA_STEP
+#undef MEGA_SGB
+
+  // epilogue as in gemm_kernel: the wave's 128 x 64 tile through its own LDS region
+  uint16_t* stage = smem + wave * 128 * EP;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < JN; ++j) {
+      const int row = i * 32 + (lane & 31);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int col = j * 32 + 8 * q4 + 4 * (lane >> 5);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[i][j][4 * q4 + e];
+        uint2 w;
+        if (DT == MEGA_BF16) {
+          w.x = pack_bf16x2(v[0], v[1]);
+          w.y = pack_bf16x2(v[2], v[3]);
+        } else {
+          w.x = static_cast<uint32_t>(float_to_f16_bits(v[0])) | (static_cast<uint32_t>(float_to_f16_bits(v[1])) << 16);
+          w.y = static_cast<uint32_t>(float_to_f16_bits(v[2])) | (static_cast<uint32_t>(float_to_f16_bits(v[3])) << 16);
+        }
+        *reinterpret_cast<uint2*>(stage + row * EP + col) = w;
+      }
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave reads back only its own region
+  const bool vec_ok = (p.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+#pragma unroll 4
+  for (int i = 0; i < 8 * JN; ++i) {
+    const int c = lane + kWave * i;
+    const int row = c / (4 * JN), kc = (c % (4 * JN)) * 8;
+    const int grow = m0 + wm * 128 + row, gcol = n0 + wn * (32 * JN) + kc;
+    if (grow < p.M && gcol < p.N) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * EP + kc);
+      uint16_t* dst = C + static_cast<int64_t>(grow) * p.ldc + gcol;
+      if (vec_ok && gcol + 8 <= p.N) {
+        *reinterpret_cast<u32x4*>(dst) = v;
+      } else {
+        const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+        for (int q = 0; q < 8; ++q)
+          if (gcol + q < p.N) dst[q] = e[q];
+      }
+    }
+  }
+  // the output regions overlap the slab buffers: every read of this tile's epilogue
+  // retires before the next tile's first slab is requested
+  lds_barrier();
+  }  // tile of the pair
+  }  // work item
+}
+
 // ---- causal softmax over rows (in place), one wavefront per row ---------------
 // `coff` < 0: every row keeps all L2 columns.  `coff` = L2 - L1 >= 0 (causal,
 // bottom-right aligned, softmax.cuh:99-100): row r keeps columns [0, n) with
@@ -713,7 +989,13 @@ int launch_gemm_t(const GemmParams& p, int batch, hipStream_t s) {
   // one per SIMD; MEGA_GEMM_W4=1 in the environment selects the latter for
   // comparison.
   const char* w4 = getenv("MEGA_GEMM_W4");
-  if (fast && !(w4 != nullptr && w4[0] == '1')) {
+  // MEGA_GEMM_DMA=0 keeps the slabs on the register path (for comparison)
+  const char* dma = getenv("MEGA_GEMM_DMA");
+  if (fast && !(w4 != nullptr && w4[0] == '1') && !(dma != nullptr && dma[0] == '0')) {
+    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<DT, TA, TB>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaLds));
+    gemm_dma_kernel<DT, TA, TB><<<grid, 2 * kThreads, kDmaLds, s>>>(q);
+  } else if (fast && !(w4 != nullptr && w4[0] == '1')) {
     const size_t lds8 = sizeof(uint16_t) * 8 * 128 * (64 + 8) > lds ? sizeof(uint16_t) * 8 * 128 * (64 + 8) : lds;
     MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, true, TA, TB, true>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds8));
