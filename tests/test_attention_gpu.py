@@ -87,6 +87,25 @@ def test_float32_tensors(B, L1, L2, NH, H1, H2, causal):
         assert torch.count_nonzero(torch.triu(w, diagonal=L2 - L1 + 1)) == 0
 
 
+@pytest.mark.parametrize("B,L1,L2,NH,H1,H2", [(1, 520, 1000, 2, 32, 64), (2, 768, 768, 2, 256, 512)])
+def test_slab_paths_agree_bit_for_bit(B, L1, L2, NH, H1, H2, monkeypatch):
+    """Aligned operands reach LDS straight from memory; MEGA_GEMM_DMA=0 sends them
+    through registers.  Both run the same products in the same order, so y, the
+    probabilities on and below the diagonal and the three gradients are identical bits."""
+    g = torch.Generator().manual_seed(L1)
+    q = (torch.randn(B, L1, NH, H1, generator=g) / H1 ** 0.5).bfloat16().cuda()
+    k = (torch.randn(B, L2, NH, H1, generator=g) / H1 ** 0.5).bfloat16().cuda()
+    v = (torch.randn(B, L2, NH, H2, generator=g) / H2 ** 0.5).bfloat16().cuda()
+    dy = torch.randn(B, L1, NH, H2, generator=g).bfloat16().cuda()
+    out = []
+    for mode in ("1", "0"):
+        monkeypatch.setenv("MEGA_GEMM_DMA", mode)
+        y, w = ops.attention_fwd(q, k, v, 1.0, 0.0, True)
+        out.append((y, torch.tril(w, diagonal=L2 - L1)) + tuple(ops.attention_bwd(dy, q, k, v, w, 1.0, True)))
+    for a, b in zip(*out):
+        assert torch.equal(a, b)
+
+
 def test_causal_with_fewer_keys_than_queries_fails_loudly():
     q = torch.zeros(1, 8, 1, 16, dtype=torch.bfloat16, device="cuda")
     k = torch.zeros(1, 4, 1, 16, dtype=torch.bfloat16, device="cuda")
