@@ -38,6 +38,8 @@ extern "C" {
 #define MEGA_F32 0
 #define MEGA_BF16 1
 #define MEGA_F16 2
+/* float64: taken by the operators that say so (the double-precision flavours) */
+#define MEGA_F64 3
 
 /* Library version (major*10000 + minor*100 + patch). */
 int mega_version(void);
@@ -228,6 +230,28 @@ int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, const void* 
                                  void* dprev_var, void* dgamma, void* dbeta,
                                  void* workspace, void* stream);
 
+/* The double-precision flavour of the two operators above
+ * (timestep_norm_kernel.cu:1567-1576 instantiates the reference's kernels for
+ * double, with float64 cummean / cumrstd, :1553-1565): every tensor float64
+ * except prev_count / count (int64) and the mask; one wavefront per (batch,
+ * group) chain walks the sequence, so there are no look-back records and the
+ * forward needs no workspace.  The backward's `workspace`: 2 * B * D doubles. */
+int mega_group_timestep_norm_fwd_f64(const double* x, const int64_t* prev_count,
+                                     const double* prev_mean, const double* prev_var,
+                                     const double* gamma, const double* beta,
+                                     const uint8_t* padding_mask, int64_t B, int64_t L,
+                                     int64_t D, int64_t G, double eps, double* y,
+                                     int64_t* count, double* mean, double* var,
+                                     double* cummean, double* cumrstd, void* stream);
+int mega_group_timestep_norm_bwd_f64(const double* dy, const double* dmean, const double* dvar,
+                                     const double* x, const double* prev_mean,
+                                     const int64_t* count, const double* cummean,
+                                     const double* cumrstd, const double* gamma,
+                                     const uint8_t* padding_mask, int64_t B, int64_t L,
+                                     int64_t D, int64_t G, double* dx, double* dprev_mean,
+                                     double* dprev_var, double* dgamma, double* dbeta,
+                                     double* workspace, void* stream);
+
 /* The tiled kernels above hand running statistics from tile to tile through
  * records in `workspace`; a tile polls for its predecessors' records at most a
  * fixed number of times (a couple of seconds), then sets a status word in the
@@ -254,10 +278,11 @@ void mega_test_timestep_norm_lookback(long long spin_limit, int mute_tile);
  *   q (B, L1, NH, H1), k (B, L2, NH, H1), v (B, L2, NH, H2), y (B, L1, NH, H2),
  *   w (B, NH, L1, L2), all of `dtype`, contiguous; B counts chunks (the
  *   module views (batch, L) as (batch*L/chunk, chunk)).  MEGA_BF16 / MEGA_F16
- *   run on the matrix cores and are what follows describes; MEGA_F32
- *   (attention_kernel.cu:269-281 dispatches over it too) keeps float32 storage
- *   and arithmetic on the vector ALUs, writes every row of w to its end, and
- *   needs twice the workspace bytes the size query returns.
+ *   run on the matrix cores and are what follows describes; MEGA_F32 and
+ *   MEGA_F64 (attention_kernel.cu:269-281 dispatches over them too) keep
+ *   storage and arithmetic of that type on the vector ALUs, write every row of
+ *   w to its end, and need two / four times the workspace bytes the size query
+ *   returns.
  *   S = scale * q k^T rounded to `dtype`; with `causal` row r keeps columns
  *   0 .. L2 - L1 + r (L2 >= L1 required: cached keys / values in front of the
  *   chunk, softmax.cuh:99-100), all columns otherwise; P = softmax in fp32,

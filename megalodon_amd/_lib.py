@@ -14,7 +14,7 @@ PKG_DIR = Path(__file__).resolve().parent
 LIB_PATH = PKG_DIR / "lib" / "libmegalodon_hip.so"
 HEADER_PATH = PKG_DIR.parent / "include" / "megalodon_hip.h"
 
-MEGA_F32, MEGA_BF16, MEGA_F16 = 0, 1, 2
+MEGA_F32, MEGA_BF16, MEGA_F16, MEGA_F64 = 0, 1, 2, 3
 
 _lib = None
 
@@ -71,8 +71,12 @@ def i32(v: int) -> ctypes.c_int:
     return ctypes.c_int(int(v))
 
 
-def dtype_code(dtype) -> int:
+def dtype_code(dtype, wide_ok: bool = False) -> int:
+    """Element type code of the C interface.  float64 is taken by the operators that have a
+    double-precision flavour (`wide_ok`); everywhere else it is refused, not narrowed."""
     import torch
+    if wide_ok and dtype == torch.float64:
+        return MEGA_F64
     try:
         return {torch.float32: MEGA_F32, torch.bfloat16: MEGA_BF16, torch.float16: MEGA_F16}[dtype]
     except KeyError:

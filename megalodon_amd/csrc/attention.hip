@@ -28,15 +28,19 @@
 
 namespace mega {
 
-// float32 tensors: attention_f32.hip
-int attention_f32_fwd(const float* q, const float* k, const float* v, int64_t B, int64_t L1, int64_t L2,
-                      int64_t NH, int64_t H1, int64_t H2, float scale, int causal, const DropKey* drop,
-                      float* y, float* w, hipStream_t s);
-int attention_f32_bwd(const float* dy, const float* q, const float* k, const float* v, const float* w,
-                      int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1, int64_t H2, float scale,
-                      int causal, float* dq, float* dk, float* dv, float* dp, hipStream_t s);
-int softmax_f32_fwd(float* x, int64_t Z, int64_t L1, int64_t L2, int causal, const DropKey* drop, hipStream_t s);
-int softmax_f32_bwd(const float* y, float* dy, int64_t Z, int64_t L1, int64_t L2, int causal, hipStream_t s);
+// float32 / float64 tensors: attention_f32.hip
+template <typename T>
+int attention_wide_fwd(const T* q, const T* k, const T* v, int64_t B, int64_t L1, int64_t L2,
+                       int64_t NH, int64_t H1, int64_t H2, double scale, int causal, const DropKey* drop,
+                       T* y, T* w, hipStream_t s);
+template <typename T>
+int attention_wide_bwd(const T* dy, const T* q, const T* k, const T* v, const T* w,
+                       int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1, int64_t H2, double scale,
+                       int causal, T* dq, T* dk, T* dv, T* dp, hipStream_t s);
+template <typename T>
+int softmax_wide_fwd(T* x, int64_t Z, int64_t L1, int64_t L2, int causal, const DropKey* drop, hipStream_t s);
+template <typename T>
+int softmax_wide_bwd(const T* y, T* dy, int64_t Z, int64_t L1, int64_t L2, int causal, hipStream_t s);
 
 namespace {
 
@@ -1032,7 +1036,7 @@ AttnWs attn_ws(int64_t B, int64_t L1, int64_t L2, int64_t NH, int64_t H1, int64_
 
 int check_attn(const char* who, int dtype, int64_t B, int64_t L1, int64_t L2, int64_t NH,
                int64_t H1, int64_t H2, int causal) {
-  MEGA_CHECK_ARG(valid_dtype(dtype), "%s: unknown dtype %d", who, dtype);
+  MEGA_CHECK_ARG(valid_dtype(dtype) || dtype == MEGA_F64, "%s: unknown dtype %d", who, dtype);
   MEGA_CHECK_ARG(B >= 0 && L1 >= 0 && L2 >= 0 && NH >= 1 && H1 >= 1 && H2 >= 1, "%s: bad sizes", who);
   MEGA_CHECK_ARG(B * NH <= 65535, "%s: batch * heads exceeds 65535", who);
   MEGA_CHECK_ARG(L1 <= (1 << 24) && L2 <= (1 << 24), "%s: sequence too long", who);
@@ -1145,9 +1149,13 @@ static int attention_fwd_entry(const char* who, const void* q, const void* k, co
   MEGA_CHECK_ARG(L2 >= 1, "%s: no keys", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == MEGA_F32)
-    return attention_f32_fwd(static_cast<const float*>(q), static_cast<const float*>(k),
-                             static_cast<const float*>(v), B, L1, L2, NH, H1, H2, (float)scale, causal, drop,
-                             static_cast<float*>(y), static_cast<float*>(w), s);
+    return attention_wide_fwd<float>(static_cast<const float*>(q), static_cast<const float*>(k),
+                                     static_cast<const float*>(v), B, L1, L2, NH, H1, H2, scale, causal, drop,
+                                     static_cast<float*>(y), static_cast<float*>(w), s);
+  if (dtype == MEGA_F64)
+    return attention_wide_fwd<double>(static_cast<const double*>(q), static_cast<const double*>(k),
+                                      static_cast<const double*>(v), B, L1, L2, NH, H1, H2, scale, causal, drop,
+                                      static_cast<double*>(y), static_cast<double*>(w), s);
   auto u = [](const void* p) { return static_cast<const uint16_t*>(p); };
   auto m = [](void* p) { return static_cast<uint16_t*>(p); };
   if (dtype == MEGA_BF16)
@@ -1190,11 +1198,17 @@ extern "C" int mega_attention_bwd(const void* dy, const void* q, const void* k, 
   MEGA_CHECK_ARG(L1 >= 1 && L2 >= 1, "mega_attention_bwd: empty sequence");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == MEGA_F32)
-    return attention_f32_bwd(static_cast<const float*>(dy), static_cast<const float*>(q),
-                             static_cast<const float*>(k), static_cast<const float*>(v),
-                             static_cast<const float*>(w), B, L1, L2, NH, H1, H2, (float)scale, causal,
-                             static_cast<float*>(dq), static_cast<float*>(dk), static_cast<float*>(dv),
-                             static_cast<float*>(workspace), s);
+    return attention_wide_bwd<float>(static_cast<const float*>(dy), static_cast<const float*>(q),
+                                     static_cast<const float*>(k), static_cast<const float*>(v),
+                                     static_cast<const float*>(w), B, L1, L2, NH, H1, H2, scale, causal,
+                                     static_cast<float*>(dq), static_cast<float*>(dk), static_cast<float*>(dv),
+                                     static_cast<float*>(workspace), s);
+  if (dtype == MEGA_F64)
+    return attention_wide_bwd<double>(static_cast<const double*>(dy), static_cast<const double*>(q),
+                                      static_cast<const double*>(k), static_cast<const double*>(v),
+                                      static_cast<const double*>(w), B, L1, L2, NH, H1, H2, scale, causal,
+                                      static_cast<double*>(dq), static_cast<double*>(dk), static_cast<double*>(dv),
+                                      static_cast<double*>(workspace), s);
   auto u = [](const void* p) { return static_cast<const uint16_t*>(p); };
   auto m = [](void* p) { return static_cast<uint16_t*>(p); };
   if (dtype == MEGA_BF16)
@@ -1206,7 +1220,7 @@ extern "C" int mega_attention_bwd(const void* dy, const void* q, const void* k, 
 
 // ---- standalone causal softmax ---------------------------------------------------
 static int check_softmax(const char* who, int dtype, int64_t Z, int64_t L1, int64_t L2, int causal) {
-  MEGA_CHECK_ARG(valid_dtype(dtype), "%s: unknown dtype %d", who, dtype);
+  MEGA_CHECK_ARG(valid_dtype(dtype) || dtype == MEGA_F64, "%s: unknown dtype %d", who, dtype);
   MEGA_CHECK_ARG(Z >= 0 && L1 >= 0 && L2 >= 0, "%s: bad sizes", who);
   MEGA_CHECK_ARG(Z <= 65535, "%s: more than 65535 matrices", who);
   MEGA_CHECK_ARG(L1 <= (1 << 24) && L2 <= (1 << 24), "%s: rows too long", who);
@@ -1220,7 +1234,8 @@ static int softmax_fwd_entry(const char* who, void* x, int dtype, int64_t Z, int
   if (rc != MEGA_OK) return rc;
   MEGA_CHECK_ARG(x != nullptr || Z * L1 * L2 == 0, "%s: null pointer", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == MEGA_F32) return softmax_f32_fwd(static_cast<float*>(x), Z, L1, L2, causal, drop, s);
+  if (dtype == MEGA_F32) return softmax_wide_fwd<float>(static_cast<float*>(x), Z, L1, L2, causal, drop, s);
+  if (dtype == MEGA_F64) return softmax_wide_fwd<double>(static_cast<double*>(x), Z, L1, L2, causal, drop, s);
   if (dtype == MEGA_BF16)
     return launch_softmax<MEGA_BF16>(nullptr, static_cast<uint16_t*>(x), Z, L1, L2, causal, s, 1, drop);
   return launch_softmax<MEGA_F16>(nullptr, static_cast<uint16_t*>(x), Z, L1, L2, causal, s, 1, drop);
@@ -1251,7 +1266,9 @@ extern "C" int mega_attention_softmax_bwd(const void* y, void* dy, int dtype, in
   if (Z * L1 * L2 == 0) return MEGA_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == MEGA_F32)
-    return softmax_f32_bwd(static_cast<const float*>(y), static_cast<float*>(dy), Z, L1, L2, causal, s);
+    return softmax_wide_bwd<float>(static_cast<const float*>(y), static_cast<float*>(dy), Z, L1, L2, causal, s);
+  if (dtype == MEGA_F64)
+    return softmax_wide_bwd<double>(static_cast<const double*>(y), static_cast<double*>(dy), Z, L1, L2, causal, s);
   if (dtype == MEGA_BF16)
     return launch_softmax<MEGA_BF16>(static_cast<const uint16_t*>(y), static_cast<uint16_t*>(dy), Z, L1,
                                      L2, causal, s, 1);

@@ -744,8 +744,9 @@ def group_timestep_norm_fwd(
     eps: float,
 ):
     """(y, count, mean, var, cummean, cumrstd); tensors other than count /
-    mask / the float32 statistics must share x's dtype, as in the reference
-    (timestep_norm_kernel.cu:1270-1273)."""
+    mask / the statistics must share x's dtype, as in the reference
+    (timestep_norm_kernel.cu:1270-1273); cummean and cumrstd are float32, float64
+    for float64 x (the accumulate type, :1553-1565)."""
     dev = _require_cuda(x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask)
     if x.dim() != 3:
         raise RuntimeError("x must be (B, L, D)")
@@ -761,9 +762,21 @@ def group_timestep_norm_fwd(
     count = torch.empty_like(prev_count, memory_format=torch.contiguous_format)
     mean = torch.empty((B, G), dtype=x.dtype, device=dev)
     var = torch.empty((B, G), dtype=x.dtype, device=dev)
-    cummean = torch.empty((B, L, G), dtype=torch.float32, device=dev)
-    cumrstd = torch.empty((B, L, G), dtype=torch.float32, device=dev)
+    stat_dtype = torch.float64 if x.dtype == torch.float64 else torch.float32
+    cummean = torch.empty((B, L, G), dtype=stat_dtype, device=dev)
+    cumrstd = torch.empty((B, L, G), dtype=stat_dtype, device=dev)
     mask = _mask_bytes(padding_mask)
+    if x.dtype == torch.float64:
+        # the double-precision flavour: one wavefront per (batch, group) chain, no workspace
+        if D % G != 0:
+            raise RuntimeError("feature count must be a multiple of num_groups")
+        with torch.cuda.device(dev):
+            _lib.call("mega_group_timestep_norm_fwd_f64", _lib.ptr(xc), _lib.ptr(prev_count.contiguous()),
+                      _lib.ptr(prev_mean.contiguous()), _lib.ptr(prev_var.contiguous()), _lib.ptr(gamma.contiguous()),
+                      _lib.ptr(beta.contiguous()), _lib.ptr(mask), _lib.i64(B), _lib.i64(L), _lib.i64(D), _lib.i64(G),
+                      _lib.f64(eps), _lib.ptr(y), _lib.ptr(count), _lib.ptr(mean), _lib.ptr(var), _lib.ptr(cummean),
+                      _lib.ptr(cumrstd), _lib.stream_ptr(dev))
+        return y, count, mean, var, cummean, cumrstd
     ws = _tsn_workspace(B, L, D, G, False, dev)
     with torch.cuda.device(dev):
         _lib.call("mega_group_timestep_norm_fwd", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
@@ -803,6 +816,18 @@ def group_timestep_norm_bwd(
     dg = torch.empty((D,), dtype=x.dtype, device=dev)
     db = torch.empty((D,), dtype=x.dtype, device=dev)
     mask = _mask_bytes(padding_mask)
+    if x.dtype == torch.float64:
+        if cummean.dtype != torch.float64 or cumrstd.dtype != torch.float64:
+            raise RuntimeError("cummean / cumrstd of float64 x must be float64")
+        ws = torch.empty((2, B, D), dtype=torch.float64, device=dev)
+        with torch.cuda.device(dev):
+            _lib.call("mega_group_timestep_norm_bwd_f64", _lib.ptr(dy), _lib.ptr(mean_grad.contiguous()),
+                      _lib.ptr(var_grad.contiguous()), _lib.ptr(xc), _lib.ptr(prev_mean.contiguous()),
+                      _lib.ptr(count.contiguous()), _lib.ptr(cummean.contiguous()), _lib.ptr(cumrstd.contiguous()),
+                      _lib.ptr(gamma.contiguous()), _lib.ptr(mask), _lib.i64(B), _lib.i64(L), _lib.i64(D), _lib.i64(G),
+                      _lib.ptr(dx), _lib.ptr(dpm), _lib.ptr(dpv), _lib.ptr(dg), _lib.ptr(db), _lib.ptr(ws),
+                      _lib.stream_ptr(dev))
+        return dx, dpm, dpv, dg, db
     ws = _tsn_workspace(B, L, D, G, True, dev)
     with torch.cuda.device(dev):
         _lib.call("mega_group_timestep_norm_bwd", _lib.ptr(dy), _lib.ptr(mean_grad.contiguous()),
@@ -835,13 +860,13 @@ def stream_copy(a: torch.Tensor, b: Optional[torch.Tensor] = None, workgroups: i
 # --------------------------------------------------------------------------
 # attention (reference: csrc/ops/attention.cc:28-29, attention_kernel.cu:261-303)
 # --------------------------------------------------------------------------
-def _attn_workspace(B, L1, L2, NH, H1, H2, backward, dev, wide=False):
-    # `wide`: float32 tensors need twice the bytes of the 16-bit layout the size query describes
+def _attn_workspace(B, L1, L2, NH, H1, H2, backward, dev, dtype=torch.bfloat16):
+    # the size query describes the 16-bit layout: float32 / float64 tensors need 2 / 4 times the bytes
     fn = _lib.load().mega_attention_workspace_bytes
     fn.restype = _lib.ctypes.c_int64
     nbytes = int(fn(_lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH), _lib.i64(H1), _lib.i64(H2),
                     _lib.i32(1 if backward else 0)))
-    return torch.empty(nbytes * (2 if wide else 1), dtype=torch.uint8, device=dev)
+    return torch.empty(nbytes * max(1, dtype.itemsize // 2), dtype=torch.uint8, device=dev)
 
 
 def _attn_dims(q, k, v):
@@ -883,11 +908,11 @@ def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: floa
         qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
         y = torch.empty((B, L1, NH, H2), dtype=v.dtype, device=dev)
         w = torch.empty((B, NH, L1, L2), dtype=v.dtype, device=dev)
-        ws = _attn_workspace(B, L1, L2, NH, H1, H2, False, dev, q.dtype == torch.float32)
+        ws = _attn_workspace(B, L1, L2, NH, H1, H2, False, dev, q.dtype)
         seed, offset = dropkey_philox_state(dev, L2)
         with torch.cuda.device(dev):
             _lib.call("mega_attention_dropkey_fwd", _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc),
-                      _lib.i32(_lib.dtype_code(q.dtype)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2),
+                      _lib.i32(_lib.dtype_code(q.dtype, True)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2),
                       _lib.i64(NH), _lib.i64(H1), _lib.i64(H2), _lib.f64(scale),
                       _lib.i32(1 if use_causal_mask else 0), _lib.f64(dropout), _lib.u64(seed),
                       _lib.u64(offset), _lib.ptr(y), _lib.ptr(w), _lib.ptr(ws), _lib.stream_ptr(dev))
@@ -895,10 +920,10 @@ def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: floa
     qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
     y = torch.empty((B, L1, NH, H2), dtype=v.dtype, device=dev)
     w = torch.empty((B, NH, L1, L2), dtype=v.dtype, device=dev)
-    ws = _attn_workspace(B, L1, L2, NH, H1, H2, False, dev, q.dtype == torch.float32)
+    ws = _attn_workspace(B, L1, L2, NH, H1, H2, False, dev, q.dtype)
     with torch.cuda.device(dev):
         _lib.call("mega_attention_fwd", _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc),
-                  _lib.i32(_lib.dtype_code(q.dtype)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH),
+                  _lib.i32(_lib.dtype_code(q.dtype, True)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH),
                   _lib.i64(H1), _lib.i64(H2), _lib.f64(scale), _lib.i32(1 if use_causal_mask else 0),
                   _lib.ptr(y), _lib.ptr(w), _lib.ptr(ws), _lib.stream_ptr(dev))
     return y, w
@@ -913,10 +938,10 @@ def attention_bwd(y_grad: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: tor
         raise RuntimeError("attention_bwd: w / y_grad shapes do not match q, k, v")
     qc, kc, vc, dy, wc = q.contiguous(), k.contiguous(), v.contiguous(), y_grad.contiguous(), w.contiguous()
     dq, dk, dv = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc)
-    ws = _attn_workspace(B, L1, L2, NH, H1, H2, True, dev, q.dtype == torch.float32)
+    ws = _attn_workspace(B, L1, L2, NH, H1, H2, True, dev, q.dtype)
     with torch.cuda.device(dev):
         _lib.call("mega_attention_bwd", _lib.ptr(dy), _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc), _lib.ptr(wc),
-                  _lib.i32(_lib.dtype_code(q.dtype)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH),
+                  _lib.i32(_lib.dtype_code(q.dtype, True)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH),
                   _lib.i64(H1), _lib.i64(H2), _lib.f64(scale), _lib.i32(1 if use_causal_mask else 0),
                   _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(ws), _lib.stream_ptr(dev))
     return dq, dk, dv
@@ -942,12 +967,12 @@ def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool
     if dropout > 0.0:
         seed, offset = dropkey_philox_state(dev, L2)
         with torch.cuda.device(dev):
-            _lib.call("mega_attention_softmax_dropkey_fwd", _lib.ptr(y), _lib.i32(_lib.dtype_code(x.dtype)),
+            _lib.call("mega_attention_softmax_dropkey_fwd", _lib.ptr(y), _lib.i32(_lib.dtype_code(x.dtype, True)),
                       _lib.i64(Z), _lib.i64(L1), _lib.i64(L2), _lib.i32(1 if use_causal_mask else 0),
                       _lib.f64(dropout), _lib.u64(seed), _lib.u64(offset), _lib.stream_ptr(dev))
         return y
     with torch.cuda.device(dev):
-        _lib.call("mega_attention_softmax_fwd", _lib.ptr(y), _lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(Z),
+        _lib.call("mega_attention_softmax_fwd", _lib.ptr(y), _lib.i32(_lib.dtype_code(x.dtype, True)), _lib.i64(Z),
                   _lib.i64(L1), _lib.i64(L2), _lib.i32(1 if use_causal_mask else 0), _lib.stream_ptr(dev))
     return y
 
@@ -961,7 +986,7 @@ def attention_softmax_bwd(y_grad: torch.Tensor, y: torch.Tensor, use_causal_mask
     yc = y.contiguous()
     dx = y_grad.contiguous().clone()
     with torch.cuda.device(dev):
-        _lib.call("mega_attention_softmax_bwd", _lib.ptr(yc), _lib.ptr(dx), _lib.i32(_lib.dtype_code(y.dtype)),
+        _lib.call("mega_attention_softmax_bwd", _lib.ptr(yc), _lib.ptr(dx), _lib.i32(_lib.dtype_code(y.dtype, True)),
                   _lib.i64(Z), _lib.i64(L1), _lib.i64(L2), _lib.i32(1 if use_causal_mask else 0),
                   _lib.stream_ptr(dev))
     return dx

@@ -14,6 +14,7 @@ from oracle import attention as oa
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
 TOL_F32 = 1e-4   # float32 tensors (the vector-ALU flavour of the operator)
+TOL_F64 = 1e-12  # float64 tensors (the same flavour in double precision)
 
 
 def _run(B, L1, L2, NH, H1, H2, causal, dtype, seed, scale=1.0):
@@ -22,14 +23,14 @@ def _run(B, L1, L2, NH, H1, H2, causal, dtype, seed, scale=1.0):
     k = (torch.randn(B, L2, NH, H1, generator=g) / H1 ** 0.5).to(dtype)
     v = (torch.randn(B, L2, NH, H2, generator=g) / H2 ** 0.5).to(dtype)
     dy = torch.randn(B, L1, NH, H2, generator=g).to(dtype)
-    TOL = TOL_F32 if dtype == torch.float32 else globals()["TOL"]
+    TOL = {torch.float32: TOL_F32, torch.float64: TOL_F64}.get(dtype, globals()["TOL"])
     y, w = ops.attention_fwd(q.cuda(), k.cuda(), v.cuda(), scale, 0.0, causal)
     wy, wp = oa.chunk_attention_fwd(q, k, v, scale, causal)
     assert y.shape == (B, L1, NH, H2) and w.shape == (B, NH, L1, L2) and y.dtype == dtype and w.dtype == dtype
     assert rel_err(y, wy) <= TOL
     if causal:
         # compare the probabilities on and below the diagonal (blocks right of the diagonal block are not written)
-        assert rel_err(torch.tril(w.float(), diagonal=L2 - L1), wp) <= TOL
+        assert rel_err(torch.tril(w.double(), diagonal=L2 - L1), wp) <= TOL
     else:
         assert rel_err(w, wp) <= TOL
     dq, dk, dv = ops.attention_bwd(dy.cuda(), q.cuda(), k.cuda(), v.cuda(), w, scale, causal)
@@ -72,17 +73,18 @@ def test_causal_with_key_value_prefix(B, L1, L2, NH, H1, H2, dtype):
     (1, 1, 40, 1, 16, 16, True),         # one new query
     (1, 520, 1000, 2, 32, 64, True),     # several row tiles, prefix of 480 keys
 ])
-def test_float32_tensors(B, L1, L2, NH, H1, H2, causal):
-    """The reference dispatches the operator over float32 too
-    (attention_kernel.cu:269-281); here float32 q, k, v keep float32 storage and
-    arithmetic: y, w and the three gradients within 1e-4 of the oracle, and w
-    holds exact zeros above the diagonal."""
-    _run(B, L1, L2, NH, H1, H2, causal, torch.float32, seed=L1 + 2 * L2, scale=0.8)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_float32_and_float64_tensors(B, L1, L2, NH, H1, H2, causal, dtype):
+    """The reference dispatches the operator over float32 and float64 too
+    (attention_kernel.cu:269-281); here such q, k, v keep their storage and
+    arithmetic: y, w and the three gradients within 1e-4 (float32) / 1e-12
+    (float64) of the oracle, and w holds exact zeros above the diagonal."""
+    _run(B, L1, L2, NH, H1, H2, causal, dtype, seed=L1 + 2 * L2, scale=0.8)
     if causal:
         g = torch.Generator().manual_seed(1)
-        q = torch.randn(B, L1, NH, H1, generator=g).cuda()
-        k = torch.randn(B, L2, NH, H1, generator=g).cuda()
-        v = torch.randn(B, L2, NH, H2, generator=g).cuda()
+        q = torch.randn(B, L1, NH, H1, generator=g).to(dtype).cuda()
+        k = torch.randn(B, L2, NH, H1, generator=g).to(dtype).cuda()
+        v = torch.randn(B, L2, NH, H2, generator=g).to(dtype).cuda()
         _, w = ops.attention_fwd(q, k, v, 1.0, 0.0, True)
         assert torch.count_nonzero(torch.triu(w, diagonal=L2 - L1 + 1)) == 0
 
@@ -172,11 +174,11 @@ def test_unsupported_cases_fail_loudly():
     q = torch.zeros(1, 8, 1, 8, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match=r"\[0, 1\]"):
         ops.attention_fwd(q, q, q, 1.0, 1.5, True)   # not a probability
-    with pytest.raises(RuntimeError, match="float64"):
-        ops.attention_fwd(q.double(), q.double(), q.double(), 1.0, 0.0, True)
+    with pytest.raises(RuntimeError, match="complex64"):
+        ops.attention_fwd(q.to(torch.complex64), q.to(torch.complex64), q.to(torch.complex64), 1.0, 0.0, True)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.float64])
 @pytest.mark.parametrize("shape,causal", [
     ((2, 3, 300, 300), True), ((1, 2, 100, 260), True), ((4, 64, 512), False), ((1, 1, 1, 40), True),
     ((2, 1, 50, 4100), False),   # rows longer than the register-resident kernels take
@@ -190,7 +192,7 @@ def test_standalone_softmax(shape, causal, dtype):
     x = (2.0 * torch.randn(*shape, generator=g)).to(dtype)
     dy = torch.randn(*shape, generator=g).to(dtype)
     L1, L2 = shape[-2], shape[-1]
-    xd = x.double().requires_grad_(True)
+    xd = x.clone().double().requires_grad_(True)   # its own leaf, also when x is float64 already
     if causal:
         r = torch.arange(L1).view(L1, 1)
         c = torch.arange(L2).view(1, L2)
@@ -200,7 +202,7 @@ def test_standalone_softmax(shape, causal, dtype):
     want.backward(dy.double())
     xg = x.cuda().requires_grad_(True)
     y = attention_softmax(xg, 0.0, causal, True)
-    tol = TOL_F32 if dtype == torch.float32 else TOL
+    tol = {torch.float32: TOL_F32, torch.float64: TOL_F64}.get(dtype, TOL)
     assert y.dtype == dtype and y.shape == x.shape
     assert rel_err(y, want.detach()) <= tol
     if causal:

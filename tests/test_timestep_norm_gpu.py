@@ -1,6 +1,6 @@
 """Parity of the HIP group TimestepNorm with the float64 oracle (forward values,
 statistics and all gradients).  Tolerances: rel err (max|a-b|/max|b|) <= 1e-4
-in float32, <= 2e-2 in bfloat16."""
+in float32, <= 2e-2 in bfloat16, <= 1e-11 in float64 (the double-precision flavour)."""
 import pytest
 import torch
 
@@ -11,7 +11,7 @@ from megalodon_amd.modules import TimestepNorm
 from oracle import timestep_norm as tn
 
 pytestmark = pytest.mark.gpu
-TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2}
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float64: 1e-11}
 
 
 def _case(B, L, H, G, seed, dtype, prior=0, mask="trailing"):
@@ -46,11 +46,12 @@ def _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed, check_stats_everywhere=Tr
     y, count, mean, var, cummean, cumrstd = ops.group_timestep_norm_fwd(cx, cpc, cpm, cpv, cg, cb, cm, G, eps)
     wy, wcount, wmean, wvar, wcm, wcr = tn.group_timestep_norm_closed_form_full(x, pc, pm, pv, gamma, beta, m, G, eps)
     tol = TOL[dtype]
-    assert y.dtype == dtype and cummean.dtype == torch.float32 and count.dtype == torch.int64
+    stat_dtype = torch.float64 if dtype == torch.float64 else torch.float32   # the accumulate type
+    assert y.dtype == dtype and cummean.dtype == stat_dtype and count.dtype == torch.int64
     assert torch.equal(count.cpu(), wcount)
     assert rel_err(y, wy) <= tol
     assert rel_err(mean, wmean) <= tol and rel_err(var, wvar) <= tol
-    assert rel_err(cummean, wcm) <= 1e-4 and rel_err(cumrstd, wcr) <= 1e-4
+    assert rel_err(cummean, wcm) <= min(tol, 1e-4) and rel_err(cumrstd, wcr) <= min(tol, 1e-4)
     # backward consumes the statistics the forward saved
     dx, dpm, dpv, dg, db = ops.group_timestep_norm_bwd(dy.cuda(), dmean.cuda(), dvar.cuda(), cx, cpm, count,
                                                        cummean, cumrstd, cg, cm, G)
@@ -75,6 +76,16 @@ def _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed, check_stats_everywhere=Tr
 ])
 def test_fwd_bwd_match_oracle(B, L, H, G, prior, mask, dtype):
     _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed=B * 1000 + L)
+
+
+@pytest.mark.parametrize("B,L,H,G,prior,mask", [
+    (2, 200, 512, 4, 3, "trailing"), (3, 300, 384, 3, 5, "holes"), (2, 50, 48, 48, 4, "holes"),
+    (2, 33, 36, 1, 0, None), (1, 40, 1200, 2, 0, "holes"),   # the last: groups wider than 256 features
+])
+def test_float64_tensors(B, L, H, G, prior, mask):
+    """The reference instantiates the operator for double (timestep_norm_kernel.cu:1567-1576,
+    float64 statistics): forward values, statistics and all gradients to 1e-11."""
+    _run_fwd_bwd(B, L, H, G, torch.float64, prior, mask, seed=B * 77 + L)
 
 
 @pytest.mark.parametrize("offset", [8.0, 40.0])
