@@ -76,6 +76,23 @@ int mega_ema_weight_bwd(const float* dw, const float* p, const float* log_q,
                         const float* gamma, int64_t D, int64_t N, int64_t L,
                         float* dp, float* dq, float* dgamma, void* stream);
 
+/* The double-precision flavours of the two operators above and of the causal
+ * convolution (ema_parameters_kernel.cu:1227 dispatches p over float64 with
+ * complex128 log_q / gamma; fftconv_kernel.cu:468-476,487-499 takes float64 x
+ * with complex128 spectra): the defining sums evaluated directly in double --
+ * every power from its own exp / sincos, the convolution as the triangular sum
+ * out[r, t] = sum_{s <= t} a[r % rows_a, s] * b[r, t - s] (rows of L doubles;
+ * a = the kernel rows (D, L), b = x (B*D, L) gives fftconv's y; the two
+ * backward sums are the same convolution of time-reversed rows).  For checking
+ * results, not for speed.  Sizes and layouts as above with double / complex128. */
+int mega_ema_weight_fwd_f64(const double* p, const double* log_q, const double* gamma,
+                            int64_t D, int64_t N, int64_t L, double* w, void* stream);
+int mega_ema_weight_bwd_f64(const double* dw, const double* p, const double* log_q,
+                            const double* gamma, int64_t D, int64_t N, int64_t L,
+                            double* dp, double* dq, double* dgamma, void* stream);
+int mega_causal_conv_f64(const double* a, const double* b, int64_t rows_a, int64_t rows,
+                         int64_t L, double* out, void* stream);
+
 /* ------------------------------------------------------------------------
  * CEMA coefficients from the raw parameters, and their gradients.
  *

@@ -32,10 +32,24 @@ def _require_cuda(*tensors) -> torch.device:
     return dev
 
 
-def _as_c64(t: torch.Tensor, name: str) -> torch.Tensor:
-    if t.dtype != torch.complex64:
-        raise RuntimeError(f"{name} must be complex64 (got {t.dtype})")
+def _as_c64(t: torch.Tensor, name: str, wide: bool = False) -> torch.Tensor:
+    """Contiguous complex64 tensor -- complex128 for the double-precision flavour (`wide`)."""
+    want = torch.complex128 if wide else torch.complex64
+    if t.dtype != want:
+        raise RuntimeError(f"{name} must be {str(want)[6:]} (got {t.dtype})")
     return t.contiguous()
+
+
+def _real_of(wide: bool) -> torch.dtype:
+    return torch.float64 if wide else torch.float32
+
+
+def _p_is_wide(p: torch.Tensor, who: str = "p") -> bool:
+    """p float32 (complex64 companions) or float64 (complex128 companions), as the reference
+    dispatches (ema_parameters_kernel.cu:1227)."""
+    if p.dtype not in (torch.float32, torch.float64):
+        raise RuntimeError(f"{who} must be float32 or float64 (got {p.dtype})")
+    return p.dtype == torch.float64
 
 
 # --------------------------------------------------------------------------
@@ -46,11 +60,12 @@ def _weight_rows(coef: torch.Tensor, log_q_rows: torch.Tensor, L: int) -> torch.
     one complex coefficient per (row, mode) (p = 1, gamma = coef)."""
     R, N = coef.shape
     dev = coef.device
-    ones = torch.ones((R, N), dtype=torch.float32, device=dev)
-    out = torch.empty((R, L), dtype=torch.float32, device=dev)
+    wide = coef.dtype == torch.complex128
+    ones = torch.ones((R, N), dtype=_real_of(wide), device=dev)
+    out = torch.empty((R, L), dtype=_real_of(wide), device=dev)
     cf, lq = coef.contiguous(), log_q_rows.contiguous()
     with torch.cuda.device(dev):
-        _lib.call("mega_ema_weight_fwd", _lib.ptr(ones), _lib.ptr(lq), _lib.ptr(cf), _lib.i64(R),
+        _lib.call("mega_ema_weight_fwd_f64" if wide else "mega_ema_weight_fwd", _lib.ptr(ones), _lib.ptr(lq), _lib.ptr(cf), _lib.i64(R),
                   _lib.i64(N), _lib.i64(L), _lib.ptr(out), _lib.stream_ptr(dev))
     return out
 
@@ -62,22 +77,23 @@ def _row_moments(rows: torch.Tensor, log_q_rows: torch.Tensor) -> Tuple[torch.Te
     R, L = rows.shape
     N = log_q_rows.shape[1]
     dev = rows.device
-    ones = torch.ones((R, N), dtype=torch.float32, device=dev)
-    onec = torch.ones((R, N), dtype=torch.complex64, device=dev)
-    dp = torch.empty((R, N), dtype=torch.float32, device=dev)
-    dq = torch.empty((R, N), dtype=torch.complex64, device=dev)
-    dg = torch.empty((R, N), dtype=torch.complex64, device=dev)
-    rw, lq = rows.contiguous(), log_q_rows.contiguous()
+    wide = log_q_rows.dtype == torch.complex128
+    ones = torch.ones((R, N), dtype=_real_of(wide), device=dev)
+    onec = torch.ones((R, N), dtype=log_q_rows.dtype, device=dev)
+    dp = torch.empty((R, N), dtype=_real_of(wide), device=dev)
+    dq = torch.empty((R, N), dtype=log_q_rows.dtype, device=dev)
+    dg = torch.empty((R, N), dtype=log_q_rows.dtype, device=dev)
+    rw, lq = rows.to(_real_of(wide)).contiguous(), log_q_rows.contiguous()
     with torch.cuda.device(dev):
-        _lib.call("mega_ema_weight_bwd", _lib.ptr(rw), _lib.ptr(ones), _lib.ptr(lq), _lib.ptr(onec),
+        _lib.call("mega_ema_weight_bwd_f64" if wide else "mega_ema_weight_bwd", _lib.ptr(rw), _lib.ptr(ones), _lib.ptr(lq), _lib.ptr(onec),
                   _lib.i64(R), _lib.i64(N), _lib.i64(L), _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg),
                   _lib.stream_ptr(dev))
     return dg.conj().resolve_conj(), dq.conj().resolve_conj()
 
 
 def _qpow(log_q: torch.Tensor, k: int) -> torch.Tensor:
-    """q^k in complex64, evaluated in complex128 (k * arg q loses bits in float32)."""
-    return torch.exp(log_q.to(torch.complex128) * float(k)).to(torch.complex64)
+    """q^k in log_q's precision, evaluated in complex128 (k * arg q loses bits in float32)."""
+    return torch.exp(log_q.to(torch.complex128) * float(k)).to(log_q.dtype)
 
 
 def ema_parameters_fwd(
@@ -89,7 +105,8 @@ def ema_parameters_fwd(
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
     """(w, b, v) = ema_parameters_fwd(p, log_q, gamma, h, L).
 
-    p (D,N[,1]) float32, log_q/gamma complex64 -> w (D, L) float32.  With the
+    p (D,N[,1]) float32, log_q/gamma complex64 -> w (D, L) float32 (float64 /
+    complex128 -> float64: the double-precision flavour).  With the
     carried state ``h`` (B, D, N) complex64 also the bias
     ``b[b,d,j] = sum_n Re(q^(j+1) gamma h[b,d,n])`` (B, D, L)
     (ema_parameters.cc:56-77): the weight kernel run on the B*D rows with the
@@ -97,19 +114,18 @@ def ema_parameters_fwd(
     is never needed and stays ``None``.
     """
     dev = _require_cuda(p, log_q, gamma, h)
-    if p.dtype != torch.float32:
-        raise RuntimeError(f"p must be float32 (got {p.dtype})")
+    wide = _p_is_wide(p)
     D, N = p.shape[0], p.shape[1]
     p_c = p.contiguous()
-    lq = _as_c64(log_q, "log_q")
-    gm = _as_c64(gamma, "gamma")
-    w = torch.empty((D, L), dtype=torch.float32, device=dev)
+    lq = _as_c64(log_q, "log_q", wide)
+    gm = _as_c64(gamma, "gamma", wide)
+    w = torch.empty((D, L), dtype=p.dtype, device=dev)
     with torch.cuda.device(dev):
-        _lib.call("mega_ema_weight_fwd", _lib.ptr(p_c), _lib.ptr(lq), _lib.ptr(gm),
-                  _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(w), _lib.stream_ptr(dev))
+        _lib.call("mega_ema_weight_fwd_f64" if wide else "mega_ema_weight_fwd", _lib.ptr(p_c), _lib.ptr(lq),
+                  _lib.ptr(gm), _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(w), _lib.stream_ptr(dev))
     if h is None:
         return w, None, None
-    hc = _as_c64(h, "h")
+    hc = _as_c64(h, "h", wide)
     if hc.dim() != 3 or hc.shape[1] != D or hc.shape[2] != N:
         raise RuntimeError(f"h must be (B, {D}, {N}) (got {tuple(hc.shape)})")
     B = hc.shape[0]
@@ -132,30 +148,31 @@ def ema_parameters_bwd(
     """(dp, dq, dgamma, dh); gradients w.r.t. q (not log q), PyTorch conjugate
     convention (ema_parameters.cc:80-98; bias part :100-117,158-188)."""
     dev = _require_cuda(w_grad, p, log_q, gamma, h, b_grad)
-    if p.dtype != torch.float32 or w_grad.dtype != torch.float32:
-        raise RuntimeError("p and w_grad must be float32")
+    wide = _p_is_wide(p)
+    if w_grad.dtype != p.dtype:
+        raise RuntimeError(f"p and w_grad must share float32 or float64 (got {p.dtype}, {w_grad.dtype})")
     D, N = p.shape[0], p.shape[1]
     L = w_grad.shape[-1]
     dw = w_grad.contiguous()
     p_c = p.contiguous()
-    lq = _as_c64(log_q, "log_q")
-    gm = _as_c64(gamma, "gamma")
+    lq = _as_c64(log_q, "log_q", wide)
+    gm = _as_c64(gamma, "gamma", wide)
     dp = torch.empty_like(p_c)
     dq = torch.empty_like(lq)
     dg = torch.empty_like(gm)
     with torch.cuda.device(dev):
-        _lib.call("mega_ema_weight_bwd", _lib.ptr(dw), _lib.ptr(p_c), _lib.ptr(lq), _lib.ptr(gm),
+        _lib.call("mega_ema_weight_bwd_f64" if wide else "mega_ema_weight_bwd", _lib.ptr(dw), _lib.ptr(p_c), _lib.ptr(lq), _lib.ptr(gm),
                   _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg),
                   _lib.stream_ptr(dev))
     if b_grad is None:
         return dp, dq, dg, (torch.zeros_like(h) if h is not None else None)
     if h is None:
         raise RuntimeError("ema_parameters_bwd: a bias gradient needs the carried state h")
-    hc = _as_c64(h, "h")
+    hc = _as_c64(h, "h", wide)
     B = hc.shape[0]
     lq2, gm2 = lq.reshape(D, N), gm.reshape(D, N)
     lq_rows = lq2.unsqueeze(0).expand(B, D, N).reshape(B * D, N)
-    s2, s1 = _row_moments(b_grad.reshape(B * D, L).float(), lq_rows)
+    s2, s1 = _row_moments(b_grad.reshape(B * D, L), lq_rows)
     s2, s1 = s2.view(B, D, N), s1.view(B, D, N)
     q = torch.exp(lq2)
     sum2 = q * s2               # sum_i db_i q^(i+1)
@@ -229,17 +246,16 @@ def ema_hidden_fwd(
     ``v`` stacks them (2, B, D, N) in place of the reference's Vandermonde tensor.
     x (B, D, L) any float dtype; p (D,N[,1]) float32; log_q complex64."""
     dev = _require_cuda(x, p, log_q, h)
-    if p.dtype != torch.float32:
-        raise RuntimeError(f"p must be float32 (got {p.dtype})")
+    wide = _p_is_wide(p)
     B, D, L = x.shape
     N = p.shape[1]
-    lq2 = _as_c64(log_q, "log_q").reshape(D, N)
+    lq2 = _as_c64(log_q, "log_q", wide).reshape(D, N)
     lq_rows = lq2.unsqueeze(0).expand(B, D, N).reshape(B * D, N)
-    s2, s1 = _row_moments(x.flip(-1).reshape(B * D, L).float(), lq_rows)
+    s2, s1 = _row_moments(x.flip(-1).reshape(B * D, L), lq_rows)
     s2, s1 = s2.view(B, D, N), s1.view(B, D, N)
     y = p.reshape(D, N) * s2
     if h is not None:
-        y = y + _qpow(lq2, L) * _as_c64(h, "h")
+        y = y + _qpow(lq2, L) * _as_c64(h, "h", wide)
     return y, torch.stack([s2, s1])
 
 
@@ -255,10 +271,11 @@ def ema_hidden_bwd(
     dev = _require_cuda(y_grad, x, p, log_q, h, v)
     B, D, L = x.shape
     N = p.shape[1]
-    lq2 = _as_c64(log_q, "log_q").reshape(D, N)
+    wide = _p_is_wide(p)
+    lq2 = _as_c64(log_q, "log_q", wide).reshape(D, N)
     lq_rows = lq2.unsqueeze(0).expand(B, D, N).reshape(B * D, N)
     p2 = p.reshape(D, N)
-    dyc = torch.conj(_as_c64(y_grad, "y_grad")).resolve_conj()
+    dyc = torch.conj(_as_c64(y_grad, "y_grad", wide)).resolve_conj()
     s2, s1 = v[0], v[1]
     # dx[j] = sum_n Re(conj(dy) p q^(L-1-j)): the weight kernel, then reversed in time
     dx = _weight_rows((dyc * p2).reshape(B * D, N), lq_rows, L).view(B, D, L).flip(-1).to(x.dtype)
@@ -266,7 +283,7 @@ def ema_hidden_bwd(
     dq_sum = (dyc * p2 * s1).sum(dim=0)
     dh = None
     if h is not None:
-        hc = _as_c64(h, "h")
+        hc = _as_c64(h, "h", wide)
         dq_sum = dq_sum + (dyc * hc).sum(dim=0) * _qpow(lq2, L - 1) * float(L)
         dh = torch.conj(dyc * _qpow(lq2, L))
     dq = torch.conj(dq_sum).reshape(log_q.shape)
@@ -350,6 +367,34 @@ def _fftconv_long_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor, bl
     return dx.view(B, D, nb * S)[..., :L].to(x.dtype), dk.view(D, nb * S)[..., :L].contiguous()
 
 
+def _causal_conv_f64(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """out[r, t] = sum_{s <= t} a[r % Ra, s] b[r, t - s] for float64 rows a (Ra, L), b (R, L): the
+    double-precision flavour's convolution, the triangular sum itself (no transform)."""
+    Ra, L = a.shape
+    R = b.shape[0]
+    ac, bc = a.contiguous(), b.contiguous()
+    out = torch.empty_like(bc)
+    with torch.cuda.device(b.device):
+        _lib.call("mega_causal_conv_f64", _lib.ptr(ac), _lib.ptr(bc), _lib.i64(Ra), _lib.i64(R), _lib.i64(L),
+                  _lib.ptr(out), _lib.stream_ptr(b.device))
+    return out
+
+
+def _fftconv_f64_fwd(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
+    B, D, L = x.shape
+    return _causal_conv_f64(k.double(), x.reshape(B * D, L)).view(B, D, L)
+
+
+def _fftconv_f64_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dx[t] = sum_s k[s] dy[t + s] and dk[j] = sum_b sum_t dy[t] x[t - j] are causal
+    convolutions of the time-reversed gradient: flip(conv(k, flip dy)), sum_b flip(conv(x, flip dy))."""
+    B, D, L = x.shape
+    dyr = y_grad.flip(-1).reshape(B * D, L)
+    dx = _causal_conv_f64(k.double(), dyr).flip(-1).view(B, D, L)
+    dk = _causal_conv_f64(x.reshape(B * D, L), dyr).flip(-1).view(B, D, L).sum(dim=0)
+    return dx, dk
+
+
 def fftconv_fwd(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     """y = causal_conv(x, k).  x (B, D, L) float32/bfloat16/float16, k (D, L).
 
@@ -365,6 +410,8 @@ def fftconv_fwd(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     if x.dim() != 3 or k.dim() != 2 or k.shape[0] != x.shape[1] or k.shape[1] != x.shape[2]:
         raise RuntimeError(f"fftconv: x {tuple(x.shape)} and k {tuple(k.shape)} do not match (B,D,L)/(D,L)")
     B, D, L = x.shape
+    if x.dtype == torch.float64:
+        return _fftconv_f64_fwd(x, k)
     if L > fftconv_max_length():
         return _fftconv_long_fwd(x, k)
     xc = x.contiguous()
@@ -387,6 +434,9 @@ def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
     B, D, L = x.shape
     if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
         raise RuntimeError("fftconv_bwd: y_grad must match x in shape and dtype")
+    if x.dtype == torch.float64:
+        dx, dk = _fftconv_f64_bwd(y_grad, x, k)
+        return dx, dk.to(k_dtype)
     if L > fftconv_max_length():
         dx, dk = _fftconv_long_bwd(y_grad, x, k)
         return dx, dk.to(k_dtype)
@@ -415,7 +465,8 @@ def _spectrum_to_row(s: torch.Tensor, L: int, what: str) -> torch.Tensor:
     if not s.is_complex() or s.shape[-1] != M + 1:
         raise RuntimeError(f"fftconv: {what} must be the complex spectrum of {M + 1} bins of rows of length {L}, "
                            f"got {tuple(s.shape)} {s.dtype}")
-    return torch.fft.irfft(s.to(torch.complex64), n=2 * M)[..., :L].contiguous()
+    wide = s.dtype == torch.complex128   # the double-precision flavour keeps its spectra in complex128
+    return torch.fft.irfft(s if wide else s.to(torch.complex64), n=2 * M)[..., :L].contiguous()
 
 
 def _fftconv_fwd_spectral(x: torch.Tensor, k_f: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -423,6 +474,8 @@ def _fftconv_fwd_spectral(x: torch.Tensor, k_f: torch.Tensor) -> Tuple[torch.Ten
     L = x.shape[-1]
     M = 1 << max(0, (L - 1).bit_length())
     y = fftconv_fwd(x, _spectrum_to_row(k_f, L, "k_f"))
+    if x.dtype == torch.float64:
+        return y, torch.fft.rfft(x, n=2 * M)
     x_f = rfft(x, False) if 32 <= M <= 16384 else torch.fft.rfft(x.float(), n=2 * M)
     return y, x_f
 
@@ -445,6 +498,8 @@ def fftconv_residual_fwd(x: torch.Tensor, k: torch.Tensor, omega: torch.Tensor) 
     if omega.numel() != x.shape[1]:
         raise RuntimeError(f"fftconv: omega has {omega.numel()} elements for D={x.shape[1]}")
     B, D, L = x.shape
+    if x.dtype == torch.float64:
+        return _fftconv_f64_fwd(x, k) + x * omega.reshape(-1, 1).double()
     if L > fftconv_max_length():  # blocks, then the skip term in float32
         y = _fftconv_long_fwd(x, k).float() + x.float() * omega.reshape(-1, 1).float()
         return y.to(x.dtype)
@@ -467,6 +522,9 @@ def fftconv_residual_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
     B, D, L = x.shape
     if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
         raise RuntimeError("fftconv_bwd: y_grad must match x in shape and dtype")
+    if x.dtype == torch.float64:
+        dx, dk = _fftconv_f64_bwd(y_grad, x, k)
+        return dx + y_grad * omega.reshape(-1, 1).double(), dk, dk[:, 0].clone()
     if L > fftconv_max_length():
         dx, dk = _fftconv_long_bwd(y_grad, x, k)
         dx = (dx.float() + y_grad.float() * omega.reshape(-1, 1).float()).to(x.dtype)
