@@ -348,6 +348,16 @@ int mega_attention_bwd(const void* dy, const void* q, const void* k, const void*
                        int64_t NH, int64_t H1, int64_t H2, double scale, int causal,
                        void* dq, void* dk, void* dv, void* workspace, void* stream);
 
+/* dw[o][i] = sum_t dy[t][o] * x[t][i]: the weight gradient of y = x W^T for dy
+ * (tokens, n_out) and x (tokens, n_in), dw (n_out, n_in), all of `dtype`
+ * (MEGA_BF16 / MEGA_F16, float32 accumulation), contiguous, on the attention
+ * operator's product kernel (both operands run across the reduction axis, as in
+ * dV = P^T dY).  Replaces the `grad_output.t().matmul(input)` of the linear layers'
+ * autograd (megalodon/modules/model_parallel/layers.py:222-235,321-341 are
+ * F.linear at model-parallel world size 1). */
+int mega_linear_weight_grad(const void* dy, const void* x, int dtype, int64_t tokens,
+                            int64_t n_out, int64_t n_in, void* dw, void* stream);
+
 /* ------------------------------------------------------------------------
  * Convolution with spectra kept between forward and backward.
  *

@@ -1218,6 +1218,26 @@ extern "C" int mega_attention_bwd(const void* dy, const void* q, const void* k, 
                                  (float)scale, causal, m(dq), m(dk), m(dv), m(workspace), s);
 }
 
+// ---- the weight gradient of a linear layer on the same product kernel ---------------
+extern "C" int mega_linear_weight_grad(const void* dy, const void* x, int dtype, int64_t tokens, int64_t n_out,
+                                       int64_t n_in, void* dw, void* stream) {
+  MEGA_CHECK_ARG(dtype == MEGA_BF16 || dtype == MEGA_F16, "mega_linear_weight_grad: bfloat16 or float16 tensors");
+  MEGA_CHECK_ARG(tokens >= 1 && n_out >= 1 && n_in >= 1 && tokens < (1ll << 31) && n_out < (1ll << 31) &&
+                     n_in < (1ll << 31),
+                 "mega_linear_weight_grad: bad sizes");
+  MEGA_CHECK_ARG(dy && x && dw, "mega_linear_weight_grad: null pointer");
+  // dw[o][i] = sum_t dy[t][o] x[t][i]: both operands k-major (k = tokens)
+  GemmParams g{};
+  g.A = static_cast<const uint16_t*>(dy);
+  g.B = static_cast<const uint16_t*>(x);
+  g.C = static_cast<uint16_t*>(dw);
+  g.M = (int)n_out; g.N = (int)n_in; g.K = (int)tokens;
+  g.lda = n_out; g.ldb = n_in; g.ldc = n_in; g.ta = 1; g.tb = 1;
+  g.nh = 1; g.alpha = 1.f;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return dtype == MEGA_BF16 ? launch_gemm<MEGA_BF16>(g, 1, s) : launch_gemm<MEGA_F16>(g, 1, s);
+}
+
 // ---- standalone causal softmax ---------------------------------------------------
 static int check_softmax(const char* who, int dtype, int64_t Z, int64_t L1, int64_t L2, int causal) {
   MEGA_CHECK_ARG(valid_dtype(dtype) || dtype == MEGA_F64, "%s: unknown dtype %d", who, dtype);

@@ -1005,6 +1005,20 @@ def attention_bwd(y_grad: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: tor
     return dq, dk, dv
 
 
+def linear_weight_grad(y_grad: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """dW (out, in) = y_grad^T x for y_grad (tokens, out), x (tokens, in), bfloat16 / float16:
+    the weight gradient of a linear layer on the attention operator's product kernel."""
+    dev = _require_cuda(y_grad, x)
+    if y_grad.dim() != 2 or x.dim() != 2 or y_grad.shape[0] != x.shape[0] or y_grad.dtype != x.dtype:
+        raise RuntimeError("linear_weight_grad: y_grad (tokens, out) and x (tokens, in) of one dtype")
+    g, xc = y_grad.contiguous(), x.contiguous()
+    dw = torch.empty((g.shape[1], xc.shape[1]), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("mega_linear_weight_grad", _lib.ptr(g), _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
+                  _lib.i64(g.shape[0]), _lib.i64(g.shape[1]), _lib.i64(xc.shape[1]), _lib.ptr(dw), _lib.stream_ptr(dev))
+    return dw
+
+
 def _softmax_dims(x: torch.Tensor):
     if x.dim() < 2:
         raise RuntimeError("attention_softmax: x needs at least two dimensions")

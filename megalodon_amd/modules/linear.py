@@ -6,8 +6,8 @@ backward forms `dx = dy @ W` with W (out, in) read along its rows.  On MI355X
 the library GEMM is 13-24 % faster when both operands run along the reduction
 axis (`dy @ Wt^T` with Wt = W^T contiguous, the same layout the forward
 `x @ W^T` uses), and the tiled transpose of W costs 15-30 us, so the backward
-makes that copy; the weight gradient of the large layers likewise copies one
-operand into its transpose (`_weight_grad`).  Values are those of `F.linear`;
+makes that copy; the weight gradient of the large layers runs on the attention
+operator's product kernel (`_weight_grad`).  Values are those of `F.linear`;
 parameters keep the names and shapes of `nn.Linear`, so state dicts are
 interchangeable."""
 from typing import Optional, Tuple
@@ -22,16 +22,17 @@ from .. import extension as megalodon_ops
 
 def _weight_grad(g2: torch.Tensor, x2: torch.Tensor) -> torch.Tensor:
     """dW = g2^T x2, (out, in) from (tokens, out) and (tokens, in).  Both operands run across
-    the reduction axis (tokens) here, the slowest layout of the library GEMM on MI355X: with one
-    of them copied into its transpose it measured 8-15 % faster at 32768 tokens (out x in =
-    8192 x 4096: 1.85 -> 1.58 ms, 11008 x 4096: 3.22 -> 3.01 ms, 4096 x 11008: 3.17 -> 2.86 ms),
-    and the tiled transpose of the operand with fewer columns costs 0.12 ms.  Small layers
-    (4096 x 4096: 0.93 -> 0.79 + 0.12 ms; 1024 x 4096: slower) keep the plain form."""
+    the reduction axis (tokens) here, the slowest layout of the library GEMM on MI355X
+    (0.9-1.2 PFLOP/s at 32768 tokens against 1.5 for the forward's layout).  The attention
+    operator's product kernel takes exactly this layout (dV = P^T dY) and measured, at 32768
+    tokens, out x in = 11008 x 4096: 2.16 ms against 3.28 (3.16 with one operand transposed
+    first), 4096 x 11008: 2.22 / 3.13, 8192 x 4096: 1.54 / 1.87, 4096 x 4096: 0.78 / 0.92;
+    below one 256 x 256 tile per compute unit (1024 x 4096: 0.50 / 0.28 ms) the library stays."""
     n_out, n_in = g2.shape[1], x2.shape[1]
-    if g2.shape[0] >= 8192 and min(n_out, n_in) >= 2048 and max(n_out, n_in) >= 8192:
-        if n_in <= n_out:
-            return g2.t() @ megalodon_ops.transpose_last2(x2).t()
-        return megalodon_ops.transpose_last2(g2) @ x2
+    tiles = ((n_out + 255) // 256) * ((n_in + 255) // 256)
+    if (g2.dtype in (torch.bfloat16, torch.float16) and g2.shape[0] >= 4096 and g2.shape[0] % 32 == 0
+            and n_out % 8 == 0 and n_in % 8 == 0 and tiles >= 256):
+        return megalodon_ops.linear_weight_grad(g2, x2)
     return g2.t() @ x2
 
 
