@@ -68,6 +68,54 @@ class LinearFunc(torch.autograd.Function):
         return dx, dw, db, (y_grad if ctx.has_residual and ctx.needs_input_grad[3] else None)
 
 
+class LinearGroupFunc(torch.autograd.Function):
+    """Several bias-optional linear layers of one input: (y_1, ..., y_n) = (x W_1^T + b_1, ...).
+    The forward is n separate products; the backward forms the input gradient as one
+    accumulation -- dx = dy_1 W_1, then dx += dy_i W_i inside the GEMM (`addmm_`) -- instead of n
+    gradients that autograd adds up with n - 1 passes over the activation."""
+
+    @staticmethod
+    def forward(ctx: FunctionCtx, x: torch.Tensor, *params: Optional[torch.Tensor]):
+        weights, biases = params[0::2], params[1::2]
+        ctx.save_for_backward(x, *weights)
+        ctx.has_bias = [b is not None for b in biases]
+        return tuple(F.linear(x, w, b) for w, b in zip(weights, biases))
+
+    @staticmethod
+    def backward(ctx: FunctionCtx, *y_grads: torch.Tensor):
+        x, *weights = ctx.saved_tensors
+        x2 = x.reshape(-1, x.shape[-1])
+        dx = None
+        grads = []
+        for i, (w, g) in enumerate(zip(weights, y_grads)):
+            g2 = g.reshape(-1, g.shape[-1])
+            if ctx.needs_input_grad[0]:
+                wt = megalodon_ops.transpose_last2(w)      # (in, out), rows along the reduction axis
+                if dx is None:
+                    dx = F.linear(g2, wt)
+                else:
+                    dx.addmm_(g2, wt.t())
+            dw = _weight_grad(g2, x2) if ctx.needs_input_grad[1 + 2 * i] else None
+            db = g2.sum(0) if ctx.has_bias[i] and ctx.needs_input_grad[2 + 2 * i] else None
+            grads += [dw, db]
+        return (None if dx is None else dx.view(x.shape), *grads)
+
+
+def linear_group(x: torch.Tensor, layers) -> Tuple[torch.Tensor, ...]:
+    """`tuple(layer(x) for layer in layers)` for `Linear` layers that read the same input; on the
+    GPU in 16 bits with gradients enabled their backward shares one input-gradient accumulation."""
+    layers = list(layers)
+    fused = (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and torch.is_grad_enabled()
+             and all(l.weight.dtype == x.dtype for l in layers)
+             and (x.requires_grad or any(l.weight.requires_grad for l in layers)))
+    if not fused or len(layers) < 2:
+        return tuple(l(x) for l in layers)
+    params = []
+    for l in layers:
+        params += [l.weight, l.bias]
+    return LinearGroupFunc.apply(x, *params)
+
+
 class Linear(nn.Linear):
     """Drop-in for `nn.Linear` (same parameters, same values); `residual`, for
     layers without bias, is added inside the GEMM."""

@@ -21,7 +21,7 @@ from .. import extension as megalodon_ops
 from ..fused_ops import memory_efficient_dropout, qk_norm_rotary, silu_mul, transpose_last2
 from .chunk_attention import _InnerAttention
 from .complex_exponential_moving_average import MultiHeadComplexEMA
-from .linear import Linear
+from .linear import Linear, linear_group
 from .layer_norm import FusedRMSNorm
 from .normalized_feedforward_network import NormalizedFeedForwardNetwork
 from .timestep_norm import TimestepNorm
@@ -89,7 +89,8 @@ class MovingAverageGatedAttention(nn.Module):
         mx = self.rmsnorm(out_cema)
         mx = memory_efficient_dropout(mx, self.hidden_dropout, self.training)
 
-        z = self.wz(mx)
+        # the three projections of mx: one accumulation of its gradient in the backward
+        z, r, h1 = linear_group(mx, (self.wz, self.wr, self.wh1))
         if (not self.znorm.elementwise_affine
                 and megalodon_ops.qk_norm_rotary_supported(z, self.gamma, self.z_head_dim)
                 and (freqs_cis is None or freqs_cis.shape[0] == min(seq_len, self.chunk_size))):
@@ -108,14 +109,13 @@ class MovingAverageGatedAttention(nn.Module):
 
         # B x L x E
         v = F.silu(self.wv(out_tsn))
-        r = self.wr(mx)
 
         attn, cache_attn = self.inner_attention(q.contiguous(), k.contiguous(), v, mask, freqs_cis, cache_attn)
         # attn * silu(r) in one pass
         attn = memory_efficient_dropout(silu_mul(r, attn), self.hidden_dropout, self.training)
 
         # B x L x E -> B x L x D
-        h = self.wh2(attn, residual=self.wh1(mx))   # wh1(mx) + wh2(attn), the sum formed inside the GEMM
+        h = self.wh2(attn, residual=h1)   # wh1(mx) + wh2(attn), the sum formed inside the GEMM
         h = memory_efficient_dropout(h, self.dropout, self.training)
         out = h + residual
         if cache is not None:

@@ -7,7 +7,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from ..fused_ops import memory_efficient_dropout, silu_mul
-from .linear import Linear
+from .linear import Linear, linear_group
 from .layer_norm import FusedLayerNorm
 
 
@@ -40,7 +40,7 @@ class NormalizedFeedForwardNetwork(nn.Module):
     def forward(self, x, residual):
         x = self.norm(x)
         if self.swiglu:
-            hidden = silu_mul(self.fc1(x), self.fc3(x))
+            hidden = silu_mul(*linear_group(x, (self.fc1, self.fc3)))
         else:
             hidden = F.silu(self.fc1(x))
         hidden = memory_efficient_dropout(hidden, self.hidden_dropout, self.training)

@@ -166,6 +166,39 @@ def test_empty_inputs_are_accepted():
     assert q.shape == (2, 0, 512) and k.shape == (2, 0, 512)
 
 
+def test_linear_group_matches_float64_and_separate_layers():
+    """Layers that read one input (`linear_group`): outputs are those of the layers one by one,
+    and the shared input gradient, accumulated inside the GEMM, and every parameter gradient
+    match float64 (2e-2, bfloat16)."""
+    from megalodon_amd.modules.linear import Linear, linear_group
+    torch.manual_seed(3)
+    layers = [Linear(256, 512, bias=True), Linear(256, 72, bias=False), Linear(256, 256, bias=True)]
+    layers = [l.cuda().bfloat16() for l in layers]
+    x = torch.randn(3, 100, 256, device="cuda").bfloat16().requires_grad_(True)
+    dys = [torch.randn(3, 100, l.out_features, device="cuda").bfloat16() for l in layers]
+    ys = linear_group(x, layers)
+    with torch.no_grad():
+        for y, l in zip(ys, layers):
+            assert torch.equal(y, l(x))
+    torch.autograd.backward(ys, dys)
+    x64 = x.detach().double().requires_grad_(True)
+    w64 = [l.weight.detach().double().requires_grad_(True) for l in layers]
+    b64 = [None if l.bias is None else l.bias.detach().double().requires_grad_(True) for l in layers]
+    torch.autograd.backward([F.linear(x64, w, b) for w, b in zip(w64, b64)], [d.double() for d in dys])
+    assert rel_err(x.grad, x64.grad) <= 2e-2
+    for l, w, b in zip(layers, w64, b64):
+        assert rel_err(l.weight.grad, w.grad) <= 2e-2
+        if b is not None:
+            assert rel_err(l.bias.grad, b.grad) <= 2e-2
+    # one output unused downstream: its gradient is taken as zero
+    x.grad = None
+    y0, _, _ = linear_group(x, layers)
+    y0.backward(dys[0])
+    x64.grad = None
+    F.linear(x64, w64[0], b64[0]).backward(dys[0].double())
+    assert rel_err(x.grad, x64.grad) <= 2e-2
+
+
 def test_linear_with_residual_inside_the_gemm():
     from megalodon_amd.modules.linear import Linear
     torch.manual_seed(4)
