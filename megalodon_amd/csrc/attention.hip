@@ -111,6 +111,9 @@ struct GemmParams {
   int per_batch;           // work items per batch index
   int items;               // per_batch * batch
   int ta, tb;   // operand is k-major: element (m, k) at [k * ld + m]
+  int n_group;  // plain schedule: tiles numbered n fastest inside bands of n_group column tiles, then m,
+                // then band (0: one band) -- the 32 tiles an XCD works on at a time then share fewer
+                // distinct operand blocks (4 x 8 instead of 2 x 16 of a 16-column problem)
 };
 
 template <bool ALIGNED>
@@ -545,8 +548,16 @@ __global__ __launch_bounds__(2 * kThreads) void gemm_dma_kernel(const GemmParams
     mt_first = p.mt_count - 1 - pr;
     if (mt_first != pr) mt_second = pr;
   } else {
-    nt = rem % p.nt_count;
-    mt_first = rem / p.nt_count;
+    if (p.n_group > 0) {
+      const int band = p.n_group * p.mt_count;       // tiles of a full band
+      const int b0 = rem / band, r2 = rem % band;
+      const int w = min(p.n_group, p.nt_count - b0 * p.n_group);  // the last band may be narrower
+      nt = b0 * p.n_group + r2 % w;
+      mt_first = r2 / w;
+    } else {
+      nt = rem % p.nt_count;
+      mt_first = rem / p.nt_count;
+    }
   }
   const int z0 = zz / p.nh, z1 = zz % p.nh;
   const uint16_t* A = p.A + z0 * p.sa0 + z1 * p.sa1;
@@ -1234,6 +1245,8 @@ extern "C" int mega_linear_weight_grad(const void* dy, const void* x, int dtype,
   g.M = (int)n_out; g.N = (int)n_in; g.K = (int)tokens;
   g.lda = n_out; g.ldb = n_in; g.ldc = n_in; g.ta = 1; g.tb = 1;
   g.nh = 1; g.alpha = 1.f;
+  const char* ng = getenv("MEGA_GEMM_NGROUP");
+  g.n_group = ng != nullptr ? atoi(ng) : 8;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return dtype == MEGA_BF16 ? launch_gemm<MEGA_BF16>(g, 1, s) : launch_gemm<MEGA_F16>(g, 1, s);
 }
