@@ -762,6 +762,260 @@ __global__ __launch_bounds__(2 * kThreads) void gemm_dma_kernel(const GemmParams
   }  // work item
 }
 
+// ---- the same with slabs of 64 k, for products of two k-contiguous operands ---------------
+// With slabs of 32 k a k-contiguous operand arrives as 64-byte pieces of its rows, half a
+// cache line each, sixteen lines per request; the products with such operands keep the matrix
+// pipe 55-57 % busy where the one with two k-major operands (whole 512-byte rows) reaches 86 %.
+// Here a slab is 64 k: k-contiguous rows come as whole 128-byte lines (1 KB = 8 rows, the chunk at
+// position c of row r holds k chunk c ^ ((r >> 1) & 7)), k-major slabs would be 64 rows of k.
+// Two slab buffers of 64 KB; slab s + 2 is requested into the buffer of slab s after the barrier
+// that ends its reads, under the last of the slab's four k-steps.  Measured in one run at the
+// attention benchmark shape: dP = dY V^T 1.15-1.27 -> 1.02-1.06 ms, forward / backward of the
+// operator 1.436 / 2.59 -> 1.425 / 2.52 ms; with one k-major operand (PV, dQ) the forward was 1 %
+// slower than with slabs of 32, so only the products of two k-contiguous operands come here (the
+// template covers the other layouts; they are not instantiated).
+constexpr int kSlab64 = 64;
+constexpr int kDma64Operand = kTile * kSlab64;  // elements of an operand slab (32 KB)
+constexpr int kDma64Stage = 2 * kDma64Operand;
+static_assert(sizeof(uint16_t) * 2 * kDma64Stage <= kDmaLds, "two slab buffers fit");
+
+template <int DT, bool TA, bool TB>
+__global__ __launch_bounds__(2 * kThreads) void gemm_dma64_kernel(const GemmParams p) {
+  extern __shared__ __align__(16) uint16_t smem[];
+  constexpr int JN = 2, NL = 4, EP = 64 + 8;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wm = wave >> 2, wn = wave & 3;
+  const int G = static_cast<int>(gridDim.x), lin = static_cast<int>(blockIdx.x);
+  int it_lo, it_hi, it_step;
+  if (G % kXcds == 0) {
+    const int xcd = lin % kXcds;
+    it_lo = static_cast<int>(static_cast<int64_t>(p.items) * xcd / kXcds) + lin / kXcds;
+    it_hi = static_cast<int>(static_cast<int64_t>(p.items) * (xcd + 1) / kXcds);
+    it_step = G / kXcds;
+  } else {
+    it_lo = lin;
+    it_hi = p.items;
+    it_step = G;
+  }
+  for (int item = it_lo; item < it_hi; item += it_step) {
+  const int zz = item / p.per_batch;
+  const int rem = item % p.per_batch;
+  int nt, mt_first, mt_second = -1;
+  if (p.tri_out) {
+    int t = rem, m = 0;
+    while (true) {
+      const int cnt = min(p.nt_count, (m * kTile + (kTile - 1) + p.off) / kTile + 1);
+      if (t < cnt) break;
+      t -= cnt;
+      ++m;
+    }
+    mt_first = m;
+    nt = t;
+  } else if (p.k_mode) {
+    nt = rem % p.nt_count;
+    const int pr = rem / p.nt_count;
+    mt_first = p.mt_count - 1 - pr;
+    if (mt_first != pr) mt_second = pr;
+  } else {
+    nt = rem % p.nt_count;
+    mt_first = rem / p.nt_count;
+  }
+  const int z0 = zz / p.nh, z1 = zz % p.nh;
+  const uint16_t* A = p.A + z0 * p.sa0 + z1 * p.sa1;
+  const uint16_t* B = p.B + z0 * p.sb0 + z1 * p.sb1;
+  uint16_t* C = p.C + z0 * p.sc0 + z1 * p.sc1;
+  for (int half = 0; half < 2; ++half) {
+  const int mt = half == 0 ? mt_first : mt_second;
+  if (mt < 0) break;
+  const int m0 = mt * kTile, n0 = nt * kTile;
+  // k range as in gemm_kernel, widened to whole slabs of 64 (K % 64 == 0): what the wider range
+  // adds are probabilities the softmax has written as zeros
+  int kb = 0, ke = p.K;
+  if (p.k_mode == 1) ke = min(p.K, ((mt + 1) * kTile + p.off + kSlab64 - 1) / kSlab64 * kSlab64);
+  if (p.k_mode == 2) kb = min(p.K, max(0, mt * kTile - p.off) / kSlab64 * kSlab64);
+  const int nslab = (ke - kb + kSlab64 - 1) / kSlab64;
+
+  floatx16 acc[4][JN];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < JN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // memory side: wave w sends the 1 KB pieces w, w + 8, w + 16, w + 24 of each operand slab
+  uint32_t offa[NL], offb[NL];
+#pragma unroll
+  for (int i = 0; i < NL; ++i) {
+    const int pc = wave + 8 * i;
+    const int krow = 2 * pc + (lane >> 5), cm = (lane & 31) ^ ((krow & 3) << 2);   // k-major piece: 2 rows of k
+    const int row = 8 * pc + (lane >> 3), ck = (lane & 7) ^ ((row >> 1) & 7);      // k-contiguous piece: 8 rows
+    if (TA) offa[i] = static_cast<uint32_t>(((kb + krow) * p.lda + min(m0 + cm * 8, p.M - 8)) * 2);
+    else offa[i] = static_cast<uint32_t>((static_cast<int64_t>(min(m0 + row, p.M - 1)) * p.lda + kb + ck * 8) * 2);
+    if (TB) offb[i] = static_cast<uint32_t>(((kb + krow) * p.ldb + min(n0 + cm * 8, p.N - 8)) * 2);
+    else offb[i] = static_cast<uint32_t>((static_cast<int64_t>(min(n0 + row, p.N - 1)) * p.ldb + kb + ck * 8) * 2);
+  }
+  const uint32_t stepa = static_cast<uint32_t>((TA ? p.lda : 1) * kSlab64 * 2);
+  const uint32_t stepb = static_cast<uint32_t>((TB ? p.ldb : 1) * kSlab64 * 2);
+  const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)(smem))) + wave * 1024);
+  // request number n of a slab: even n the pieces of A, odd n those of B
+  auto request_one = [&](int s, int stage, int n) {
+    const uint32_t sc = static_cast<uint32_t>(min(s, nslab - 1));
+    const uint32_t dst = lds_wave + static_cast<uint32_t>(stage * kDma64Stage + (n >> 1) * 8 * 512 + (n & 1) * kDma64Operand) * 2;
+    if (n & 1) load_to_lds16(B, offb[n >> 1] + sc * stepb, dst);
+    else load_to_lds16(A, offa[n >> 1] + sc * stepa, dst);
+  };
+  auto request = [&](int s, int stage) {
+#pragma unroll
+    for (int n = 0; n < 2 * NL; ++n) request_one(s, stage, n);
+  };
+
+  // fragment side: k-step `set` (0 .. 3) of a slab takes k = 16 set + 8 g + e for lane half g
+  const int g = lane >> 5, r = lane & 31;
+  const int ta_a = (lane & 15) >> 2, ta_h = (lane >> 4) & 1, ta_b = lane & 3;
+  int fra[4], frb[JN];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (TA) fra[i] = (8 * g + ta_a) * kTile + (((wm * 16 + 4 * i + 2 * ta_h + (ta_b >> 1)) ^ (ta_a << 2)) * 8) + 4 * (ta_b & 1);
+    else fra[i] = (wm * 128 + 32 * i + r) * kSlab64 + ((g ^ ((r >> 1) & 7)) * 8);
+  }
+#pragma unroll
+  for (int j = 0; j < JN; ++j) {
+    if (TB) frb[j] = kDma64Operand + (8 * g + ta_a) * kTile + (((wn * 8 + 4 * j + 2 * ta_h + (ta_b >> 1)) ^ (ta_a << 2)) * 8) + 4 * (ta_b & 1);
+    else frb[j] = kDma64Operand + (wn * 64 + 32 * j + r) * kSlab64 + ((g ^ ((r >> 1) & 7)) * 8);
+  }
+  u32x4 fa0[4], fb0[JN], fa1[4], fb1[JN];
+  // fragments lo .. hi - 1 of a k-step: number i = row block i of A and, for i < JN, column block i of B
+  auto fread = [&](u32x4* fa, u32x4* fb, int set, int stage, int lo = 0, int hi = 4) {
+    const uint16_t* base = smem + stage * kDma64Stage;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (i < lo || i >= hi) continue;
+      if (TA) {
+        const uint16_t* q = base + fra[i] + set * 16 * kTile;
+        const uint2 lo = lds_read_tr(q), hi = lds_read_tr(q + 4 * kTile);
+        fa[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+      } else {
+        // chunk 2 set + g sits at position (2 set + g) ^ swizzle = (g ^ swizzle) ^ (2 set)
+        fa[i] = *reinterpret_cast<const u32x4*>(base + (fra[i] ^ (set * 16)));
+      }
+      if (i < JN) {
+        if (TB) {
+          const uint16_t* q = base + frb[i] + set * 16 * kTile;
+          const uint2 lo = lds_read_tr(q), hi = lds_read_tr(q + 4 * kTile);
+          fb[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        } else {
+          fb[i] = *reinterpret_cast<const u32x4*>(base + (frb[i] ^ (set * 16)));
+        }
+      }
+    }
+  };
+  auto mma = [&](const u32x4* fa, const u32x4* fb, int lo, int hi) {
+#pragma unroll
+    for (int n = 0; n < 4 * JN; ++n)
+      if (n >= lo && n < hi) acc[n >> 1][n & 1] = Mma<DT>::run(fb[n & 1], fa[n >> 1], acc[n >> 1][n & 1]);
+  };
+
+  // One step per slab of 64 k = four k-steps; the fragments of the next k-step are read under the
+  // products of the current one.  Before the last k-step: this wave's pieces of the next slab have
+  // landed (nothing else of its requests is in flight) and its reads of this slab have returned;
+  // barrier; then the first fragments of the next slab, the requests for the slab after it into
+  // the buffer just left (one per product), the last 8 products.
+#define MEGA_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+  constexpr int kFragReads = (TA ? 2 : 1) + (TB ? JN / 2 : (JN + 3) / 4);
+#define MEGA_DMA64_KSTEP(FA, FB, NFA, NFB, SET, STAGE)                     \
+  {                                                                        \
+    fread(NFA, NFB, (SET) + 1, (STAGE));                                   \
+    mma(FA, FB, 0, 8);                                                     \
+    _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
+      MEGA_SGB(0x008, 1);                                                  \
+      MEGA_SGB(0x100, kFragReads);                                         \
+    }                                                                      \
+    MEGA_SGB(0x008, 4);                                                    \
+    __builtin_amdgcn_sched_barrier(0);                                     \
+  }
+#define MEGA_DMA64_STEP(R)                                                 \
+  {                                                                        \
+    const int cur = it + (R);                                              \
+    MEGA_DMA64_KSTEP(fa0, fb0, fa1, fb1, 0, (R))                           \
+    MEGA_DMA64_KSTEP(fa1, fb1, fa0, fb0, 1, (R))                           \
+    MEGA_DMA64_KSTEP(fa0, fb0, fa1, fb1, 2, (R))                           \
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); \
+    _Pragma("unroll") for (int n = 0; n < 2 * NL; ++n) {                   \
+      if (n < 4) fread(fa0, fb0, 0, (R) ^ 1, n, n + 1);                    \
+      request_one(cur + 2, (R), n);                                        \
+      mma(fa1, fb1, n, n + 1);                                             \
+      __builtin_amdgcn_sched_barrier(0);                                   \
+    }                                                                      \
+  }
+  if (nslab > 0) {
+    request(0, 0);
+    request(1, 1);
+    asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+    fread(fa0, fb0, 0, 0);
+    int it = 0;
+    for (; it + 2 <= nslab; it += 2) {
+      MEGA_DMA64_STEP(0)
+      MEGA_DMA64_STEP(1)
+    }
+    if (it < nslab) MEGA_DMA64_STEP(0)
+    // nothing may land in the buffers once they hold the output tiles
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  }
+#undef MEGA_DMA64_STEP
+#undef MEGA_DMA64_KSTEP
+#undef MEGA_SGB
+
+  // epilogue as in gemm_kernel: the wave's 128 x 64 tile through its own LDS region
+  uint16_t* stage = smem + wave * 128 * EP;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < JN; ++j) {
+      const int row = i * 32 + (lane & 31);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int col = j * 32 + 8 * q4 + 4 * (lane >> 5);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[i][j][4 * q4 + e];
+        uint2 w;
+        if (DT == MEGA_BF16) {
+          w.x = pack_bf16x2(v[0], v[1]);
+          w.y = pack_bf16x2(v[2], v[3]);
+        } else {
+          w.x = static_cast<uint32_t>(float_to_f16_bits(v[0])) | (static_cast<uint32_t>(float_to_f16_bits(v[1])) << 16);
+          w.y = static_cast<uint32_t>(float_to_f16_bits(v[2])) | (static_cast<uint32_t>(float_to_f16_bits(v[3])) << 16);
+        }
+        *reinterpret_cast<uint2*>(stage + row * EP + col) = w;
+      }
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  const bool vec_ok = (p.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+#pragma unroll 4
+  for (int i = 0; i < 8 * JN; ++i) {
+    const int c = lane + kWave * i;
+    const int row = c / (4 * JN), kc = (c % (4 * JN)) * 8;
+    const int grow = m0 + wm * 128 + row, gcol = n0 + wn * (32 * JN) + kc;
+    if (grow < p.M && gcol < p.N) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * EP + kc);
+      uint16_t* dst = C + static_cast<int64_t>(grow) * p.ldc + gcol;
+      if (vec_ok && gcol + 8 <= p.N) {
+        *reinterpret_cast<u32x4*>(dst) = v;
+      } else {
+        const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+        for (int q = 0; q < 8; ++q)
+          if (gcol + q < p.N) dst[q] = e[q];
+      }
+    }
+  }
+  lds_barrier();
+  }  // tile of the pair
+  }  // work item
+}
+
 // ---- causal softmax over rows (in place), one wavefront per row ---------------
 // `coff` < 0: every row keeps all L2 columns.  `coff` = L2 - L1 >= 0 (causal,
 // bottom-right aligned, softmax.cuh:99-100): row r keeps columns [0, n) with
@@ -1006,7 +1260,20 @@ int launch_gemm_t(const GemmParams& p, int batch, hipStream_t s) {
   const char* w4 = getenv("MEGA_GEMM_W4");
   // MEGA_GEMM_DMA=0 keeps the slabs on the register path (for comparison)
   const char* dma = getenv("MEGA_GEMM_DMA");
-  if (fast && !(w4 != nullptr && w4[0] == '1') && !(dma != nullptr && dma[0] == '0')) {
+  // products of two k-contiguous operands (S = Q K^T, dP = dY V^T) take slabs of 64 k;
+  // MEGA_GEMM_SLAB64=0 keeps slabs of 32 k for every product
+  const char* s64 = getenv("MEGA_GEMM_SLAB64");
+  bool slab64 = false;
+  if constexpr (!TA && !TB)
+    slab64 = fast && p.K % kSlab64 == 0 && !(w4 != nullptr && w4[0] == '1') && !(dma != nullptr && dma[0] == '0') &&
+             !(s64 != nullptr && s64[0] == '0');
+  if (slab64) {
+    if constexpr (!TA && !TB) {
+      MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma64_kernel<DT, TA, TB>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaLds));
+      gemm_dma64_kernel<DT, TA, TB><<<grid, 2 * kThreads, kDmaLds, s>>>(q);
+    }
+  } else if (fast && !(w4 != nullptr && w4[0] == '1') && !(dma != nullptr && dma[0] == '0')) {
     MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<DT, TA, TB>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaLds));
     gemm_dma_kernel<DT, TA, TB><<<grid, 2 * kThreads, kDmaLds, s>>>(q);
