@@ -30,8 +30,10 @@ def _weight_grad(g2: torch.Tensor, x2: torch.Tensor) -> torch.Tensor:
     below one 256 x 256 tile per compute unit (1024 x 4096: 0.50 / 0.28 ms) the library stays."""
     n_out, n_in = g2.shape[1], x2.shape[1]
     tiles = ((n_out + 255) // 256) * ((n_in + 255) // 256)
+    # (operands of 2^30 elements and more leave the kernel's aligned path, whose offsets are 32-bit)
     if (g2.dtype in (torch.bfloat16, torch.float16) and g2.shape[0] >= 4096 and g2.shape[0] % 32 == 0
-            and n_out % 8 == 0 and n_in % 8 == 0 and tiles >= 256):
+            and n_out % 8 == 0 and n_in % 8 == 0 and tiles >= 256
+            and g2.shape[0] * max(n_out, n_in) < (1 << 30)):
         return megalodon_ops.linear_weight_grad(g2, x2)
     return g2.t() @ x2
 
