@@ -166,6 +166,25 @@ def test_empty_inputs_are_accepted():
     assert q.shape == (2, 0, 512) and k.shape == (2, 0, 512)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tokens,n_out,n_in", [(4096, 512, 768), (4128, 2304, 264), (64, 8, 8), (8200, 1000, 520),
+                                               (4099, 130, 77)])   # the last: off the aligned path
+def test_linear_weight_grad_matches_float64(tokens, n_out, n_in, dtype, monkeypatch):
+    """dW = dy^T x on the attention product kernel against float64 (2e-2, 16-bit output of a
+    float32 accumulation), for every band width of the tile order (identical bits: the order of
+    the tiles does not enter a tile's sum)."""
+    g = torch.Generator().manual_seed(tokens + n_out)
+    dy = torch.randn(tokens, n_out, generator=g).to(dtype).cuda()
+    x = torch.randn(tokens, n_in, generator=g).to(dtype).cuda()
+    want = dy.double().t() @ x.double()
+    got = ops.linear_weight_grad(dy, x)
+    assert got.shape == (n_out, n_in) and got.dtype == dtype
+    assert rel_err(got, want) <= 2e-2
+    for ng in ("0", "3", "16"):
+        monkeypatch.setenv("MEGA_GEMM_NGROUP", ng)
+        assert torch.equal(ops.linear_weight_grad(dy, x), got)
+
+
 def test_linear_group_matches_float64_and_separate_layers():
     """Layers that read one input (`linear_group`): outputs are those of the layers one by one,
     and the shared input gradient, accumulated inside the GEMM, and every parameter gradient
