@@ -44,3 +44,22 @@ def test_saved_none_is_allowed():
     a = torch.ones(3, requires_grad=True)
     op.apply(a, None).sum().backward()
     assert torch.equal(a.grad, torch.full((3,), 2.0))
+
+
+def test_linear_layers_on_cpu_tensors_are_plain_linear():
+    """`Linear` / `linear_group` off the GPU (or in float32): the values and gradients of
+    `F.linear`, layer by layer -- the grouped backward and the own weight-gradient kernel are for
+    16-bit tensors on the GPU only."""
+    import torch.nn.functional as F
+    from megalodon_amd.modules.linear import Linear, linear_group
+    torch.manual_seed(0)
+    layers = [Linear(12, 7, bias=True).double(), Linear(12, 5, bias=False).double()]
+    x = torch.randn(3, 4, 12, dtype=torch.float64, requires_grad=True)
+    ys = linear_group(x, layers)
+    for y, l in zip(ys, layers):
+        assert torch.equal(y, F.linear(x, l.weight, l.bias))
+    (ys[0].sum() + 2.0 * ys[1].sum()).backward()
+    want = layers[0].weight.detach().sum(0) + 2.0 * layers[1].weight.detach().sum(0)
+    assert torch.allclose(x.grad, want.expand_as(x.grad))
+    r = torch.randn(3, 4, 5, dtype=torch.float64)
+    assert torch.allclose(layers[1](x, residual=r), F.linear(x, layers[1].weight) + r)
