@@ -1016,6 +1016,277 @@ __global__ __launch_bounds__(2 * kThreads) void gemm_dma64_kernel(const GemmPara
   }  // work item
 }
 
+// ---- one k-contiguous and one k-major operand: A in slabs of 64 k, B in slabs of 32 k ------
+// (PV and dQ: A = P or dS, rows of keys; B = V or K, rows of k.)  With slabs of 32 k the rows of A
+// arrive as half cache lines, and the L2 answers a 64-byte request no faster than a 128-byte one:
+// such a product sends 1.5 times the requests of one with two k-major operands and keeps the
+// matrix pipe 55-68 % busy where that one reaches 86 %.  Slabs of 64 k for both operands leave
+// room for two buffers only (gemm_dma64_kernel) and were 1 % slower here.  This form keeps the
+// depth: three A buffers of 32 KB (256 rows x 64 k, whole lines) and four B buffers of 16 KB
+// (32 rows of k), all 160 KB of the LDS; a step is 32 k as in gemm_dma_kernel.
+constexpr int kA64Operand = kTile * kSlab64;        // elements of an A slab (32 KB)
+constexpr int kA64BBase = 3 * kA64Operand;          // the B buffers start behind the three A buffers
+constexpr size_t kA64Lds = sizeof(uint16_t) * (kA64BBase + kStages * kDmaOperand);
+static_assert(kA64Lds <= 160 * 1024 && sizeof(uint16_t) * 8 * 128 * (64 + 8) <= kA64Lds, "fits the LDS, holds the output tiles");
+
+template <int DT>
+__global__ __launch_bounds__(2 * kThreads) void gemm_dma_a64_kernel(const GemmParams p) {
+  extern __shared__ __align__(16) uint16_t smem[];
+  constexpr int JN = 2, EP = 64 + 8;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wm = wave >> 2, wn = wave & 3;
+  // work items as in gemm_kernel
+  const int G = static_cast<int>(gridDim.x), lin = static_cast<int>(blockIdx.x);
+  int it_lo, it_hi, it_step;
+  if (G % kXcds == 0) {
+    const int xcd = lin % kXcds;
+    it_lo = static_cast<int>(static_cast<int64_t>(p.items) * xcd / kXcds) + lin / kXcds;
+    it_hi = static_cast<int>(static_cast<int64_t>(p.items) * (xcd + 1) / kXcds);
+    it_step = G / kXcds;
+  } else {
+    it_lo = lin;
+    it_hi = p.items;
+    it_step = G;
+  }
+  for (int item = it_lo; item < it_hi; item += it_step) {
+  const int zz = item / p.per_batch;
+  const int rem = item % p.per_batch;
+  int nt, mt_first, mt_second = -1;
+  if (p.tri_out) {
+    int t = rem, m = 0;
+    while (true) {
+      const int cnt = min(p.nt_count, (m * kTile + (kTile - 1) + p.off) / kTile + 1);
+      if (t < cnt) break;
+      t -= cnt;
+      ++m;
+    }
+    mt_first = m;
+    nt = t;
+  } else if (p.k_mode) {
+    nt = rem % p.nt_count;
+    const int pr = rem / p.nt_count;
+    mt_first = p.mt_count - 1 - pr;
+    if (mt_first != pr) mt_second = pr;
+  } else {
+    if (p.n_group > 0) {
+      const int band = p.n_group * p.mt_count;       // tiles of a full band
+      const int b0 = rem / band, r2 = rem % band;
+      const int w = min(p.n_group, p.nt_count - b0 * p.n_group);  // the last band may be narrower
+      nt = b0 * p.n_group + r2 % w;
+      mt_first = r2 / w;
+    } else {
+      nt = rem % p.nt_count;
+      mt_first = rem / p.nt_count;
+    }
+  }
+  const int z0 = zz / p.nh, z1 = zz % p.nh;
+  const uint16_t* A = p.A + z0 * p.sa0 + z1 * p.sa1;
+  const uint16_t* B = p.B + z0 * p.sb0 + z1 * p.sb1;
+  uint16_t* C = p.C + z0 * p.sc0 + z1 * p.sc1;
+  for (int half = 0; half < 2; ++half) {
+  const int mt = half == 0 ? mt_first : mt_second;
+  if (mt < 0) break;
+  const int m0 = mt * kTile, n0 = nt * kTile;
+  // k range as in gemm_kernel, widened to whole slabs of 64 (K % 64 == 0): what the wider range
+  // adds are probabilities the softmax has written as zeros
+  int kb = 0, ke = p.K;
+  if (p.k_mode == 1) ke = min(p.K, ((mt + 1) * kTile + p.off + kSlab64 - 1) / kSlab64 * kSlab64);
+  if (p.k_mode == 2) kb = min(p.K, max(0, mt * kTile - p.off) / kSlab64 * kSlab64);
+  const int nslab = (ke - kb) / kSlab;   // steps of 32 k, an even number
+  const int nslab_a = nslab / 2;         // slabs of A
+
+  floatx16 acc[4][JN];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < JN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // memory side.  A: wave w sends the 1 KB pieces w, w + 8, w + 16, w + 24 of a slab (8 rows of
+  // 128 bytes each, the chunk at position c of row r holds k chunk c ^ ((r >> 1) & 7)); B: the
+  // pieces w, w + 8 (2 rows of k, 512 bytes each).  Addresses are clamped into the matrix.
+  uint32_t offa[4], offb[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int pc = wave + 8 * i;
+    const int row = 8 * pc + (lane >> 3), ck = (lane & 7) ^ ((row >> 1) & 7);
+    offa[i] = static_cast<uint32_t>((static_cast<int64_t>(min(m0 + row, p.M - 1)) * p.lda + kb + ck * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int pc = wave + 8 * i;
+    const int krow = 2 * pc + (lane >> 5), cm = (lane & 31) ^ ((krow & 3) << 2);
+    offb[i] = static_cast<uint32_t>(((kb + krow) * p.ldb + min(n0 + cm * 8, p.N - 8)) * 2);
+  }
+  const uint32_t stepa = static_cast<uint32_t>(kSlab64 * 2);
+  const uint32_t stepb = static_cast<uint32_t>(p.ldb * kSlab * 2);
+  const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)(smem))) + wave * 1024);
+  // A slab ja into A buffer ab (4 requests), B slab s into B buffer bb (2 requests); slabs past the
+  // end ask for the last one again, so that every step issues the same number of requests
+  auto request_a = [&](int ja, int ab, int n) {
+    const uint32_t sc = static_cast<uint32_t>(min(ja, nslab_a - 1));
+    load_to_lds16(A, offa[n] + sc * stepa, lds_wave + static_cast<uint32_t>(ab * kA64Operand + n * 8 * 512) * 2);
+  };
+  auto request_b = [&](int sb, int bb, int n) {
+    const uint32_t sc = static_cast<uint32_t>(min(sb, nslab - 1));
+    load_to_lds16(B, offb[n] + sc * stepb, lds_wave + static_cast<uint32_t>(kA64BBase + bb * kDmaOperand + n * 8 * 512) * 2);
+  };
+
+  // fragment side: as in gemm_dma_kernel, k-step `set` of a 32-k step takes k = 16 g + 8 set + e
+  // for lane half g; in the A slab that is chunk 4 h + 2 g + set of the row (h: which half of the
+  // 64 k the step is), at position ((2 g) ^ swizzle) ^ (4 h + set)
+  const int g = lane >> 5, r = lane & 31;
+  const int ta_a = (lane & 15) >> 2, ta_h = (lane >> 4) & 1, ta_b = lane & 3;
+  int fra[4], frb[JN];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) fra[i] = (wm * 128 + 32 * i + r) * kSlab64 + (((2 * g) ^ ((r >> 1) & 7)) * 8);
+#pragma unroll
+  for (int j = 0; j < JN; ++j)
+    frb[j] = kA64BBase + (16 * g + ta_a) * kTile + (((wn * 8 + 4 * j + 2 * ta_h + (ta_b >> 1)) ^ (ta_a << 2)) * 8) + 4 * (ta_b & 1);
+  u32x4 fa0[4], fb0[JN], fa1[4], fb1[JN];
+  // fragments of k-step `set` of a 32-k step: A buffer ab, chunk selector x = 4 h + set; B buffer bb
+  auto fread = [&](u32x4* fa, u32x4* fb, int x, int ab, int set, int bb) {
+    const uint16_t* abase = smem + ab * kA64Operand;
+    const uint16_t* bbase = smem + bb * kDmaOperand;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      fa[i] = *reinterpret_cast<const u32x4*>(abase + (fra[i] ^ (x * 8)));
+      if (i < JN) {
+        const uint16_t* q = bbase + frb[i] + set * 8 * kTile;
+        const uint2 lo = lds_read_tr(q), hi = lds_read_tr(q + 4 * kTile);
+        fb[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+      }
+    }
+  };
+  auto mma = [&](const u32x4* fa, const u32x4* fb, int lo, int hi) {
+#pragma unroll
+    for (int n = 0; n < 4 * JN; ++n)
+      if (n >= lo && n < hi) acc[n >> 1][n & 1] = Mma<DT>::run(fb[n & 1], fa[n >> 1], acc[n >> 1][n & 1]);
+  };
+
+  // One step per 32 k as in gemm_dma_kernel.  An odd step also ends the reads of its A slab and
+  // requests A slab (s >> 1) + 3 into that buffer, before the step's B requests.  In front of the
+  // barrier of step s the requests of the two steps before it may still be in flight: two B slabs
+  // and one A slab, 8 per wave; B slab s + 1 and, at odd s, A slab (s + 1) / 2 are older.
+#define MEGA_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+  constexpr int kFragReads = 1 + JN / 2;
+#define MEGA_A64_STEP(R)                                                   \
+  {                                                                        \
+    const int cur = it + (R);                                              \
+    fread(fa1, fb1, 4 * ((R) & 1) + 1, ab, 1, (R));                        \
+    mma(fa0, fb0, 0, 8);                                                   \
+    _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
+      MEGA_SGB(0x008, 1);                                                  \
+      MEGA_SGB(0x100, kFragReads);                                         \
+    }                                                                      \
+    MEGA_SGB(0x008, 4 * JN - 4);                                           \
+    __builtin_amdgcn_sched_barrier(0);                                     \
+    asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory"); \
+    const int ab_next = ((R) & 1) ? (ab == 2 ? 0 : ab + 1) : ab;           \
+    fread(fa0, fb0, ((R) & 1) ? 0 : 4, ab_next, 0, ((R) + 1) & 3);         \
+    mma(fa1, fb1, 0, 2);                                                   \
+    _Pragma("unroll") for (int sg = 0; sg < 2; ++sg) {                     \
+      MEGA_SGB(0x008, 1);                                                  \
+      MEGA_SGB(0x100, 2 * kFragReads);                                     \
+    }                                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                     \
+    _Pragma("unroll") for (int n = 0; n < 6; ++n) {                        \
+      if ((R) & 1) {                                                       \
+        if (n < 4) request_a((cur >> 1) + 3, ab, n);                       \
+        else request_b(cur + kStages, (R), n - 4);                         \
+      } else if (n < 2) {                                                  \
+        request_b(cur + kStages, (R), n);                                  \
+      }                                                                    \
+      mma(fa1, fb1, 2 + n, 3 + n);                                         \
+      __builtin_amdgcn_sched_barrier(0);                                   \
+    }                                                                      \
+    ab = ab_next;                                                          \
+  }
+  if (nslab > 0) {
+    int ab = 0;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) request_a(0, 0, n);
+#pragma unroll
+    for (int n = 0; n < 2; ++n) request_b(0, 0, n);
+#pragma unroll
+    for (int n = 0; n < 2; ++n) request_b(1, 1, n);
+#pragma unroll
+    for (int n = 0; n < 4; ++n) request_a(1, 1, n);
+#pragma unroll
+    for (int n = 0; n < 2; ++n) request_b(2, 2, n);
+#pragma unroll
+    for (int n = 0; n < 2; ++n) request_b(3, 3, n);
+#pragma unroll
+    for (int n = 0; n < 4; ++n) request_a(2, 2, n);
+    asm volatile("s_waitcnt vmcnt(14)\n\ts_barrier" ::: "memory");
+    fread(fa0, fb0, 0, 0, 0, 0);
+    for (int it = 0; it < nslab; it += 4) {
+      MEGA_A64_STEP(0)
+      MEGA_A64_STEP(1)
+      if (it + 2 < nslab) {
+        MEGA_A64_STEP(2)
+        MEGA_A64_STEP(3)
+      }
+    }
+    // nothing may land in the buffers once they hold the output tiles
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  }
+#undef MEGA_A64_STEP
+#undef MEGA_SGB
+
+  // epilogue as in gemm_kernel: the wave's 128 x 64 tile through its own LDS region
+  uint16_t* stage = smem + wave * 128 * EP;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < JN; ++j) {
+      const int row = i * 32 + (lane & 31);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int col = j * 32 + 8 * q4 + 4 * (lane >> 5);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[i][j][4 * q4 + e];
+        uint2 w;
+        if (DT == MEGA_BF16) {
+          w.x = pack_bf16x2(v[0], v[1]);
+          w.y = pack_bf16x2(v[2], v[3]);
+        } else {
+          w.x = static_cast<uint32_t>(float_to_f16_bits(v[0])) | (static_cast<uint32_t>(float_to_f16_bits(v[1])) << 16);
+          w.y = static_cast<uint32_t>(float_to_f16_bits(v[2])) | (static_cast<uint32_t>(float_to_f16_bits(v[3])) << 16);
+        }
+        *reinterpret_cast<uint2*>(stage + row * EP + col) = w;
+      }
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave reads back only its own region
+  const bool vec_ok = (p.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+#pragma unroll 4
+  for (int i = 0; i < 8 * JN; ++i) {
+    const int c = lane + kWave * i;
+    const int row = c / (4 * JN), kc = (c % (4 * JN)) * 8;
+    const int grow = m0 + wm * 128 + row, gcol = n0 + wn * (32 * JN) + kc;
+    if (grow < p.M && gcol < p.N) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * EP + kc);
+      uint16_t* dst = C + static_cast<int64_t>(grow) * p.ldc + gcol;
+      if (vec_ok && gcol + 8 <= p.N) {
+        *reinterpret_cast<u32x4*>(dst) = v;
+      } else {
+        const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+        for (int q = 0; q < 8; ++q)
+          if (gcol + q < p.N) dst[q] = e[q];
+      }
+    }
+  }
+  // the output regions overlap the slab buffers: every read of this tile's epilogue
+  // retires before the next tile's first slab is requested
+  lds_barrier();
+  }  // tile of the pair
+  }  // work item
+}
+
 // ---- causal softmax over rows (in place), one wavefront per row ---------------
 // `coff` < 0: every row keeps all L2 columns.  `coff` = L2 - L1 >= 0 (causal,
 // bottom-right aligned, softmax.cuh:99-100): row r keeps columns [0, n) with
@@ -1267,11 +1538,23 @@ int launch_gemm_t(const GemmParams& p, int batch, hipStream_t s) {
   if constexpr (!TA && !TB)
     slab64 = fast && p.K % kSlab64 == 0 && !(w4 != nullptr && w4[0] == '1') && !(dma != nullptr && dma[0] == '0') &&
              !(s64 != nullptr && s64[0] == '0');
+  // one k-contiguous and one k-major operand: A in slabs of 64 k (MEGA_GEMM_A64=0: slabs of 32 k for both)
+  const char* a64e = getenv("MEGA_GEMM_A64");
+  bool a64 = false;
+  if constexpr (!TA && TB)
+    a64 = fast && p.K % kSlab64 == 0 && !(w4 != nullptr && w4[0] == '1') && !(dma != nullptr && dma[0] == '0') &&
+          !(a64e != nullptr && a64e[0] == '0');
   if (slab64) {
     if constexpr (!TA && !TB) {
       MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma64_kernel<DT, TA, TB>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaLds));
       gemm_dma64_kernel<DT, TA, TB><<<grid, 2 * kThreads, kDmaLds, s>>>(q);
+    }
+  } else if (a64) {
+    if constexpr (!TA && TB) {
+      MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_a64_kernel<DT>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kA64Lds));
+      gemm_dma_a64_kernel<DT><<<grid, 2 * kThreads, kA64Lds, s>>>(q);
     }
   } else if (fast && !(w4 != nullptr && w4[0] == '1') && !(dma != nullptr && dma[0] == '0')) {
     MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<DT, TA, TB>),

@@ -89,27 +89,34 @@ def test_float32_and_float64_tensors(B, L1, L2, NH, H1, H2, causal, dtype):
         assert torch.count_nonzero(torch.triu(w, diagonal=L2 - L1 + 1)) == 0
 
 
-@pytest.mark.parametrize("B,L1,L2,NH,H1,H2", [(1, 520, 1000, 2, 32, 64), (2, 768, 768, 2, 256, 512)])
+@pytest.mark.parametrize("B,L1,L2,NH,H1,H2", [(1, 520, 1000, 2, 32, 64), (2, 768, 768, 2, 256, 512), (1, 512, 1088, 2, 64, 192)])
 def test_slab_paths_agree(B, L1, L2, NH, H1, H2, monkeypatch):
-    """Aligned operands reach LDS straight from memory, in slabs of 64 k when both operands of a
-    product are k-contiguous and of 32 k otherwise; MEGA_GEMM_SLAB64=0 keeps 32 everywhere and
-    MEGA_GEMM_DMA=0 sends the slabs through registers.  The two forms with slabs of 32 add up
-    the same products in the same order: identical bits.  Slabs of 64 group the k-steps
-    differently (float32 accumulation, one rounding at the end): within one bfloat16 ulp."""
+    """Aligned operands reach LDS straight from memory: in slabs of 64 k when both operands of a
+    product are k-contiguous, with A in slabs of 64 k and B in slabs of 32 k when one is k-major
+    and the other k-contiguous, in slabs of 32 k otherwise.  MEGA_GEMM_SLAB64=0 and
+    MEGA_GEMM_A64=0 keep 32 everywhere, MEGA_GEMM_DMA=0 sends the slabs through registers.  The
+    forms whose steps are 32 k add up the same products in the same order: identical bits.
+    Slabs of 64 for both operands group the k-steps differently (float32 accumulation, one
+    rounding at the end): within one bfloat16 ulp."""
     g = torch.Generator().manual_seed(L1)
     q = (torch.randn(B, L1, NH, H1, generator=g) / H1 ** 0.5).bfloat16().cuda()
     k = (torch.randn(B, L2, NH, H1, generator=g) / H1 ** 0.5).bfloat16().cuda()
     v = (torch.randn(B, L2, NH, H2, generator=g) / H2 ** 0.5).bfloat16().cuda()
     dy = torch.randn(B, L1, NH, H2, generator=g).bfloat16().cuda()
     out = {}
-    for mode, env in (("default", {}), ("slab32", {"MEGA_GEMM_SLAB64": "0"}), ("registers", {"MEGA_GEMM_DMA": "0"})):
-        monkeypatch.delenv("MEGA_GEMM_SLAB64", raising=False)
-        monkeypatch.delenv("MEGA_GEMM_DMA", raising=False)
+    switches = ("MEGA_GEMM_SLAB64", "MEGA_GEMM_A64", "MEGA_GEMM_DMA")
+    for mode, env in (("default", {}), ("a32", {"MEGA_GEMM_A64": "0"}),
+                      ("slab32", {"MEGA_GEMM_SLAB64": "0", "MEGA_GEMM_A64": "0"}),
+                      ("slab32_a64", {"MEGA_GEMM_SLAB64": "0"}), ("registers", {"MEGA_GEMM_DMA": "0"})):
+        for name in switches:
+            monkeypatch.delenv(name, raising=False)
         for name, val in env.items():
             monkeypatch.setenv(name, val)
         y, w = ops.attention_fwd(q, k, v, 1.0, 0.0, True)
         out[mode] = (y, torch.tril(w, diagonal=L2 - L1)) + tuple(ops.attention_bwd(dy, q, k, v, w, 1.0, True))
-    for a, b in zip(out["slab32"], out["registers"]):
+    for a, b, c in zip(out["slab32"], out["registers"], out["slab32_a64"]):
+        assert torch.equal(a, b) and torch.equal(a, c)
+    for a, b in zip(out["default"], out["a32"]):
         assert torch.equal(a, b)
     for a, b in zip(out["default"], out["registers"]):
         assert rel_err(a, b) <= 8e-3
