@@ -10,7 +10,8 @@ synthetic, seeded inputs that are resident in HBM before the timed region.
 Beside it, in the same JSON line:
   roofline      the dominant kernel of the CEMA + convolution sub-layer
                 (config 1: B=1, L=32768, D=4096, ndim=16, x / dy bf16), timed
-                live with device events on the launch stream
+                live with device events on the launch stream around twenty
+                launches back to back
   cema_layer    the config-1 step (layer forward + backward) on the default
                 path (chunked recurrence on the matrix cores, float32-equivalent
                 arithmetic) and on the two FFT-convolution engines
@@ -258,11 +259,24 @@ def cema_leg(torch, dev, steps, warmup, copy_calibration):
     _lib.set_event_log(None)
     avg = {k: (sum(a.elapsed_time(b) for a, b in v) / max(1, len(v))) for k, v in log.items()}
     E = B * D * L
+    # the two recurrence kernels launched back to back on the layer's own operands, device events
+    # around the run: the launch duration without the host's time to issue it (inside a step the
+    # device is idle when the first event of a call is recorded, so `kernels_ms` above holds the
+    # 10-25 us the host takes to launch as well)
+    from megalodon_amd import extension as ops
+    n_k = 20 if steps >= 5 else max(1, steps)
+    with torch.no_grad():
+        cp, clq, cgm = ops.cema_coeffs_fwd(layer.alpha.float(), layer.delta.float(), layer.theta.float(),
+                                           layer.gamma.float())
+        xd = x.detach()
+        ms_f = dev_ms(torch, lambda: ops.cema_scan_fwd(xd, cp, clq, cgm, layer.omega), n_k, warm=min(3, n_k))
+        ms_b = dev_ms(torch, lambda: ops.cema_scan_bwd(dy, xd, cp, clq, cgm, layer.omega), n_k, warm=min(3, n_k))
     res = {"ms_per_step": dt * 1e3, "tokens_per_s": B * L / dt,
            "GBps_on_10E": 10 * E / dt / 1e9, "frac_hbm_on_10E": 10 * E / dt / 1e9 / HBM_PEAK_GBS,
            "kernels_ms": avg,
-           "scan_fwd_GBps": 4 * E / (avg["mega_cema_scan_fwd"] * 1e-3) / 1e9,
-           "scan_bwd_GBps": 6 * E / (avg["mega_cema_scan_bwd"] * 1e-3) / 1e9}
+           "scan_launch_ms": {"fwd": ms_f, "bwd": ms_b, "launches": n_k},
+           "scan_fwd_GBps": 4 * E / (ms_f * 1e-3) / 1e9,
+           "scan_bwd_GBps": 6 * E / (ms_b * 1e-3) / 1e9}
     # the same step on the FFT-convolution operators: float32 transforms, then the fp16-stage engine
     n_alt = max(1, min(5, steps))
     os.environ["MEGA_CEMA_FFT"] = "1"
