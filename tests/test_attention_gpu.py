@@ -122,6 +122,34 @@ def test_slab_paths_agree(B, L1, L2, NH, H1, H2, monkeypatch):
         assert rel_err(a, b) <= 8e-3
 
 
+def test_whole_line_slabs_random_shapes(monkeypatch):
+    """Seeded random shapes with a key count that is a multiple of 64 (PV and dQ then take A in
+    slabs of 64 k): ragged query counts, key/value prefixes of any length, causal and not --
+    against the oracle (2e-2) and, bit for bit, against the same products on slabs of 32 k."""
+    import random
+    rnd = random.Random(6464)
+    for case in range(10):
+        L2 = 64 * rnd.randint(1, 20)
+        L1 = rnd.choice([L2, rnd.randint(1, L2), max(1, L2 - 64 * rnd.randint(0, 3))])
+        B, NH = rnd.randint(1, 2), rnd.randint(1, 3)
+        H1, H2 = 8 * rnd.randint(1, 12), 8 * rnd.randint(1, 40)
+        causal = rnd.random() < 0.7
+        _run(B, L1, L2, NH, H1, H2, causal, torch.bfloat16, seed=case)
+        g = torch.Generator().manual_seed(100 + case)
+        q = (torch.randn(B, L1, NH, H1, generator=g) / H1 ** 0.5).bfloat16().cuda()
+        k = (torch.randn(B, L2, NH, H1, generator=g) / H1 ** 0.5).bfloat16().cuda()
+        v = (torch.randn(B, L2, NH, H2, generator=g) / H2 ** 0.5).bfloat16().cuda()
+        dy = torch.randn(B, L1, NH, H2, generator=g).bfloat16().cuda()
+        out = []
+        for a64 in ("1", "0"):
+            monkeypatch.setenv("MEGA_GEMM_A64", a64)
+            y, w = ops.attention_fwd(q, k, v, 0.7, 0.0, causal)
+            out.append((y,) + tuple(ops.attention_bwd(dy, q, k, v, w, 0.7, causal)))
+        monkeypatch.delenv("MEGA_GEMM_A64")
+        for a, b in zip(*out):
+            assert torch.equal(a, b), (case, B, L1, L2, NH, H1, H2, causal)
+
+
 def test_causal_with_fewer_keys_than_queries_fails_loudly():
     q = torch.zeros(1, 8, 1, 16, dtype=torch.bfloat16, device="cuda")
     k = torch.zeros(1, 4, 1, 16, dtype=torch.bfloat16, device="cuda")
