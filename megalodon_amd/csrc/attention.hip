@@ -41,6 +41,9 @@ template <typename T>
 int softmax_wide_fwd(T* x, int64_t Z, int64_t L1, int64_t L2, int causal, const DropKey* drop, hipStream_t s);
 template <typename T>
 int softmax_wide_bwd(const T* y, T* dy, int64_t Z, int64_t L1, int64_t L2, int causal, hipStream_t s);
+// scores + softmax in one kernel (attention_scores.hip); -1: shape outside that kernel
+int attention_probs_fused(int dtype, const uint16_t* q, const uint16_t* k, uint16_t* w, int64_t B, int64_t L1,
+                          int64_t L2, int64_t NH, int64_t H1, float scale, int causal, int fill, hipStream_t s);
 
 namespace {
 
@@ -1609,9 +1612,12 @@ int check_attn(const char* who, int dtype, int64_t B, int64_t L1, int64_t L2, in
 template <int DT>
 int attn_fwd_impl(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64_t B, int64_t L1,
                   int64_t L2, int64_t NH, int64_t H1, int64_t H2, float scale, int causal,
-                  uint16_t* y, uint16_t* w, uint16_t* ws, hipStream_t s, const DropKey* drop) {
+                  uint16_t* y, uint16_t* w, uint16_t* ws, hipStream_t s, const DropKey* drop, int fill) {
   (void)ws;
   const int Z = static_cast<int>(B * NH);
+  int rc = drop ? -1 : attention_probs_fused(DT, q, k, w, B, L1, L2, NH, H1, scale, causal, fill, s);
+  if (rc > 0) return rc;
+  if (rc < 0) {
   // S = scale Q K^T  -> w
   GemmParams g{};
   g.A = q; g.B = k; g.C = w; g.M = (int)L1; g.N = (int)L2; g.K = (int)H1;
@@ -1619,10 +1625,10 @@ int attn_fwd_impl(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64
   g.sa0 = L1 * NH * H1; g.sa1 = H1; g.sb0 = L2 * NH * H1; g.sb1 = H1;
   g.sc0 = NH * L1 * L2; g.sc1 = L1 * L2; g.nh = (int)NH; g.alpha = scale;
   g.tri_out = causal; g.k_mode = 0; g.off = causal ? (int)(L2 - L1) : 0;
-  int rc = launch_gemm<DT>(g, Z, s);
-  if (rc != MEGA_OK) return rc;
+  if ((rc = launch_gemm<DT>(g, Z, s)) != MEGA_OK) return rc;
   // P = softmax(S) in place
-  if ((rc = launch_softmax<DT>(nullptr, w, Z, L1, L2, causal, s, 0, drop)) != MEGA_OK) return rc;
+  if ((rc = launch_softmax<DT>(nullptr, w, Z, L1, L2, causal, s, fill, drop)) != MEGA_OK) return rc;
+  }
   // Y = P V: V[key][c] is the k-major B operand
   GemmParams o{};
   o.A = w; o.B = v; o.C = y; o.M = (int)L1; o.N = (int)H2; o.K = (int)L2;
@@ -1709,6 +1715,9 @@ static int attention_fwd_entry(const char* who, const void* q, const void* k, co
   MEGA_CHECK_ARG(q && k && v && y && w && workspace, "%s: null pointer", who);
   MEGA_CHECK_ARG(L2 >= 1, "%s: no keys", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // causal == 2: as 1, but w need only hold what mega_attention_bwd reads
+  const int fill = causal == 2 ? 0 : 1;
+  causal = causal != 0;
   if (dtype == MEGA_F32)
     return attention_wide_fwd<float>(static_cast<const float*>(q), static_cast<const float*>(k),
                                      static_cast<const float*>(v), B, L1, L2, NH, H1, H2, scale, causal, drop,
@@ -1721,9 +1730,9 @@ static int attention_fwd_entry(const char* who, const void* q, const void* k, co
   auto m = [](void* p) { return static_cast<uint16_t*>(p); };
   if (dtype == MEGA_BF16)
     return attn_fwd_impl<MEGA_BF16>(u(q), u(k), u(v), B, L1, L2, NH, H1, H2, (float)scale, causal,
-                                    m(y), m(w), m(workspace), s, drop);
+                                    m(y), m(w), m(workspace), s, drop, fill);
   return attn_fwd_impl<MEGA_F16>(u(q), u(k), u(v), B, L1, L2, NH, H1, H2, (float)scale, causal,
-                                 m(y), m(w), m(workspace), s, drop);
+                                 m(y), m(w), m(workspace), s, drop, fill);
 }
 
 extern "C" int mega_attention_fwd(const void* q, const void* k, const void* v, int dtype, int64_t B,

@@ -953,15 +953,21 @@ def dropkey_philox_state(dev: torch.device, columns: int) -> Tuple[int, int]:
 
 
 def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, dropout: float,
-                  use_causal_mask: bool) -> Tuple[torch.Tensor, torch.Tensor]:
-    """(y, w): y (B, L1, N, H2), w = softmax probabilities (B, N, L1, L2).
+                  use_causal_mask: bool, lower_only: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(y, w): y (B, L1, N, H2), w = softmax probabilities (B, N, L1, L2), every
+    row written to its end (zeros behind the causal limit, as the reference's
+    softmax writes them, softmax.cuh:99-105,127-129).
     `dropout` > 0 is DropKey (softmax.cuh:135-196): keys leave a row with that
     probability before the softmax, drawn from the device generator's
-    (seed, offset)."""
+    (seed, offset).  `lower_only` (no counterpart in the reference) is for callers
+    that hand w to `attention_bwd` and nowhere else: with a causal mask and 16-bit
+    tensors the zeros to the right of the block that holds a row's diagonal are
+    then not written (half of w at L1 = L2), and those entries are undefined."""
     dev = _require_cuda(q, k, v)
     if not 0.0 <= dropout <= 1.0:
         raise RuntimeError("attention_fwd: dropout must lie in [0, 1]")
     B, L1, L2, NH, H1, H2 = _attn_dims(q, k, v)
+    causal = (2 if lower_only else 1) if use_causal_mask else 0
     if dropout > 0.0:
         qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
         y = torch.empty((B, L1, NH, H2), dtype=v.dtype, device=dev)
@@ -972,7 +978,7 @@ def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: floa
             _lib.call("mega_attention_dropkey_fwd", _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc),
                       _lib.i32(_lib.dtype_code(q.dtype, True)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2),
                       _lib.i64(NH), _lib.i64(H1), _lib.i64(H2), _lib.f64(scale),
-                      _lib.i32(1 if use_causal_mask else 0), _lib.f64(dropout), _lib.u64(seed),
+                      _lib.i32(causal), _lib.f64(dropout), _lib.u64(seed),
                       _lib.u64(offset), _lib.ptr(y), _lib.ptr(w), _lib.ptr(ws), _lib.stream_ptr(dev))
         return y, w
     qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
@@ -982,7 +988,7 @@ def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: floa
     with torch.cuda.device(dev):
         _lib.call("mega_attention_fwd", _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(vc),
                   _lib.i32(_lib.dtype_code(q.dtype, True)), _lib.i64(B), _lib.i64(L1), _lib.i64(L2), _lib.i64(NH),
-                  _lib.i64(H1), _lib.i64(H2), _lib.f64(scale), _lib.i32(1 if use_causal_mask else 0),
+                  _lib.i64(H1), _lib.i64(H2), _lib.f64(scale), _lib.i32(causal),
                   _lib.ptr(y), _lib.ptr(w), _lib.ptr(ws), _lib.stream_ptr(dev))
     return y, w
 

@@ -1,65 +1,57 @@
-"""`FusedLayerNorm` / `FusedRMSNorm` with the reference's parameterisation
-(megalodon/modules/layer_norm.py:14-66: stored weight is `gamma - 1`; the
-reference adds 1 and calls apex's fused_layer_norm_cuda).  On the GPU the
-normalisation over the last axis runs as one streaming kernel that takes the
-stored weight as it is; CPU tensors and multi-axis shapes use PyTorch's
-layer_norm / rms_norm."""
-import numbers
+"""`FusedLayerNorm` / `FusedRMSNorm`: normalisation over the trailing axes with
+the reference's parameterisation (megalodon/modules/layer_norm.py:14-66): the
+stored `weight` is `gamma - 1` and starts at zero, so the state dict matches.
+On the GPU a normalisation over the last axis is one streaming kernel that
+reads the stored weight as it is (no `weight + 1` tensor is formed); CPU
+tensors and multi-axis shapes go through PyTorch's layer_norm / rms_norm."""
+from typing import Sequence, Union
 
 import torch
-import torch.nn as nn
 import torch.nn.functional as F
+from torch import nn
 
 from ..fused_ops import layer_norm_plus_one
 
 
-def _param_dtype(weight, input_):
-    return input_.dtype if weight is None else weight.dtype
+class _PlusOneNorm(nn.Module):
+    """State and dispatch shared by the two norms.  `rms` drops the mean and the bias."""
 
+    rms = False
 
-class FusedLayerNorm(nn.Module):
-    def __init__(self, normalized_shape, eps=1e-5, elementwise_affine=True):
+    def __init__(self, normalized_shape: Union[int, Sequence[int]], eps: float = 1e-5,
+                 elementwise_affine: bool = True):
         super().__init__()
-        if isinstance(normalized_shape, numbers.Integral):
-            normalized_shape = (normalized_shape,)
-        self.normalized_shape = torch.Size(normalized_shape)
+        shape = (int(normalized_shape),) if isinstance(normalized_shape, int) else tuple(normalized_shape)
+        self.normalized_shape = torch.Size(shape)
         self.eps = eps
         self.elementwise_affine = elementwise_affine
-        if self.elementwise_affine:
-            self.weight = nn.Parameter(torch.zeros(*normalized_shape))
-            self.bias = nn.Parameter(torch.zeros(*normalized_shape))
-        else:
-            self.register_parameter("weight", None)
-            self.register_parameter("bias", None)
+        names = ("weight",) if self.rms else ("weight", "bias")
+        for name in names:
+            if elementwise_affine:
+                setattr(self, name, nn.Parameter(torch.zeros(shape)))
+            else:
+                self.register_parameter(name, None)
 
-    def forward(self, input_):
-        if input_.is_cuda and len(self.normalized_shape) == 1 and input_.dtype == _param_dtype(self.weight, input_):
-            return layer_norm_plus_one(input_, self.weight, self.bias, self.eps, False)
-        weight = None if self.weight is None else self.weight + 1.0
-        return F.layer_norm(input_, self.normalized_shape, weight, self.bias, self.eps)
+    def _fused(self, x: torch.Tensor) -> bool:
+        same = self.weight is None or self.weight.dtype == x.dtype
+        return x.is_cuda and len(self.normalized_shape) == 1 and same
 
-    def extra_repr(self):
-        return "{normalized_shape}, eps={eps}, elementwise_affine={elementwise_affine}".format(**self.__dict__)
+    def forward(self, input_: torch.Tensor) -> torch.Tensor:
+        bias = None if self.rms else self.bias
+        if self._fused(input_):
+            return layer_norm_plus_one(input_, self.weight, bias, self.eps, self.rms)
+        gamma = self.weight + 1.0 if self.weight is not None else None
+        if self.rms:
+            return F.rms_norm(input_, self.normalized_shape, gamma, self.eps)
+        return F.layer_norm(input_, self.normalized_shape, gamma, bias, self.eps)
+
+    def extra_repr(self) -> str:
+        return f"{tuple(self.normalized_shape)}, eps={self.eps}, elementwise_affine={self.elementwise_affine}"
 
 
-class FusedRMSNorm(nn.Module):
-    def __init__(self, normalized_shape, eps=1e-5, elementwise_affine=True):
-        super().__init__()
-        if isinstance(normalized_shape, numbers.Integral):
-            normalized_shape = (normalized_shape,)
-        self.normalized_shape = torch.Size(normalized_shape)
-        self.eps = eps
-        self.elementwise_affine = elementwise_affine
-        if self.elementwise_affine:
-            self.weight = nn.Parameter(torch.zeros(*normalized_shape))
-        else:
-            self.register_parameter("weight", None)
+class FusedLayerNorm(_PlusOneNorm):
+    rms = False
 
-    def forward(self, input_):
-        if input_.is_cuda and len(self.normalized_shape) == 1 and input_.dtype == _param_dtype(self.weight, input_):
-            return layer_norm_plus_one(input_, self.weight, None, self.eps, True)
-        weight = None if self.weight is None else self.weight + 1.0
-        return F.rms_norm(input_, self.normalized_shape, weight, self.eps)
 
-    def extra_repr(self):
-        return "{normalized_shape}, eps={eps}, elementwise_affine={elementwise_affine}".format(**self.__dict__)
+class FusedRMSNorm(_PlusOneNorm):
+    rms = True
