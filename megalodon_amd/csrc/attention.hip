@@ -24,7 +24,6 @@
 #include "dropkey.hpp"
 
 #include <algorithm>
-#include <cstdlib>
 
 namespace mega {
 
@@ -161,18 +160,20 @@ __device__ __forceinline__ uint2 lds_read_tr(const uint16_t* q) {
 
 // C[m][n] = alpha * sum_k A(m, k) B(n, k).  An operand is either k-contiguous
 // (rows m, `ld` between rows) or, with TA / TB, k-major (rows k, m contiguous).
-template <int DT, bool FAST, bool TA, bool TB, bool W8>
-__global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(const GemmParams p) {
+// This is the form for operands of any alignment and extent: four waves of 128 x 128, slabs of
+// 32 k through a ring of three register sets (bounds-checked element loads) and two LDS buffers.
+// Aligned operands take the kernels below, whose slabs go from memory straight into LDS.
+template <int DT, bool TA, bool TB>
+__global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
   extern __shared__ __align__(16) uint16_t smem[];
   // main loop: [buf][A|B] operand slabs; epilogue: [wave][128][pitch]
   constexpr int kOperand = kOperandElems;
-  // W8: eight waves (two per SIMD) of 128 x 64 each instead of four of 128 x 128
-  constexpr int T = W8 ? 2 * kThreads : kThreads;  // threads
-  constexpr int JN = W8 ? 2 : 4;                   // 32-column blocks per wave
-  constexpr int NL = W8 ? 2 : 4;                   // 16-byte chunks per thread, operand and slab
-  constexpr int EP = W8 ? 64 + 8 : kEpiPitch;      // staging pitch
+  constexpr int T = kThreads;  // threads
+  constexpr int JN = 4;        // 32-column blocks per wave
+  constexpr int NL = 4;        // 16-byte chunks per thread, operand and slab
+  constexpr int EP = kEpiPitch;
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const int wm = W8 ? wave >> 2 : wave >> 1, wn = W8 ? wave & 3 : wave & 1;
+  const int wm = wave >> 1, wn = wave & 1;
 
   // Persistent workgroups (one per CU) walk a list of work items of equal
   // weight, so nothing is launched for skipped tiles and no CU ends up with
@@ -245,43 +246,19 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
 
   // register ring: slab s lives in ring slot s % 3 from its issue (three steps
   // before use) until it is written to LDS
-  constexpr int RING = W8 ? 4 : kRing;  // slabs in flight from memory
-  u32x4 ra0[NL], ra1[NL], ra2[NL], ra3[W8 ? NL : 1], rb0[NL], rb1[NL], rb2[NL], rb3[W8 ? NL : 1];
+  u32x4 ra0[NL], ra1[NL], ra2[NL], rb0[NL], rb1[NL], rb2[NL];
 
-  // Global -> register chunk i of a thread (16 bytes):
+  // Global -> register chunk i of a thread (16 bytes), bounds-checked element loads:
   //   k-contiguous operand: row (tid >> 2) + T / 4 i, k chunk tid & 3
   //   k-major operand:      k row (tid >> 5) + T / 32 i, m chunk tid & 31
-  // FAST (16-byte aligned rows, K % 32 == 0, extents % 8 == 0 and below 1 GiB):
-  // branch-free loads from a uniform base plus 32-bit byte offsets with rows,
-  // columns and slab index clamped into the matrix, so nothing forces a wait
-  // on the loads in flight.  Otherwise: bounds-checked element loads.
-  uint32_t offa[NL], offb[NL];
-#pragma unroll
-  for (int i = 0; i < NL; ++i) {
-    if (TA) offa[i] = static_cast<uint32_t>(((kb + (tid >> 5) + (T / 32) * i) * p.lda + min(m0 + (tid & 31) * 8, p.M - 8)) * 2);
-    else offa[i] = static_cast<uint32_t>((static_cast<int64_t>(min(m0 + (tid >> 2) + (T / 4) * i, p.M - 1)) * p.lda + kb + (tid & 3) * 8) * 2);
-    if (TB) offb[i] = static_cast<uint32_t>(((kb + (tid >> 5) + (T / 32) * i) * p.ldb + min(n0 + (tid & 31) * 8, p.N - 8)) * 2);
-    else offb[i] = static_cast<uint32_t>((static_cast<int64_t>(min(n0 + (tid >> 2) + (T / 4) * i, p.N - 1)) * p.ldb + kb + (tid & 3) * 8) * 2);
-  }
-  const uint32_t stepa = static_cast<uint32_t>((TA ? p.lda : 1) * kSlab * 2);
-  const uint32_t stepb = static_cast<uint32_t>((TB ? p.ldb : 1) * kSlab * 2);
   auto gload = [&](u32x4* qa, u32x4* qb, int s) {
-    if (FAST) {
-      const uint32_t sc = static_cast<uint32_t>(min(s, nslab - 1));
+    const int k0 = kb + s * kSlab;
 #pragma unroll
-      for (int i = 0; i < NL; ++i) {
-        qa[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(A) + (offa[i] + sc * stepa));
-        qb[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(B) + (offb[i] + sc * stepb));
-      }
-    } else {
-      const int k0 = kb + s * kSlab;
-#pragma unroll
-      for (int i = 0; i < NL; ++i) {
-        if (TA) qa[i] = load_chunk<false>(A, p.lda, k0 + (tid >> 5) + (T / 32) * i, ke, m0 + (tid & 31) * 8, p.M);
-        else qa[i] = load_chunk<false>(A, p.lda, m0 + (tid >> 2) + (T / 4) * i, p.M, k0 + (tid & 3) * 8, ke);
-        if (TB) qb[i] = load_chunk<false>(B, p.ldb, k0 + (tid >> 5) + (T / 32) * i, ke, n0 + (tid & 31) * 8, p.N);
-        else qb[i] = load_chunk<false>(B, p.ldb, n0 + (tid >> 2) + (T / 4) * i, p.N, k0 + (tid & 3) * 8, ke);
-      }
+    for (int i = 0; i < NL; ++i) {
+      if (TA) qa[i] = load_chunk<false>(A, p.lda, k0 + (tid >> 5) + (T / 32) * i, ke, m0 + (tid & 31) * 8, p.M);
+      else qa[i] = load_chunk<false>(A, p.lda, m0 + (tid >> 2) + (T / 4) * i, p.M, k0 + (tid & 3) * 8, ke);
+      if (TB) qb[i] = load_chunk<false>(B, p.ldb, k0 + (tid >> 5) + (T / 32) * i, ke, n0 + (tid & 31) * 8, p.N);
+      else qb[i] = load_chunk<false>(B, p.ldb, n0 + (tid >> 2) + (T / 4) * i, p.N, k0 + (tid & 3) * 8, ke);
     }
   };
   // register -> LDS: chunk layout for k-contiguous operands, padded rows of k
@@ -320,13 +297,11 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
       } else {
         fa[i] = *reinterpret_cast<const u32x4*>(qa + i * 32 * 8);
       }
-      if (i < JN) {
-        if (TB) {
-          const uint2 lo = lds_read_tr(qb + i * 32), hi = lds_read_tr(qb + i * 32 + 4 * kPitchT);
-          fb[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
-        } else {
-          fb[i] = *reinterpret_cast<const u32x4*>(qb + i * 32 * 8);
-        }
+      if (TB) {
+        const uint2 lo = lds_read_tr(qb + i * 32), hi = lds_read_tr(qb + i * 32 + 4 * kPitchT);
+        fb[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+      } else {
+        fb[i] = *reinterpret_cast<const u32x4*>(qb + i * 32 * 8);
       }
     }
   };
@@ -345,88 +320,39 @@ __global__ __launch_bounds__(W8 ? 2 * kThreads : kThreads) void gemm_kernel(cons
   //                cur+3, 16 MFMAs on the second set.
   // Loads and LDS stores are unconditional, so every path has the same number
   // of loads in flight and the waits can count.
-  // Inside each half the 16 MFMAs and the half's memory instructions are one
-  // scheduling region, interleaved by sched_group_barrier: one MFMA, then one
-  // LDS write or global load, then one LDS read.  An MFMA occupies the matrix
-  // pipe for 8 passes while the wave may issue other instructions, and a wave
-  // issues in order -- memory instructions bunched in front of the MFMAs leave
-  // the matrix pipe idle while they issue (one or two waves per SIMD: hardly anybody else
-  // feeds it).
-#define MEGA_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-  // What the barrier waits for goes first: the fragment reads of this slab
-  // (their buffer is overwritten after the barrier) under the first four
-  // MFMAs, the LDS writes of the next slab under the next eight; the global
-  // loads (nobody waits for them here) go under the MFMAs of the second half,
-  // behind the fragment reads for the next slab.
-  constexpr int kFragReads = (TA ? 2 : 1) + (TB ? JN / 2 : (JN + 3) / 4);  // LDS reads per MFMA of the first four
-  constexpr int kRest = 4 * JN - 4 - 2 * NL;  // MFMAs of a half with nothing to carry
 #define MEGA_GEMM_STEP(R, CA, CB, NA, NB)                                  \
   {                                                                        \
     const int cur = it + (R);                                              \
     fread(fa1, fb1, 1, cur & 1);                                           \
     sstore(NA, NB, cur + 1);                                               \
     mma(fa0, fb0);                                                         \
-    _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
-      MEGA_SGB(0x008, 1);                                                  \
-      MEGA_SGB(0x100, kFragReads);                                         \
-    }                                                                      \
-    _Pragma("unroll") for (int sg = 0; sg < 2 * NL; ++sg) {                \
-      MEGA_SGB(0x008, 1);                                                  \
-      MEGA_SGB(0x200, 1);                                                  \
-    }                                                                      \
-    if (kRest > 0) MEGA_SGB(0x008, kRest);                                 \
-    __builtin_amdgcn_sched_barrier(0);                                     \
     lds_barrier();                                                         \
     fread(fa0, fb0, 0, (cur + 1) & 1);                                     \
-    gload(CA, CB, cur + RING);                                             \
+    gload(CA, CB, cur + kRing);                                            \
     mma(fa1, fb1);                                                         \
-    _Pragma("unroll") for (int sg = 0; sg < 4; ++sg) {                     \
-      MEGA_SGB(0x008, 1);                                                  \
-      MEGA_SGB(0x100, kFragReads);                                         \
-    }                                                                      \
-    _Pragma("unroll") for (int sg = 0; sg < 2 * NL; ++sg) {                \
-      MEGA_SGB(0x008, 1);                                                  \
-      MEGA_SGB(0x020, 1);                                                  \
-    }                                                                      \
-    if (kRest > 0) MEGA_SGB(0x008, kRest);                                 \
-    __builtin_amdgcn_sched_barrier(0);                                     \
   }
   if (nslab > 0) {
     gload(ra0, rb0, 0);
     gload(ra1, rb1, 1);
     gload(ra2, rb2, 2);
-    if constexpr (RING == 4) gload(ra3, rb3, 3);
     sstore(ra0, rb0, 0);
     lds_barrier();
     fread(fa0, fb0, 0, 0);
     // ring slot R held slab cur, already written to LDS, so it is free for
     // slab cur + kRing
     int it = 0;
-    if constexpr (RING == 4) {
-      for (; it + 4 <= nslab; it += 4) {
-        MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
-        MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
-        MEGA_GEMM_STEP(2, ra2, rb2, ra3, rb3)
-        MEGA_GEMM_STEP(3, ra3, rb3, ra0, rb0)
-      }
-      if (it < nslab) MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
-      if (it + 1 < nslab) MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
-      if (it + 2 < nslab) MEGA_GEMM_STEP(2, ra2, rb2, ra3, rb3)
-    } else {
-      for (; it + kRing <= nslab; it += kRing) {
-        MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
-        MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
-        MEGA_GEMM_STEP(2, ra2, rb2, ra0, rb0)
-      }
-      if (it < nslab) MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
-      if (it + 1 < nslab) MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
+    for (; it + kRing <= nslab; it += kRing) {
+      MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
+      MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
+      MEGA_GEMM_STEP(2, ra2, rb2, ra0, rb0)
     }
+    if (it < nslab) MEGA_GEMM_STEP(0, ra0, rb0, ra1, rb1)
+    if (it + 1 < nslab) MEGA_GEMM_STEP(1, ra1, rb1, ra2, rb2)
     lds_barrier();  // every wave is done with the slab buffers before they are reused
   }
 #undef MEGA_GEMM_STEP
-#undef MEGA_SGB
 
-  // epilogue: stage the wave's 128 x 32 JN tile in LDS ([row][col], element type),
+  // epilogue: stage the wave's 128 x 128 tile in LDS ([row][col], element type),
   // then write it with 16-byte row segments.  The products are issued as
   // B-fragment x A-fragment, so a 32x32 MFMA tile holds C transposed: lane l has
   // row m = l % 32 and register r the column n = 8 (r / 4) + 4 (l / 32) + r % 4,
@@ -1527,55 +1453,35 @@ int launch_gemm_t(const GemmParams& p, int batch, hipStream_t s) {
   if (g >= kXcds) g -= g % kXcds;
   const dim3 grid(static_cast<unsigned>(g));
   const size_t lds = kGemmLds;
-  // Eight waves of 128 x 64 (two per SIMD, accumulators in the unified register
-  // file, a ring of four slabs) hide more latency than four of 128 x 128 with
-  // one per SIMD; MEGA_GEMM_W4=1 in the environment selects the latter for
-  // comparison.
-  const char* w4 = getenv("MEGA_GEMM_W4");
-  // MEGA_GEMM_DMA=0 keeps the slabs on the register path (for comparison)
-  const char* dma = getenv("MEGA_GEMM_DMA");
-  // products of two k-contiguous operands (S = Q K^T, dP = dY V^T) take slabs of 64 k;
-  // MEGA_GEMM_SLAB64=0 keeps slabs of 32 k for every product
-  const char* s64 = getenv("MEGA_GEMM_SLAB64");
-  bool slab64 = false;
-  if constexpr (!TA && !TB)
-    slab64 = fast && p.K % kSlab64 == 0 && !(w4 != nullptr && w4[0] == '1') && !(dma != nullptr && dma[0] == '0') &&
-             !(s64 != nullptr && s64[0] == '0');
-  // one k-contiguous and one k-major operand: A in slabs of 64 k (MEGA_GEMM_A64=0: slabs of 32 k for both)
-  const char* a64e = getenv("MEGA_GEMM_A64");
-  bool a64 = false;
-  if constexpr (!TA && TB)
-    a64 = fast && p.K % kSlab64 == 0 && !(w4 != nullptr && w4[0] == '1') && !(dma != nullptr && dma[0] == '0') &&
-          !(a64e != nullptr && a64e[0] == '0');
-  if (slab64) {
-    if constexpr (!TA && !TB) {
+  // Aligned operands: slabs from memory straight into LDS, eight waves of 128 x 64.  Products of
+  // two k-contiguous operands (S = Q K^T, dP = dY V^T) take slabs of 64 k; one k-contiguous and
+  // one k-major operand (P V, dS K) take A in slabs of 64 k and B in slabs of 32 k; the rest
+  // slabs of 32 k.
+  bool done = false;
+  if constexpr (!TA && !TB) {
+    if (fast && p.K % kSlab64 == 0) {
       MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma64_kernel<DT, TA, TB>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaLds));
       gemm_dma64_kernel<DT, TA, TB><<<grid, 2 * kThreads, kDmaLds, s>>>(q);
+      done = true;
     }
-  } else if (a64) {
-    if constexpr (!TA && TB) {
+  }
+  if constexpr (!TA && TB) {
+    if (fast && p.K % kSlab64 == 0) {
       MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_a64_kernel<DT>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kA64Lds));
       gemm_dma_a64_kernel<DT><<<grid, 2 * kThreads, kA64Lds, s>>>(q);
+      done = true;
     }
-  } else if (fast && !(w4 != nullptr && w4[0] == '1') && !(dma != nullptr && dma[0] == '0')) {
+  }
+  if (!done && fast) {
     MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<DT, TA, TB>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaLds));
     gemm_dma_kernel<DT, TA, TB><<<grid, 2 * kThreads, kDmaLds, s>>>(q);
-  } else if (fast && !(w4 != nullptr && w4[0] == '1')) {
-    const size_t lds8 = sizeof(uint16_t) * 8 * 128 * (64 + 8) > lds ? sizeof(uint16_t) * 8 * 128 * (64 + 8) : lds;
-    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, true, TA, TB, true>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds8));
-    gemm_kernel<DT, true, TA, TB, true><<<grid, 2 * kThreads, lds8, s>>>(q);
-  } else if (fast) {
-    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, true, TA, TB, false>),
+  } else if (!done) {
+    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, TA, TB>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    gemm_kernel<DT, true, TA, TB, false><<<grid, kThreads, lds, s>>>(q);
-  } else {
-    MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<DT, false, TA, TB, false>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    gemm_kernel<DT, false, TA, TB, false><<<grid, kThreads, lds, s>>>(q);
+    gemm_kernel<DT, TA, TB><<<grid, kThreads, lds, s>>>(q);
   }
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
@@ -1804,8 +1710,7 @@ extern "C" int mega_linear_weight_grad(const void* dy, const void* x, int dtype,
   g.M = (int)n_out; g.N = (int)n_in; g.K = (int)tokens;
   g.lda = n_out; g.ldb = n_in; g.ldc = n_in; g.ta = 1; g.tb = 1;
   g.nh = 1; g.alpha = 1.f;
-  const char* ng = getenv("MEGA_GEMM_NGROUP");
-  g.n_group = ng != nullptr ? atoi(ng) : 8;
+  g.n_group = 8;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return dtype == MEGA_BF16 ? launch_gemm<MEGA_BF16>(g, 1, s) : launch_gemm<MEGA_F16>(g, 1, s);
 }

@@ -484,7 +484,7 @@ extern "C" int mega_ema_weight_fwd(const float* p, const float* log_q,
   const cf* lq = reinterpret_cast<const cf*>(log_q);
   const cf* gm = reinterpret_cast<const cf*>(gamma);
   const bool vec = (L % 4 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0);
-  if (N <= 16 && (L + 1023) / 1024 <= 32 * 65535 && getenv("MEGA_EMA_FWD_VALU") == nullptr) {
+  if (N <= 16 && (L + 1023) / 1024 <= 32 * 65535) {
     const int64_t hrows = (L + 1023) / 1024;
     dim3 grid(static_cast<unsigned>(D), static_cast<unsigned>((hrows + 31) / 32));
     ema_weight_fwd_mfma_kernel<<<grid, kThreads, 0, s>>>(p, lq, gm, (int)N, L, w);
@@ -527,8 +527,7 @@ extern "C" int mega_ema_weight_bwd(const float* dw, const float* p,
   cf* dgc = reinterpret_cast<cf*>(dgamma);
   const bool vec = (L % 2 == 0) && (reinterpret_cast<uintptr_t>(dw) % 8 == 0);
   dim3 grid(static_cast<unsigned>(D));
-  if (N <= 16 && L >= 1 && reinterpret_cast<uintptr_t>(dw) % 16 == 0 && L % 4 == 0 &&
-      getenv("MEGA_EMA_BWD_VALU") == nullptr) {
+  if (N <= 16 && L >= 1 && reinterpret_cast<uintptr_t>(dw) % 16 == 0 && L % 4 == 0) {
     ema_weight_bwd_mfma_kernel<<<grid, kThreads, 0, s>>>(dw, p, lq, gm, (int)N, L, dp, dqc, dgc);
   } else if (N <= 16) {
     if (vec)

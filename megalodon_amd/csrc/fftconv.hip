@@ -544,8 +544,7 @@ int fftconv_bwd_impl(const char* who, const void* dy, const void* x, int dtype, 
     return MEGA_OK;
   }
   if (fftm::applicable(dtype, L, dy, x, dx) && reinterpret_cast<uintptr_t>(k) % 16 == 0 &&
-      reinterpret_cast<uintptr_t>(dk) % 16 == 0 && f16_stages_enabled() &&
-      getenv("MEGA_FFTCONV_SPLIT_BWD") == nullptr)
+      reinterpret_cast<uintptr_t>(dk) % 16 == 0 && f16_stages_enabled())
     return fftm::launch_backward(dtype, dy, x, k, dx, dk, B, D, L, omega, s);
   int rc = dispatch_conv<0>(dtype, dy, k, dx, B, D, L, 1, omega, s);
   if (rc != MEGA_OK) return rc;

@@ -14,8 +14,10 @@
   pass; everything must be finite.
 
 Bars: <= 2e-2 for bfloat16 tensors, <= 1e-4 for float32 tensors computed by a
-single operator chain (the CEMA parameter gradients), <= 5e-2 through the
-whole block (about 15 bf16-rounded operators)."""
+single operator chain (the CEMA parameter gradients); through the whole block
+(about 15 bf16-rounded operators) <= 2e-2 on the output, dx and the CEMA parameter
+gradients and <= 3e-2 on the other parameter gradients (the measured errors are
+printed, run with -s)."""
 import pytest
 import torch
 
@@ -151,10 +153,13 @@ def test_config4_block_prefix_equals_small_run_equals_oracle():
     want = oblock.mega_block_forward(p64, xo, num_heads=CFG4["num_heads"], ndim=CFG4["cema_ndim"],
                                      chunk_size=CFG4["chunk_size"], groups=CFG4["norm_num_groups"])
     want.backward(dy[:, :P].double())
-    assert rel_err(out_small, want) <= 5e-2
-    assert rel_err(xs.grad, xo.grad) <= 5e-2
+    errs = {"out": rel_err(out_small, want), "dx": rel_err(xs.grad, xo.grad)}
     for n_ in checked:
-        assert rel_err(small_grads[n_], p64[n_].grad) <= 5e-2, n_
+        errs["d " + n_] = rel_err(small_grads[n_], p64[n_].grad)
+    print("config-4 block, first 256 tokens, errors vs float64 oracle:", {k: f"{v:.2e}" for k, v in errs.items()})
+    tight = lambda k: k in ("out", "dx") or ".cema." in k
+    bad = {k: v for k, v in errs.items() if not v <= (2e-2 if tight(k) else 3e-2)}
+    assert not bad, bad
 
 
 def test_config4_block_two_piece_cached_pass_equals_single_pass():
