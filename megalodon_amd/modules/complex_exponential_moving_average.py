@@ -89,7 +89,7 @@ class MultiHeadComplexEMA(nn.Module):
             # coefficients cached for evaluation (:100-101,119-125); every branch below does the same
             self._coeffs = None
         stateless = hx is None and not compute_last_state
-        needs_grad = torch.is_grad_enabled() and (x.requires_grad or self.alpha.requires_grad
+        needs_grad = torch.is_grad_enabled() and (x.requires_grad or any(t.requires_grad for t in self.parameters())
                                                   or (hx is not None and hx.requires_grad))
         if self.alpha.is_cuda and os.environ.get("MEGA_CEMA_FFT") is None:
             # the layer as a chunked recurrence on the matrix cores (no kernel row, no

@@ -1,8 +1,12 @@
 """The hot operators under HIP graph capture: a captured launch sequence is
 replayed several times, with eager work and synchronisations of the program's
 own between the replays, and every replay is held against the eager result.
-None of the captured entry points allocates, synchronises or records a memset
-(scratch is cleared by kernels), which is what makes them capturable."""
+None of the captured C entry points allocates, synchronises or records a memset
+(scratch is cleared by kernels).  The Python shim does allocate -- outputs, and
+one TimestepNorm workspace per (device, stream, direction) -- so the capture runs
+on the stream the warm-up ran on: the workspace then exists before the capture
+and only the outputs come from the graph's private pool.  Graphs captured on one
+stream share that stream's workspace, so their replays must not overlap."""
 import pytest
 import torch
 
@@ -25,7 +29,7 @@ def _replay_and_compare(build, inputs, refresh):
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
+    with torch.cuda.graph(g, stream=side):
         outs = build()
     for i in (0, 1, 2, 1):
         refresh(i)
