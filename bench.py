@@ -42,8 +42,28 @@ CFG4 = dict(model_dim=4096, z_dim=1024, value_dim=8192, num_heads=4, cema_ndim=1
 
 
 def host_cores():
+    """Threads for the CPU baselines: the cores this process may run on (OMP_NUM_THREADS, when the
+    environment sets it, is the share of the box a job is given and wins)."""
     env = os.environ.get("OMP_NUM_THREADS")
-    return int(env) if env else min(os.cpu_count() or 1, 16)
+    if env:
+        return int(env)
+    try:
+        return len(os.sched_getaffinity(0))
+    except AttributeError:
+        return os.cpu_count() or 1
+
+
+def host_info():
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"nproc": os.cpu_count(), "cpu_model": model, "omp_num_threads_env": os.environ.get("OMP_NUM_THREADS")}
 
 
 # --------------------------------------------------------------------------- CPU baselines
@@ -144,19 +164,88 @@ def cpu_attention(cores, budget_s=12.0):
                       f"scaled by {pairs}"}
 
 
-def cpu_block(cores, budget_s=25.0):
-    """Config 4 on the host: the float64 composition of the oracles (TimestepNorm
-    closed form, CEMA kernel + torch.fft convolution, matmul + softmax attention,
-    F.linear projections), forward + backward by autograd, on a prefix of the
-    sequence (every stage but attention is linear in L; attention is cheaper per
-    token below one chunk, so the figure flatters the CPU)."""
+def cpu_block_forward(p, x, cfg):
+    """One block on CPU tensors in float32, the reference's CPU arithmetic: TimestepNorm and the CEMA
+    kernel row through the C/OpenMP restatements of its loop nests (csrc/ops/timestep_norm.cc:218-450,
+    csrc/ops/ema_parameters.cc:17-98), the convolution through torch.fft (fused_ops/fftconv.py:30-75),
+    attention as matmul + causal mask + float32 softmax + matmul
+    (modules/moving_average_gated_attention.py:116-129), projections and norms through
+    torch.nn.functional; differentiable.  `p` is keyed like MegaBlock.named_parameters(); x (1, L, D)
+    with L at most one chunk."""
+    import math
     import torch
-    from oracle import block as oblock
+    import torch.nn.functional as F
+    from oracle import native
+    lib = native.port()
+    _, Ls, D = x.shape
+    Z, H = cfg["z_dim"], cfg["value_dim"]
+    N, NH, G = cfg["cema_ndim"], cfg["num_heads"], cfg["norm_num_groups"]
+    assert x.shape[0] == 1 and Ls <= cfg["chunk_size"]
+    pc, pm, pv = torch.zeros(1, dtype=torch.int64), torch.zeros(1, G), torch.ones(1, G)
+
+    class TimestepNormCPU(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x_, gamma, beta):
+            y, count, mean, var, cm, cr = native.group_timestep_norm_fwd(lib, "oracle_", x_, pc, pm, pv, gamma, beta,
+                                                                         None, G, 1e-5)
+            ctx.save_for_backward(x_, count, cm, cr, gamma)
+            return y
+
+        @staticmethod
+        def backward(ctx, gy):
+            x_, count, cm, cr, gamma = ctx.saved_tensors
+            dx, _, _, dgam, dbet = native.group_timestep_norm_bwd(lib, "oracle_", gy.contiguous(), torch.zeros(1, G),
+                                                                  torch.zeros(1, G), x_, pm, count, cm, cr, gamma, None, G)
+            return dx, dgam, dbet
+
+    class EmaWeightCPU(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, pp, q, gam):
+            ctx.save_for_backward(pp, q, gam)
+            return native.ema_weight_fwd(lib, "oracle_", pp, q.log(), gam, Ls)
+
+        @staticmethod
+        def backward(ctx, gk):
+            pp, q, gam = ctx.saved_tensors
+            # the operator returns the gradients with respect to (p, q, gamma), as the reference's does
+            dp, dq, dg = native.ema_weight_bwd(lib, "oracle_", gk.contiguous(), pp, q.log(), gam)
+            return dp.view_as(pp), dq.view_as(q), dg.view_as(gam)
+
+    rms = lambda t, w: t * torch.rsqrt((t * t).mean(-1, keepdim=True) + 1e-5) * (1.0 if w is None else w + 1.0)
+    tsn = TimestepNormCPU.apply(x, p["mega.timenorm.weight"] + 1.0, p["mega.timenorm.bias"])
+    pp = torch.sigmoid(p["mega.cema.alpha"])
+    ang = torch.sigmoid(p["mega.cema.theta"]) * (2 * math.pi / N) * torch.arange(1, N + 1).view(1, N, 1)
+    q = torch.polar(1.0 - pp * torch.sigmoid(p["mega.cema.delta"]), ang)
+    k = EmaWeightCPU.apply(pp, q.squeeze(-1), torch.view_as_complex(p["mega.cema.gamma"]) * math.sqrt(1.0 / N))
+    xt = tsn.transpose(1, 2)
+    n = 2 * (Ls if (Ls & (Ls - 1)) == 0 else (1 << Ls.bit_length()))
+    conv = torch.fft.irfft(torch.fft.rfft(xt, n=n) * torch.fft.rfft(k, n=n, norm="forward"), n=n, norm="forward")[..., :Ls]
+    mx = rms((conv + xt * p["mega.cema.omega"]).transpose(1, 2), p["mega.rmsnorm.weight"])
+    zh = Z // NH
+    z = rms(F.linear(mx, p["mega.wz.weight"], p["mega.wz.bias"]).view(1, Ls, NH, zh), None).view(1, Ls, Z)
+    z = z.unsqueeze(2) * ((p["mega.gamma"] + 1.0) / math.sqrt(zh)) + p["mega.beta"]
+    qq, kk = (t.reshape(1, Ls, NH, zh).transpose(1, 2) for t in torch.unbind(z, dim=2))
+    v = F.silu(F.linear(tsn, p["mega.wv.weight"], p["mega.wv.bias"])).view(1, Ls, NH, H // NH).transpose(1, 2)
+    rr = F.silu(F.linear(mx, p["mega.wr.weight"], p["mega.wr.bias"]))
+    mask = torch.full((Ls, Ls), float("-inf")).triu(1)
+    prob = torch.softmax(torch.matmul(qq, kk.transpose(2, 3)) + mask, dim=-1, dtype=torch.float32)
+    attn = torch.matmul(prob, v).transpose(1, 2).reshape(1, Ls, H) * rr
+    y1 = F.linear(mx, p["mega.wh1.weight"], p["mega.wh1.bias"]) + F.linear(attn, p["mega.wh2.weight"]) + x
+    nn_ = F.layer_norm(y1, (D,), p["nffn.norm.weight"] + 1.0, p["nffn.norm.bias"], 1e-5)
+    hid = F.silu(F.linear(nn_, p["nffn.fc1.weight"])) * F.linear(nn_, p["nffn.fc3.weight"])
+    return F.linear(hid, p["nffn.fc2.weight"]) + x
+
+
+def cpu_block(cores, budget_s=25.0):
+    """Config 4 on the host in float32 (cpu_block_forward, backward by autograd) on a prefix of the
+    sequence: every stage but attention is linear in L and attention is cheaper per token below one
+    chunk, so the figure flatters the CPU."""
+    import torch
     Ls = 1024
     g = torch.Generator().manual_seed(1004)
     D, Z, H, F_ = CFG4["model_dim"], CFG4["z_dim"], CFG4["value_dim"], CFG4["ffn_hidden_dim"]
     N = CFG4["cema_ndim"]
-    r = lambda *s: (torch.randn(*s, generator=g, dtype=torch.float64) * 0.02).requires_grad_(True)
+    r = lambda *s: (torch.randn(*s, generator=g) * 0.02).requires_grad_(True)
     p = {"mega.timenorm.weight": r(D), "mega.timenorm.bias": r(D), "mega.cema.alpha": r(D, N, 1),
          "mega.cema.delta": r(D, N, 1), "mega.cema.theta": r(D, 1, 1), "mega.cema.gamma": r(D, N, 2),
          "mega.cema.omega": r(D, 1), "mega.rmsnorm.weight": r(D), "mega.wz.weight": r(Z, D), "mega.wz.bias": r(Z),
@@ -164,20 +253,19 @@ def cpu_block(cores, budget_s=25.0):
          "mega.wh1.weight": r(D, D), "mega.wh1.bias": r(D), "mega.wh2.weight": r(D, H), "mega.gamma": r(2, Z),
          "mega.beta": r(2, Z), "nffn.norm.weight": r(D), "nffn.norm.bias": r(D), "nffn.fc1.weight": r(F_, D),
          "nffn.fc2.weight": r(D, F_), "nffn.fc3.weight": r(F_, D)}
-    x = (torch.rand(1, Ls, D, generator=g, dtype=torch.float64) * 2 - 1).requires_grad_(True)
-    dy = torch.randn(1, Ls, D, generator=g, dtype=torch.float64)
+    x = (torch.rand(1, Ls, D, generator=g) * 2 - 1).requires_grad_(True)
+    dy = torch.randn(1, Ls, D, generator=g)
 
     def step():
         for t in list(p.values()) + [x]:
             t.grad = None
-        out = oblock.mega_block_forward(p, x, num_heads=CFG4["num_heads"], ndim=N, chunk_size=CFG4["chunk_size"],
-                                        groups=CFG4["norm_num_groups"])
-        out.backward(dy)
+        cpu_block_forward(p, x, CFG4).backward(dy)
 
     dt, reps = _timed(step, budget_s, max_reps=3)
-    return {"value": Ls / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"the first {Ls} of 32768 tokens through the float64 oracle of the block "
-                      f"(oracle/block.py), {reps} rep(s), {dt:.2f} s each"}
+    return {"value": Ls / dt, "unit": "tokens/s", "cores": cores, "kind": "port", "dtype": "f32", **host_info(),
+            "sample": f"the first {Ls} of 32768 tokens of the block in float32 (C/OpenMP restatements of the reference's "
+                      f"TimestepNorm and ema_parameters loop nests, torch.fft convolution, matmul + softmax attention, "
+                      f"F.linear projections; autograd backward), {reps} rep(s), {dt:.2f} s each"}
 
 
 # --------------------------------------------------------------------------- GPU legs
@@ -345,9 +433,16 @@ def other_ops(torch, dev):
     aio = {k_: v_.to(dev) for k_, v_ in synthetic.attention_inputs(8, 4096, 4, 256, 2048, 1003).items()}
     pairs = 4096 * 4097 // 2
     f_fwd, f_bwd = 2 * pairs * (256 + 2048) * 32, 2 * pairs * (2 * 256 + 2 * 2048) * 32
-    ay, aw = ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True)
+    # forward as the modules run it (w goes to the backward pass only: the zeros right of the diagonal
+    # block stay unwritten), and as the operator-level call returns it (every row of w written to its
+    # end, as the reference's softmax does: 0.55 GB of zeros more)
+    ay, aw = ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True, lower_only=True)
+    ms = dev_ms(torch, lambda: ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True, lower_only=True), 50, warm=10)
+    other["attention_fwd"] = {"ms": ms, "TFLOPs": f_fwd / ms / 1e9, "frac_mfma_bf16": f_fwd / ms / 1e9 / 2516.6,
+                              "w": "lower blocks only (module path)"}
     ms = dev_ms(torch, lambda: ops.attention_fwd(aio["q"], aio["k"], aio["v"], 1.0, 0.0, True), 50, warm=10)
-    other["attention_fwd"] = {"ms": ms, "TFLOPs": f_fwd / ms / 1e9, "frac_mfma_bf16": f_fwd / ms / 1e9 / 2516.6}
+    other["attention_fwd_full_w"] = {"ms": ms, "TFLOPs": f_fwd / ms / 1e9, "frac_mfma_bf16": f_fwd / ms / 1e9 / 2516.6,
+                                     "w": "every row to its end (operator-level call)"}
     ms = dev_ms(torch, lambda: ops.attention_bwd(aio["dy"], aio["q"], aio["k"], aio["v"], aw, 1.0, True), 50, warm=10)
     other["attention_bwd"] = {"ms": ms, "TFLOPs": f_bwd / ms / 1e9, "frac_mfma_bf16": f_bwd / ms / 1e9 / 2516.6}
     del aio, ay, aw
@@ -417,6 +512,7 @@ def main():
         torch.set_num_threads(cores)
         os.environ.setdefault("OMP_NUM_THREADS", str(cores))
         result["cpu_baseline"] = cpu_block(cores)
+        result["host"] = host_info()
         result["cpu_ops"] = {"cema_conv_config1": cpu_cema(1, 4096, 16, 32768, 1001, cores),
                              "timestep_norm_config2": cpu_timestep_norm(cores),
                              "attention_config3": cpu_attention(cores)}
