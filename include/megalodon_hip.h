@@ -597,16 +597,33 @@ int mega_cema_scan_bwd(const void* dy, const void* x, int dtype, const float* p,
                        int64_t D, int64_t N, int64_t L, void* dx, float* dp, float* dq,
                        float* dgamma, float* domega, void* stream);
 
+/* The same backward for a forward that had a carried state h0 (B, D, N)
+ * complex64: the state adds b[t] = Re sum_n gamma_n q_n^(t+1) h0_n to the output
+ * (csrc/ops/ema_parameters.cc:56-77), and its backward
+ * (ema_parameters.cc:100-117,158-188) adds conj(q h0 R0) to dgamma and
+ * conj(gamma h0 (R0 + q R0')) to dq, with R0 = sum_t dy[t] q^t, R0' = dR0/dq --
+ * what the kernel's reverse scan has carried to the start of the row -- and
+ * returns dh0 = conj(gamma q R0), (B, D, N) complex64 (NULL: not wanted).
+ * h0 == NULL is mega_cema_scan_bwd.  The gradient of a last state taken from
+ * the forward is a separate operator (ema_hidden_bwd, csrc/ops/ema_hidden.cc:63-159). */
+int mega_cema_scan_bwd_state(const void* dy, const void* x, int dtype, const float* p,
+                             const float* log_q, const float* gamma, const float* omega,
+                             const float* h0, int64_t B, int64_t D, int64_t N, int64_t L, void* dx,
+                             float* dp, float* dq, float* dgamma, float* domega, float* dh0,
+                             void* stream);
+
 /* mega_cema_scan_bwd on bfloat16 dy and x with dx written in float32, or not at
  * all when `dx` is NULL.  The backward is linear in dy and, for the parameter
  * gradients, in x: a caller with float16 or float32 tensors (the reference's
  * operators take them, fused_ops/fftconv.py:37-44 upcasts to float32) runs
  * this on the bfloat16 pieces of dy and x and adds the results up
- * (extension.py:cema_scan_bwd does). */
+ * (extension.py:cema_scan_bwd does); h0 / dh0 as in mega_cema_scan_bwd_state, to be
+ * passed with the pieces of dy and the leading piece of x only (the state's terms
+ * do not depend on x). */
 int mega_cema_scan_bwd_wide(const void* dy, const void* x, const float* p, const float* log_q,
-                            const float* gamma, const float* omega, int64_t B, int64_t D,
-                            int64_t N, int64_t L, float* dx, float* dp, float* dq, float* dgamma,
-                            float* domega, void* stream);
+                            const float* gamma, const float* omega, const float* h0, int64_t B,
+                            int64_t D, int64_t N, int64_t L, float* dx, float* dp, float* dq,
+                            float* dgamma, float* domega, float* dh0, void* stream);
 
 /* ------------------------------------------------------------------------
  * Streaming reference kernel for measurements (no counterpart in the

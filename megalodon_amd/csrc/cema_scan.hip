@@ -617,8 +617,9 @@ template <int DT, bool DX32>
 __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
     const void* __restrict__ dy, const void* __restrict__ x, void* __restrict__ dx,
     const float* __restrict__ p, const cf* __restrict__ log_q, const cf* __restrict__ gamma,
-    const float* __restrict__ omega, float* __restrict__ dp, cf* __restrict__ dq,
-    cf* __restrict__ dgamma, float* __restrict__ domega, int64_t rows, int D, int N, int64_t L) {
+    const float* __restrict__ omega, const cf* __restrict__ h0, float* __restrict__ dp, cf* __restrict__ dq,
+    cf* __restrict__ dgamma, float* __restrict__ domega, cf* __restrict__ dh0, int64_t rows, int D, int N,
+    int64_t L) {
   static_assert(XOp<DT>::XP == 1, "the backward kernel takes bfloat16 rows");
   constexpr int NC = kBwdNC, CPS = kBwdCPS;
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -891,8 +892,27 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
       const float pp = sm.pn[n];
       dp[row * N + n] = A.x * gm.x - A.y * gm.y;
       const cf t = cmul(Bq, cf{pp * gm.x, pp * gm.y});
-      dq[row * N + n] = cf{t.x, -t.y};
-      dgamma[row * N + n] = cf{A.x * pp, -A.y * pp};
+      cf dqv{t.x, -t.y}, dgv{A.x * pp, -A.y * pp};
+      if (h0 != nullptr) {
+        // A carried state h0 adds b[t] = Re(gamma q^(t+1) h0) to the output (ema_parameters.cc:56-77).
+        // With R0 = sum_t dy[t] q^t and R0' = dR0 / dq -- what the reverse scan has carried to the
+        // start of the row -- its gradients are (ema_parameters.cc:158-188, PyTorch's convention)
+        //   dgamma += conj(q h0 R0),  dq += conj(gamma h0 (R0 + q R0')),  dh0 = conj(gamma q R0).
+        const cf r0 = sm.carry[cur][0][n], r0d = sm.carry[cur][1][n];
+        const cf h = h0[row * N + n];
+        const cf e1 = cmul(cmul(qq, h), r0);
+        dgv.x += e1.x;
+        dgv.y -= e1.y;
+        const cf e2 = cmul(cmul(gm, h), cadd(r0, cmul(qq, r0d)));
+        dqv.x += e2.x;
+        dqv.y -= e2.y;
+        if (dh0 != nullptr) {
+          const cf e3 = cmul(cmul(gm, qq), r0);
+          dh0[row * N + n] = cf{e3.x, -e3.y};
+        }
+      }
+      dq[row * N + n] = dqv;
+      dgamma[row * N + n] = dgv;
     }
     // the skip term sat on the diagonal of K, not in M: domega = sum dy x = dkin[0]
     if (tid == 0) domega[row] = sm.dkin[0];
@@ -1157,8 +1177,8 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
 
 template <bool DX32>
 int launch_bwd(const void* dy, const void* x, void* dx, const float* p, const cf* log_q,
-               const cf* gamma, const float* omega, float* dp, cf* dq, cf* dgamma, float* domega,
-               int64_t B, int64_t D, int64_t N, int64_t L, hipStream_t stream) {
+               const cf* gamma, const float* omega, const cf* h0, float* dp, cf* dq, cf* dgamma, float* domega,
+               cf* dh0, int64_t B, int64_t D, int64_t N, int64_t L, hipStream_t stream) {
   const int lds = static_cast<int>(sizeof(BwdSmem));
   MEGA_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&cema_scan_bwd_kernel<MEGA_BF16, DX32>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -1168,7 +1188,7 @@ int launch_bwd(const void* dy, const void* x, void* dx, const float* p, const cf
   const int64_t rows = B * D, slots = 2 * static_cast<int64_t>(cus);  // two workgroups fit a compute unit
   const unsigned grid = static_cast<unsigned>(rows < slots ? rows : slots);
   cema_scan_bwd_kernel<MEGA_BF16, DX32><<<dim3(grid), kThreads, lds, stream>>>(
-      dy, x, dx, p, log_q, gamma, omega, dp, dq, dgamma, domega, rows, static_cast<int>(D),
+      dy, x, dx, p, log_q, gamma, omega, h0, dp, dq, dgamma, domega, dh0, rows, static_cast<int>(D),
       static_cast<int>(N), L);
   MEGA_CHECK_LAUNCH();
   return MEGA_OK;
@@ -1213,10 +1233,11 @@ extern "C" int mega_cema_scan_bwd_supported(int dtype, int64_t N, int64_t L) {
   return dtype == MEGA_BF16 && N >= 1 && N <= 16 && L >= 8 && L % 8 == 0;
 }
 
-extern "C" int mega_cema_scan_bwd(const void* dy, const void* x, int dtype, const float* p,
-                                  const float* log_q, const float* gamma, const float* omega,
-                                  int64_t B, int64_t D, int64_t N, int64_t L, void* dx, float* dp,
-                                  float* dq, float* dgamma, float* domega, void* stream) {
+extern "C" int mega_cema_scan_bwd_state(const void* dy, const void* x, int dtype, const float* p,
+                                        const float* log_q, const float* gamma, const float* omega,
+                                        const float* h0, int64_t B, int64_t D, int64_t N, int64_t L, void* dx,
+                                        float* dp, float* dq, float* dgamma, float* domega, float* dh0,
+                                        void* stream) {
   const char* who = "mega_cema_scan_bwd";
   MEGA_CHECK_ARG(dy && x && p && log_q && gamma && dx && dp && dq && dgamma && domega, "%s: null pointer", who);
   MEGA_CHECK_ARG(B >= 0 && D >= 0 && L >= 0, "%s: negative size", who);
@@ -1228,15 +1249,25 @@ extern "C" int mega_cema_scan_bwd(const void* dy, const void* x, int dtype, cons
   const auto al = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
   MEGA_CHECK_ARG(al(dy) && al(x) && al(dx), "%s: dy, x and dx must be 16-byte aligned", who);
   if (B == 0 || D == 0) return MEGA_OK;
+  MEGA_CHECK_ARG(dh0 == nullptr || h0 != nullptr, "%s: dh0 without h0", who);
   return launch_bwd<false>(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
-                           omega, dp, reinterpret_cast<cf*>(dq), reinterpret_cast<cf*>(dgamma), domega, B, D, N, L,
+                           omega, reinterpret_cast<const cf*>(h0), dp, reinterpret_cast<cf*>(dq),
+                           reinterpret_cast<cf*>(dgamma), domega, reinterpret_cast<cf*>(dh0), B, D, N, L,
                            static_cast<hipStream_t>(stream));
 }
 
+extern "C" int mega_cema_scan_bwd(const void* dy, const void* x, int dtype, const float* p,
+                                  const float* log_q, const float* gamma, const float* omega,
+                                  int64_t B, int64_t D, int64_t N, int64_t L, void* dx, float* dp,
+                                  float* dq, float* dgamma, float* domega, void* stream) {
+  return mega_cema_scan_bwd_state(dy, x, dtype, p, log_q, gamma, omega, nullptr, B, D, N, L, dx, dp, dq, dgamma,
+                                  domega, nullptr, stream);
+}
+
 extern "C" int mega_cema_scan_bwd_wide(const void* dy, const void* x, const float* p, const float* log_q,
-                                       const float* gamma, const float* omega, int64_t B, int64_t D,
-                                       int64_t N, int64_t L, float* dx, float* dp, float* dq, float* dgamma,
-                                       float* domega, void* stream) {
+                                       const float* gamma, const float* omega, const float* h0, int64_t B,
+                                       int64_t D, int64_t N, int64_t L, float* dx, float* dp, float* dq,
+                                       float* dgamma, float* domega, float* dh0, void* stream) {
   const char* who = "mega_cema_scan_bwd_wide";
   MEGA_CHECK_ARG(dy && x && p && log_q && gamma && dp && dq && dgamma && domega, "%s: null pointer", who);
   MEGA_CHECK_ARG(B >= 0 && D >= 0 && L >= 0, "%s: negative size", who);
@@ -1247,7 +1278,9 @@ extern "C" int mega_cema_scan_bwd_wide(const void* dy, const void* x, const floa
   const auto al = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
   MEGA_CHECK_ARG(al(dy) && al(x) && al(dx), "%s: dy, x and dx must be 16-byte aligned", who);
   if (B == 0 || D == 0) return MEGA_OK;
+  MEGA_CHECK_ARG(dh0 == nullptr || h0 != nullptr, "%s: dh0 without h0", who);
   return launch_bwd<true>(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
-                          omega, dp, reinterpret_cast<cf*>(dq), reinterpret_cast<cf*>(dgamma), domega, B, D, N, L,
+                          omega, reinterpret_cast<const cf*>(h0), dp, reinterpret_cast<cf*>(dq),
+                          reinterpret_cast<cf*>(dgamma), domega, reinterpret_cast<cf*>(dh0), B, D, N, L,
                           static_cast<hipStream_t>(stream));
 }

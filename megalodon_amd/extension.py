@@ -612,11 +612,11 @@ def fftconv_residual_bwd_saved(y_grad: torch.Tensor, spec_x: torch.Tensor, spec_
 # --------------------------------------------------------------------------
 def cema_scan_supported(x: torch.Tensor, ndim: int) -> bool:
     """Whether `cema_scan_fwd` takes this input: bfloat16 / float16 / float32 rows
-    on the GPU, at most 16 modes, a length that is a multiple of 8."""
-    if not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+    on the GPU, at most 32 modes (16 per launch), a length that is a multiple of 8."""
+    if not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float16, torch.float32) or ndim > 32:
         return False
     fn = _lib.load().mega_cema_scan_supported
-    return bool(fn(_lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(ndim), _lib.i64(x.shape[-1])))
+    return bool(fn(_lib.i32(_lib.dtype_code(x.dtype)), _lib.i64(min(ndim, 16)), _lib.i64(x.shape[-1])))
 
 
 def cema_scan_fwd(x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor, gamma: torch.Tensor,
@@ -637,7 +637,16 @@ def cema_scan_fwd(x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor, gamma: 
     pc = p.reshape(D, N).contiguous().float()
     lq, gm = _as_c64(log_q, "log_q").reshape(D, N), _as_c64(gamma, "gamma").reshape(D, N)
     wc = None if omega is None else omega.reshape(-1).contiguous().float()
-    hc = None if h0 is None else _as_c64(h0, "h0").reshape(B, D, N)
+    hc = None if h0 is None else _as_c64(h0, "h0").reshape(B, D, N).contiguous()
+    if N > 16:
+        # mode groups of at most 16: the outputs add up (float32 sum, one rounding), the states are per mode
+        ys, hs = None, []
+        for i, (lo, hi) in enumerate(_mode_groups(N)):
+            yi, hi_ = cema_scan_fwd(xc, pc[:, lo:hi], lq[:, lo:hi], gm[:, lo:hi], wc if i == 0 else None,
+                                    None if hc is None else hc[:, :, lo:hi], compute_last_state)
+            ys = yi.float() if ys is None else ys.add_(yi.float())
+            hs.append(hi_)
+        return ys.to(x.dtype), (torch.cat(hs, dim=2) if compute_last_state else None)
     y = torch.empty_like(xc)
     h_last = torch.empty((B, D, N), dtype=torch.complex64, device=dev) if compute_last_state else None
     with torch.cuda.device(dev):
@@ -654,10 +663,10 @@ def cema_scan_bwd_supported(x: torch.Tensor, ndim: int) -> bool:
     `cema_scan_bwd` itself also takes float32 rows (six launches on three pieces each),
     but that measured slower than the float32 FFT path (5.9 against 4.6 ms), so float32
     training is left there."""
-    if not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float16):
+    if not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float16) or ndim > 32:
         return False
     fn = _lib.load().mega_cema_scan_bwd_supported
-    return bool(fn(_lib.i32(_lib.dtype_code(torch.bfloat16)), _lib.i64(ndim), _lib.i64(x.shape[-1])))
+    return bool(fn(_lib.i32(_lib.dtype_code(torch.bfloat16)), _lib.i64(min(ndim, 16)), _lib.i64(x.shape[-1])))
 
 
 def _bf16_pieces(t: torch.Tensor, n: int = 2):
@@ -672,9 +681,9 @@ def _bf16_pieces(t: torch.Tensor, n: int = 2):
     return pieces
 
 
-def _cema_scan_bwd_wide(dy, x, pc, lq, gm, wc, want_dx: bool):
+def _cema_scan_bwd_wide(dy, x, pc, lq, gm, wc, hc, want_dx: bool):
     """One launch of the backward kernel on bfloat16 pieces: float32 dx (or none), per-row
-    parameter gradients summed over the batch."""
+    parameter gradients summed over the batch, dh0 (or none)."""
     dev = x.device
     B, D, L = x.shape
     N = pc.shape[1]
@@ -683,65 +692,89 @@ def _cema_scan_bwd_wide(dy, x, pc, lq, gm, wc, want_dx: bool):
     dq = torch.empty((B, D, N), dtype=torch.complex64, device=dev)
     dg = torch.empty((B, D, N), dtype=torch.complex64, device=dev)
     dw = torch.empty((B, D), dtype=torch.float32, device=dev)
+    dh = None if hc is None else torch.empty((B, D, N), dtype=torch.complex64, device=dev)
     with torch.cuda.device(dev):
         _lib.call("mega_cema_scan_bwd_wide", _lib.ptr(dy), _lib.ptr(x), _lib.ptr(pc), _lib.ptr(lq), _lib.ptr(gm),
-                  _lib.ptr(wc), _lib.i64(B), _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(dx), _lib.ptr(dp),
-                  _lib.ptr(dq), _lib.ptr(dg), _lib.ptr(dw), _lib.stream_ptr(dev))
-    return dx, [dp.sum(0), dq.sum(0), dg.sum(0), dw.sum(0)]
+                  _lib.ptr(wc), _lib.ptr(hc), _lib.i64(B), _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(dx),
+                  _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg), _lib.ptr(dw), _lib.ptr(dh), _lib.stream_ptr(dev))
+    return dx, [dp.sum(0), dq.sum(0), dg.sum(0), dw.sum(0)], dh
+
+
+def _mode_groups(N: int):
+    """The kernels hold 16 modes; the modes of a channel are independent and their outputs add up,
+    so more (the reference allows N <= 32, ema_parameters_kernel.cu:1026) run as several launches."""
+    return [(lo, min(lo + 16, N)) for lo in range(0, N, 16)]
 
 
 def cema_scan_bwd(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor,
-                  gamma: torch.Tensor, omega: Optional[torch.Tensor]):
-    """(dx, dp, dq, dgamma, domega) of ``cema_scan_fwd(x, p, log_q, gamma, omega)[0]``
-    (no carried state): dp (D, N) float32, dq and dgamma (D, N) complex64 in
-    the convention of ``ema_parameters_bwd`` (gradient w.r.t. q, conjugated),
-    domega (D,) float32."""
-    dev = _require_cuda(y_grad, x, p, log_q, gamma, omega)
+                  gamma: torch.Tensor, omega: Optional[torch.Tensor], h0: Optional[torch.Tensor] = None):
+    """(dx, dp, dq, dgamma, domega[, dh0]) of ``cema_scan_fwd(x, p, log_q, gamma, omega, h0)[0]``:
+    dp (D, N) float32, dq and dgamma (D, N) complex64 in the convention of
+    ``ema_parameters_bwd`` (gradient w.r.t. q, conjugated), domega (D,) float32 and,
+    when a carried state h0 (B, D, N) is given, its gradient dh0 (B, D, N) complex64
+    (ema_parameters.cc:158-188)."""
+    dev = _require_cuda(y_grad, x, p, log_q, gamma, omega, h0)
     B, D, L = x.shape
     N = p.shape[1]
     if y_grad.shape != x.shape or y_grad.dtype != x.dtype:
         raise RuntimeError("cema_scan_bwd: y_grad must match x in shape and dtype")
+    pc = p.reshape(D, N).contiguous().float()
+    lq, gm = _as_c64(log_q, "log_q").reshape(D, N), _as_c64(gamma, "gamma").reshape(D, N)
+    wc = None if omega is None else omega.reshape(-1).contiguous().float()
+    hc = None if h0 is None else _as_c64(h0, "h0").reshape(B, D, N).contiguous()
+    if N > 16:
+        # mode groups of at most 16: dx and domega add up (the skip term rides on the first group),
+        # the other gradients are per mode
+        parts = []
+        for i, (lo, hi) in enumerate(_mode_groups(N)):
+            parts.append(cema_scan_bwd(y_grad, x, pc[:, lo:hi], lq[:, lo:hi], gm[:, lo:hi], wc if i == 0 else None,
+                                       None if hc is None else hc[:, :, lo:hi]))
+        dx = parts[0][0].float()
+        for q_ in parts[1:]:
+            dx += q_[0].float()
+        out = [dx.to(x.dtype)] + [torch.cat([q_[j] for q_ in parts], dim=1) for j in (1, 2, 3)] + [parts[0][4]]
+        if hc is not None:
+            out.append(torch.cat([q_[5] for q_ in parts], dim=2))
+        return tuple(out)
     if x.dtype != torch.bfloat16:
         # The backward is linear in y_grad and, for the parameter gradients, in x as well: the
         # bfloat16 kernel runs on pairs of pieces (dy_i, x_j) with i + j below the number of
         # pieces (what is left out is 2^-16 of the result for float16, 2^-24 for float32); dx
-        # comes from the pairs with x_0, in float32, and is rounded once.
+        # comes from the pairs with x_0, in float32, and is rounded once; so do the terms of a
+        # carried state, which do not depend on x.
         n = 2 if x.dtype == torch.float16 else 3
         gp = [t.contiguous() for t in _bf16_pieces(y_grad, n)]
         xp = [t.contiguous() for t in _bf16_pieces(x, n)]
-        pc = p.reshape(D, N).contiguous().float()
-        lq, gm = _as_c64(log_q, "log_q").reshape(D, N), _as_c64(gamma, "gamma").reshape(D, N)
-        wc = None if omega is None else omega.reshape(-1).contiguous().float()
-        dx_sum, grads = None, None
+        dx_sum, grads, dh_sum = None, None, None
         for i in range(n):
             for j in range(n - i):
-                dxi, g = _cema_scan_bwd_wide(gp[i], xp[j], pc, lq, gm, wc, want_dx=(j == 0))
+                dxi, g, dh = _cema_scan_bwd_wide(gp[i], xp[j], pc, lq, gm, wc, hc if j == 0 else None, want_dx=(j == 0))
                 if dxi is not None:
                     dx_sum = dxi if dx_sum is None else dx_sum.add_(dxi)
+                if dh is not None:
+                    dh_sum = dh if dh_sum is None else dh_sum.add_(dh)
                 grads = g if grads is None else [a + b for a, b in zip(grads, g)]
-        return (dx_sum.to(x.dtype), *grads)
+        out = (dx_sum.to(x.dtype), *grads)
+        return out if hc is None else out + (dh_sum,)
 
     def aligned(t):
         t = t.contiguous()
         return t if t.data_ptr() % 16 == 0 else t.clone(memory_format=torch.contiguous_format)
 
     dy, xc = aligned(y_grad), aligned(x)
-    pc = p.reshape(D, N).contiguous().float()
-    lq, gm = _as_c64(log_q, "log_q").reshape(D, N), _as_c64(gamma, "gamma").reshape(D, N)
-    wc = None if omega is None else omega.reshape(-1).contiguous().float()
     dx = torch.empty_like(xc)
     dp = torch.empty((B, D, N), dtype=torch.float32, device=dev)
     dq = torch.empty((B, D, N), dtype=torch.complex64, device=dev)
     dg = torch.empty((B, D, N), dtype=torch.complex64, device=dev)
     dw = torch.empty((B, D), dtype=torch.float32, device=dev)
+    dh = None if hc is None else torch.empty((B, D, N), dtype=torch.complex64, device=dev)
     with torch.cuda.device(dev):
-        _lib.call("mega_cema_scan_bwd", _lib.ptr(dy), _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
-                  _lib.ptr(pc), _lib.ptr(lq), _lib.ptr(gm), _lib.ptr(wc), _lib.i64(B), _lib.i64(D), _lib.i64(N),
-                  _lib.i64(L), _lib.ptr(dx), _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg), _lib.ptr(dw),
-                  _lib.stream_ptr(dev))
-    if B == 1:
-        return dx, dp[0], dq[0], dg[0], dw[0]
-    return dx, dp.sum(0), dq.sum(0), dg.sum(0), dw.sum(0)
+        _lib.call("mega_cema_scan_bwd_state", _lib.ptr(dy), _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
+                  _lib.ptr(pc), _lib.ptr(lq), _lib.ptr(gm), _lib.ptr(wc), _lib.ptr(hc), _lib.i64(B), _lib.i64(D),
+                  _lib.i64(N), _lib.i64(L), _lib.ptr(dx), _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg), _lib.ptr(dw),
+                  _lib.ptr(dh), _lib.stream_ptr(dev))
+    out = (dx, dp[0], dq[0], dg[0], dw[0]) if B == 1 else (dx, dp.sum(0), dq.sum(0), dg.sum(0), dw.sum(0))
+    return out if hc is None else out + (dh,)
 
 
 # --------------------------------------------------------------------------

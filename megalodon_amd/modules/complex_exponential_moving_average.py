@@ -15,6 +15,7 @@ import torch
 from torch import nn
 
 from .. import extension as megalodon_ops
+from ..fused_ops.cema_scan import cema_scan_state
 from ..fused_ops import (cema_kernel, cema_scan, cema_scan_applicable, ema_hidden, ema_parameters,
                          fftconv_residual)
 
@@ -62,6 +63,7 @@ class MultiHeadComplexEMA(nn.Module):
         sigmoid(theta) 2 pi / N (D, N, 1) complex; gamma_hat = gamma / sqrt(N)
         (D, N) complex (:100-117)."""
         self._coeffs = None
+        self._coeffs_kernel = None
         n_modes = self.ndim
         p = torch.sigmoid(self.alpha.float())
         base = torch.sigmoid(self.theta.float()) * (2 * math.pi / n_modes)
@@ -76,6 +78,19 @@ class MultiHeadComplexEMA(nn.Module):
             self._coeffs = self._calc_coeffs()
         return self._coeffs
 
+    @torch.no_grad()
+    def _kernel_coeffs(self):
+        """(p, log q, gamma_hat) from the coefficient kernel, for the branches that need no gradient;
+        cached in evaluation mode beside (and dropped with) the coefficients of `coeffs()`."""
+        make = lambda: megalodon_ops.cema_coeffs_fwd(self.alpha.float(), self.delta.float(), self.theta.float(),
+                                                     self.gamma.float())
+        if self.training:
+            return make()
+        self.coeffs()
+        if getattr(self, "_coeffs_kernel", None) is None:
+            self._coeffs_kernel = make()
+        return self._coeffs_kernel
+
     def forward(
         self,
         x: torch.Tensor,
@@ -88,6 +103,7 @@ class MultiHeadComplexEMA(nn.Module):
             # the reference's training forward goes through _calc_coeffs(), which drops the
             # coefficients cached for evaluation (:100-101,119-125); every branch below does the same
             self._coeffs = None
+            self._coeffs_kernel = None
         stateless = hx is None and not compute_last_state
         needs_grad = torch.is_grad_enabled() and (x.requires_grad or any(t.requires_grad for t in self.parameters())
                                                   or (hx is not None and hx.requires_grad))
@@ -99,9 +115,15 @@ class MultiHeadComplexEMA(nn.Module):
                 out = cema_scan(x, self.alpha.float(), self.delta.float(), self.theta.float(), self.gamma.float(),
                                 self.omega)
                 return out, None
+            if not stateless and needs_grad and cema_scan_applicable(x, self.ndim, True):
+                # carried state in, last state out, all differentiable (dh0 included)
+                return cema_scan_state(x, self.alpha.float(), self.delta.float(), self.theta.float(),
+                                       self.gamma.float(), self.omega, hx, compute_last_state)
             if not stateless and not needs_grad and cema_scan_applicable(x, self.ndim, False):
-                p, q, gamma = self.coeffs()
-                return megalodon_ops.cema_scan_fwd(x, p, q.log(), gamma, self.omega, hx, compute_last_state)
+                # log q from the coefficient kernel, the one the stateless branch uses: a prefill
+                # and its carried continuation see the same decay rates
+                p, log_q, gamma = self._kernel_coeffs()
+                return megalodon_ops.cema_scan_fwd(x, p, log_q, gamma, self.omega, hx, compute_last_state)
         if stateless and self.alpha.is_cuda:
             # no carried state: coefficients and kernel as one autograd node
             # (two launches per direction instead of the coefficient graph)
