@@ -375,6 +375,27 @@ def cema_leg(torch, dev, steps, warmup, copy_calibration):
     finally:
         os.environ.pop("MEGA_CEMA_FFT", None)
         os.environ.pop("MEGA_FFTCONV_F16_STAGES", None)
+    # the same layer step on float32 rows: the recurrence kernels on two bfloat16 pieces per tensor
+    # (16 significant bits, parameter gradients within 1e-4), three backward launches
+    x32 = io["x"].float().to(dev).requires_grad_(True)
+    dy32 = io["dy"].float().to(dev)
+
+    def step32():
+        x32.grad = None
+        for prm in layer.parameters():
+            prm.grad = None
+        out, _ = layer(x32, None, False)
+        out.backward(dy32)
+
+    for _ in range(2):
+        step32()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n_alt):
+        step32()
+    torch.cuda.synchronize()
+    res["float32_rows"] = {"ms_per_step": (time.perf_counter() - t0) / n_alt * 1e3, "steps": n_alt}
+    del x32, dy32
     if copy_calibration:
         src = torch.ones(1 << 29, dtype=torch.bfloat16, device=dev)
         dst = torch.empty_like(src)

@@ -613,7 +613,7 @@ int mega_cema_scan_bwd_state(const void* dy, const void* x, int dtype, const flo
                              void* stream);
 
 /* mega_cema_scan_bwd on bfloat16 dy and x with dx written in float32, or not at
- * all when `dx` is NULL.  The backward is linear in dy and, for the parameter
+ * all when `dx` is NULL; with `accumulate_dx` the launch adds to what dx holds.  The backward is linear in dy and, for the parameter
  * gradients, in x: a caller with float16 or float32 tensors (the reference's
  * operators take them, fused_ops/fftconv.py:37-44 upcasts to float32) runs
  * this on the bfloat16 pieces of dy and x and adds the results up
@@ -622,8 +622,13 @@ int mega_cema_scan_bwd_state(const void* dy, const void* x, int dtype, const flo
  * do not depend on x). */
 int mega_cema_scan_bwd_wide(const void* dy, const void* x, const float* p, const float* log_q,
                             const float* gamma, const float* omega, const float* h0, int64_t B,
-                            int64_t D, int64_t N, int64_t L, float* dx, float* dp, float* dq,
-                            float* dgamma, float* domega, float* dh0, void* stream);
+                            int64_t D, int64_t N, int64_t L, float* dx, int accumulate_dx, float* dp,
+                            float* dq, float* dgamma, float* domega, float* dh0, void* stream);
+
+/* src (n elements, MEGA_F32 or MEGA_F16, n % 8 == 0, 16-byte aligned) as the sum of two
+ * bfloat16 tensors: hi = bf16(src), lo = bf16(src - hi) -- 16 significant bits of a float32
+ * value, every bit of a float16 one.  The pieces mega_cema_scan_bwd_wide runs on. */
+int mega_split_bf16(const void* src, int dtype, int64_t n, void* hi, void* lo, void* stream);
 
 /* ------------------------------------------------------------------------
  * Streaming reference kernel for measurements (no counterpart in the

@@ -12,6 +12,8 @@
 // and one write of every element.
 #include "common.hpp"
 
+#include <algorithm>
+
 namespace mega {
 namespace {
 
@@ -204,6 +206,33 @@ int launch_silu_mul(const void* dout, const void* a, const void* b, void* o0, vo
   return MEGA_OK;
 }
 
+// ---- a float32 / float16 tensor as the sum of two bfloat16 tensors ------------------------
+// hi = bf16(v), lo = bf16(v - hi): 16 significant bits of a float32 value, all 11 of a float16
+// one.  The backward of the CEMA recurrence is linear in dy and, for the parameter gradients,
+// in x, and runs on such pieces (mega_cema_scan_bwd_wide).  8 elements per lane and pass.
+template <int DT>
+__global__ __launch_bounds__(kThreads) void split_bf16_kernel(const void* __restrict__ src, uint16_t* __restrict__ hi,
+                                                             uint16_t* __restrict__ lo, int64_t n8) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n8;
+       i += static_cast<int64_t>(gridDim.x) * kThreads) {
+    float v[8];
+    if (DT == MEGA_F32) {
+      const float4 a = reinterpret_cast<const float4*>(src)[2 * i], b = reinterpret_cast<const float4*>(src)[2 * i + 1];
+      v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+      unpack8<MEGA_F16>(reinterpret_cast<const uint4*>(src)[i], v);
+    }
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      h[e] = pack_bf16x2(v[2 * e], v[2 * e + 1]);
+      l[e] = pack_bf16x2(v[2 * e] - __uint_as_float(h[e] << 16), v[2 * e + 1] - __uint_as_float(h[e] & 0xffff0000u));
+    }
+    reinterpret_cast<uint4*>(hi)[i] = make_uint4(h[0], h[1], h[2], h[3]);
+    reinterpret_cast<uint4*>(lo)[i] = make_uint4(l[0], l[1], l[2], l[3]);
+  }
+}
+
 }  // namespace
 }  // namespace mega
 
@@ -259,4 +288,22 @@ extern "C" int mega_silu_mul_bwd(const void* dout, const void* a, const void* b,
   if (dtype == MEGA_F32) return launch_silu_mul<MEGA_F32>(dout, a, b, da, db, n, s);
   if (dtype == MEGA_BF16) return launch_silu_mul<MEGA_BF16>(dout, a, b, da, db, n, s);
   return launch_silu_mul<MEGA_F16>(dout, a, b, da, db, n, s);
+}
+
+extern "C" int mega_split_bf16(const void* src, int dtype, int64_t n, void* hi, void* lo, void* stream) {
+  MEGA_CHECK_ARG(dtype == MEGA_F32 || dtype == MEGA_F16, "mega_split_bf16: float32 or float16 input");
+  MEGA_CHECK_ARG(n >= 0 && n % 8 == 0, "mega_split_bf16: the element count must be a multiple of 8");
+  if (n == 0) return MEGA_OK;
+  MEGA_CHECK_ARG(src && hi && lo, "mega_split_bf16: null pointer");
+  const auto al = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  MEGA_CHECK_ARG(al(src) && al(hi) && al(lo), "mega_split_bf16: operands must be 16-byte aligned");
+  const int64_t n8 = n / 8;
+  const unsigned grid = static_cast<unsigned>(std::min<int64_t>((n8 + kThreads - 1) / kThreads, 16384));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MEGA_F32)
+    split_bf16_kernel<MEGA_F32><<<grid, kThreads, 0, s>>>(src, static_cast<uint16_t*>(hi), static_cast<uint16_t*>(lo), n8);
+  else
+    split_bf16_kernel<MEGA_F16><<<grid, kThreads, 0, s>>>(src, static_cast<uint16_t*>(hi), static_cast<uint16_t*>(lo), n8);
+  MEGA_CHECK_LAUNCH();
+  return MEGA_OK;
 }

@@ -612,8 +612,9 @@ __device__ __forceinline__ void rstep(cf& h, cf& hd, cf g, cf gd, cf m, cf md) {
 }
 
 // DX32: dx is written in float32 (or, with a null pointer, not at all) instead of the rows'
-// own type -- for callers that add up the backward of several bfloat16 pieces of one tensor.
-template <int DT, bool DX32>
+// own type -- for callers that add up the backward of several bfloat16 pieces of one tensor;
+// DX32 == 2 adds to what dx holds instead of overwriting it.
+template <int DT, int DX32>
 __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
     const void* __restrict__ dy, const void* __restrict__ x, void* __restrict__ dx,
     const float* __restrict__ p, const cf* __restrict__ log_q, const cf* __restrict__ gamma,
@@ -928,7 +929,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
       return u32x4{lo.x, lo.y, hi.x, hi.y};
     };
     if (seg0 == seg_last) setup_row(row);
-    using dx_t = typename std::conditional<DX32, float, uint16_t>::type;
+    using dx_t = typename std::conditional<DX32 != 0, float, uint16_t>::type;
     dx_t* dxrow = static_cast<dx_t*>(dx) + row * L;
     const int nc = static_cast<int>(C - seg0 < NC ? C - seg0 : NC);
     const int c0 = wave * 32;
@@ -1114,9 +1115,15 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
               const int64_t elem = chunk * kT + 16 * (2 * jt + pr) + 8 * h + 4 * g;
-              if (dx != nullptr && elem + 4 <= L)
-                *reinterpret_cast<float4*>(dxrow + elem) = make_float4(acc[8 * pr + 4 * h], acc[8 * pr + 4 * h + 1],
-                                                                       acc[8 * pr + 4 * h + 2], acc[8 * pr + 4 * h + 3]);
+              if (dx != nullptr && elem + 4 <= L) {
+                float4 v = make_float4(acc[8 * pr + 4 * h], acc[8 * pr + 4 * h + 1], acc[8 * pr + 4 * h + 2],
+                                       acc[8 * pr + 4 * h + 3]);
+                if constexpr (DX32 == 2) {
+                  const float4 o = *reinterpret_cast<const float4*>(dxrow + elem);
+                  v = make_float4(v.x + o.x, v.y + o.y, v.z + o.z, v.w + o.w);
+                }
+                *reinterpret_cast<float4*>(dxrow + elem) = v;
+              }
             }
           } else {
             const uint4 oct = octet_of<DT>(acc, pr);
@@ -1175,7 +1182,7 @@ __global__ __launch_bounds__(kThreads, 2) void cema_scan_bwd_kernel(
 #undef MEGA_LANE_IDS
 }
 
-template <bool DX32>
+template <int DX32>
 int launch_bwd(const void* dy, const void* x, void* dx, const float* p, const cf* log_q,
                const cf* gamma, const float* omega, const cf* h0, float* dp, cf* dq, cf* dgamma, float* domega,
                cf* dh0, int64_t B, int64_t D, int64_t N, int64_t L, hipStream_t stream) {
@@ -1250,7 +1257,7 @@ extern "C" int mega_cema_scan_bwd_state(const void* dy, const void* x, int dtype
   MEGA_CHECK_ARG(al(dy) && al(x) && al(dx), "%s: dy, x and dx must be 16-byte aligned", who);
   if (B == 0 || D == 0) return MEGA_OK;
   MEGA_CHECK_ARG(dh0 == nullptr || h0 != nullptr, "%s: dh0 without h0", who);
-  return launch_bwd<false>(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
+  return launch_bwd<0>(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
                            omega, reinterpret_cast<const cf*>(h0), dp, reinterpret_cast<cf*>(dq),
                            reinterpret_cast<cf*>(dgamma), domega, reinterpret_cast<cf*>(dh0), B, D, N, L,
                            static_cast<hipStream_t>(stream));
@@ -1266,8 +1273,8 @@ extern "C" int mega_cema_scan_bwd(const void* dy, const void* x, int dtype, cons
 
 extern "C" int mega_cema_scan_bwd_wide(const void* dy, const void* x, const float* p, const float* log_q,
                                        const float* gamma, const float* omega, const float* h0, int64_t B,
-                                       int64_t D, int64_t N, int64_t L, float* dx, float* dp, float* dq,
-                                       float* dgamma, float* domega, float* dh0, void* stream) {
+                                       int64_t D, int64_t N, int64_t L, float* dx, int accumulate_dx, float* dp,
+                                       float* dq, float* dgamma, float* domega, float* dh0, void* stream) {
   const char* who = "mega_cema_scan_bwd_wide";
   MEGA_CHECK_ARG(dy && x && p && log_q && gamma && dp && dq && dgamma && domega, "%s: null pointer", who);
   MEGA_CHECK_ARG(B >= 0 && D >= 0 && L >= 0, "%s: negative size", who);
@@ -1279,8 +1286,13 @@ extern "C" int mega_cema_scan_bwd_wide(const void* dy, const void* x, const floa
   MEGA_CHECK_ARG(al(dy) && al(x) && al(dx), "%s: dy, x and dx must be 16-byte aligned", who);
   if (B == 0 || D == 0) return MEGA_OK;
   MEGA_CHECK_ARG(dh0 == nullptr || h0 != nullptr, "%s: dh0 without h0", who);
-  return launch_bwd<true>(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
-                          omega, reinterpret_cast<const cf*>(h0), dp, reinterpret_cast<cf*>(dq),
-                          reinterpret_cast<cf*>(dgamma), domega, reinterpret_cast<cf*>(dh0), B, D, N, L,
-                          static_cast<hipStream_t>(stream));
+  if (accumulate_dx && dx != nullptr)
+    return launch_bwd<2>(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
+                         omega, reinterpret_cast<const cf*>(h0), dp, reinterpret_cast<cf*>(dq),
+                         reinterpret_cast<cf*>(dgamma), domega, reinterpret_cast<cf*>(dh0), B, D, N, L,
+                         static_cast<hipStream_t>(stream));
+  return launch_bwd<1>(dy, x, dx, p, reinterpret_cast<const cf*>(log_q), reinterpret_cast<const cf*>(gamma),
+                       omega, reinterpret_cast<const cf*>(h0), dp, reinterpret_cast<cf*>(dq),
+                       reinterpret_cast<cf*>(dgamma), domega, reinterpret_cast<cf*>(dh0), B, D, N, L,
+                       static_cast<hipStream_t>(stream));
 }

@@ -658,36 +658,38 @@ def cema_scan_fwd(x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor, gamma: 
 
 def cema_scan_bwd_supported(x: torch.Tensor, ndim: int) -> bool:
     """Whether the layer should train through `cema_scan_bwd` for this input: bfloat16
-    rows (one launch) and float16 rows (three launches on their bfloat16 pieces: 4.0 ms
-    against 5.8 ms on the FFT path at B=1, L=32768, D=4096); otherwise as the forward.
-    `cema_scan_bwd` itself also takes float32 rows (six launches on three pieces each),
-    but that measured slower than the float32 FFT path (5.9 against 4.6 ms), so float32
-    training is left there."""
-    if not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float16) or ndim > 32:
+    rows (one launch), float16 and float32 rows (three launches on their two bfloat16
+    pieces: 16 significant bits, what the forward takes of float32 rows as well);
+    otherwise as the forward."""
+    if not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float16, torch.float32) or ndim > 32:
         return False
     fn = _lib.load().mega_cema_scan_bwd_supported
     return bool(fn(_lib.i32(_lib.dtype_code(torch.bfloat16)), _lib.i64(min(ndim, 16)), _lib.i64(x.shape[-1])))
 
 
-def _bf16_pieces(t: torch.Tensor, n: int = 2):
-    """A float16 tensor as the sum of two bfloat16 tensors (11 significant bits = 8 + 3),
-    a float32 tensor as the sum of three (24 = 8 + 8 + 8): exact while the low pieces stay
-    above the bfloat16 underflow threshold."""
-    pieces, rest = [], t.float()
-    for _ in range(n):
-        piece = rest.to(torch.bfloat16)
-        pieces.append(piece)
-        rest = rest - piece.float()
-    return pieces
+def split_bf16(t: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """A float32 / float16 tensor as the sum of two bfloat16 tensors, hi = bf16(t) and
+    lo = bf16(t - hi): 16 significant bits of a float32 value (what the recurrence's forward
+    takes of float32 rows), every bit of a float16 one; one streaming kernel."""
+    dev = _require_cuda(t)
+    tc = t.contiguous()
+    if tc.numel() % 8 != 0 or tc.data_ptr() % 16 != 0 or tc.dtype not in (torch.float32, torch.float16):
+        hi = tc.to(torch.bfloat16)
+        return hi, (tc.float() - hi.float()).to(torch.bfloat16)
+    hi = torch.empty(tc.shape, dtype=torch.bfloat16, device=dev)
+    lo = torch.empty_like(hi)
+    with torch.cuda.device(dev):
+        _lib.call("mega_split_bf16", _lib.ptr(tc), _lib.i32(_lib.dtype_code(tc.dtype)), _lib.i64(tc.numel()),
+                  _lib.ptr(hi), _lib.ptr(lo), _lib.stream_ptr(dev))
+    return hi, lo
 
 
-def _cema_scan_bwd_wide(dy, x, pc, lq, gm, wc, hc, want_dx: bool):
-    """One launch of the backward kernel on bfloat16 pieces: float32 dx (or none), per-row
-    parameter gradients summed over the batch, dh0 (or none)."""
+def _cema_scan_bwd_wide(dy, x, pc, lq, gm, wc, hc, dx: Optional[torch.Tensor], accumulate: bool):
+    """One launch of the backward kernel on bfloat16 pieces: float32 dx written, added to, or
+    (None) left out; per-row parameter gradients summed over the batch; dh0 (or none)."""
     dev = x.device
     B, D, L = x.shape
     N = pc.shape[1]
-    dx = torch.empty((B, D, L), dtype=torch.float32, device=dev) if want_dx else None
     dp = torch.empty((B, D, N), dtype=torch.float32, device=dev)
     dq = torch.empty((B, D, N), dtype=torch.complex64, device=dev)
     dg = torch.empty((B, D, N), dtype=torch.complex64, device=dev)
@@ -696,8 +698,9 @@ def _cema_scan_bwd_wide(dy, x, pc, lq, gm, wc, hc, want_dx: bool):
     with torch.cuda.device(dev):
         _lib.call("mega_cema_scan_bwd_wide", _lib.ptr(dy), _lib.ptr(x), _lib.ptr(pc), _lib.ptr(lq), _lib.ptr(gm),
                   _lib.ptr(wc), _lib.ptr(hc), _lib.i64(B), _lib.i64(D), _lib.i64(N), _lib.i64(L), _lib.ptr(dx),
-                  _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg), _lib.ptr(dw), _lib.ptr(dh), _lib.stream_ptr(dev))
-    return dx, [dp.sum(0), dq.sum(0), dg.sum(0), dw.sum(0)], dh
+                  _lib.i32(1 if accumulate else 0), _lib.ptr(dp), _lib.ptr(dq), _lib.ptr(dg), _lib.ptr(dw),
+                  _lib.ptr(dh), _lib.stream_ptr(dev))
+    return [dp.sum(0), dq.sum(0), dg.sum(0), dw.sum(0)], dh
 
 
 def _mode_groups(N: int):
@@ -738,24 +741,18 @@ def cema_scan_bwd(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, log_q:
         return tuple(out)
     if x.dtype != torch.bfloat16:
         # The backward is linear in y_grad and, for the parameter gradients, in x as well: the
-        # bfloat16 kernel runs on pairs of pieces (dy_i, x_j) with i + j below the number of
-        # pieces (what is left out is 2^-16 of the result for float16, 2^-24 for float32); dx
-        # comes from the pairs with x_0, in float32, and is rounded once; so do the terms of a
-        # carried state, which do not depend on x.
-        n = 2 if x.dtype == torch.float16 else 3
-        gp = [t.contiguous() for t in _bf16_pieces(y_grad, n)]
-        xp = [t.contiguous() for t in _bf16_pieces(x, n)]
-        dx_sum, grads, dh_sum = None, None, None
-        for i in range(n):
-            for j in range(n - i):
-                dxi, g, dh = _cema_scan_bwd_wide(gp[i], xp[j], pc, lq, gm, wc, hc if j == 0 else None, want_dx=(j == 0))
-                if dxi is not None:
-                    dx_sum = dxi if dx_sum is None else dx_sum.add_(dxi)
-                if dh is not None:
-                    dh_sum = dh if dh_sum is None else dh_sum.add_(dh)
-                grads = g if grads is None else [a + b for a, b in zip(grads, g)]
-        out = (dx_sum.to(x.dtype), *grads)
-        return out if hc is None else out + (dh_sum,)
+        # bfloat16 kernel runs on the pairs of pieces (dy_hi, x_hi), (dy_lo, x_hi), (dy_hi, x_lo)
+        # -- what is left out is 2^-16 of the result.  dx is linear in dy alone: the first two
+        # launches write and add to it in float32, one rounding at the end; so the terms of a
+        # carried state, which do not depend on x either.
+        (g_hi, g_lo), (x_hi, x_lo) = split_bf16(y_grad), split_bf16(x)
+        dx32 = torch.empty((B, D, L), dtype=torch.float32, device=dev)
+        grads, dh = _cema_scan_bwd_wide(g_hi, x_hi, pc, lq, gm, wc, hc, dx32, False)
+        g2, dh2 = _cema_scan_bwd_wide(g_lo, x_hi, pc, lq, gm, wc, hc, dx32, True)
+        g3, _ = _cema_scan_bwd_wide(g_hi, x_lo, pc, lq, gm, wc, None, None, False)
+        grads = [a_ + b_ + c_ for a_, b_, c_ in zip(grads, g2, g3)]
+        out = (dx32 if x.dtype == torch.float32 else dx32.to(x.dtype), *grads)
+        return out if hc is None else out + (dh + dh2,)
 
     def aligned(t):
         t = t.contiguous()

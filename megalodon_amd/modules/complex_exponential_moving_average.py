@@ -4,9 +4,10 @@
 ``dim_per_partition == embed_dim`` and the theta permutation is drawn locally
 instead of being broadcast (:21-26).  On the GPU the layer runs as a chunked
 recurrence (fused_ops/cema_scan.py) wherever its kernels take the case --
-bfloat16 / float16 rows with gradients, every dtype without; MEGA_CEMA_FFT=1
-in the environment keeps everything on the kernel-row + FFT-convolution
-operators that the remaining cases (float32 training, odd lengths) use."""
+rows of a length that is a multiple of 8, at most 32 modes, with or without
+gradients, carried state and last state; MEGA_CEMA_FFT=1 in the environment
+keeps everything on the kernel-row + FFT-convolution operators that the
+remaining cases (other lengths) use."""
 from typing import Optional, Tuple
 import math
 import os

@@ -74,8 +74,7 @@ def test_unsupported_shapes_are_refused():
     x = torch.zeros(1, 2, 100, dtype=torch.bfloat16, device="cuda")   # L % 8 != 0
     assert not ops.cema_scan_supported(x, 16)
     assert ops.cema_scan_supported(torch.zeros(1, 2, 64, device="cuda"), 16)       # float32 rows
-    # float32 rows: cema_scan_bwd takes them (tested below) but the layer trains them on the FFT path
-    assert not ops.cema_scan_bwd_supported(torch.zeros(1, 2, 64, device="cuda"), 16)
+    assert ops.cema_scan_bwd_supported(torch.zeros(1, 2, 64, device="cuda"), 16)   # float32 rows: two bf16 pieces
     assert ops.cema_scan_bwd_supported(torch.zeros(1, 2, 64, dtype=torch.float16, device="cuda"), 16)
     assert ops.cema_scan_supported(torch.zeros(1, 2, 64, dtype=torch.bfloat16, device="cuda"), 17)   # two launches
     assert not ops.cema_scan_supported(torch.zeros(1, 2, 64, dtype=torch.bfloat16, device="cuda"), 33)
@@ -95,9 +94,8 @@ def test_backward_matches_oracle(B, D, N, L, dtype):
     g = torch.Generator().manual_seed(L + 1)
     x = torch.randn(B, D, L, generator=g).to(dtype)
     dy = torch.randn(B, D, L, generator=g).to(dtype)
-    # the layer trains bfloat16 / float16 rows through this operator; float32 rows are taken too
-    # (the layer leaves them on the FFT path, which measured faster)
-    assert ops.cema_scan_bwd_supported(x.cuda(), N) == (dtype != torch.float32)
+    # bfloat16 rows in one launch, float16 / float32 rows in three launches on two bfloat16 pieces each
+    assert ops.cema_scan_bwd_supported(x.cuda(), N)
     dx, dp, dq, dg, dw = ops.cema_scan_bwd(dy.cuda(), x.cuda(), p.cuda(), q.log().cuda(), gam.cuda(), omega.cuda())
     lq = q.to(torch.complex128).log()
     k = ocema.ema_weight_fwd(p.double(), lq, gam.to(torch.complex128), L)
@@ -166,7 +164,7 @@ def _oracle_bwd(dy, x, p, q, gam, omega, h0):
 
 
 @pytest.mark.parametrize("B,D,N,L", [(2, 3, 16, 64), (1, 2, 16, 8264), (3, 2, 7, 1000), (1, 3, 16, 32768)])
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_backward_with_carried_state(B, D, N, L, dtype):
     """The backward of a forward that had a carried state: the state's terms in dq and dgamma and
     its own gradient dh0 (ema_parameters.cc:100-117,158-188) from what the reverse scan carries to
@@ -179,7 +177,7 @@ def test_backward_with_carried_state(B, D, N, L, dtype):
     dx, dp, dq, dg, dw, dh = ops.cema_scan_bwd(dy.cuda(), x.cuda(), p.cuda(), q.log().cuda(), gam.cuda(), omega.cuda(),
                                                h0.cuda())
     wdx, wdp, wdq, wdg, wdw, wdh = _oracle_bwd(dy, x, p, q, gam, omega, h0)
-    assert rel_err(dx, wdx) <= 2e-2
+    assert dx.dtype == dtype and rel_err(dx, wdx) <= (1e-4 if dtype == torch.float32 else 2e-2)
     assert rel_err(dp, wdp) <= 1e-4 and rel_err(dq, wdq) <= 1e-4 and rel_err(dg, wdg) <= 1e-4
     assert rel_err(dw, wdw) <= 1e-4
     assert dh.shape == (B, D, N) and rel_err(dh, wdh) <= 1e-4
