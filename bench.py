@@ -341,7 +341,7 @@ def cema_leg(torch, dev, steps, warmup, copy_calibration):
 
     for _ in range(warmup):
         step()
-    log = {"mega_cema_scan_fwd": [], "mega_cema_scan_bwd": [], "mega_cema_coeffs_fwd": [], "mega_cema_coeffs_bwd": []}
+    log = {"mega_cema_scan_fwd": [], "mega_cema_scan_bwd_state": [], "mega_cema_coeffs_fwd": [], "mega_cema_coeffs_bwd": []}
     _lib.set_event_log(log)
     dt = timed(steps)
     _lib.set_event_log(None)

@@ -29,12 +29,19 @@
 // wave works through the finished tile t - 1 in the other, one 32-key block per slab, a piece
 // of it per k-step.
 // Measured on the way (8 chunks x 4 heads, 4096 x 4096, head width 256; this kernel 0.31 ms
-// against 0.27 + 0.23 ms for product and softmax as two kernels): the stores straight from the
-// registers (32 bytes of a line per row and instruction) cost 0.03 ms over no stores at all and
-// the HBM writes behind them another 0.06 ms; the same tile staged through LDS and stored as
+// against 0.27 + 0.23 ms for product and softmax as two kernels).  With parts switched off
+// (timing only): no stores 0.27 ms, neither barrier nor slab requests 0.26 ms, neither of the
+// two 0.24 ms -- the products and the passes themselves, at the clock the part sustains with
+// every matrix pipe busy; a quarter of the (batch, head) pairs, half the compute units idle,
+// runs the same code a quarter faster per row block.  A wave's `s_waitcnt vmcnt` counts its
+// stores of P with its slab requests, so the waits for slabs also wait for stores; letting four
+// waves request for all eight changed nothing.  The same tile staged through LDS and stored as
 // whole lines was slower (0.38 ms), non-temporal stores of the 32-byte pieces three times
 // slower; four waves per workgroup and two workgroups per compute unit 0.33 ms; taking the
 // (batch, head) pairs of an XCD two at a time instead of all at once 0.33 -> 0.31 ms.
+// On this part an MFMA of this shape holds the matrix pipe for 32 clocks and its wave's issue
+// for about 14; beside it a SIMD issues six ordinary vector instructions (v_exp_f32 counts
+// two) per MFMA before the vector port, not the matrix pipe, sets the pace.
 #include "common.hpp"
 
 #include <type_traits>
