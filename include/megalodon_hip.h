@@ -303,13 +303,22 @@ void mega_test_timestep_norm_lookback(long long spin_limit, int mute_tile);
  *   S = scale * q k^T rounded to `dtype`; with `causal` row r keeps columns
  *   0 .. L2 - L1 + r (L2 >= L1 required: cached keys / values in front of the
  *   chunk, softmax.cuh:99-100), all columns otherwise; P = softmax in fp32,
- *   stored in `dtype` into w; y = P v.  With `causal` and L1 == L2, w is
- *   written only up to the end of the 256-column block holding the diagonal of
- *   each row (zeros above the diagonal inside that block); the blocks to the
- *   right are never read by the backward and are left untouched.  With
- *   L2 > L1 every row of w is written to its end.  Without dropout use
- *   mega_attention_fwd; with DropKey dropout (softmax.cuh:135-196,
- *   attention_kernel.cu:99-116) mega_attention_dropkey_fwd, below.
+ *   stored in `dtype` into w; y = P v.
+ *   `causal`: 0 = every key; 1 = the causal mask, every row of w written to
+ *   its end as the reference's softmax does (masked columns are exp(-inf) = 0,
+ *   softmax.cuh:99-105,127-129); 2 = the same mask and the same y, but with
+ *   L1 == L2 a row of w is written only up to the end of the 256-column block
+ *   that holds its diagonal (zeros above the diagonal inside that block) and
+ *   the blocks to the right are left untouched -- for a caller that hands w
+ *   to mega_attention_bwd and nowhere else (the backward never reads them;
+ *   the zero fill is 0.1 ms of 1.3 at 32 x 4096 x 4096).  With L2 > L1 both
+ *   values write every row to its end.
+ *   For head widths H1 of 64, 128 or 256 (16-byte aligned tensors, L2 % 8 == 0,
+ *   no dropout) scores and softmax are one kernel and S never reaches memory;
+ *   other shapes form S in w and run the softmax over it in place.
+ *   Without dropout use mega_attention_fwd; with DropKey dropout
+ *   (softmax.cuh:135-196, attention_kernel.cu:99-116)
+ *   mega_attention_dropkey_fwd, below.
  *   `workspace`: mega_attention_workspace_bytes(B, L1, L2, NH, H1, H2, 0) bytes.
  * ---------------------------------------------------------------------- */
 int64_t mega_attention_workspace_bytes(int64_t B, int64_t L1, int64_t L2, int64_t NH,

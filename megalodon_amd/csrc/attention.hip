@@ -1510,6 +1510,7 @@ int check_attn(const char* who, int dtype, int64_t B, int64_t L1, int64_t L2, in
   MEGA_CHECK_ARG(B >= 0 && L1 >= 0 && L2 >= 0 && NH >= 1 && H1 >= 1 && H2 >= 1, "%s: bad sizes", who);
   MEGA_CHECK_ARG(B * NH <= 65535, "%s: batch * heads exceeds 65535", who);
   MEGA_CHECK_ARG(L1 <= (1 << 24) && L2 <= (1 << 24), "%s: sequence too long", who);
+  MEGA_CHECK_ARG(causal >= 0 && causal <= 2, "%s: causal must be 0, 1 or 2", who);
   MEGA_CHECK_ARG(!causal || L2 >= L1,
                  "%s: causal attention needs L2 >= L1 (row r sees keys 0 .. L2 - L1 + r)", who);
   return MEGA_OK;
@@ -1673,6 +1674,7 @@ extern "C" int mega_attention_bwd(const void* dy, const void* q, const void* k, 
                  "mega_attention_bwd: null pointer");
   MEGA_CHECK_ARG(L1 >= 1 && L2 >= 1, "mega_attention_bwd: empty sequence");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  causal = causal != 0;  // the forward's 1 and 2 are the same mask
   if (dtype == MEGA_F32)
     return attention_wide_bwd<float>(static_cast<const float*>(dy), static_cast<const float*>(q),
                                      static_cast<const float*>(k), static_cast<const float*>(v),
