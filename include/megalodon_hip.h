@@ -300,7 +300,9 @@ void mega_test_timestep_norm_lookback(long long spin_limit, int mute_tile);
  *   storage and arithmetic of that type on the vector ALUs, write every row of
  *   w to its end, and need two / four times the workspace bytes the size query
  *   returns.
- *   S = scale * q k^T rounded to `dtype`; with `causal` row r keeps columns
+ *   S = scale * q k^T (rounded to `dtype` as in the reference where S passes
+ *   through w; the one-kernel path below feeds it to the softmax in float32);
+ *   with `causal` row r keeps columns
  *   0 .. L2 - L1 + r (L2 >= L1 required: cached keys / values in front of the
  *   chunk, softmax.cuh:99-100), all columns otherwise; P = softmax in fp32,
  *   stored in `dtype` into w; y = P v.

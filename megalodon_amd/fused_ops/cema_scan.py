@@ -78,8 +78,8 @@ cema_scan_state = CEMAScanStateFunc.apply
 
 def cema_scan_applicable(x: torch.Tensor, ndim: int, needs_grad: bool) -> bool:
     """The recurrence kernels take bfloat16 / float16 / float32 rows of a length that
-    is a multiple of 8 with at most 16 modes; the backward bfloat16 rows, and float16
-    rows through their bfloat16 pieces."""
+    is a multiple of 8 with at most 32 modes (16 per launch), forward and backward;
+    the backward runs float16 and float32 rows through their bfloat16 pieces."""
     if needs_grad:
         return megalodon_ops.cema_scan_bwd_supported(x, ndim)
     return megalodon_ops.cema_scan_supported(x, ndim)

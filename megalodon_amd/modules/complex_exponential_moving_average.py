@@ -16,8 +16,7 @@ import torch
 from torch import nn
 
 from .. import extension as megalodon_ops
-from ..fused_ops.cema_scan import cema_scan_state
-from ..fused_ops import (cema_kernel, cema_scan, cema_scan_applicable, ema_hidden, ema_parameters,
+from ..fused_ops import (cema_kernel, cema_scan, cema_scan_applicable, cema_scan_state, ema_hidden, ema_parameters,
                          fftconv_residual)
 
 
