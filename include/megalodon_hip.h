@@ -144,14 +144,23 @@ int mega_cema_coeffs_bwd(const float* dp, const float* dq, const float* dgamma_h
  *   L <= mega_fftconv_max_length() (32768); longer rows return
  *   MEGA_ERR_UNSUPPORTED.
  *   The float32 engine needs twiddle tables (one per device and transform
- *   size) and a per-workgroup scratch block (one per device, transform size
- *   and stream, so launches on different streams never share slots); both are
- *   kept until process exit.  mega_fftconv_prepare(L, stream) makes them ahead
- *   of time (it allocates and synchronises `stream` once; not capturable);
- *   after it, the convolution entry points on that stream only enqueue.
- *   Without it the first call for a size / stream does the same work itself.
+ *   size) and per-workgroup scratch blocks (per device and transform size:
+ *   a stream gets a block of its own, so launches on different streams never
+ *   share slots, up to four blocks; a fifth stream takes over the block that
+ *   has been idle longest and waits on the device for the last launch that
+ *   used it); they are kept until process exit (64 MiB per block at the
+ *   largest size on 256 compute units).  mega_fftconv_prepare(L, stream) makes
+ *   them ahead of time (it allocates and synchronises `stream` once; not
+ *   capturable); after it, the convolution entry points on that stream only
+ *   enqueue.  Without it the first call for a size / stream does the same
+ *   work itself.  To capture a convolution into a graph, prepare the stream
+ *   the capture runs on; a block used under capture belongs to that graph's
+ *   replays and is never handed to another stream.
+ *   mega_fftconv_scratch_blocks(L): blocks held on the current device for the
+ *   transform size of rows of L samples.
  * ---------------------------------------------------------------------- */
 int mega_fftconv_prepare(int64_t L, void* stream);
+int mega_fftconv_scratch_blocks(int64_t L);
 int mega_fftconv_max_length(void);
 int mega_fftconv_fwd(const void* x, int dtype, const float* k, int64_t B,
                      int64_t D, int64_t L, void* y, void* stream);

@@ -26,27 +26,44 @@ using namespace fftc;
 
 // ------------------------------ tables --------------------------------------
 constexpr int kMaxDevices = 16;
+constexpr int kMaxScratch = 4;  // scratch blocks per device and size before streams start taking turns
 struct StreamScratch {
-  hipStream_t stream;
+  hipStream_t stream;  // the stream whose launches used the block last
   float* ptr;
+  hipEvent_t done;     // recorded behind the last launch that used the block
+  uint64_t tick;       // when that was
+  bool pinned;         // used under stream capture: the graph's replays own the block from then on
 };
 struct TableCache {
   c32* ptr[kMaxDevices][4] = {};
   int slots[kMaxDevices][4] = {};
-  // one scratch block per stream that has run this transform size: launches
-  // on different streams of a device may overlap, and a workgroup's slot is
-  // picked by its index alone
+  // Launches on different streams of a device may overlap, and a workgroup's
+  // slot is picked by its index alone, so a stream gets a block of its own --
+  // up to kMaxScratch of them per device and size.  A further stream takes
+  // over the block that has been idle longest and first waits (on the device,
+  // through the block's event) for the last launch that used it.  Blocks used
+  // under stream capture are never handed on.
   std::vector<StreamScratch> scratch[kMaxDevices][4];
+  uint64_t tick = 0;
   std::mutex mu;
 };
 TableCache g_tables;
 
+bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st != hipStreamCaptureStatusNone;
+}
+
 // Twiddle tables (one per device and transform size) and the per-workgroup
-// scratch slots (one block per device, transform size and stream) live for the
-// life of the process.  They are made on first use, or ahead of time by
-// mega_fftconv_prepare; making them allocates and, for the tables,
-// synchronises the stream once, so that call cannot be captured into a graph.
-// Scratch is 2*M floats per resident workgroup (at most 2 workgroups per CU).
+// scratch slots live for the life of the process.  They are made on first use,
+// or ahead of time by mega_fftconv_prepare; making them allocates and, for the
+// tables, synchronises the stream once, so that call cannot be captured into a
+// graph.  Scratch is 2*M floats per resident workgroup (at most 2 workgroups
+// per CU).
 template <int LOGM>
 int get_tables(hipStream_t stream, const c32** out, float** scratch, int* slots) {
   using C = Cfg<LOGM>;
@@ -73,16 +90,51 @@ int get_tables(hipStream_t stream, const c32** out, float** scratch, int* slots)
     slot = p;
   }
   const int nslots = g_tables.slots[dev][LOGM - 11];
-  float* sc = nullptr;
-  for (const StreamScratch& s : g_tables.scratch[dev][LOGM - 11])
-    if (s.stream == stream) sc = s.ptr;
-  if (sc == nullptr) {
-    MEGA_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&sc), sizeof(float) * 2 * C::M * nslots));
-    g_tables.scratch[dev][LOGM - 11].push_back(StreamScratch{stream, sc});
+  std::vector<StreamScratch>& blocks = g_tables.scratch[dev][LOGM - 11];
+  StreamScratch* mine = nullptr;
+  int open_blocks = 0;
+  for (StreamScratch& s : blocks) {
+    if (s.stream == stream) mine = &s;
+    open_blocks += s.pinned ? 0 : 1;
   }
+  const bool capturing = stream_is_capturing(stream);
+  if (mine == nullptr && open_blocks >= kMaxScratch && !capturing) {
+    // take over the block that has been idle longest, behind its last launch
+    for (StreamScratch& s : blocks)
+      if (!s.pinned && (mine == nullptr || s.tick < mine->tick)) mine = &s;
+    MEGA_CHECK_HIP(hipStreamWaitEvent(stream, mine->done, 0));
+    mine->stream = stream;
+  }
+  if (mine == nullptr) {
+    float* sc = nullptr;
+    hipEvent_t ev = nullptr;
+    MEGA_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&sc), sizeof(float) * 2 * C::M * nslots));
+    hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+    if (e != hipSuccess) {
+      (void)hipFree(sc);
+      return set_error(MEGA_ERR_HIP, "fftconv scratch event: %s", hipGetErrorString(e));
+    }
+    blocks.push_back(StreamScratch{stream, sc, ev, 0, false});
+    mine = &blocks.back();
+  }
+  mine->tick = ++g_tables.tick;
+  if (capturing) mine->pinned = true;
   *out = slot;
-  *scratch = sc;
+  *scratch = mine->ptr;
   *slots = nslots;
+  return MEGA_OK;
+}
+
+// Marks the end of the launches that used `stream`'s scratch block, so that a
+// later take-over can order itself behind them.  Not recorded under capture
+// (the block is pinned there).
+template <int LOGM>
+int scratch_used(hipStream_t stream) {
+  int dev = 0;
+  MEGA_CHECK_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_tables.mu);
+  for (StreamScratch& s : g_tables.scratch[dev][LOGM - 11])
+    if (s.stream == stream && !s.pinned) MEGA_CHECK_HIP(hipEventRecord(s.done, stream));
   return MEGA_OK;
 }
 
@@ -380,7 +432,7 @@ int launch_fft_v(const void* a, const void* b, void* out, int64_t B, int64_t D, 
       MEGA_CHECK_LAUNCH();
     }
   }
-  return MEGA_OK;
+  return scratch_used<LOGM>(stream);
 }
 
 template <int LOGM, int DT, int MODE>
@@ -511,6 +563,17 @@ extern "C" int mega_fftconv_prepare(int64_t L, void* stream) {
   if (L <= 8192) return get_tables<12>(s, &tab, &scratch, &slots);
   if (L <= 16384) return get_tables<13>(s, &tab, &scratch, &slots);
   return get_tables<14>(s, &tab, &scratch, &slots);
+}
+
+// Scratch blocks held on the current device for the transform size that rows
+// of L samples take (0 for rows the time-domain kernel takes).
+extern "C" int mega_fftconv_scratch_blocks(int64_t L) {
+  if (L <= kDirectMaxL || L > kMaxL) return 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  const int size = L <= 4096 ? 0 : L <= 8192 ? 1 : L <= 16384 ? 2 : 3;
+  std::lock_guard<std::mutex> lock(g_tables.mu);
+  return static_cast<int>(g_tables.scratch[dev][size].size());
 }
 
 namespace {

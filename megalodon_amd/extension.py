@@ -542,13 +542,28 @@ def fftconv_residual_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor,
     return dx, dk, dk[:, 0].clone()
 
 
-def fftconv_prepare(L: int, device=None) -> None:
-    """Make the float32 convolution engine's tables and the current stream's
-    scratch block for rows of L samples ahead of time (allocates and
-    synchronises once); later convolution calls on that stream only enqueue."""
+def fftconv_prepare(L: int, device=None, stream=None) -> None:
+    """Make the float32 convolution engine's tables and a scratch block for rows of
+    L samples ahead of time, for `stream` (a torch.cuda.Stream; default: the current
+    stream).  It allocates and synchronises once; later convolution calls on that
+    stream only enqueue -- which is what a graph capture on that stream needs:
+        fftconv_prepare(L, stream=s);  with torch.cuda.graph(g, stream=s): ..."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    if stream is not None:
+        dev = stream.device
+    with torch.cuda.device(dev):
+        ptr = _lib.stream_ptr(dev) if stream is None else _lib.ctypes.c_void_p(stream.cuda_stream)
+        _lib.call("mega_fftconv_prepare", _lib.i64(min(int(L), fftconv_max_length())), ptr)
+
+
+def fftconv_scratch_blocks(L: int, device=None) -> int:
+    """Scratch blocks the float32 convolution engine holds on `device` for the
+    transform size of rows of L samples (at most four plus those owned by graphs)."""
     dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
     with torch.cuda.device(dev):
-        _lib.call("mega_fftconv_prepare", _lib.i64(min(int(L), fftconv_max_length())), _lib.stream_ptr(dev))
+        fn = _lib.load().mega_fftconv_scratch_blocks
+        fn.restype = _lib.ctypes.c_int
+        return int(fn(_lib.i64(int(L))))
 
 
 def fftconv_spectrum_bytes(dtype: torch.dtype, B: int, D: int, L: int) -> int:

@@ -84,3 +84,60 @@ def test_timestep_norm_under_graph_replay():
         return y, mean, var, dx, dg, db
 
     _replay_and_compare(build, (x, dy), refresh)
+
+
+def test_float32_convolution_under_graph_replay_after_prepare():
+    """The float32 FFT engine keeps a scratch block per stream.  `fftconv_prepare(L, stream=s)`
+    makes it (and the tables) for the capture stream ahead of time, so the captured call only
+    enqueues; the block then belongs to the graph and is not handed to other streams."""
+    L, D = 4096, 64
+    g_ = torch.Generator().manual_seed(11)
+    x = torch.randn(2, D, L, generator=g_).cuda()
+    k = (torch.randn(D, L, generator=g_) / L ** 0.5).cuda()
+    base = [x.clone(), x.flip(-1).clone(), (2 * x).clone()]
+
+    def refresh(i):
+        x.copy_(base[i])
+
+    refresh(0)
+    eager0 = ops.fftconv_fwd(x, k).clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    ops.fftconv_prepare(L, stream=side)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        y = ops.fftconv_fwd(x, k)
+    for i in (0, 1, 2, 1):
+        refresh(i)
+        want = ops.fftconv_fwd(x, k).clone()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), "replay differs from the eager launch"
+    refresh(0)
+    g.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y, eager0)
+
+
+def test_float32_convolution_scratch_blocks_are_bounded():
+    """Six streams run the float32 engine at one transform size: at most four scratch blocks
+    (plus those a graph owns) exist afterwards, and a stream that took a block over gets the
+    same result as the first."""
+    L, D = 8192, 48
+    g_ = torch.Generator().manual_seed(12)
+    x = torch.randn(1, D, L, generator=g_).cuda()
+    k = (torch.randn(D, L, generator=g_) / L ** 0.5).cuda()
+    want = ops.fftconv_fwd(x, k)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(6)]
+    outs = []
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            for _ in range(3):
+                outs.append(ops.fftconv_fwd(x, k))
+    torch.cuda.synchronize()
+    for o in outs:
+        assert torch.equal(o, want)
+    assert 1 <= ops.fftconv_scratch_blocks(L) <= 4
