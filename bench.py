@@ -307,6 +307,12 @@ def block_leg(torch, dev, steps, warmup):
         step()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
+    # outside the timed region: a TimestepNorm tile that gave up its bounded wait would have
+    # written NaN; the status word turns that into an error instead of a quietly wrong number
+    from megalodon_amd import extension as ops
+    ops.timestep_norm_status(dev)
+    if not torch.isfinite(bx.grad.float()).all():
+        raise RuntimeError("bench: the block's input gradient is not finite")
     del blk, bx, bdy
     torch.cuda.empty_cache()
     return dt
