@@ -112,6 +112,32 @@ def test_scores_and_softmax_in_one_kernel(B, L1, L2, NH, H1, H2, causal, dtype):
     _run(B, L1, L2, NH, H1, H2, causal, dtype, seed=L1 + L2 + H1)
 
 
+@pytest.mark.parametrize("B,L1,L2,NH,H1,H2,causal", [
+    (1, 8, 8, 1, 64, 64, True),           # fewer keys than one slab holds
+    (2, 5, 40, 1, 128, 32, True),         # five new rows on a prefix of 35 keys
+    (1, 24, 24, 2, 256, 8, False),
+    (3, 1, 8, 1, 64, 16, False),          # one row, eight keys
+])
+def test_one_kernel_scores_on_tiny_shapes(B, L1, L2, NH, H1, H2, causal):
+    _run(B, L1, L2, NH, H1, H2, causal, torch.bfloat16, seed=3 * L1 + L2)
+
+
+def test_one_kernel_scores_with_large_logits():
+    """Scores of several hundred in magnitude: the exponentials are taken relative to the row maximum
+    (in both passes), so rows whose probabilities are all but one-hot come out exact and nothing
+    overflows; compared with the float64 oracle on the same bf16 inputs."""
+    g = torch.Generator().manual_seed(5)
+    B, L, NH, H1, H2 = 1, 320, 2, 128, 64
+    q = (6 * torch.randn(B, L, NH, H1, generator=g)).bfloat16()
+    k = (6 * torch.randn(B, L, NH, H1, generator=g)).bfloat16()
+    v = torch.randn(B, L, NH, H2, generator=g).bfloat16()
+    y, w = ops.attention_fwd(q.cuda(), k.cuda(), v.cuda(), 1.0, 0.0, True)
+    wy, ww = oa.chunk_attention_fwd(q, k, v, 1.0, True)
+    assert torch.isfinite(w.float()).all() and torch.isfinite(y.float()).all()
+    assert rel_err(w, ww) <= TOL and rel_err(y, wy) <= TOL
+    assert torch.allclose(w.float().sum(-1).cpu(), torch.ones(B, NH, L), atol=2e-2)
+
+
 def test_random_shapes():
     """Seeded random shapes with a key count that is a multiple of 64: ragged query counts,
     key/value prefixes of any length, causal and not, any head width that is a multiple of 8."""
