@@ -676,7 +676,7 @@ __global__ __launch_bounds__(2 * kThreads) void gemm_dma_kernel(const GemmParams
       const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * EP + kc);
       uint16_t* dst = C + static_cast<int64_t>(grow) * p.ldc + gcol;
       if (vec_ok && gcol + 8 <= p.N) {
-        *reinterpret_cast<u32x4*>(dst) = v;
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));  // whole lines, read by a later kernel
       } else {
         const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
         for (int q = 0; q < 8; ++q)
@@ -932,7 +932,7 @@ __global__ __launch_bounds__(2 * kThreads) void gemm_dma64_kernel(const GemmPara
       const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * EP + kc);
       uint16_t* dst = C + static_cast<int64_t>(grow) * p.ldc + gcol;
       if (vec_ok && gcol + 8 <= p.N) {
-        *reinterpret_cast<u32x4*>(dst) = v;
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));  // whole lines, read by a later kernel
       } else {
         const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
         for (int q = 0; q < 8; ++q)
@@ -1201,7 +1201,7 @@ __global__ __launch_bounds__(2 * kThreads) void gemm_dma_a64_kernel(const GemmPa
       const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * EP + kc);
       uint16_t* dst = C + static_cast<int64_t>(grow) * p.ldc + gcol;
       if (vec_ok && gcol + 8 <= p.N) {
-        *reinterpret_cast<u32x4*>(dst) = v;
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));  // whole lines, read by a later kernel
       } else {
         const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
         for (int q = 0; q < 8; ++q)

@@ -173,4 +173,17 @@ __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t
   out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
 }
 
+// 16-byte accesses with the non-temporal hint: for tensors a kernel writes once in whole
+// 128-byte lines and does not read again (stores), or reads once (loads).  Such stores do not
+// displace what the kernel still reads; partial lines written with the hint are slow.
+typedef uint32_t nt_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_streaming(void* ptr, uint4 v) {
+  nt_u32x4 w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, static_cast<nt_u32x4*>(ptr));
+}
+__device__ __forceinline__ uint4 load_once(const void* ptr) {
+  const nt_u32x4 v = __builtin_nontemporal_load(static_cast<const nt_u32x4*>(ptr));
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
 }  // namespace mega

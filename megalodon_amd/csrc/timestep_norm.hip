@@ -227,15 +227,6 @@ __device__ __forceinline__ void stT(void* p, int64_t i, float v) {
 // hint on its loads the forward is 0.114 ms, the backward 0.179 ms), and so are the statistics:
 // they leave four bytes per lane, and partial lines written with the hint are slow (forward
 // 0.167 ms).
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ uint4 ld_once(const void* ptr) {
-  const u32x4_t v = __builtin_nontemporal_load(static_cast<const u32x4_t*>(ptr));
-  return make_uint4(v[0], v[1], v[2], v[3]);
-}
-__device__ __forceinline__ void st_stream(void* ptr, uint4 v) {
-  u32x4_t w = {v.x, v.y, v.z, v.w};
-  __builtin_nontemporal_store(w, static_cast<u32x4_t*>(ptr));
-}
 __device__ __forceinline__ uint4 reload(uint4 v) {
   asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
   return v;
@@ -499,7 +490,7 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
 #pragma unroll
       for (int e = 0; e < VEC; ++e) o[e] = valid ? (f[e] - u) * rs * gm[e] + bt[e] : 0.f;
       const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
-      st_stream(static_cast<typename Elem<DT>::type*>(p.y) + off, Vec<DT>::pack(o));
+      store_streaming(static_cast<typename Elem<DT>::type*>(p.y) + off, Vec<DT>::pack(o));
     }
   }
 }
@@ -652,7 +643,7 @@ void tsn_fwd_wave_kernel(const TsnParams p, int tiles) {
       for (int e = 0; e < VEC; ++e) o[e] = fmaf(fmaf(f[e], rs, nur), gm[e], bt[e]);
       uint4 packed = Vec<DT>::pack(o);
       if (sv[r] == 0) packed = make_uint4(0, 0, 0, 0);
-      st_stream(yp + q * pass_stride, packed);
+      store_streaming(yp + q * pass_stride, packed);
     }
   }
 }
@@ -821,7 +812,7 @@ void tsn_bwd_kernel(const TsnParams p) {
     if (((live >> r) & 1) && col_ok) {
       const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
       xv[q] = *reinterpret_cast<const uint4*>(static_cast<const typename Elem<DT>::type*>(p.x) + off);
-      dv[q] = ld_once(static_cast<const typename Elem<DT>::type*>(p.dy) + off);
+      dv[q] = load_once(static_cast<const typename Elem<DT>::type*>(p.dy) + off);
     }
   }
   uint4 gmv = make_uint4(0, 0, 0, 0);
@@ -955,7 +946,7 @@ void tsn_bwd_kernel(const TsnParams p) {
         pb[e] += d[e];
       }
       const int64_t off = (static_cast<int64_t>(b) * p.L + t) * p.D + g * p.Dg + col * VEC;
-      st_stream(static_cast<typename Elem<DT>::type*>(p.y) + off, Vec<DT>::pack(o));
+      store_streaming(static_cast<typename Elem<DT>::type*>(p.y) + off, Vec<DT>::pack(o));
     }
   }
   // per-tile column sums of the gamma / beta gradients
