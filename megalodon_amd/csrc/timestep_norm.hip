@@ -218,15 +218,16 @@ __device__ __forceinline__ void stT(void* p, int64_t i, float v) {
   Elem<DT>::store(static_cast<typename Elem<DT>::type*>(p) + i, v);
 }
 
-// Hides a loaded vector from common-subexpression elimination: the unpacked
-// floats of an earlier phase are recomputed instead of being kept in registers.
-// Streamed accesses.  y (dx) is written once, in whole 128-byte lines, and read by another
+// Streamed accesses (store_streaming / load_once).  y (dx) is written once, in whole 128-byte lines, and read by another
 // kernel much later: stored with the non-temporal hint it does not displace what the kernel
 // still reads (config 2, forward 0.129 -> 0.104 ms, backward 0.193 -> 0.185 ms).  dy in the
 // backward is read once: loaded with the hint, 0.185 -> 0.175 ms.  x is left alone (with the
 // hint on its loads the forward is 0.114 ms, the backward 0.179 ms), and so are the statistics:
 // they leave four bytes per lane, and partial lines written with the hint are slow (forward
 // 0.167 ms).
+
+// Hides a loaded vector from common-subexpression elimination: the unpacked
+// floats of an earlier phase are recomputed instead of being kept in registers.
 __device__ __forceinline__ uint4 reload(uint4 v) {
   asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
   return v;
