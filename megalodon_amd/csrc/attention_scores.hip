@@ -399,7 +399,8 @@ __global__ __launch_bounds__(64 * kWaves) void attn_probs_kernel(const ProbsPara
     if (nb * kKeys < zend) {
       for (int rr = 0; rr < 32 && r0 + rr < p.L1; ++rr) {
         uint16_t* dst = p.w + (static_cast<int64_t>(z) * p.L1 + r0 + rr) * p.L2;
-        for (int c = nb * kKeys + lane * 8; c < zend; c += 64 * 8) *reinterpret_cast<u32x4*>(dst + c) = zero;
+        // whole lines, not read by this kernel: non-temporal (forward with full rows 1.312 -> 1.291 ms)
+        for (int c = nb * kKeys + lane * 8; c < zend; c += 64 * 8) __builtin_nontemporal_store(zero, reinterpret_cast<u32x4*>(dst + c));
       }
     }
   }
