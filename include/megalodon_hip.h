@@ -219,6 +219,23 @@ int mega_group_timestep_norm_fwd(const void* x, int dtype, const int64_t* prev_c
                                  float* cummean, float* cumrstd, void* workspace,
                                  void* stream);
 
+/* mega_group_timestep_norm_fwd / _bwd with the saved statistics time-last:
+ * cummean, cumrstd (B, G, L) instead of the reference's (B, L, G)
+ * (timestep_norm_kernel.cu:1553-1565 allocates them as {B, L, G}).  For a caller
+ * that hands them from the forward to the backward and nowhere else: a
+ * wavefront owns 64 steps of one group, so time-last it writes and reads 256
+ * contiguous bytes per array where the reference layout has it touch 64 lines
+ * for 4 bytes each.  Everything else as the two entry points without _tl
+ * (declared here for the forward, below for the backward). */
+int mega_group_timestep_norm_fwd_tl(const void* x, int dtype, const int64_t* prev_count,
+                                    const void* prev_mean, const void* prev_var,
+                                    const void* gamma, const void* beta,
+                                    const uint8_t* padding_mask, int64_t B, int64_t L,
+                                    int64_t D, int64_t G, double eps, void* y,
+                                    int64_t* count, void* mean, void* var,
+                                    float* cummean, float* cumrstd, void* workspace,
+                                    void* stream);
+
 /* The forward above for callers that cannot allocate (code under graph
  * capture, serving loops, harnesses that forbid it).  No counterpart in the
  * reference, whose operators allocate their own scratch (torch::empty in
@@ -255,6 +272,15 @@ int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, const void* 
                                  int64_t D, int64_t G, void* dx, void* dprev_mean,
                                  void* dprev_var, void* dgamma, void* dbeta,
                                  void* workspace, void* stream);
+/* the same with cummean, cumrstd (B, G, L), as mega_group_timestep_norm_fwd_tl writes them */
+int mega_group_timestep_norm_bwd_tl(const void* dy, const void* dmean, const void* dvar,
+                                    const void* x, int dtype, const void* prev_mean,
+                                    const int64_t* count, const float* cummean,
+                                    const float* cumrstd, const void* gamma,
+                                    const uint8_t* padding_mask, int64_t B, int64_t L,
+                                    int64_t D, int64_t G, void* dx, void* dprev_mean,
+                                    void* dprev_var, void* dgamma, void* dbeta,
+                                    void* workspace, void* stream);
 
 /* The double-precision flavour of the two operators above
  * (timestep_norm_kernel.cu:1567-1576 instantiates the reference's kernels for

@@ -71,8 +71,14 @@ struct TsnParams {
   long long spin_limit;    // polls of one record before a wait is given up
   int mute_tile;           // test hook: this tile index publishes nothing (-1: none)
   int B, L, D, G, Dg, NT;
+  // element strides of cummean / cumrstd: (B, L, G) as the reference stores them, or (B, G, L)
+  int64_t st_b, st_t, st_g;
   float eps;
 };
+
+__device__ __forceinline__ int64_t stat_index(const TsnParams& p, int b, int64_t t, int g) {
+  return b * p.st_b + t * p.st_t + g * p.st_g;
+}
 
 // A wait for another tile's record is bounded: tiles of a chain start in time
 // order, so in a healthy launch the record arrives within the predecessor's own
@@ -457,7 +463,7 @@ __global__ __launch_bounds__(kThreads) void tsn_fwd_kernel(const TsnParams p) {
     const Wel st = wel_merge(prefix, me);
     const float rstd = 1.f / sqrtf(st.v + p.eps);
     if (t < p.L) {
-      const int64_t o = (static_cast<int64_t>(b) * p.L + t) * p.G + g;
+      const int64_t o = stat_index(p, b, t, g);
       p.cummean[o] = st.u;
       p.cumrstd[o] = rstd;
     }
@@ -610,7 +616,7 @@ void tsn_fwd_wave_kernel(const TsnParams p, int tiles) {
   const Wel st = wel_merge(prefix, me);
   const float rstd = 1.f / sqrtf(st.v + p.eps);
   if (t < p.L) {
-    const int64_t o = (static_cast<int64_t>(b) * p.L + t) * p.G + g;
+    const int64_t o = stat_index(p, b, t, g);
     p.cummean[o] = st.u;
     p.cumrstd[o] = rstd;
   }
@@ -676,7 +682,7 @@ __global__ __launch_bounds__(kWave) void tsn_fwd_serial_kernel(const TsnParams p
     }
     const float rstd = 1.f / sqrtf(st.v + p.eps);
     if (lane == 0) {
-      const int64_t o = (static_cast<int64_t>(b) * p.L + t) * p.G + g;
+      const int64_t o = stat_index(p, b, t, g);
       p.cummean[o] = st.u;
       p.cumrstd[o] = rstd;
     }
@@ -822,7 +828,7 @@ void tsn_bwd_kernel(const TsnParams p) {
   const int64_t chain64 = static_cast<int64_t>(b) * p.G + g;
   // wave 0 only uses these; loading them in every wave keeps the code uniform
   const float before_u = t0 == 0 ? ldT<DT>(p.prev_mean, chain64)
-                                 : p.cummean_in[(static_cast<int64_t>(b) * p.L + t0 - 1) * p.G + g];
+                                 : p.cummean_in[stat_index(p, b, t0 - 1, g)];
   const State2 init{ldT<DT>(p.dmean, chain64), ldT<DT>(p.dvar, chain64)};
   const int* nb = p.nbefore + b * (p.NT + 1);
   const int64_t n0 = p.prev_count[b] - nb[p.NT];  // prior count
@@ -833,7 +839,7 @@ void tsn_bwd_kernel(const TsnParams p) {
     const int t = t0 + lane;
     if (wave == 0) {
       const bool in = t < p.L;
-      const int64_t o = (static_cast<int64_t>(b) * p.L + (in ? t : 0)) * p.G + g;
+      const int64_t o = stat_index(p, b, in ? t : 0, g);
       s_u[lane] = in ? p.cummean_in[o] : 0.f;
       s_r[lane] = in ? p.cumrstd_in[o] : 0.f;
       s_valid[lane] = (in && (p.mask == nullptr || p.mask[static_cast<int64_t>(b) * p.L + t] == 0)) ? 1 : 0;
@@ -999,9 +1005,9 @@ __global__ __launch_bounds__(kWave) void tsn_bwd_serial_kernel(const TsnParams p
       for (int i = lane; i < p.Dg; i += kWave) stT<DT>(p.y, row + i, 0.f);
       continue;
     }
-    const int64_t so = (static_cast<int64_t>(b) * p.L + t) * p.G + g;
+    const int64_t so = stat_index(p, b, t, g);
     const float u = p.cummean_in[so], r = p.cumrstd_in[so];
-    const float prev_u = t == 0 ? ldT<DT>(p.prev_mean, chain) : p.cummean_in[so - p.G];
+    const float prev_u = t == 0 ? ldT<DT>(p.prev_mean, chain) : p.cummean_in[so - p.st_t];
     const float c1 = static_cast<float>(m0 - 1) / static_cast<float>(m0);
     const float c2 = 1.f / static_cast<float>(m0);
     --m0;
@@ -1242,13 +1248,20 @@ static int check_dims(const char* who, int64_t B, int64_t L, int64_t D, int64_t 
   return MEGA_OK;
 }
 
-extern "C" int mega_group_timestep_norm_fwd(const void* x, int dtype, const int64_t* prev_count,
-                                            const void* prev_mean, const void* prev_var,
-                                            const void* gamma, const void* beta,
-                                            const uint8_t* padding_mask, int64_t B, int64_t L,
-                                            int64_t D, int64_t G, double eps, void* y,
-                                            int64_t* count, void* mean, void* var, float* cummean,
-                                            float* cumrstd, void* workspace, void* stream) {
+// time_last: cummean / cumrstd are (B, G, L) instead of the reference's (B, L, G)
+static void set_stat_strides(TsnParams& p, bool time_last) {
+  if (time_last) {
+    p.st_b = static_cast<int64_t>(p.G) * p.L; p.st_g = p.L; p.st_t = 1;
+  } else {
+    p.st_b = static_cast<int64_t>(p.L) * p.G; p.st_t = p.G; p.st_g = 1;
+  }
+}
+
+static int tsn_fwd_entry(bool time_last, const void* x, int dtype, const int64_t* prev_count,
+                         const void* prev_mean, const void* prev_var, const void* gamma, const void* beta,
+                         const uint8_t* padding_mask, int64_t B, int64_t L, int64_t D, int64_t G, double eps,
+                         void* y, int64_t* count, void* mean, void* var, float* cummean, float* cumrstd,
+                         void* workspace, void* stream) {
   MEGA_CHECK_ARG(valid_dtype(dtype), "mega_group_timestep_norm_fwd: bad dtype %d", dtype);
   int rc = check_dims("mega_group_timestep_norm_fwd", B, L, D, G);
   if (rc != MEGA_OK) return rc;
@@ -1262,6 +1275,7 @@ extern "C" int mega_group_timestep_norm_fwd(const void* x, int dtype, const int6
   p.var = var; p.cummean = cummean; p.cumrstd = cumrstd;
   p.B = (int)B; p.L = (int)L; p.D = (int)D; p.G = (int)G; p.Dg = (int)(D / G);
   p.NT = (int)((L + kTL - 1) / kTL); p.eps = (float)eps;
+  set_stat_strides(p, time_last);
   hipStream_t s = static_cast<hipStream_t>(stream);
   MEGA_CHECK_ARG(L >= 1, "mega_group_timestep_norm_fwd: empty sequence");
   switch (dtype) {
@@ -1271,14 +1285,33 @@ extern "C" int mega_group_timestep_norm_fwd(const void* x, int dtype, const int6
   }
 }
 
-extern "C" int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, const void* dvar,
-                                            const void* x, int dtype, const void* prev_mean,
-                                            const int64_t* count, const float* cummean,
-                                            const float* cumrstd, const void* gamma,
+extern "C" int mega_group_timestep_norm_fwd(const void* x, int dtype, const int64_t* prev_count,
+                                            const void* prev_mean, const void* prev_var,
+                                            const void* gamma, const void* beta,
                                             const uint8_t* padding_mask, int64_t B, int64_t L,
-                                            int64_t D, int64_t G, void* dx, void* dprev_mean,
-                                            void* dprev_var, void* dgamma, void* dbeta,
-                                            void* workspace, void* stream) {
+                                            int64_t D, int64_t G, double eps, void* y,
+                                            int64_t* count, void* mean, void* var, float* cummean,
+                                            float* cumrstd, void* workspace, void* stream) {
+  return tsn_fwd_entry(false, x, dtype, prev_count, prev_mean, prev_var, gamma, beta, padding_mask, B, L, D, G,
+                       eps, y, count, mean, var, cummean, cumrstd, workspace, stream);
+}
+
+extern "C" int mega_group_timestep_norm_fwd_tl(const void* x, int dtype, const int64_t* prev_count,
+                                               const void* prev_mean, const void* prev_var,
+                                               const void* gamma, const void* beta,
+                                               const uint8_t* padding_mask, int64_t B, int64_t L,
+                                               int64_t D, int64_t G, double eps, void* y,
+                                               int64_t* count, void* mean, void* var, float* cummean,
+                                               float* cumrstd, void* workspace, void* stream) {
+  return tsn_fwd_entry(true, x, dtype, prev_count, prev_mean, prev_var, gamma, beta, padding_mask, B, L, D, G,
+                       eps, y, count, mean, var, cummean, cumrstd, workspace, stream);
+}
+
+static int tsn_bwd_entry(bool time_last, const void* dy, const void* dmean, const void* dvar, const void* x,
+                         int dtype, const void* prev_mean, const int64_t* count, const float* cummean,
+                         const float* cumrstd, const void* gamma, const uint8_t* padding_mask, int64_t B,
+                         int64_t L, int64_t D, int64_t G, void* dx, void* dprev_mean, void* dprev_var,
+                         void* dgamma, void* dbeta, void* workspace, void* stream) {
   MEGA_CHECK_ARG(valid_dtype(dtype), "mega_group_timestep_norm_bwd: bad dtype %d", dtype);
   int rc = check_dims("mega_group_timestep_norm_bwd", B, L, D, G);
   if (rc != MEGA_OK) return rc;
@@ -1292,12 +1325,37 @@ extern "C" int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, c
   p.cumrstd_in = cumrstd; p.y = dx; p.mean = dprev_mean; p.var = dprev_var;
   p.B = (int)B; p.L = (int)L; p.D = (int)D; p.G = (int)G; p.Dg = (int)(D / G);
   p.NT = (int)((L + kTL - 1) / kTL);
+  set_stat_strides(p, time_last);
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
     case MEGA_F32: return tsn_bwd_impl<MEGA_F32>(p, dgamma, dbeta, workspace, s);
     case MEGA_BF16: return tsn_bwd_impl<MEGA_BF16>(p, dgamma, dbeta, workspace, s);
     default: return tsn_bwd_impl<MEGA_F16>(p, dgamma, dbeta, workspace, s);
   }
+}
+
+extern "C" int mega_group_timestep_norm_bwd(const void* dy, const void* dmean, const void* dvar,
+                                            const void* x, int dtype, const void* prev_mean,
+                                            const int64_t* count, const float* cummean,
+                                            const float* cumrstd, const void* gamma,
+                                            const uint8_t* padding_mask, int64_t B, int64_t L,
+                                            int64_t D, int64_t G, void* dx, void* dprev_mean,
+                                            void* dprev_var, void* dgamma, void* dbeta,
+                                            void* workspace, void* stream) {
+  return tsn_bwd_entry(false, dy, dmean, dvar, x, dtype, prev_mean, count, cummean, cumrstd, gamma, padding_mask,
+                       B, L, D, G, dx, dprev_mean, dprev_var, dgamma, dbeta, workspace, stream);
+}
+
+extern "C" int mega_group_timestep_norm_bwd_tl(const void* dy, const void* dmean, const void* dvar,
+                                               const void* x, int dtype, const void* prev_mean,
+                                               const int64_t* count, const float* cummean,
+                                               const float* cumrstd, const void* gamma,
+                                               const uint8_t* padding_mask, int64_t B, int64_t L,
+                                               int64_t D, int64_t G, void* dx, void* dprev_mean,
+                                               void* dprev_var, void* dgamma, void* dbeta,
+                                               void* workspace, void* stream) {
+  return tsn_bwd_entry(true, dy, dmean, dvar, x, dtype, prev_mean, count, cummean, cumrstd, gamma, padding_mask,
+                       B, L, D, G, dx, dprev_mean, dprev_var, dgamma, dbeta, workspace, stream);
 }
 
 // Test hook: look-back poll limit (<= 0 restores the default) and a tile index

@@ -845,11 +845,19 @@ def group_timestep_norm_fwd(
     padding_mask: Optional[torch.Tensor],
     num_groups: int,
     eps: float,
+    stats_time_last: bool = False,
 ):
     """(y, count, mean, var, cummean, cumrstd); tensors other than count /
     mask / the statistics must share x's dtype, as in the reference
     (timestep_norm_kernel.cu:1270-1273); cummean and cumrstd are float32, float64
-    for float64 x (the accumulate type, :1553-1565)."""
+    for float64 x (the accumulate type, :1553-1565).
+
+    `stats_time_last`: cummean and cumrstd come back as (B, G, L) instead of the
+    reference's (B, L, G) -- for a caller that hands them to
+    group_timestep_norm_bwd (with the same flag) and nowhere else, as the autograd
+    node of the module does: a wavefront owns 64 steps of one group, so in that
+    layout it writes and reads the statistics as whole lines (not available for
+    float64 x)."""
     dev = _require_cuda(x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask)
     if x.dim() != 3:
         raise RuntimeError("x must be (B, L, D)")
@@ -866,8 +874,11 @@ def group_timestep_norm_fwd(
     mean = torch.empty((B, G), dtype=x.dtype, device=dev)
     var = torch.empty((B, G), dtype=x.dtype, device=dev)
     stat_dtype = torch.float64 if x.dtype == torch.float64 else torch.float32
-    cummean = torch.empty((B, L, G), dtype=stat_dtype, device=dev)
-    cumrstd = torch.empty((B, L, G), dtype=stat_dtype, device=dev)
+    if stats_time_last and x.dtype == torch.float64:
+        raise RuntimeError("stats_time_last is not available for float64 x")
+    stat_shape = (B, G, L) if stats_time_last else (B, L, G)
+    cummean = torch.empty(stat_shape, dtype=stat_dtype, device=dev)
+    cumrstd = torch.empty(stat_shape, dtype=stat_dtype, device=dev)
     mask = _mask_bytes(padding_mask)
     if x.dtype == torch.float64:
         # the double-precision flavour: one wavefront per (batch, group) chain, no workspace
@@ -882,7 +893,8 @@ def group_timestep_norm_fwd(
         return y, count, mean, var, cummean, cumrstd
     ws = _tsn_workspace(B, L, D, G, False, dev)
     with torch.cuda.device(dev):
-        _lib.call("mega_group_timestep_norm_fwd", _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
+        _lib.call("mega_group_timestep_norm_fwd_tl" if stats_time_last else "mega_group_timestep_norm_fwd",
+                  _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
                   _lib.ptr(prev_count.contiguous()), _lib.ptr(prev_mean.contiguous()),
                   _lib.ptr(prev_var.contiguous()), _lib.ptr(gamma.contiguous()), _lib.ptr(beta.contiguous()),
                   _lib.ptr(mask), _lib.i64(B), _lib.i64(L), _lib.i64(D), _lib.i64(G), _lib.f64(eps),
@@ -903,11 +915,18 @@ def group_timestep_norm_bwd(
     gamma: torch.Tensor,
     padding_mask: Optional[torch.Tensor],
     num_groups: int,
+    stats_time_last: bool = False,
 ):
-    """(dx, dprev_mean, dprev_var, dgamma, dbeta)."""
+    """(dx, dprev_mean, dprev_var, dgamma, dbeta).  `stats_time_last`: cummean and
+    cumrstd are (B, G, L), as group_timestep_norm_fwd returns them under the same flag."""
     dev = _require_cuda(y_grad, mean_grad, var_grad, x, prev_mean, count, cummean, cumrstd, gamma, padding_mask)
     B, L, D = x.shape
     G = int(num_groups)
+    want = (B, G, L) if stats_time_last else (B, L, G)
+    if tuple(cummean.shape) != want or tuple(cumrstd.shape) != want:
+        raise RuntimeError(f"cummean / cumrstd must be {want} (got {tuple(cummean.shape)}, {tuple(cumrstd.shape)})")
+    if stats_time_last and x.dtype == torch.float64:
+        raise RuntimeError("stats_time_last is not available for float64 x")
     for name, t in (("y_grad", y_grad), ("mean_grad", mean_grad), ("var_grad", var_grad),
                     ("prev_mean", prev_mean), ("gamma", gamma)):
         if t.dtype != x.dtype:
@@ -933,7 +952,8 @@ def group_timestep_norm_bwd(
         return dx, dpm, dpv, dg, db
     ws = _tsn_workspace(B, L, D, G, True, dev)
     with torch.cuda.device(dev):
-        _lib.call("mega_group_timestep_norm_bwd", _lib.ptr(dy), _lib.ptr(mean_grad.contiguous()),
+        _lib.call("mega_group_timestep_norm_bwd_tl" if stats_time_last else "mega_group_timestep_norm_bwd",
+                  _lib.ptr(dy), _lib.ptr(mean_grad.contiguous()),
                   _lib.ptr(var_grad.contiguous()), _lib.ptr(xc), _lib.i32(_lib.dtype_code(x.dtype)),
                   _lib.ptr(prev_mean.contiguous()), _lib.ptr(count.contiguous()),
                   _lib.ptr(cummean.contiguous()), _lib.ptr(cumrstd.contiguous()), _lib.ptr(gamma.contiguous()),

@@ -16,18 +16,23 @@ from ..fused_ops._autograd import fused_op
 
 def _run(x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask=None, num_groups=None, eps=1e-5):
     groups = x.size(-1) if num_groups is None else num_groups
+    # cummean / cumrstd go to the backward and nowhere else, so they are kept time-last, (B, G, L):
+    # the kernels then write and read them as whole lines
+    time_last = x.dtype != torch.float64
     y, count, mean, var, cummean, cumrstd = ops.group_timestep_norm_fwd(
-        x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask, groups, eps)
-    return (y, count, mean, var), (x, prev_mean, count, cummean, cumrstd, gamma, padding_mask), groups
+        x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask, groups, eps, stats_time_last=time_last)
+    return (y, count, mean, var), (x, prev_mean, count, cummean, cumrstd, gamma, padding_mask), (groups, time_last)
 
 
-def _grad(groups, saved, y_grad, _count_grad, mean_grad, var_grad):
+def _grad(consts, saved, y_grad, _count_grad, mean_grad, var_grad):
+    groups, time_last = consts
     x, prev_mean, count, cummean, cumrstd, gamma, padding_mask = saved
     # an output nobody used arrives as None
     mean_grad = torch.zeros_like(prev_mean) if mean_grad is None else mean_grad
     var_grad = torch.zeros_like(prev_mean) if var_grad is None else var_grad
     dx, dprev_mean, dprev_var, dgamma, dbeta = ops.group_timestep_norm_bwd(
-        y_grad, mean_grad, var_grad, x, prev_mean, count, cummean, cumrstd, gamma, padding_mask, groups)
+        y_grad, mean_grad, var_grad, x, prev_mean, count, cummean, cumrstd, gamma, padding_mask, groups,
+        stats_time_last=time_last)
     #      x   count  prev_mean   prev_var   gamma   beta   mask  groups eps
     return dx, None, dprev_mean, dprev_var, dgamma, dbeta, None, None, None
 

@@ -39,12 +39,16 @@ def _cuda(*ts):
     return [None if t is None else t.cuda() for t in ts]
 
 
-def _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed, check_stats_everywhere=True):
+def _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed, check_stats_everywhere=True, time_last=False):
     x, pc, pm, pv, gamma, beta, m, dy, dmean, dvar = _case(B, L, H, G, seed, dtype, prior, mask)
     eps = 1e-5
     cx, cpc, cpm, cpv, cg, cb, cm = _cuda(x, pc, pm, pv, gamma, beta, m)
-    y, count, mean, var, cummean, cumrstd = ops.group_timestep_norm_fwd(cx, cpc, cpm, cpv, cg, cb, cm, G, eps)
+    y, count, mean, var, cummean, cumrstd = ops.group_timestep_norm_fwd(cx, cpc, cpm, cpv, cg, cb, cm, G, eps,
+                                                                        stats_time_last=time_last)
     wy, wcount, wmean, wvar, wcm, wcr = tn.group_timestep_norm_closed_form_full(x, pc, pm, pv, gamma, beta, m, G, eps)
+    if time_last:   # the saved statistics as (B, G, L)
+        assert cummean.shape == (B, G, L) and cumrstd.shape == (B, G, L)
+        wcm, wcr = wcm.transpose(1, 2), wcr.transpose(1, 2)
     tol = TOL[dtype]
     stat_dtype = torch.float64 if dtype == torch.float64 else torch.float32   # the accumulate type
     assert y.dtype == dtype and cummean.dtype == stat_dtype and count.dtype == torch.int64
@@ -54,7 +58,7 @@ def _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed, check_stats_everywhere=Tr
     assert rel_err(cummean, wcm) <= min(tol, 1e-4) and rel_err(cumrstd, wcr) <= min(tol, 1e-4)
     # backward consumes the statistics the forward saved
     dx, dpm, dpv, dg, db = ops.group_timestep_norm_bwd(dy.cuda(), dmean.cuda(), dvar.cuda(), cx, cpm, count,
-                                                       cummean, cumrstd, cg, cm, G)
+                                                       cummean, cumrstd, cg, cm, G, stats_time_last=time_last)
     want = tn.group_timestep_norm_bwd_autograd(dy, dmean, dvar, x, pc, pm, pv, gamma, beta, m, G, eps)
     for name, a, b_ in zip(["dx", "dprev_mean", "dprev_var", "dgamma", "dbeta"], (dx, dpm, dpv, dg, db), want):
         assert a.dtype == dtype
@@ -76,6 +80,27 @@ def _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed, check_stats_everywhere=Tr
 ])
 def test_fwd_bwd_match_oracle(B, L, H, G, prior, mask, dtype):
     _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed=B * 1000 + L)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,L,H,G,prior,mask", [
+    (2, 200, 512, 4, 3, "trailing"),   # tile-per-wave forward, ragged last tile
+    (3, 1000, 384, 3, 5, "holes"),
+    (2, 77, 1024, 2, 1, "trailing"),   # workgroup forward kernel (64 lanes per row)
+    (2, 50, 48, 48, 4, "holes"),       # serial kernels
+    (1, 1, 128, 1, 0, None),
+])
+def test_statistics_kept_time_last(B, L, H, G, prior, mask, dtype):
+    """`stats_time_last`: cummean / cumrstd travel from the forward to the backward as (B, G, L)
+    (what the module's autograd node uses); values, statistics and gradients against the oracle as
+    in the reference layout, and a layout the backward was not told about is refused."""
+    _run_fwd_bwd(B, L, H, G, dtype, prior, mask, seed=B * 1000 + L + 1, time_last=True)
+    if L != G:
+        x, pc, pm, pv, gamma, beta, m, dy, dmean, dvar = _case(B, L, H, G, 1, dtype, prior, mask)
+        cx, cpc, cpm, cpv, cg, cb, cm = _cuda(x, pc, pm, pv, gamma, beta, m)
+        _, count, _, _, cmn, crs = ops.group_timestep_norm_fwd(cx, cpc, cpm, cpv, cg, cb, cm, G, 1e-5, stats_time_last=True)
+        with pytest.raises(RuntimeError, match="cummean / cumrstd must be"):
+            ops.group_timestep_norm_bwd(dy.cuda(), dmean.cuda(), dvar.cuda(), cx, cpm, count, cmn, crs, cg, cm, G)
 
 
 @pytest.mark.parametrize("B,L,H,G,prior,mask", [

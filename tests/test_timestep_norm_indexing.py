@@ -25,7 +25,7 @@ def _fast_path_ok(D, Dg, vec):
     return Dg % vec == 0 and D % vec == 0 and Dg // vec <= 64
 
 
-def _emulate(B, L, D, G, vec, wave_kernel, backward):
+def _emulate(B, L, D, G, vec, wave_kernel, backward, time_last=False):
     Dg = D // G
     assert _fast_path_ok(D, Dg, vec)
     LPR = _lanes_per_row(Dg, vec)
@@ -34,6 +34,8 @@ def _emulate(B, L, D, G, vec, wave_kernel, backward):
     tiles = NC * NT
     written = np.zeros(B * L * D // vec, dtype=np.int32)     # 16-byte vectors of y / dx
     stats = np.zeros(B * L * G, dtype=np.int32)              # cummean / cumrstd slots
+    # element strides of the statistics: (B, L, G) as the reference stores them, or (B, G, L)
+    st_b, st_t, st_g = (G * L, 1, L) if time_last else (L * G, G, 1)
     rec_words = 3 if backward else 2
     n_rec = NC * NT * rec_words
     lane = np.arange(K_WAVE)
@@ -64,7 +66,7 @@ def _emulate(B, L, D, G, vec, wave_kernel, backward):
                 np.add.at(written, off[ok] // vec, 1)
         # wave 0, lane = time step: the saved statistics
         t = t0 + lane
-        o = (b * L + t[t < L]) * G + g
+        o = b * st_b + t[t < L] * st_t + g * st_g
         assert (o >= 0).all() and (o < B * L * G).all()
         np.add.at(stats, o, 1)
         # records: own slot, and the window of predecessors (forward) / successors (backward)
@@ -96,11 +98,13 @@ SHAPES = [
 
 
 @pytest.mark.parametrize("B,L,D,G,vec", SHAPES)
+@pytest.mark.parametrize("time_last", [False, True])
 @pytest.mark.parametrize("kernel", ["fwd_workgroup", "fwd_wave", "bwd_workgroup"])
-def test_tile_kernels_stay_inside_their_tensors(B, L, D, G, vec, kernel):
+def test_tile_kernels_stay_inside_their_tensors(B, L, D, G, vec, kernel, time_last):
     Dg = D // G
     if not _fast_path_ok(D, Dg, vec):
         pytest.skip("shape goes to the serial kernels")
     if kernel == "fwd_wave" and Dg // vec > 16:
         pytest.skip("the tile-per-wave kernel takes groups of at most 16 lanes")
-    _emulate(B, L, D, G, vec, wave_kernel=(kernel == "fwd_wave"), backward=(kernel == "bwd_workgroup"))
+    _emulate(B, L, D, G, vec, wave_kernel=(kernel == "fwd_wave"), backward=(kernel == "bwd_workgroup"),
+             time_last=time_last)
