@@ -23,7 +23,7 @@ import torch
 
 from conftest import rel_err
 from megalodon_amd import synthetic
-from megalodon_amd.modules import MegaBlock, MultiHeadComplexEMA
+from megalodon_amd.modules import MegaBlock, RotaryEmbedding, MultiHeadComplexEMA
 from oracle import block as oblock
 from oracle import cema as ocema
 from oracle import fftconv as offt
@@ -160,6 +160,48 @@ def test_config4_block_prefix_equals_small_run_equals_oracle():
     tight = lambda k: k in ("out", "dx") or ".cema." in k
     bad = {k: v for k, v in errs.items() if not v <= (2e-2 if tight(k) else 3e-2)}
     assert not bad, bad
+
+
+def test_config4_width_across_chunk_boundaries_against_oracle():
+    """The block at config 4's widths (model 4096, z 1024, values 8192, FFN 11008, 32 groups, 4 heads) with a
+    chunk of 512 and 1536 tokens -- three chunks -- and rotary angles by position in the
+    chunk: output, dx and every parameter gradient against the float64 oracle over the whole sequence, and the
+    output chunk by chunk and on the two tokens either side of each boundary."""
+    cfg = dict(CFG4, chunk_size=512)
+    L = 1536
+    torch.manual_seed(1005)
+    blk = MegaBlock(**cfg).cuda().bfloat16()
+    with torch.no_grad():
+        for n_, p_ in blk.named_parameters():
+            if n_.endswith(("timenorm.weight", "timenorm.bias", "rmsnorm.weight", "mega.gamma", "mega.beta",
+                            "norm.weight", "norm.bias", "wz.bias", "wv.bias", "wr.bias", "wh1.bias")):
+                p_.normal_(0, 0.1)
+    rope = RotaryEmbedding(cfg["z_dim"] // cfg["num_heads"], cfg["chunk_size"])
+    freqs = rope.get_freqs_cis(0, cfg["chunk_size"])
+    g = torch.Generator().manual_seed(1005)
+    x = (torch.rand(1, L, 4096, generator=g) * 2 - 1).bfloat16()
+    dy = torch.randn(1, L, 4096, generator=g).bfloat16()
+    xc = x.cuda().requires_grad_(True)
+    out, _ = blk(xc, freqs.cuda())
+    out.backward(dy.cuda())
+    print("config-4 widths, 1536 tokens in chunks of 512: float64 oracle running on the host ...", flush=True)
+    p64 = {n_: p_.detach().cpu().double().requires_grad_(True) for n_, p_ in blk.named_parameters()}
+    xo = x.double().requires_grad_(True)
+    want = oblock.mega_block_forward(p64, xo, num_heads=cfg["num_heads"], ndim=cfg["cema_ndim"],
+                                     chunk_size=cfg["chunk_size"], groups=cfg["norm_num_groups"], freqs_cis=freqs)
+    want.backward(dy.double())
+    errs = {"out": rel_err(out, want), "dx": rel_err(xc.grad, xo.grad)}
+    for n_, p_ in blk.named_parameters():
+        errs["d " + n_] = rel_err(p_.grad, p64[n_].grad)
+    print("errors vs float64 oracle:", {k: f"{v:.2e}" for k, v in errs.items()})
+    tight = lambda k: k in ("out", "dx") or ".cema." in k
+    bad = {k: v for k, v in errs.items() if not v <= (2e-2 if tight(k) else 3e-2)}
+    assert not bad, bad
+    C = cfg["chunk_size"]
+    for c in range(-(-L // C)):
+        assert rel_err(out[:, c * C:(c + 1) * C], want[:, c * C:(c + 1) * C]) <= 2e-2, c
+    for c in range(1, -(-L // C)):
+        assert rel_err(out[:, c * C - 1:c * C + 1], want[:, c * C - 1:c * C + 1]) <= 2e-2, c
 
 
 def test_config4_block_two_piece_cached_pass_equals_single_pass():
